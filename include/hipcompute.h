@@ -1,0 +1,259 @@
+/*
+ * libhipcompute -- gfx950 (MI355X) kernels for the quantized matrix-product
+ * operators, behind a plain C ABI.
+ *
+ * The library is the HIP sibling of the reference's `vk-compute` runtime plus
+ * the host functions of `onnx-vulkan-core` that sit on the quantized matmul
+ * path. Every entry point names the reference interface it stands in for
+ * (paths relative to the reference tree). Conventions shared by all calls:
+ *
+ *   - every function returns an int status: 0 ok, HIPC_ERR_* otherwise; the text
+ *     of the last failure on a context is `hipc_last_error(ctx)`
+ *     (the reference flattens every backend failure to `Error::Backend(String)`,
+ *     crates/onnx-vulkan-core/src/error.rs:6-13, interp.rs:892-894);
+ *   - tensor arguments are raw DEVICE pointers (a `hipc_alloc` result plus any
+ *     byte offset the caller likes -- the reference's `BufferSlice{buf,offset}`,
+ *     crates/vk-compute/src/pipeline.rs:12-21) in the ONNX layout of the operator;
+ *   - operator calls only ENQUEUE on the context's stream, in call order; the
+ *     host blocks only in `hipc_flush` and `hipc_download`
+ *     (crates/vk-compute/src/stream.rs:8-28, 370-383, 702);
+ *   - zero points of the integer operators are read ON THE DEVICE, never read
+ *     back (crates/onnx-vulkan-core/src/shaders/matmul_integer.rs:55-56);
+ *   - a context may be used from any thread; calls are serialised inside
+ *     (`submit_lock`, crates/vk-compute/src/stream.rs:77).
+ */
+#ifndef HIPCOMPUTE_H
+#define HIPCOMPUTE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPC_OK 0
+#define HIPC_ERR_INVALID 1     /* bad shape / short buffer / null pointer  (Error::InvalidShape, ::InvalidTensor) */
+#define HIPC_ERR_UNSUPPORTED 2 /* a form of the operator this library refuses (Error::Unsupported) */
+#define HIPC_ERR_BACKEND 3     /* a HIP call failed                        (Error::Backend) */
+
+/* element types, numbered as ONNX TensorProto.DataType (crates/onnx-vulkan-core/src/host_ops.rs) */
+#define HIPC_F32 1
+#define HIPC_U8 2
+#define HIPC_I8 3
+#define HIPC_I32 6
+#define HIPC_F16 10
+
+typedef struct hipc_ctx hipc_ctx;
+typedef struct hipc_graph hipc_graph;
+typedef struct hipc_nbits_weight hipc_nbits_weight; /* prepacked MatMulNBits weight */
+typedef struct hipc_int8_weight hipc_int8_weight;   /* prepacked MatMulInteger / QLinearMatMul B */
+typedef struct hipc_conv_weight hipc_conv_weight;   /* prepacked ConvInteger / QLinearConv W */
+
+/* ------------------------------------------------------------------ context */
+
+/* `VkContext::new` (crates/vk-compute/src/lib.rs:16-20; one per process in the
+ * plugin, crates/vulkan-ep/src/vk.rs:6-18). Creates one in-order stream at the
+ * default priority on `device`. */
+int hipc_ctx_create(int device, hipc_ctx **out);
+/* Same, but enqueue on a stream the caller owns (a `hipStream_t`, e.g. the one a
+ * host framework already uses), so work interleaves with the caller's in order. */
+int hipc_ctx_create_on_stream(int device, void *stream, hipc_ctx **out);
+void hipc_ctx_destroy(hipc_ctx *ctx);
+const char *hipc_last_error(hipc_ctx *ctx);
+const char *hipc_version(void);
+/* the `hipStream_t` operators are enqueued on */
+void *hipc_stream(hipc_ctx *ctx);
+
+/* ------------------------------------------------------------------ buffers */
+
+/* `create_storage_buffer` (crates/vk-compute/src/buffer.rs:239). 256-byte aligned. */
+int hipc_alloc(hipc_ctx *ctx, size_t bytes, void **dptr);
+/* `defer_destroy` (crates/vk-compute/src/stream.rs:691): the memory stays valid for
+ * everything already enqueued and is released at the next flush. */
+int hipc_free_deferred(hipc_ctx *ctx, void *dptr);
+/* `stream_upload_at` (stream.rs:310-321): `host` may be reused when the call returns. */
+int hipc_upload(hipc_ctx *ctx, void *dst, size_t dst_offset, const void *host, size_t bytes);
+/* `stream_download` (stream.rs:773-918): flushes, then copies to `host`. */
+int hipc_download(hipc_ctx *ctx, void *host, const void *src, size_t src_offset, size_t bytes);
+/* `stream_copy_range` (stream.rs:431) */
+int hipc_copy(hipc_ctx *ctx, void *dst, size_t dst_offset, const void *src, size_t src_offset, size_t bytes);
+/* `stream_fill` (stream.rs:481): `bytes` must be a multiple of 4; done by a fill kernel,
+ * so it may be recorded into a captured graph. */
+int hipc_fill(hipc_ctx *ctx, void *dst, size_t dst_offset, size_t bytes, uint32_t word);
+/* `flush` (stream.rs:702): the only host<->device synchronisation. */
+int hipc_flush(hipc_ctx *ctx);
+
+/* ------------------------------------------------------- capture and replay */
+
+/* `begin_capture` / `end_capture` / `replay` (crates/vk-compute/src/stream.rs:537-572):
+ * everything enqueued between begin and end is recorded instead of run, and
+ * `hipc_graph_launch` re-issues it. Buffers named while recording must stay alive
+ * and keep their addresses (the reference's preconditions, crates/onnx-vulkan-core/src/plan.rs:21-29). */
+int hipc_capture_begin(hipc_ctx *ctx);
+int hipc_capture_end(hipc_ctx *ctx, hipc_graph **out);
+int hipc_graph_launch(hipc_ctx *ctx, hipc_graph *graph);
+void hipc_graph_destroy(hipc_ctx *ctx, hipc_graph *graph);
+
+/* `measure_dispatch_gpu` (crates/vk-compute/src/pipeline.rs:246): time `samples`
+ * groups of `launches_per_sample` launches of a recorded graph with device
+ * events on the context's stream; writes nanoseconds PER LAUNCH to ns_out[samples]. */
+int hipc_measure_graph(hipc_ctx *ctx, hipc_graph *graph, int samples, int launches_per_sample, double *ns_out);
+
+/* -------------------------------------------------------------- MatMulNBits */
+
+/*
+ * `interp::matmul_nbits` (crates/onnx-vulkan-core/src/interp.rs:6429-6561) on the
+ * tensor format of shaders/matmul_nbits.rs:1-25:
+ *   A      [M, K]  f32 or f16 (a_dtype)
+ *   B      [N, n_blocks, block_size/2] u8, element 2i in the low nibble of byte i
+ *   scales [N * n_blocks]  f32 or f16 (scale_dtype)
+ *   zp     [N, ceil(n_blocks/2)] u8, packed like B; NULL => 8 for every block
+ *   Y      [M, N]  the dtype of A (crates/onnx-vulkan-frontend/src/shape.rs:497-512)
+ * bits is fixed at 4; block_size is a power of two >= 16; g_idx and bias are
+ * refused as in the reference (interp.rs:447-464). `accuracy_level` must be 0
+ * (unset) or 1..3: level 4 asks for int8 activations and is refused.
+ * Buffer lengths are in elements and are checked against K, N and block_size
+ * as the reference does (interp.rs:6455-6472); M*N == 0 is a no-op.
+ */
+int hipc_matmul_nbits(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, size_t b_len,
+                      const void *scales, int scale_dtype, size_t scales_len, const void *zp,
+                      size_t zp_len, void *Y, int64_t M, int64_t K, int64_t N, int64_t block_size,
+                      int accuracy_level);
+
+/* Repack a constant weight once (the role `packed_b` plays for MatMulInteger,
+ * interp.rs:2712-2768; the reference feeds MatMulNBits the ONNX layout directly).
+ * The operands are device pointers in the ONNX layout above and may be released
+ * after the next flush. */
+int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales,
+                              int scale_dtype, size_t scales_len, const void *zp, size_t zp_len,
+                              int64_t K, int64_t N, int64_t block_size, hipc_nbits_weight **out);
+void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w);
+/* bytes of device memory the prepacked form occupies */
+size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w);
+int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w,
+                             void *Y, int64_t M);
+
+/* ---------------------------------------------------- DynamicQuantizeLinear */
+
+/*
+ * `interp::dynamic_quantize` + `quantize_on_device` (interp.rs:1945-2085),
+ * arithmetic of shaders/dynamic_quantize.rs:106-222:
+ *   X [n] f32 -> Y [n] u8, scale (one f32, device), zero point (one u8, device).
+ * n == 0 writes scale 1 and zero point 0 (interp.rs:1949-1966).
+ * `range` is an 8-byte device slot {bits(-min), bits(max)}; NULL lets the call use
+ * the context's own. When `range_ready` != 0 the slot already holds the range of X
+ * (a producer folded it, `computed_range`) and the min/max pass is skipped.
+ */
+int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out,
+                                 void *zp_out, void *range, int range_ready);
+
+/* ------------------------------------------------------------ MatMulInteger */
+
+/* `packed_b` + `flipped_const` (interp.rs:2673-2768; shaders/matmul_integer.rs:135-158):
+ * B [K, N] u8 / i8 (b_dtype) -> the layout the GEMM reads, plus per-column sums
+ * for the zero-point correction. */
+int hipc_prepack_int8_b(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, int64_t N,
+                        hipc_int8_weight **out);
+void hipc_int8_weight_destroy(hipc_ctx *ctx, hipc_int8_weight *w);
+
+/*
+ * `interp::matmul_integer` (interp.rs:2090-2183), definition host_ops.rs:1157-1199:
+ *   Y [M, N] i32 = sum_k (A[m,k] - a_zp) * (B[k,n] - b_zp)
+ * A [M, K] u8 / i8 (a_dtype); a_zp / b_zp are device pointers to ONE byte of the
+ * operand's dtype, or NULL for 0. Any K (the reference needs a second kernel
+ * for K % 4 != 0, interp.rs:2193). K <= 33025 so the i32 sum cannot overflow
+ * (interp.rs:2216-2218) is NOT required here: sums wrap as the reference's.
+ */
+int hipc_matmul_integer(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_int8_weight *B,
+                        const void *a_zp, const void *b_zp, void *Y, int64_t M);
+/* The same with B in the ONNX layout [K, N]; packs into scratch on every call. */
+int hipc_matmul_integer_raw(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, int b_dtype,
+                            const void *a_zp, const void *b_zp, void *Y, int64_t M, int64_t K, int64_t N);
+
+/*
+ * `matmul_integer_scale_bias` (interp.rs:2405-2572; epilogue rounding
+ * shaders/glsl/matmul_integer_coop.comp:39-60): the fused
+ * MatMulInteger -> Cast -> Mul(scale) -> Add(bias) [-> Relu]:
+ *   Y [M, N] f32 = fadd(fmul(float(acc), s[n]), bias[n]),  s[n] = scale[n*scale_step] (* product[n*product_step])
+ * two roundings, no fused multiply-add. scale / product / bias are DEVICE f32
+ * pointers; *_step is 0 (scalar) or 1 (per column); product and bias may be NULL.
+ * With `range` != NULL the output's {bits(-min), bits(max)} are folded into that
+ * 8-byte slot (which the caller cleared), ready for a following
+ * hipc_dynamic_quantize_linear(range_ready = 1).
+ */
+int hipc_matmul_integer_scale_bias(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_int8_weight *B,
+                                   const void *a_zp, const void *b_zp, const void *scale, int scale_step,
+                                   const void *product, int product_step, const void *bias, int bias_step,
+                                   int relu, void *range, void *Y, int64_t M);
+
+/* ------------------------------------------------ Requantize / QLinearMatMul */
+
+/*
+ * `requantize` (interp.rs:4714-4788; shaders/qlinear.rs:28-63):
+ *   c = (i / inner) % axis_len
+ *   out[i] = sat(int32(rte(float(acc[i] + bias[c]) * ratio[c])) + y_zp)   as u8 / i8 (out_dtype)
+ * ratio [axis_len] f32 and bias [axis_len] i32 (or NULL) are device pointers.
+ */
+int hipc_requantize(hipc_ctx *ctx, const void *acc, const void *bias, const void *ratio, int64_t n,
+                    int64_t inner, int64_t axis_len, int32_t y_zp, int out_dtype, void *out);
+
+/*
+ * `qlinear_matmul` (interp.rs:4845-4875) within the envelope of
+ * `unsupported_quantization` (interp.rs:781-847): per-tensor activation and
+ * output quantisation given as HOST constants; weight scale per tensor or per
+ * column (n_b_scale == 1 or N), per-column weights must have zero point 0.
+ * ratio[c] = a_scale * b_scale[c] / y_scale in f32, left to right (interp.rs:4693).
+ * `b_scale` is a HOST array.
+ */
+int hipc_qlinear_matmul(hipc_ctx *ctx, const void *A, int a_dtype, float a_scale, int32_t a_zp,
+                        const hipc_int8_weight *B, const float *b_scale, int64_t n_b_scale, int32_t b_zp,
+                        float y_scale, int32_t y_zp, int y_dtype, void *Y, int64_t M);
+
+/* ------------------------------------------------- ConvInteger / QLinearConv */
+
+/* `ConvGeom` (interp.rs:3361-3536): NCHW, 1-D given as H = 1. */
+typedef struct {
+    int64_t n, c_in, h, w;
+    int64_t c_out, kh, kw;
+    int64_t stride_h, stride_w, dil_h, dil_w;
+    int64_t pad_top, pad_left, pad_bottom, pad_right;
+    int64_t group;
+} hipc_conv_geom;
+
+/* output extents of a geometry; HIPC_ERR_INVALID if the window does not fit */
+int hipc_conv_out_shape(const hipc_conv_geom *g, int64_t *h_out, int64_t *w_out);
+/* `same_pads` (interp.rs:3427-3436): auto_pad SAME_UPPER (upper != 0) / SAME_LOWER for one axis */
+void hipc_same_pads(int64_t in, int64_t kernel, int64_t stride, int64_t dilation, int upper,
+                    int64_t *pad_begin, int64_t *pad_end);
+
+/* `hwc_weight` (interp.rs:5719-5748): W [c_out, c_in/group, kh, kw] u8 / i8 -> the
+ * layout the implicit-GEMM kernel reads (K ordered (kh, kw, c)). */
+int hipc_prepack_conv_w(hipc_ctx *ctx, const void *W, int w_dtype, const hipc_conv_geom *g,
+                        hipc_conv_weight **out);
+void hipc_conv_weight_destroy(hipc_ctx *ctx, hipc_conv_weight *w);
+
+/*
+ * `conv_integer_with` (interp.rs:4421-4651), definition tests/conv_integer_im2col.rs:58-89:
+ *   Y [n, c_out, h_out, w_out] i32; out-of-bounds taps contribute 0.
+ * x_zp / w_zp are device pointers to one byte, or NULL for 0.
+ */
+int hipc_conv_integer(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *W,
+                      const void *x_zp, const void *w_zp, const hipc_conv_geom *g, void *Y);
+
+/*
+ * `qlinear_conv` (interp.rs:4796-4837): ConvInteger, then Requantize with
+ * ratio[c] = x_scale * w_scale[c] / y_scale; a per-tensor w_scale (n_w_scale == 1)
+ * is broadcast to c_out so `bias` [c_out] i32 (device, may be NULL) stays per channel.
+ * Scales and zero points are HOST constants; per-channel weights need w_zp == 0
+ * (interp.rs:830-835). Y is u8 / i8 (y_dtype).
+ */
+int hipc_qlinear_conv(hipc_ctx *ctx, const void *X, int x_dtype, float x_scale, int32_t x_zp,
+                      const hipc_conv_weight *W, const float *w_scale, int64_t n_w_scale, int32_t w_zp,
+                      float y_scale, int32_t y_zp, int y_dtype, const void *bias,
+                      const hipc_conv_geom *g, void *Y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

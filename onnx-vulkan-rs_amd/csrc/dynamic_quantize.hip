@@ -1,0 +1,145 @@
+// DynamicQuantizeLinear for gfx950.
+//
+// Reference: crates/onnx-vulkan-core/src/shaders/dynamic_quantize.rs:106-222 (the two
+// passes and the range slot), interp.rs:1945-2085 (host side), definition
+// tests/dynamic_quantize.rs:16-26.
+//
+// The range slot is 8 bytes {bits(-min), bits(max)}. The range always contains 0,
+// so both values are >= 0 and their bit patterns order like the values: an
+// unsigned atomicMax on the words is a float max, independent of the order the
+// workgroups arrive in. The reference replaces `/` by a double-single reciprocal
+// because Vulkan's OpFDiv may be 2.5 ULP off; here `__fdiv_rn` is the IEEE
+// division, so the operator's definition is evaluated as written.
+#include "internal.h"
+
+namespace hipc {
+
+__global__ void dql_clear_range_kernel(uint32_t *range) {
+    if (threadIdx.x < 2) range[threadIdx.x] = 0u;
+}
+
+__global__ void __launch_bounds__(256)
+dql_range_kernel(const float *__restrict__ x, long n, uint32_t *__restrict__ range, int vec_ok) {
+    float mn = 0.f, mx = 0.f;
+    const long tid = (long)blockIdx.x * 256 + threadIdx.x;
+    const long nthreads = (long)gridDim.x * 256;
+    if (vec_ok) {
+        const long n4 = n >> 2;
+        const float4 *x4 = reinterpret_cast<const float4 *>(x);
+        for (long i = tid; i < n4; i += nthreads) {
+            const float4 v = x4[i];
+            mn = fminf(mn, fminf(fminf(v.x, v.y), fminf(v.z, v.w)));
+            mx = fmaxf(mx, fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
+        }
+        for (long i = (n4 << 2) + tid; i < n; i += nthreads) {
+            mn = fminf(mn, x[i]);
+            mx = fmaxf(mx, x[i]);
+        }
+    } else {
+        for (long i = tid; i < n; i += nthreads) {
+            mn = fminf(mn, x[i]);
+            mx = fmaxf(mx, x[i]);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        mn = fminf(mn, __shfl_xor(mn, off, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    }
+    __shared__ float smn[4], smx[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) smn[wave] = mn, smx[wave] = mx;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        mn = fminf(fminf(smn[0], smn[1]), fminf(smn[2], smn[3]));
+        mx = fmaxf(fmaxf(smx[0], smx[1]), fmaxf(smx[2], smx[3]));
+        // -0.0 counts as 0: drop the sign bit
+        atomicMax(&range[0], __float_as_uint(-mn) & 0x7fffffffu);
+        atomicMax(&range[1], __float_as_uint(mx) & 0x7fffffffu);
+    }
+}
+
+__device__ __forceinline__ void dql_params(const uint32_t *range, float &scale, float &zp) {
+    const float neg_min = __uint_as_float(range[0]);
+    const float mx = __uint_as_float(range[1]);
+    // max - min with min = -neg_min; max == min only when both are 0
+    const float span = __fadd_rn(mx, neg_min);
+    scale = span == 0.f ? 1.f : __fdiv_rn(span, 255.f);
+    zp = rintf(fminf(fmaxf(__fdiv_rn(neg_min, scale), 0.f), 255.f));
+}
+
+__device__ __forceinline__ uint32_t dql_one(float v, float scale, float zp) {
+    const float q = __fadd_rn(rintf(__fdiv_rn(v, scale)), zp);
+    return (uint32_t)fminf(fmaxf(q, 0.f), 255.f);
+}
+
+// four values per thread, packed into one 32-bit store where the output allows it
+__global__ void __launch_bounds__(256)
+dql_quantize_kernel(const float *__restrict__ x, long n, const uint32_t *__restrict__ range,
+                    uint8_t *__restrict__ y, float *__restrict__ scale_out, uint8_t *__restrict__ zp_out, int vec_ok) {
+    float scale, zp;
+    dql_params(range, scale, zp);
+    const long i4 = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i4 == 0) {
+        *scale_out = scale;
+        *zp_out = (uint8_t)zp;
+    }
+    const long base = i4 << 2;
+    if (base >= n) return;
+    if (vec_ok && base + 4 <= n) {
+        const float4 v = reinterpret_cast<const float4 *>(x)[i4];
+        const uint32_t packed = dql_one(v.x, scale, zp) | dql_one(v.y, scale, zp) << 8 |
+                                dql_one(v.z, scale, zp) << 16 | dql_one(v.w, scale, zp) << 24;
+        reinterpret_cast<uint32_t *>(y)[i4] = packed;
+    } else {
+        for (long i = base; i < n && i < base + 4; i++) y[i] = (uint8_t)dql_one(x[i], scale, zp);
+    }
+}
+
+__global__ void dql_empty_kernel(float *scale_out, uint8_t *zp_out) {
+    if (threadIdx.x == 0) {
+        *scale_out = 1.f;
+        *zp_out = 0;
+    }
+}
+
+}  // namespace hipc
+
+using namespace hipc;
+
+extern "C" int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out,
+                                            void *zp_out, void *range, int range_ready) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, n >= 0, "DynamicQuantizeLinear: negative length");
+    HIPC_REQUIRE(ctx, scale_out && zp_out, "DynamicQuantizeLinear: null scale or zero-point output");
+    HIPC_REQUIRE(ctx, aligned(scale_out, 4), "DynamicQuantizeLinear: scale output must be 4-byte aligned");
+    if (n == 0) {  // empty input: y empty, scale 1, zero point 0 (interp.rs:1949-1966)
+        dql_empty_kernel<<<1, 64, 0, ctx->stream>>>(static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out));
+        HIPC_LAUNCHED(ctx);
+        return HIPC_OK;
+    }
+    HIPC_REQUIRE(ctx, X && Y, "DynamicQuantizeLinear: null tensor");
+    HIPC_REQUIRE(ctx, aligned(X, 4), "DynamicQuantizeLinear: input must be 4-byte aligned");
+    uint32_t *slot = static_cast<uint32_t *>(range ? range : static_cast<void *>(static_cast<char *>(ctx->params) + kParamRange));
+    HIPC_REQUIRE(ctx, aligned(slot, 4), "DynamicQuantizeLinear: range slot must be 4-byte aligned");
+    HIPC_REQUIRE(ctx, !(range_ready && !range), "DynamicQuantizeLinear: range_ready needs a caller-owned range slot");
+    const int vec_ok = aligned(X, 16) && aligned(Y, 4);
+    const float *x = static_cast<const float *>(X);
+    if (!range_ready) {
+        dql_clear_range_kernel<<<1, 64, 0, ctx->stream>>>(slot);
+        HIPC_LAUNCHED(ctx);
+        // enough workgroups to pull from every HBM channel, few enough that the atomics are noise
+        const long want = ceil_div(n, 256 * 16);
+        const unsigned grid = (unsigned)std::min<long>(std::max<long>(want, 1), 8L * ctx->cu_count);
+        dql_range_kernel<<<grid, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok);
+        HIPC_LAUNCHED(ctx);
+    }
+    const long quads = ceil_div(n, 4);
+    HIPC_REQUIRE(ctx, ceil_div(quads, 256) < (int64_t(1) << 31), "DynamicQuantizeLinear: tensor too large");
+    dql_quantize_kernel<<<(unsigned)ceil_div(quads, 256), 256, 0, ctx->stream>>>(
+        x, (long)n, slot, static_cast<uint8_t *>(Y), static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out),
+        vec_ok);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}

@@ -1,0 +1,280 @@
+// The int8 MFMA contraction shared by MatMulInteger / QLinearMatMul and
+// ConvInteger / QLinearConv:
+//
+//     C[i][j] = sum_k P[i][k] * Q[j][k]          (both operands k-contiguous, signed bytes)
+//
+// One 256-thread workgroup owns a 128x128 tile of C; its four wavefronts own
+// 64x64 each as 2x2 v_mfma_i32_32x32x32_i8 accumulators. Each k stage moves a
+// 128x64-byte slab of P and of Q through LDS with 128-bit accesses (row pitch
+// 80 bytes, conflict-free for ds_read_b128), the next slab's global loads
+// being in flight while the current one is multiplied.
+//
+// gfx950's int8 MFMA is signed x signed, so uint8 operands are shifted by 128
+// (x ^ 0x80), their zero points with them -- the identity the reference uses
+// the other way round (crates/onnx-vulkan-core/src/shaders/matmul_integer.rs:11-24) --
+// and the zero points leave in the epilogue
+// (shaders/glsl/matmul_integer_coop.comp:22-31):
+//     sum (p-zp)(q-zq) = sum p*q - zq*sum_k p - zp*sum_k q + K*zp*zq
+// The constant operand's sums come from prepacking; the dynamic operand's are
+// taken from its MFMA operand registers with v_dot4 only when the other zero
+// point is not 0.
+#pragma once
+
+#include "internal.h"
+
+namespace hipc {
+
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+
+constexpr int kBM = 128, kBN = 128, kBK = 64, kPitch = kBK + 16;
+
+enum { EPI_I32 = 0, EPI_SCALE_BIAS = 1, EPI_REQUANT = 2 };
+enum { MODE_MM = 0, MODE_CONV = 1 };
+
+struct GemmArgs {
+    // P operand: MODE_MM  -> the activation matrix A [I, K] (u8 / i8, pitch K)
+    //            MODE_CONV -> prepacked weight [I_pad, K_pad] signed
+    const uint8_t *P;
+    // Q operand: MODE_MM  -> prepacked B [J_pad, K_pad] signed
+    //            MODE_CONV -> NHWC activations, already signed
+    const uint8_t *Q;
+    const int32_t *const_sum;  // sums over k of the prepacked operand (per j in MM, per i in CONV)
+    const uint8_t *dyn_zp;     // device zero point of the dynamic operand (may be null)
+    const uint8_t *const_zp;   // device zero point of the prepacked operand (may be null)
+    int dyn_shift, const_shift;    // 128 when that operand is uint8, else 0
+    int dyn_signed, const_signed;  // how to read the zero-point byte
+    int host_zp;                   // zero points given by value instead of by pointer
+    int dyn_zp_value, const_zp_value;
+    int I, J, K, K_pad;
+    int p_aligned;  // MODE_MM: rows of A can be read with 128-bit loads
+
+    // conv geometry (MODE_CONV); Q is [n][H][W][C]
+    int C, H, W, Ho, Wo, kh, kw, sh, sw, dh, dw, pt, pl;
+
+    // epilogue
+    void *Y;
+    const float *scale, *product, *bias;   // EPI_SCALE_BIAS (per j)
+    int scale_step, product_step, bias_step, relu;
+    uint32_t *range;
+    const float *ratio;                    // EPI_REQUANT: per j in MM, per i in CONV
+    int ratio_step;
+    const int32_t *qbias;                  // EPI_REQUANT int32 bias (per i in CONV)
+    int y_zp, out_signed;
+};
+
+__device__ __forceinline__ int zp_byte(const uint8_t *ptr, int is_signed) {
+    if (!ptr) return 0;
+    const uint8_t v = *ptr;
+    return is_signed ? (int)(int8_t)v : (int)v;
+}
+
+__device__ __forceinline__ uint4 xor4(uint4 v, uint32_t m) { return make_uint4(v.x ^ m, v.y ^ m, v.z ^ m, v.w ^ m); }
+
+__device__ __forceinline__ int dot_ones(uint4 v) {
+    int s = __builtin_amdgcn_sdot4((int)v.x, 0x01010101, 0, false);
+    s = __builtin_amdgcn_sdot4((int)v.y, 0x01010101, s, false);
+    s = __builtin_amdgcn_sdot4((int)v.z, 0x01010101, s, false);
+    return __builtin_amdgcn_sdot4((int)v.w, 0x01010101, s, false);
+}
+
+template <int MODE, int EPI>
+__global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_p[2][kBM * kPitch];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_q[2][kBN * kPitch];
+    __shared__ int lds_sum[4][64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r32 = lane & 31, kg = lane >> 5;
+    const int i0 = blockIdx.y * kBM, j0 = blockIdx.x * kBN;
+    const int img = blockIdx.z;
+
+    // zero points in the shifted (signed) domain
+    const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
+    const int zc = (p.host_zp ? p.const_zp_value : zp_byte(p.const_zp, p.const_signed)) - p.const_shift;
+    const bool need_dyn_sum = zc != 0;
+    const uint32_t flip = p.dyn_shift ? 0x80808080u : 0u;
+    const uint32_t pad_word = (uint32_t)(zd & 0xff) * 0x01010101u;
+
+    // the two 16-byte chunks of each operand slab this thread moves
+    int row_[2], kc_[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int c = tid + 256 * u;
+        row_[u] = c >> 2;
+        kc_[u] = c & 3;
+    }
+    // MODE_CONV: where this thread's two positions sit in the input
+    int base_h[2] = {0, 0}, base_w[2] = {0, 0};
+    bool pos_ok[2] = {false, false};
+    const uint8_t *q_img = p.Q;
+    if (MODE == MODE_CONV) {
+        q_img = p.Q + (size_t)img * p.H * p.W * p.C;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int gj = j0 + row_[u];
+            pos_ok[u] = gj < p.J;
+            const int oh = gj / p.Wo, ow = gj - oh * p.Wo;
+            base_h[u] = oh * p.sh - p.pt;
+            base_w[u] = ow * p.sw - p.pl;
+        }
+    }
+
+    auto load_p = [&](int u, int k0) -> uint4 {
+        const int gi = i0 + row_[u], gk = k0 + kc_[u] * 16;
+        if (MODE == MODE_CONV) {
+            return *reinterpret_cast<const uint4 *>(p.P + (size_t)gi * p.K_pad + gk);
+        } else {
+            if (gi >= p.I || gk >= p.K) return make_uint4(0, 0, 0, 0);
+            const uint8_t *src = p.P + (size_t)gi * p.K + gk;
+            if (p.p_aligned) return xor4(*reinterpret_cast<const uint4 *>(src), flip);
+            uint32_t w[4] = {0, 0, 0, 0};
+            for (int b = 0; b < 16; b++)
+                if (gk + b < p.K) w[b >> 2] |= (uint32_t)(src[b] ^ (flip & 0xff)) << (8 * (b & 3));
+            return make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    };
+    auto load_q = [&](int u, int k0) -> uint4 {
+        const int gk = k0 + kc_[u] * 16;
+        if (MODE == MODE_MM) {
+            const int gj = j0 + row_[u];
+            return *reinterpret_cast<const uint4 *>(p.Q + (size_t)gj * p.K_pad + gk);
+        } else {
+            if (!pos_ok[u] || gk >= p.K) return make_uint4(0, 0, 0, 0);
+            const int tap = gk / p.C, c0 = gk - tap * p.C;
+            const int r = tap / p.kw, s = tap - r * p.kw;
+            const int ih = base_h[u] + r * p.dh, iw = base_w[u] + s * p.dw;
+            if (ih < 0 || ih >= p.H || iw < 0 || iw >= p.W) return make_uint4(pad_word, pad_word, pad_word, pad_word);
+            return *reinterpret_cast<const uint4 *>(q_img + ((size_t)ih * p.W + iw) * p.C + c0);
+        }
+    };
+
+    i32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    int dsum[2] = {0, 0};
+
+    const int nk = p.K_pad / kBK;
+    uint4 rp[2], rq[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) rp[u] = load_p(u, 0), rq[u] = load_q(u, 0);
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        *reinterpret_cast<uint4 *>(&lds_p[0][row_[u] * kPitch + kc_[u] * 16]) = rp[u];
+        *reinterpret_cast<uint4 *>(&lds_q[0][row_[u] * kPitch + kc_[u] * 16]) = rq[u];
+    }
+    __syncthreads();
+
+    for (int ks = 0; ks < nk; ks++) {
+        const int buf = ks & 1;
+        const bool more = ks + 1 < nk;
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) rp[u] = load_p(u, (ks + 1) * kBK), rq[u] = load_q(u, (ks + 1) * kBK);
+        }
+#pragma unroll
+        for (int step = 0; step < kBK / 32; step++) {
+            uint4 pf[2], qf[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                pf[i] = *reinterpret_cast<const uint4 *>(
+                    &lds_p[buf][(wm * 64 + i * 32 + r32) * kPitch + step * 32 + kg * 16]);
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                qf[j] = *reinterpret_cast<const uint4 *>(
+                    &lds_q[buf][(wn * 64 + j * 32 + r32) * kPitch + step * 32 + kg * 16]);
+            if (need_dyn_sum) {
+#pragma unroll
+                for (int f = 0; f < 2; f++) dsum[f] += dot_ones(MODE == MODE_MM ? pf[f] : qf[f]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, pf[i]),
+                                                                      __builtin_bit_cast(i32x4, qf[j]), acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                *reinterpret_cast<uint4 *>(&lds_p[buf ^ 1][row_[u] * kPitch + kc_[u] * 16]) = rp[u];
+                *reinterpret_cast<uint4 *>(&lds_q[buf ^ 1][row_[u] * kPitch + kc_[u] * 16]) = rq[u];
+            }
+        }
+        __syncthreads();
+    }
+
+    // sums of the dynamic operand over k: the two k halves of a row live in lanes l and l+32
+    if (need_dyn_sum) {
+#pragma unroll
+        for (int f = 0; f < 2; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
+        if (MODE == MODE_MM) {
+            if (kg == 0) lds_sum[wave][r32] = dsum[0], lds_sum[wave][32 + r32] = dsum[1];
+        }
+    }
+    __syncthreads();
+
+    const int kzz = p.K * zd * zc;
+    float fmn = 0.f, fmx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int gj = j0 + wn * 64 + j * 32 + r32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);  // row inside the 32x32 fragment
+                const int gi = i0 + wm * 64 + i * 32 + rf;
+                if (gi >= p.I || gj >= p.J) continue;
+                int v = acc[i][j][r];
+                const int csum = p.const_sum[MODE == MODE_MM ? gj : gi];
+                v = v - zd * csum + kzz;
+                if (need_dyn_sum) v -= zc * (MODE == MODE_MM ? lds_sum[wave][i * 32 + rf] : dsum[j]);
+                const size_t at = MODE == MODE_MM ? (size_t)gi * p.J + gj : ((size_t)img * p.I + gi) * p.J + gj;
+                if (EPI == EPI_I32) {
+                    static_cast<int32_t *>(p.Y)[at] = v;
+                } else if (EPI == EPI_SCALE_BIAS) {
+                    float s = p.scale[(size_t)gj * p.scale_step];
+                    if (p.product) s = __fmul_rn(s, p.product[(size_t)gj * p.product_step]);
+                    float o = __fmul_rn((float)v, s);
+                    if (p.bias) o = __fadd_rn(o, p.bias[(size_t)gj * p.bias_step]);
+                    if (p.relu) o = o > 0.f ? o : 0.f;
+                    static_cast<float *>(p.Y)[at] = o;
+                    fmn = fminf(fmn, o);
+                    fmx = fmaxf(fmx, o);
+                } else {
+                    const int c = MODE == MODE_MM ? gj : gi;
+                    if (p.qbias) v += p.qbias[c];
+                    const float t = __fmul_rn((float)v, p.ratio[(size_t)c * p.ratio_step]);
+                    int q = (int)rintf(t) + p.y_zp;
+                    if (p.out_signed) {
+                        q = min(max(q, -128), 127);
+                        static_cast<int8_t *>(p.Y)[at] = (int8_t)q;
+                    } else {
+                        q = min(max(q, 0), 255);
+                        static_cast<uint8_t *>(p.Y)[at] = (uint8_t)q;
+                    }
+                }
+            }
+        }
+    }
+    if (EPI == EPI_SCALE_BIAS && p.range) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            fmn = fminf(fmn, __shfl_xor(fmn, off, 64));
+            fmx = fmaxf(fmx, __shfl_xor(fmx, off, 64));
+        }
+        if (lane == 0) {
+            atomicMax(&p.range[0], __float_as_uint(-fmn) & 0x7fffffffu);
+            atomicMax(&p.range[1], __float_as_uint(fmx) & 0x7fffffffu);
+        }
+    }
+}
+
+}  // namespace hipc

@@ -1,0 +1,100 @@
+// Shared internals of libhipcompute: the context object, status plumbing and
+// launch helpers. Nothing here is part of the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/hipcompute.h"
+
+namespace hipc {
+
+constexpr int kScratchSlots = 4;
+
+// grow-only device scratch reused by operators that need a temporary (packed
+// B of a raw call, the i32 accumulator of a QLinear op). One in-order stream
+// makes sequential reuse safe: the next user starts after the previous one ended.
+struct Scratch {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+
+}  // namespace hipc
+
+struct hipc_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool owns_stream = false;
+    bool capturing = false;
+    std::mutex mu;
+    std::string err;
+    std::vector<void *> deferred;        // released at the next flush
+    hipc::Scratch scratch[hipc::kScratchSlots];
+    void *params = nullptr;              // small device block: range slot + scalars (256 B)
+    int cu_count = 256;
+};
+
+struct hipc_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+namespace hipc {
+
+inline int fail(hipc_ctx *ctx, int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (ctx) ctx->err = buf;
+    return code;
+}
+
+// RAII: serialise the call and make the context's device current.
+struct Guard {
+    std::unique_lock<std::mutex> lock;
+    explicit Guard(hipc_ctx *ctx) : lock(ctx->mu) { (void)hipSetDevice(ctx->device); }
+};
+
+#define HIPC_TRY(ctx, expr)                                                                      \
+    do {                                                                                         \
+        hipError_t e_ = (expr);                                                                  \
+        if (e_ != hipSuccess)                                                                    \
+            return hipc::fail((ctx), HIPC_ERR_BACKEND, "%s: %s (%s:%d)", #expr,                  \
+                              hipGetErrorString(e_), __FILE__, __LINE__);                        \
+    } while (0)
+
+#define HIPC_REQUIRE(ctx, cond, ...)                                                             \
+    do {                                                                                         \
+        if (!(cond)) return hipc::fail((ctx), HIPC_ERR_INVALID, __VA_ARGS__);                    \
+    } while (0)
+
+#define HIPC_REFUSE(ctx, cond, ...)                                                              \
+    do {                                                                                         \
+        if (cond) return hipc::fail((ctx), HIPC_ERR_UNSUPPORTED, __VA_ARGS__);                   \
+    } while (0)
+
+// status of the launch just made (configuration errors surface here, not at the next sync)
+#define HIPC_LAUNCHED(ctx) HIPC_TRY((ctx), hipGetLastError())
+
+// Returns ctx->scratch[slot] grown to at least `bytes`. Growth allocates, so it is
+// refused while a capture is open.
+int scratch_get(hipc_ctx *ctx, int slot, size_t bytes, void **out);
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+inline bool is_byte_dtype(int dt) { return dt == HIPC_U8 || dt == HIPC_I8; }
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// offsets inside ctx->params
+constexpr size_t kParamRange = 0;   // 8 B  {bits(-min), bits(max)}
+constexpr size_t kParamBytes = 256;
+
+}  // namespace hipc

@@ -1,0 +1,301 @@
+// MatMulInteger, its fused dequantising epilogue, Requantize and QLinearMatMul.
+//
+// Reference: crates/onnx-vulkan-core/src/interp.rs:2090-2183 (matmul_integer),
+// :2405-2572 (matmul_integer_scale_bias), :2712-2768 (packed_b), :4682-4788
+// (requantize), :4845-4875 (qlinear_matmul); kernels shaders/matmul_integer.rs and
+// shaders/glsl/matmul_integer_coop_smem.comp; definition host_ops.rs:1157-1199.
+#include <algorithm>
+
+#include "int8_gemm.h"
+
+namespace hipc {
+
+// B [K, N] (N contiguous) -> Bp [N_pad, K_pad] (k contiguous), signed domain, zero padded.
+// One thread writes one 32-bit word (4 consecutive k of one column); reads are
+// coalesced along n.
+__global__ void __launch_bounds__(256)
+pack_b_kernel(const uint8_t *__restrict__ B, uint32_t *__restrict__ Bp, int K, int N, int K_pad, int N_pad,
+              uint32_t flip) {
+    const int n = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int kw = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (n >= N_pad || kw >= K_pad / 4) return;
+    uint32_t word = 0;
+    if (n < N) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int k = kw * 4 + b;
+            if (k < K) word |= (uint32_t)(B[(size_t)k * N + n] ^ (flip & 0xff)) << (8 * b);
+        }
+    }
+    Bp[(size_t)n * (K_pad / 4) + kw] = word;
+}
+
+// per-column sums of the shifted weight
+__global__ void __launch_bounds__(256)
+col_sum_kernel(const uint8_t *__restrict__ B, int32_t *__restrict__ sums, int K, int N, int N_pad, int is_signed,
+               int shift) {
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if (n >= N_pad) return;
+    int s = 0;
+    if (n < N) {
+        for (int k = 0; k < K; k++) {
+            const uint8_t v = B[(size_t)k * N + n];
+            s += (is_signed ? (int)(int8_t)v : (int)v) - shift;
+        }
+    }
+    sums[n] = s;
+}
+
+__global__ void __launch_bounds__(256)
+requantize_kernel(const int32_t *__restrict__ acc, const int32_t *__restrict__ bias, const float *__restrict__ ratio,
+                  long n, long inner, long axis_len, int y_zp, int out_signed, uint8_t *__restrict__ out) {
+    const long word = (long)blockIdx.x * 256 + threadIdx.x;
+    const long base = word * 4;
+    if (base >= n) return;
+    uint32_t packed = 0;
+    int count = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const long i = base + j;
+        if (i >= n) break;
+        const long c = (i / inner) % axis_len;
+        int a = acc[i];
+        if (bias) a += bias[c];
+        int q = (int)rintf(__fmul_rn((float)a, ratio[c])) + y_zp;
+        q = out_signed ? min(max(q, -128), 127) : min(max(q, 0), 255);
+        packed |= ((uint32_t)q & 0xffu) << (8 * j);
+        count++;
+    }
+    if (count == 4 && ((reinterpret_cast<uintptr_t>(out) & 3) == 0)) {
+        reinterpret_cast<uint32_t *>(out)[word] = packed;
+    } else {
+        for (int j = 0; j < count; j++) out[base + j] = (uint8_t)(packed >> (8 * j));
+    }
+}
+
+}  // namespace hipc
+
+using namespace hipc;
+
+struct hipc_int8_weight {
+    int64_t K = 0, N = 0;
+    int K_pad = 0, N_pad = 0;
+    int b_dtype = HIPC_I8;
+    uint8_t *Bp = nullptr;
+    int32_t *colsum = nullptr;
+};
+
+namespace {
+
+int pack_into(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, int64_t N, int K_pad, int N_pad, uint8_t *Bp,
+              int32_t *colsum) {
+    const uint32_t flip = b_dtype == HIPC_U8 ? 0x80808080u : 0u;
+    pack_b_kernel<<<dim3((unsigned)ceil_div(N_pad, 64), (unsigned)ceil_div(K_pad / 4, 4)), 256, 0, ctx->stream>>>(
+        static_cast<const uint8_t *>(B), reinterpret_cast<uint32_t *>(Bp), (int)K, (int)N, K_pad, N_pad, flip);
+    HIPC_LAUNCHED(ctx);
+    col_sum_kernel<<<dim3((unsigned)ceil_div(N_pad, 256)), 256, 0, ctx->stream>>>(
+        static_cast<const uint8_t *>(B), colsum, (int)K, (int)N, N_pad, b_dtype == HIPC_I8, b_dtype == HIPC_U8 ? 128 : 0);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+struct MmOperands {
+    const void *A;
+    int a_dtype;
+    const uint8_t *Bp;
+    const int32_t *colsum;
+    int b_dtype;
+    int64_t M, K, N;
+    int K_pad;
+};
+
+int fill_common(hipc_ctx *ctx, const MmOperands &o, GemmArgs &g) {
+    HIPC_REFUSE(ctx, !is_byte_dtype(o.a_dtype), "MatMulInteger: A must be uint8 or int8, got %d", o.a_dtype);
+    HIPC_REQUIRE(ctx, o.M >= 0 && o.M < (int64_t(1) << 30), "MatMulInteger: bad M=%ld", (long)o.M);
+    g = GemmArgs{};
+    g.P = static_cast<const uint8_t *>(o.A);
+    g.Q = o.Bp;
+    g.const_sum = o.colsum;
+    g.dyn_shift = o.a_dtype == HIPC_U8 ? 128 : 0;
+    g.const_shift = o.b_dtype == HIPC_U8 ? 128 : 0;
+    g.dyn_signed = o.a_dtype == HIPC_I8;
+    g.const_signed = o.b_dtype == HIPC_I8;
+    g.I = (int)o.M, g.J = (int)o.N, g.K = (int)o.K, g.K_pad = o.K_pad;
+    g.p_aligned = (o.K % 16 == 0) && aligned(o.A, 16);
+    return HIPC_OK;
+}
+
+template <int EPI>
+int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
+    if (g.I == 0 || g.J == 0) return HIPC_OK;
+    const dim3 grid((unsigned)ceil_div(g.J, kBN), (unsigned)ceil_div(g.I, kBM), 1);
+    int8_gemm_kernel<MODE_MM, EPI><<<grid, 256, 0, ctx->stream>>>(g);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hipc_prepack_int8_b(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, int64_t N, hipc_int8_weight **out) {
+    if (!ctx || !out) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    *out = nullptr;
+    HIPC_REFUSE(ctx, ctx->capturing, "MatMulInteger prepack while a capture is open");
+    HIPC_REFUSE(ctx, !is_byte_dtype(b_dtype), "MatMulInteger: B must be uint8 or int8, got %d", b_dtype);
+    HIPC_REQUIRE(ctx, B && K > 0 && N > 0 && K < (int64_t(1) << 30) && N < (int64_t(1) << 30),
+                 "MatMulInteger prepack: bad shape K=%ld N=%ld", (long)K, (long)N);
+    hipc_int8_weight *w = new hipc_int8_weight();
+    w->K = K, w->N = N, w->b_dtype = b_dtype;
+    w->K_pad = (int)(ceil_div(K, kBK) * kBK);
+    w->N_pad = (int)(ceil_div(N, kBN) * kBN);
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->Bp), (size_t)w->K_pad * w->N_pad);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&w->colsum), (size_t)w->N_pad * 4);
+    if (e != hipSuccess) {
+        if (w->Bp) (void)hipFree(w->Bp);
+        delete w;
+        return fail(ctx, HIPC_ERR_BACKEND, "MatMulInteger prepack: %s", hipGetErrorString(e));
+    }
+    int rc = pack_into(ctx, B, b_dtype, K, N, w->K_pad, w->N_pad, w->Bp, w->colsum);
+    if (rc != HIPC_OK) {
+        (void)hipFree(w->Bp);
+        (void)hipFree(w->colsum);
+        delete w;
+        return rc;
+    }
+    *out = w;
+    return HIPC_OK;
+}
+
+void hipc_int8_weight_destroy(hipc_ctx *ctx, hipc_int8_weight *w) {
+    if (!ctx || !w) return;
+    Guard g(ctx);
+    if (w->Bp) ctx->deferred.push_back(w->Bp);
+    if (w->colsum) ctx->deferred.push_back(w->colsum);
+    delete w;
+}
+
+int hipc_matmul_integer(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_int8_weight *B, const void *a_zp,
+                        const void *b_zp, void *Y, int64_t M) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, B, "MatMulInteger: null weight");
+    GemmArgs ga;
+    int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
+    if (rc != HIPC_OK) return rc;
+    if (M == 0) return HIPC_OK;
+    HIPC_REQUIRE(ctx, A && Y, "MatMulInteger: null operand");
+    ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
+    ga.const_zp = static_cast<const uint8_t *>(b_zp);
+    ga.Y = Y;
+    return launch_mm<EPI_I32>(ctx, ga);
+}
+
+int hipc_matmul_integer_raw(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, int b_dtype, const void *a_zp,
+                            const void *b_zp, void *Y, int64_t M, int64_t K, int64_t N) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REFUSE(ctx, !is_byte_dtype(b_dtype), "MatMulInteger: B must be uint8 or int8, got %d", b_dtype);
+    HIPC_REQUIRE(ctx, K > 0 && N >= 0 && K < (int64_t(1) << 30) && N < (int64_t(1) << 30),
+                 "MatMulInteger: bad shape K=%ld N=%ld", (long)K, (long)N);
+    if (M == 0 || N == 0) return HIPC_OK;
+    HIPC_REQUIRE(ctx, A && B && Y, "MatMulInteger: null operand");
+    const int K_pad = (int)(ceil_div(K, kBK) * kBK), N_pad = (int)(ceil_div(N, kBN) * kBN);
+    void *scratch = nullptr;
+    const size_t bp_bytes = (size_t)K_pad * N_pad;
+    int rc = scratch_get(ctx, 1, bp_bytes + (size_t)N_pad * 4, &scratch);
+    if (rc != HIPC_OK) return rc;
+    uint8_t *Bp = static_cast<uint8_t *>(scratch);
+    int32_t *colsum = reinterpret_cast<int32_t *>(Bp + bp_bytes);
+    rc = pack_into(ctx, B, b_dtype, K, N, K_pad, N_pad, Bp, colsum);
+    if (rc != HIPC_OK) return rc;
+    GemmArgs ga;
+    rc = fill_common(ctx, MmOperands{A, a_dtype, Bp, colsum, b_dtype, M, K, N, K_pad}, ga);
+    if (rc != HIPC_OK) return rc;
+    ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
+    ga.const_zp = static_cast<const uint8_t *>(b_zp);
+    ga.Y = Y;
+    return launch_mm<EPI_I32>(ctx, ga);
+}
+
+int hipc_matmul_integer_scale_bias(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_int8_weight *B,
+                                   const void *a_zp, const void *b_zp, const void *scale, int scale_step,
+                                   const void *product, int product_step, const void *bias, int bias_step, int relu,
+                                   void *range, void *Y, int64_t M) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, B, "MatMulIntegerScaleBias: null weight");
+    HIPC_REQUIRE(ctx, scale, "MatMulIntegerScaleBias: null scale");
+    HIPC_REQUIRE(ctx, (scale_step | 1) == 1 && (product_step | 1) == 1 && (bias_step | 1) == 1,
+                 "MatMulIntegerScaleBias: broadcast steps must be 0 (scalar) or 1 (per column)");
+    GemmArgs ga;
+    int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
+    if (rc != HIPC_OK) return rc;
+    if (M == 0) return HIPC_OK;
+    HIPC_REQUIRE(ctx, A && Y, "MatMulIntegerScaleBias: null operand");
+    ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
+    ga.const_zp = static_cast<const uint8_t *>(b_zp);
+    ga.Y = Y;
+    ga.scale = static_cast<const float *>(scale), ga.scale_step = scale_step;
+    ga.product = static_cast<const float *>(product), ga.product_step = product_step;
+    ga.bias = static_cast<const float *>(bias), ga.bias_step = bias_step;
+    ga.relu = relu;
+    ga.range = static_cast<uint32_t *>(range);
+    return launch_mm<EPI_SCALE_BIAS>(ctx, ga);
+}
+
+int hipc_requantize(hipc_ctx *ctx, const void *acc, const void *bias, const void *ratio, int64_t n, int64_t inner,
+                    int64_t axis_len, int32_t y_zp, int out_dtype, void *out) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REFUSE(ctx, !is_byte_dtype(out_dtype), "Requantize: output must be uint8 or int8, got %d", out_dtype);
+    HIPC_REQUIRE(ctx, n >= 0, "Requantize: negative length");
+    HIPC_REQUIRE(ctx, axis_len > 0, "Requantize: empty scale");  // interp.rs:4732
+    if (n == 0) return HIPC_OK;
+    HIPC_REQUIRE(ctx, acc && ratio && out, "Requantize: null operand");
+    const long words = ceil_div(n, 4);
+    requantize_kernel<<<dim3((unsigned)ceil_div(words, 256)), 256, 0, ctx->stream>>>(
+        static_cast<const int32_t *>(acc), static_cast<const int32_t *>(bias), static_cast<const float *>(ratio), (long)n,
+        (long)std::max<int64_t>(inner, 1), (long)axis_len, y_zp, out_dtype == HIPC_I8, static_cast<uint8_t *>(out));
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+int hipc_qlinear_matmul(hipc_ctx *ctx, const void *A, int a_dtype, float a_scale, int32_t a_zp,
+                        const hipc_int8_weight *B, const float *b_scale, int64_t n_b_scale, int32_t b_zp, float y_scale,
+                        int32_t y_zp, int y_dtype, void *Y, int64_t M) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, B && b_scale, "QLinearMatMul: null weight or scale");
+    HIPC_REFUSE(ctx, !is_byte_dtype(y_dtype), "QLinearMatMul: output must be uint8 or int8, got %d", y_dtype);
+    // the accepted envelope of `unsupported_quantization` (interp.rs:781-847, :4862-4866)
+    HIPC_REQUIRE(ctx, n_b_scale == 1 || n_b_scale == B->N, "QLinearMatMul: %ld scales for %ld columns", (long)n_b_scale,
+                 (long)B->N);
+    HIPC_REFUSE(ctx, n_b_scale > 1 && b_zp != 0, "QLinearMatMul: b per-channel zero point is not zero (asymmetric weights)");
+    HIPC_REQUIRE(ctx, y_scale != 0.f, "QLinear: y_scale is zero");
+    GemmArgs ga;
+    int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
+    if (rc != HIPC_OK) return rc;
+    if (M == 0) return HIPC_OK;
+    HIPC_REQUIRE(ctx, A && Y, "QLinearMatMul: null operand");
+    // ratio[c] = a_scale * b_scale[c] / y_scale, f32, left to right (interp.rs:4693)
+    std::vector<float> ratio((size_t)n_b_scale);
+    for (int64_t c = 0; c < n_b_scale; c++) {
+        volatile float t = a_scale * b_scale[c];
+        ratio[(size_t)c] = t / y_scale;
+    }
+    void *dratio = nullptr;
+    rc = scratch_get(ctx, 2, ratio.size() * 4, &dratio);
+    if (rc != HIPC_OK) return rc;
+    HIPC_REFUSE(ctx, ctx->capturing, "QLinearMatMul uploads its requantisation ratios: not capturable");
+    HIPC_TRY(ctx, hipMemcpyAsync(dratio, ratio.data(), ratio.size() * 4, hipMemcpyHostToDevice, ctx->stream));
+    HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    ga.host_zp = 1, ga.dyn_zp_value = a_zp, ga.const_zp_value = b_zp;
+    ga.Y = Y;
+    ga.ratio = static_cast<const float *>(dratio), ga.ratio_step = n_b_scale > 1 ? 1 : 0;
+    ga.y_zp = y_zp, ga.out_signed = y_dtype == HIPC_I8;
+    return launch_mm<EPI_REQUANT>(ctx, ga);
+}
+
+}  // extern "C"

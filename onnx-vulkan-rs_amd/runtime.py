@@ -1,0 +1,221 @@
+"""ctypes binding of libhipcompute.so: context, device buffers, capture/replay, timing.
+
+Mirrors the method set of the reference's ``VkContext`` (crates/vk-compute/src/lib.rs:16-20):
+enqueue-only calls, one explicit ``flush``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+F32, U8, I8, I32, F16 = 1, 2, 3, 6, 10
+_NP_TO_HIPC = {np.dtype(np.float32): F32, np.dtype(np.uint8): U8, np.dtype(np.int8): I8,
+               np.dtype(np.int32): I32, np.dtype(np.float16): F16}
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+class HipComputeError(RuntimeError):
+    """A call into libhipcompute failed; ``code`` is the HIPC_ERR_* status."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"hipcompute error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class ConvGeom(C.Structure):
+    """``hipc_conv_geom`` -- the reference's ``ConvGeom`` (interp.rs:3361-3536)."""
+    _fields_ = [(n, C.c_int64) for n in (
+        "n", "c_in", "h", "w", "c_out", "kh", "kw", "stride_h", "stride_w", "dil_h", "dil_w",
+        "pad_top", "pad_left", "pad_bottom", "pad_right", "group")]
+
+    @classmethod
+    def make(cls, x_shape, w_shape, strides=(1, 1), dilations=(1, 1), pads=(0, 0, 0, 0), group=1):
+        n, c_in, h, w = x_shape
+        c_out, _, kh, kw = w_shape
+        return cls(n, c_in, h, w, c_out, kh, kw, strides[0], strides[1], dilations[0], dilations[1],
+                   pads[0], pads[1], pads[2], pads[3], group)
+
+
+def library_path() -> str:
+    return os.path.join(_HERE, "libhipcompute.so")
+
+
+_lib = None
+
+# name -> (restype, argtypes); every symbol include/hipcompute.h declares
+_vp, _i64, _sz, _int, _f = C.c_void_p, C.c_int64, C.c_size_t, C.c_int, C.c_float
+SIGNATURES = {
+    "hipc_ctx_create": (_int, [_int, C.POINTER(_vp)]),
+    "hipc_ctx_create_on_stream": (_int, [_int, _vp, C.POINTER(_vp)]),
+    "hipc_ctx_destroy": (None, [_vp]),
+    "hipc_last_error": (C.c_char_p, [_vp]),
+    "hipc_version": (C.c_char_p, []),
+    "hipc_stream": (_vp, [_vp]),
+    "hipc_alloc": (_int, [_vp, _sz, C.POINTER(_vp)]),
+    "hipc_free_deferred": (_int, [_vp, _vp]),
+    "hipc_upload": (_int, [_vp, _vp, _sz, _vp, _sz]),
+    "hipc_download": (_int, [_vp, _vp, _vp, _sz, _sz]),
+    "hipc_copy": (_int, [_vp, _vp, _sz, _vp, _sz, _sz]),
+    "hipc_fill": (_int, [_vp, _vp, _sz, _sz, C.c_uint32]),
+    "hipc_flush": (_int, [_vp]),
+    "hipc_capture_begin": (_int, [_vp]),
+    "hipc_capture_end": (_int, [_vp, C.POINTER(_vp)]),
+    "hipc_graph_launch": (_int, [_vp, _vp]),
+    "hipc_graph_destroy": (None, [_vp, _vp]),
+    "hipc_measure_graph": (_int, [_vp, _vp, _int, _int, C.POINTER(C.c_double)]),
+    "hipc_matmul_nbits": (_int, [_vp, _vp, _int, _vp, _sz, _vp, _int, _sz, _vp, _sz, _vp, _i64, _i64, _i64,
+                                 _i64, _int]),
+    "hipc_prepack_matmul_nbits": (_int, [_vp, _vp, _sz, _vp, _int, _sz, _vp, _sz, _i64, _i64, _i64,
+                                         C.POINTER(_vp)]),
+    "hipc_nbits_weight_destroy": (None, [_vp, _vp]),
+    "hipc_nbits_weight_bytes": (_sz, [_vp]),
+    "hipc_matmul_nbits_packed": (_int, [_vp, _vp, _int, _vp, _vp, _i64]),
+    "hipc_dynamic_quantize_linear": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _int]),
+    "hipc_prepack_int8_b": (_int, [_vp, _vp, _int, _i64, _i64, C.POINTER(_vp)]),
+    "hipc_int8_weight_destroy": (None, [_vp, _vp]),
+    "hipc_matmul_integer": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _i64]),
+    "hipc_matmul_integer_raw": (_int, [_vp, _vp, _int, _vp, _int, _vp, _vp, _vp, _i64, _i64, _i64]),
+    "hipc_matmul_integer_scale_bias": (_int, [_vp, _vp, _int, _vp, _vp, _vp, _vp, _int, _vp, _int, _vp, _int,
+                                              _int, _vp, _vp, _i64]),
+    "hipc_requantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, C.c_int32, _int, _vp]),
+    "hipc_qlinear_matmul": (_int, [_vp, _vp, _int, _f, C.c_int32, _vp, C.POINTER(_f), _i64, C.c_int32, _f,
+                                   C.c_int32, _int, _vp, _i64]),
+    "hipc_conv_out_shape": (_int, [C.POINTER(ConvGeom), C.POINTER(_i64), C.POINTER(_i64)]),
+    "hipc_same_pads": (None, [_i64, _i64, _i64, _i64, _int, C.POINTER(_i64), C.POINTER(_i64)]),
+    "hipc_prepack_conv_w": (_int, [_vp, _vp, _int, C.POINTER(ConvGeom), C.POINTER(_vp)]),
+    "hipc_conv_weight_destroy": (None, [_vp, _vp]),
+    "hipc_conv_integer": (_int, [_vp, _vp, _int, _vp, _vp, _vp, C.POINTER(ConvGeom), _vp]),
+    "hipc_qlinear_conv": (_int, [_vp, _vp, _int, _f, C.c_int32, _vp, C.POINTER(_f), _i64, C.c_int32, _f,
+                                 C.c_int32, _int, _vp, C.POINTER(ConvGeom), _vp]),
+}
+
+
+def load_library():
+    """Load libhipcompute.so and declare its signatures. Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise HipComputeError(3, f"{path} is missing: build it with __graft_entry__.build() "
+                                     f"(make -C onnx-vulkan-rs_amd/csrc); there is no fallback path")
+        lib = C.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError here means the header and the library disagree
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def hipc_dtype(dt) -> int:
+    return _NP_TO_HIPC[np.dtype(dt)]
+
+
+class Buffer:
+    """A device allocation (``GpuBuffer``). ``ptr`` is the raw device address."""
+
+    def __init__(self, ctx: "Context", nbytes: int):
+        self.ctx = ctx
+        self.nbytes = int(nbytes)
+        p = _vp()
+        ctx._check(ctx.lib.hipc_alloc(ctx.handle, self.nbytes, C.byref(p)))
+        self.ptr = p.value
+
+    def at(self, offset: int) -> int:
+        return self.ptr + int(offset)
+
+    def free(self):
+        if self.ptr:
+            self.ctx.lib.hipc_free_deferred(self.ctx.handle, self.ptr)
+            self.ptr = None
+
+
+class Context:
+    """One device, one in-order stream (``VkContext``)."""
+
+    def __init__(self, device: int = 0, stream: int | None = None):
+        self.lib = load_library()
+        h = _vp()
+        if stream is None:
+            rc = self.lib.hipc_ctx_create(device, C.byref(h))
+        else:
+            rc = self.lib.hipc_ctx_create_on_stream(device, stream, C.byref(h))
+        if rc != 0:
+            raise HipComputeError(rc, f"cannot create a context on device {device} (no GPU?)")
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            self.lib.hipc_ctx_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def _check(self, rc: int):
+        if rc != 0:
+            raise HipComputeError(rc, self.lib.hipc_last_error(self.handle).decode())
+
+    @property
+    def stream(self) -> int:
+        return self.lib.hipc_stream(self.handle)
+
+    # ---- buffers
+    def alloc(self, nbytes: int) -> Buffer:
+        return Buffer(self, nbytes)
+
+    def upload(self, array: np.ndarray, buf: Buffer | None = None, offset: int = 0) -> Buffer:
+        a = np.ascontiguousarray(array)
+        if buf is None:
+            buf = self.alloc(max(a.nbytes, 4))
+        self._check(self.lib.hipc_upload(self.handle, buf.ptr, offset, a.ctypes.data, a.nbytes))
+        return buf
+
+    def download(self, buf, dtype, shape, offset: int = 0) -> np.ndarray:
+        out = np.empty(shape, dtype)
+        ptr = buf.ptr if isinstance(buf, Buffer) else buf
+        self._check(self.lib.hipc_download(self.handle, out.ctypes.data, ptr, offset, out.nbytes))
+        return out
+
+    def copy(self, dst, dst_offset, src, src_offset, nbytes):
+        self._check(self.lib.hipc_copy(self.handle, _ptr(dst), dst_offset, _ptr(src), src_offset, nbytes))
+
+    def fill(self, buf, offset, nbytes, word):
+        self._check(self.lib.hipc_fill(self.handle, _ptr(buf), offset, nbytes, word))
+
+    def flush(self):
+        self._check(self.lib.hipc_flush(self.handle))
+
+    # ---- capture / replay / timing
+    def capture_begin(self):
+        self._check(self.lib.hipc_capture_begin(self.handle))
+
+    def capture_end(self):
+        g = _vp()
+        self._check(self.lib.hipc_capture_end(self.handle, C.byref(g)))
+        return g
+
+    def graph_launch(self, graph):
+        self._check(self.lib.hipc_graph_launch(self.handle, graph))
+
+    def graph_destroy(self, graph):
+        self.lib.hipc_graph_destroy(self.handle, graph)
+
+    def measure_graph(self, graph, samples: int, launches_per_sample: int) -> np.ndarray:
+        """Nanoseconds per launch for each sample (``measure_dispatch_gpu``)."""
+        out = (C.c_double * samples)()
+        self._check(self.lib.hipc_measure_graph(self.handle, graph, samples, launches_per_sample, out))
+        return np.array(out[:], dtype=np.float64)
+
+
+def _ptr(b):
+    if b is None:
+        return None
+    return b.ptr if isinstance(b, Buffer) else int(b)

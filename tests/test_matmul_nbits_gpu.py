@@ -1,0 +1,141 @@
+"""MatMulNBits on the GPU against the oracle, through the C ABI.
+
+Tolerance (the one the task states for this operator): |got - ref| <= atol + rtol * |ref| with
+atol = 1e-3 and rtol = 1e-4 for f32 tensors, rtol = 1e-3 for f16 tensors.
+"""
+import numpy as np
+import pytest
+
+import refcases as rc
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL32, RTOL16 = 1e-3, 1e-4, 1e-3
+
+
+def close(got, ref, rtol):
+    got, ref = got.astype(np.float64), ref.astype(np.float64)
+    return np.all(np.abs(got - ref) <= ATOL + rtol * np.abs(ref))
+
+
+def worst(got, ref):
+    return float(np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64))))
+
+
+@pytest.mark.parametrize("case", rc.MATMUL_NBITS_CASES, ids=lambda c: "M%d_K%d_N%d_bs%d" % c)
+def test_reference_cases_as_nodes(ctx, pkg, oracle, case):
+    """The seven cases of crates/onnx-vulkan-core/tests/matmul_nbits.rs, built as the reference
+    builds them: one com.microsoft::MatMulNBits node, tensors by name."""
+    m, k, n, bs = case
+    a, nib, zp, scale = rc.matmul_nbits_case(m, k, n, bs)
+    B, Z = pkg.synth.pack_nibbles(nib, bs), pkg.synth.pack_zero_points(zp)
+    node = pkg.graph.NodeIr("MatMulNBits", ["a", "quant", "scales", "zp"], ["out"],
+                            {"K": k, "N": n, "bits": 4, "block_size": bs}, domain="com.microsoft", name="mmnb")
+    assert pkg.graph.is_implemented_node(node)
+    env = {"a": a, "quant": B, "scales": scale.reshape(-1), "zp": Z}
+    pkg.graph.execute(ctx, [node], env)
+    want = oracle.matmul_nbits(a, B, scale.reshape(-1), Z, k, n, bs)
+    got = env["out"]
+    assert got.shape == (m, n) and got.dtype == np.float32
+    assert close(got, want, RTOL32), worst(got, want)
+    # and the reference's own bound against the mathematics
+    f64 = rc.matmul_nbits_f64(a, nib, zp, scale, bs)
+    assert np.all(np.abs(got - f64) <= 1e-4 * np.maximum(np.abs(f64), 1.0))
+
+
+@pytest.mark.parametrize("case", [c for c in rc.MATMUL_NBITS_CASES if c[3] >= 32], ids=lambda c: "M%d_K%d_N%d_bs%d" % c)
+def test_reference_cases_on_the_prepacked_path(ctx, pkg, oracle, case):
+    m, k, n, bs = case
+    a, nib, zp, scale = rc.matmul_nbits_case(m, k, n, bs)
+    B, Z = pkg.synth.pack_nibbles(nib, bs), pkg.synth.pack_zero_points(zp)
+    w = pkg.ops.NBitsWeight(ctx, B, scale.reshape(-1), Z, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    want = oracle.matmul_nbits(a, B, scale.reshape(-1), Z, k, n, bs)
+    assert close(got, want, RTOL32), worst(got, want)
+
+
+SHAPES = [  # (M, K, N, block_size, with_zp)
+    (1, 1152, 6912, 32, True),    # gemma3 up / gate projection
+    (1, 6912, 1152, 32, True),    # down projection
+    (1, 1152, 1024, 32, True), (1, 1024, 1152, 32, True), (1, 1152, 256, 32, True),
+    (2, 2048, 2560, 128, False),  # qwen-style block 128 without zero points
+    (4, 300, 100, 64, True),      # partial last block, N not a multiple of 16
+    (5, 4096, 48, 256, True),
+    (8, 1152, 512, 32, True), (9, 512, 80, 32, False), (16, 640, 96, 32, True),
+    (17, 256, 64, 32, True),      # more than one group of 16 rows
+    (3, 7000, 40, 32, True),      # K large enough to split across workgroups
+    (8, 6912, 1152, 32, True),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_seeded_shapes_both_paths(ctx, pkg, oracle, shape):
+    m, k, n, bs, with_zp = shape
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=100 + n, with_zp=with_zp)
+    a = pkg.synth.normal_f32(m * k, 7).reshape(m, k)
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs)
+    assert close(got, want, RTOL32), ("direct", worst(got, want))
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    assert close(got, want, RTOL32), ("gemv", worst(got, want))
+
+
+def test_block_size_16_runs_direct_and_refuses_prepack(ctx, pkg, oracle):
+    k, n, bs = 208, 50, 16   # 13 blocks: odd, zero-point rows off word boundaries
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=3)
+    a = pkg.synth.normal_f32(3 * k, 8).reshape(3, k)
+    got = pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs)
+    assert close(got, oracle.matmul_nbits(a, B, scales, zp, k, n, bs), RTOL32)
+    with pytest.raises(pkg.HipComputeError) as e:
+        pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    assert e.value.code == 2
+
+
+@pytest.mark.parametrize("shape", [(1, 2048, 2560, 128), (6, 1024, 300, 32), (40, 512, 128, 128)],
+                         ids=lambda s: "M%d_K%d_N%d_bs%d" % s)
+def test_f16_tensors(ctx, pkg, oracle, shape):
+    m, k, n, bs = shape
+    B, scales, _ = pkg.synth.nbits_weight(n, k, bs, seed=5, with_zp=False, scale_dtype=np.float16)
+    a = pkg.synth.normal_f32(m * k, 9).reshape(m, k).astype(np.float16)
+    want = oracle.matmul_nbits(a, B, scales, None, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, B, scales, None, k, n, bs)
+    assert got.dtype == np.float16 and close(got, want, RTOL16), ("direct", worst(got, want))
+    w = pkg.ops.NBitsWeight(ctx, B, scales, None, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    assert got.dtype == np.float16 and close(got, want, RTOL16), ("gemv", worst(got, want))
+
+
+def test_unembedding_width_full_size(ctx, pkg, oracle):
+    """lm_head of the decoder configuration: K = 1152, N = 262144, every column checked."""
+    k, n, bs = 1152, 262144, 32
+    B, scales, zp = pkg.synth.fast_nbits_weight(n, k, bs, seed=17)
+    a = pkg.synth.normal_f32(k, 18).reshape(1, k)
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    assert close(got, want, RTOL32), worst(got, want)
+    # linearity in A, a size-independent property: f(2a) == 2 f(a) exactly (power-of-two scaling)
+    got2 = pkg.ops.matmul_nbits(ctx, 2 * a, None, None, None, k, n, bs, weight=w)
+    assert np.array_equal(got2, 2 * got)
+    w.destroy()
+
+
+def test_refusals_and_short_buffers(ctx, pkg):
+    k, n, bs = 128, 16, 32
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=1)
+    a = np.zeros((1, k), np.float32)
+    with pytest.raises(pkg.HipComputeError) as e:   # level 4 asks for int8 activations
+        pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs, accuracy_level=4)
+    assert e.value.code == 2
+    with pytest.raises(pkg.HipComputeError) as e:   # the weight is short for N (interp.rs:6465-6472)
+        pkg.ops.matmul_nbits(ctx, a, B[: n - 1], scales, zp, k, n, bs)
+    assert e.value.code == 1 and "short" in e.value.message
+    with pytest.raises(pkg.HipComputeError) as e:
+        pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, 24)
+    assert e.value.code == 1
+    y = pkg.ops.matmul_nbits(ctx, np.zeros((0, k), np.float32), B, scales, zp, k, n, bs)   # no rows: a no-op
+    assert y.shape == (0, n)

@@ -1,0 +1,305 @@
+"""Pins of the CPU oracle (no GPU): every oracle function is checked against something that is
+not its own formula -- known answers, the reference's closed-form test inputs evaluated by an
+independent route, committed golden literals, or an invariant the mathematics fixes.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import refcases as rc
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+# ------------------------------------------------------------------ binary16
+
+def test_f16_conversions_match_numpy(oracle):
+    lib = oracle.lib()
+    rng = np.random.default_rng(1)
+    vals = np.concatenate([
+        rng.standard_normal(4000).astype(np.float32) * np.float32(100.0),
+        rng.standard_normal(2000).astype(np.float32) * np.float32(1e-6),
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, -1e9, 6e-8, 2.98e-8, 2.99e-8, 6.1e-5, 1.0009765625,
+                  1.00048828125, 1.00146484375, np.inf, -np.inf], np.float32)])
+    for v in vals:
+        got = lib.oracle_f32_to_f16(float(v))
+        want = int(np.float32(v).astype(np.float16).view(np.uint16))
+        assert got == want, (v, got, want)
+    for h in list(range(0, 0x7C01, 37)) + [0x8000, 0x8001, 0xFBFF, 0x0001, 0x03FF, 0x0400]:
+        got = np.float32(lib.oracle_f16_to_f32(h))
+        want = np.array([h], np.uint16).view(np.float16).astype(np.float32)[0]
+        assert got.tobytes() == want.tobytes(), hex(h)
+
+
+# --------------------------------------------------------------- MatMulNBits
+
+def _packed(pkg, nib, zp, bs):
+    return pkg.synth.pack_nibbles(nib, bs), pkg.synth.pack_zero_points(zp)
+
+
+def test_nbits_one_hot_weights_pin_the_nibble_and_block_order(oracle, pkg):
+    """A single non-zero (q - zp) at (n, k) must give Y[n] = a[k] * scale(n, k/bs): a swapped
+    nibble, a transposed block index or a wrong zero-point nibble moves or changes it."""
+    K, N, bs = 100, 7, 16  # 7 blocks: odd, so zero-point rows are 4 bytes with a dangling nibble
+    nb = -(-K // bs)
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((1, K)).astype(np.float32)
+    for (n, k) in [(0, 0), (0, 1), (3, 16), (3, 17), (6, 99), (2, 31), (5, 64), (4, 95)]:
+        zp = rng.integers(0, 16, (N, nb)).astype(np.uint8)
+        nib = zp[:, np.arange(K) // bs].copy()          # every weight dequantises to exactly 0
+        nib[n, k] = (nib[n, k] + 5) % 16                # ... except one: q - zp = +5 or -11
+        scale = rng.uniform(0.5, 2.0, (N, nb)).astype(np.float32)
+        B, Z = _packed(pkg, nib, zp, bs)
+        y = oracle.matmul_nbits(a, B, scale.reshape(-1), Z, K, N, bs)
+        want = np.zeros((1, N), np.float32)
+        d = np.float32(int(nib[n, k]) - int(zp[n, k // bs]))
+        want[0, n] = a[0, k] * (d * scale[n, k // bs])
+        assert np.array_equal(y, want), (n, k)
+
+
+def test_nbits_all_ones_is_the_row_sum(oracle, pkg):
+    K, N, bs = 96, 5, 32
+    a = (np.arange(K, dtype=np.float32) - 40).reshape(1, K)
+    nib = np.full((N, K), 9, np.uint8)
+    B = pkg.synth.pack_nibbles(nib, bs)
+    scales = np.ones(N * 3, np.float32)
+    y = oracle.matmul_nbits(a, B, scales, None, K, N, bs)   # zp omitted => 8 => every weight is 1
+    assert np.array_equal(y, np.full((1, N), a.sum(), np.float32))
+
+
+def test_nbits_missing_zero_points_mean_eight(oracle, pkg):
+    a, nib, zp, scale = rc.matmul_nbits_case(3, 200, 19, 32)
+    B = pkg.synth.pack_nibbles(nib, 32)
+    eight = pkg.synth.pack_zero_points(np.full_like(zp, 8))
+    y0 = oracle.matmul_nbits(a, B, scale.reshape(-1), None, 200, 19, 32)
+    y8 = oracle.matmul_nbits(a, B, scale.reshape(-1), eight, 200, 19, 32)
+    assert np.array_equal(y0, y8)
+
+
+@pytest.mark.parametrize("case", rc.MATMUL_NBITS_CASES, ids=lambda c: "M%d_K%d_N%d_bs%d" % c)
+def test_nbits_reference_cases_against_the_float64_product(oracle, pkg, case):
+    m, k, n, bs = case
+    a, nib, zp, scale = rc.matmul_nbits_case(m, k, n, bs)
+    B, Z = _packed(pkg, nib, zp, bs)
+    y = oracle.matmul_nbits(a, B, scale.reshape(-1), Z, k, n, bs)
+    want = rc.matmul_nbits_f64(a, nib, zp, scale, bs)
+    # the reference's own bound (tests/matmul_nbits.rs:159-163)
+    assert np.all(np.abs(y - want) <= 1e-4 * np.maximum(np.abs(want), 1.0))
+
+
+def test_nbits_padding_of_a_partial_block_is_ignored(oracle, pkg):
+    """K = 100 with 32-wide blocks: the 28 padding nibbles of the last block must not count."""
+    a, nib, zp, scale = rc.matmul_nbits_case(2, 100, 17, 32)
+    B, Z = _packed(pkg, nib, zp, 32)
+    y = oracle.matmul_nbits(a, B, scale.reshape(-1), Z, 100, 17, 32)
+    B2 = B.copy()
+    B2[:, 3, 2:] = 0xFF  # k = 100..127 live in bytes 2.. of block 3
+    assert np.array_equal(y, oracle.matmul_nbits(a, B2, scale.reshape(-1), Z, 100, 17, 32))
+
+
+def test_nbits_f16_is_the_f32_computation_rounded_once(oracle, pkg):
+    a, nib, zp, scale = rc.matmul_nbits_case(4, 256, 24, 128)
+    B, Z = _packed(pkg, nib, zp, 128)
+    a16, s16 = a.astype(np.float16), scale.astype(np.float16)
+    y16 = oracle.matmul_nbits(a16, B, s16.reshape(-1), Z, 256, 24, 128)
+    y32 = oracle.matmul_nbits(a16.astype(np.float32), B, s16.astype(np.float32).reshape(-1), Z, 256, 24, 128)
+    assert y16.dtype == np.float16 and np.array_equal(y16, y32.astype(np.float16))
+
+
+# ----------------------------------------------------- DynamicQuantizeLinear
+
+@pytest.mark.parametrize("r,want_zp", [(0.6, 128), (1.0, 127), (0.5, 127), (2.0, 127), (3.7, 127)])
+def test_dql_symmetric_range_zero_point_sits_on_the_tie(oracle, r, want_zp):
+    """-min/scale is 127.5 up to rounding (tests/dynamic_quantize.rs:1-7, 78-88): for r = 0.6 the
+    correctly rounded quotient is exactly 127.5 and ties to the even 128, for the other ranges
+    it is the float just below and gives 127 -- a quotient one ULP off flips either."""
+    x = rc.dql_symmetric(r)
+    y, scale, zp = oracle.dynamic_quantize_linear(x)
+    want_scale = np.float32(np.float64(np.float32(x.max() - x.min())) / 255.0)
+    assert np.float32(scale).tobytes() == want_scale.tobytes()
+    # f64 quotient of two f32, cast once: the correctly rounded f32 quotient
+    q = np.float32(np.float64(-x.min()) / np.float64(want_scale))
+    assert zp == int(np.rint(q)) == want_zp
+    assert y[0] == 0 and y[-1] == min(255, int(np.rint(q)) + want_zp) and np.all(np.diff(y.astype(int)) >= 0)
+
+
+def test_dql_integer_ramp_is_the_identity(oracle):
+    x = np.arange(256, dtype=np.float32)
+    y, scale, zp = oracle.dynamic_quantize_linear(x)
+    assert scale == 1.0 and zp == 0 and np.array_equal(y, np.arange(256, dtype=np.uint8))
+    y, scale, zp = oracle.dynamic_quantize_linear(x - 100)
+    assert scale == 1.0 and zp == 100 and np.array_equal(y, np.arange(256, dtype=np.uint8))
+
+
+def test_dql_range_always_contains_zero_and_constants(oracle):
+    y, scale, zp = oracle.dynamic_quantize_linear(np.full(9, 5.1, np.float32))
+    assert zp == 0 and np.float32(scale).tobytes() == np.float32(np.float64(np.float32(5.1)) / 255).tobytes()
+    assert np.all(y == 255)
+    y, scale, zp = oracle.dynamic_quantize_linear(np.zeros(5, np.float32))
+    assert scale == 1.0 and zp == 0 and np.all(y == 0)
+    y, scale, zp = oracle.dynamic_quantize_linear(np.zeros(0, np.float32))   # interp.rs:1949-1966
+    assert y.size == 0 and scale == 1.0 and zp == 0
+
+
+def test_dql_division_agrees_with_the_reference_double_single_reciprocal(oracle):
+    """The reference replaces d/255 by fma(d, hi, d*lo) with the constants of
+    shaders/dynamic_quantize.rs:183 and proves it equal to the rounded quotient on xorshift values
+    (:255-285). The oracle's plain division must land on the same floats."""
+    hi, lo = np.float32(3.921568859e-3), np.float32(-2.319175824e-10)
+    assert hi == np.float32(1.0 / 255.0) and lo == np.float32(1.0 / 255.0 - np.float64(hi))
+    mask = (1 << 64) - 1
+    s = 0x2545F4914F6CDD1D
+    for _ in range(3000):
+        s ^= (s << 13) & mask
+        s ^= s >> 7
+        s ^= (s << 17) & mask
+        d = np.float32(np.float32(s >> 40) / np.float32(512.0))
+        if d == 0:
+            continue
+        _, scale, _ = oracle.dynamic_quantize_linear(np.array([0.0, d], np.float32))
+        # fma in exact arithmetic: d*hi + fl(d*lo), rounded once
+        fma = np.float32(np.float64(d) * np.float64(hi) + np.float64(np.float32(d * lo)))
+        assert np.float32(scale).tobytes() == fma.tobytes(), d
+
+
+def test_dql_codes_follow_the_rounded_quotient(oracle):
+    x = rc.dql_xorshift(1 << 14)
+    y, scale, zp = oracle.dynamic_quantize_linear(x)
+    q = np.float64(x) / np.float64(scale)          # f64 quotient of two f32: rounds like the exact one
+    want = np.clip(np.rint(q.astype(np.float32)) + zp, 0, 255).astype(np.uint8)
+    assert np.array_equal(y, want)
+
+
+# ------------------------------------------------------------- MatMulInteger
+
+def test_matmul_integer_reference_cases_against_big_integers(oracle):
+    # tests/matmul_integer_variants.rs:113-137: M7 K12 N5, both zero points non-zero
+    a = rc.pseudo_plus1(7 * 12, 11).reshape(7, 12)
+    b = rc.pseudo_plus1(12 * 5, 29).reshape(12, 5)
+    assert np.array_equal(oracle.matmul_integer(a, b, 37, 211), rc.matmul_integer_bigint(a, b, 37, 211))
+    # :255-282: int8 B reinterpreted from the same bytes, negative zero point
+    a = rc.pseudo_plus1(20 * 64, 3).reshape(20, 64)
+    b = rc.pseudo_plus1(64 * 18, 41).view(np.int8).reshape(64, 18)
+    assert np.array_equal(oracle.matmul_integer(a, b, 37, -73), rc.matmul_integer_bigint(a, b, 37, -73))
+    # signed A as well
+    a8 = a.view(np.int8)
+    assert np.array_equal(oracle.matmul_integer(a8, b, -5, 9), rc.matmul_integer_bigint(a8, b, -5, 9))
+
+
+def test_matmul_integer_extremes(oracle):
+    """255 * 255 * K with zero points 0: a dropped sign or a narrow accumulator shows at once."""
+    K = 300
+    a = np.full((2, K), 255, np.uint8)
+    b = np.full((K, 3), 255, np.uint8)
+    assert np.all(oracle.matmul_integer(a, b, 0, 0) == 255 * 255 * K)
+    bi = np.full((K, 3), -128, np.int8)
+    assert np.all(oracle.matmul_integer(a, bi, 0, 127) == 255 * (-255) * K)
+
+
+def test_rescale_rounds_twice(oracle):
+    rng = np.random.default_rng(5)
+    acc = rng.integers(-2 ** 22, 2 ** 22, (6, 40)).astype(np.int32)
+    scale = rng.uniform(1e-4, 1e-2, 40).astype(np.float32)
+    bias = rng.uniform(-1, 1, 40).astype(np.float32)
+    got = oracle.rescale(acc, scale, bias)
+    # acc < 2^24 is exact in f32; the product of two f32 is exact in f64; one cast rounds it
+    prod = (acc.astype(np.float64) * scale.astype(np.float64)).astype(np.float32)
+    want = (prod.astype(np.float64) + bias.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    fused = (acc.astype(np.float64) * scale.astype(np.float64) + bias.astype(np.float64)).astype(np.float32)
+    assert np.any(fused.view(np.uint32) != want.view(np.uint32)), "the case must tell an fma from two roundings"
+    relu = oracle.rescale(acc, scale, bias, relu=True)
+    assert np.array_equal(relu, np.maximum(want, 0)) and not np.signbit(relu).any()
+    # the product of scales is formed first, with its own rounding
+    p = np.float32(0.0123)
+    got = oracle.rescale(acc, p, bias, product=scale)
+    s2 = (np.float64(p) * scale.astype(np.float64)).astype(np.float32)
+    want = ((acc.astype(np.float64) * s2.astype(np.float64)).astype(np.float32).astype(np.float64)
+            + bias.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+# ------------------------------------------- Requantize / QLinear literals
+
+def test_requantize_against_exact_rationals(oracle):
+    rng = np.random.default_rng(7)
+    acc = rng.integers(-60000, 60000, 400).astype(np.int32)
+    for (xs, ws, ys, zp, signed) in [(0.02, 0.01, 0.05, 10, False), (0.03, 0.02, 0.1, -3, True),
+                                     (0.5, 0.5, 0.25, 128, False)]:   # the last lands on exact .5 ties
+        ratio = oracle.requantize_ratio(xs, [ws], ys)
+        got = oracle.requantize(acc, None, ratio, 1, zp, signed)
+        want = [rc.requantize_exact(int(a), xs, ws, ys, zp, signed) for a in acc]
+        assert np.array_equal(got.astype(int), np.array(want))
+
+
+def test_requantize_channel_index_and_bias(oracle):
+    # conv layout: c = (i / inner) % axis_len, bias added before the scaling
+    acc = np.arange(2 * 3 * 4, dtype=np.int32).reshape(2, 3, 4) * 100
+    ratio = np.array([0.01, 0.02, 0.04], np.float32)
+    bias = np.array([1000, -500, 0], np.int32)
+    got = oracle.requantize(acc, bias, ratio, 4, 3, False)
+    for n in range(2):
+        for c in range(3):
+            for i in range(4):
+                v = int(acc[n, c, i]) + int(bias[c])
+                want = min(255, max(0, int(np.rint(np.float32(v) * ratio[c])) + 3))
+                assert got[n, c, i] == want
+
+
+def _golden():
+    with open(os.path.join(GOLDEN, "qlinear_golden.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("case", _golden(), ids=lambda c: c["name"])
+def test_qlinear_golden_literals(oracle, case):
+    if case["op"] == "QLinearConv":
+        X = np.array(case["x"], np.uint8).reshape(case["x_shape"])
+        W = np.array(case["w"], np.int8).reshape(case["w_shape"])
+        g = oracle.conv_geom(X.shape, W.shape)
+        bias = None if case["bias"] is None else np.array(case["bias"], np.int32)
+        got = oracle.qlinear_conv(X, case["x_scale"], case["x_zp"], W, np.array(case["w_scale"], np.float32),
+                                  case["w_zp"][0], case["y_scale"], case["y_zp"], bias, g)
+    else:
+        A = np.array(case["a"], np.uint8).reshape(case["a_shape"])
+        B = np.array(case["b"], np.int8).reshape(case["b_shape"])
+        got = oracle.qlinear_matmul(A, case["a_scale"], case["a_zp"], B, np.array(case["b_scale"], np.float32),
+                                    case["b_zp"][0], case["y_scale"], case["y_zp"])
+    assert got.reshape(-1).tolist() == case["want"]
+
+
+# --------------------------------------------------------------- ConvInteger
+
+@pytest.mark.parametrize("case", rc.CONV_CASES, ids=lambda c: "c%d_o%d_%dx%d_s%d_d%d" % (
+    c["c_in"], c["c_out"], c["h"], c["w"], c["stride"], c["dilation"]))
+def test_conv_integer_reference_cases_against_the_dense_route(oracle, case):
+    X, W, x_zp, w_zp = rc.conv_case_operands(case)
+    s, d = case["stride"], case["dilation"]
+    g = oracle.conv_geom(X.shape, W.shape, (s, s), (d, d), case["pads"])
+    got = oracle.conv_integer(X, W, x_zp, w_zp, g)
+    want = rc.conv_integer_dense(X, W, x_zp, w_zp, (s, s), (d, d), case["pads"])
+    assert got.shape == want.shape and np.array_equal(got, want)
+
+
+def test_conv_integer_groups_and_1d(oracle):
+    rng = np.random.default_rng(9)
+    X = rng.integers(0, 256, (2, 8, 1, 50)).astype(np.uint8)
+    W = rng.integers(-128, 128, (12, 2, 1, 7)).astype(np.int8)   # group 4
+    g = oracle.conv_geom(X.shape, W.shape, (1, 2), (1, 3), (0, 9, 0, 9), group=4)
+    got = oracle.conv_integer(X, W, 128, 0, g)
+    want = rc.conv_integer_dense(X, W, 128, 0, (1, 2), (1, 3), (0, 9, 0, 9), group=4)
+    assert np.array_equal(got, want)
+
+
+def test_conv_geometry_known_answers(oracle):
+    lib = oracle.lib()
+    assert lib.oracle_conv_out_dim(4096, 3, 3, 7, 1, 1) == 4096
+    assert lib.oracle_conv_out_dim(4096, 15, 15, 7, 1, 5) == 4096
+    assert lib.oracle_conv_out_dim(224, 3, 3, 7, 2, 1) == 112       # resnet stem
+    assert lib.oracle_conv_out_dim(5, 0, 0, 7, 1, 1) == 0
+    assert oracle.same_pads(4096, 7, 1, 5) == (15, 15)
+    assert oracle.same_pads(224, 7, 2, 1, upper=True) == (2, 3)      # odd total: the extra goes last
+    assert oracle.same_pads(224, 7, 2, 1, upper=False) == (3, 2)
+    assert oracle.same_pads(10, 1, 1, 1) == (0, 0)

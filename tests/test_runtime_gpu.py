@@ -1,0 +1,86 @@
+"""The runtime half of the boundary: buffers, ordering, capture / replay, timing, errors."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_upload_copy_fill_download(ctx):
+    a = np.arange(1000, dtype=np.int32)
+    d = ctx.upload(a)
+    e = ctx.alloc(4000)
+    ctx.fill(e, 0, 4000, 0xDEADBEEF)
+    ctx.copy(e, 400, d, 0, 2000)
+    out = ctx.download(e, np.uint32, (1000,))
+    assert np.all(out[:100] == 0xDEADBEEF) and np.array_equal(out[100:600], a[:500].astype(np.uint32))
+    assert np.all(out[600:] == 0xDEADBEEF)
+    d.free(), e.free()
+    ctx.flush()
+
+
+def test_capture_replays_equal_eager_every_time(ctx, pkg, oracle):
+    """A captured MatMulNBits decode step + DynamicQuantizeLinear, replayed several times with
+    eager work and synchronisations in between; every replay must equal the eager result."""
+    k, n, bs = 1152, 1024, 32
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=31)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    dA, dY = ctx.alloc(4 * k), ctx.alloc(4 * n)
+    dQ, dP = ctx.alloc(n), ctx.alloc(8)
+
+    def step():
+        pkg.ops.matmul_nbits_packed_device(ctx, dA, pkg.F32, w, dY, 1)
+        pkg.ops.dynamic_quantize_linear_device(ctx, dY, n, dQ, dP, dP.at(4))
+
+    a0 = pkg.synth.normal_f32(k, 32).reshape(1, k)
+    ctx.upload(a0, dA)
+    step()                                  # warm: scratch is sized before the capture
+    ctx.flush()
+    ctx.capture_begin()
+    step()
+    graph = ctx.capture_end()
+    for i in range(4):
+        a = pkg.synth.normal_f32(k, 40 + i).reshape(1, k)
+        ctx.upload(a, dA)
+        ctx.fill(dY, 0, 4 * n, 0)           # eager work between replays
+        ctx.flush()
+        ctx.graph_launch(graph)
+        y = ctx.download(dY, np.float32, (1, n))
+        want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+        assert np.all(np.abs(y - want) <= 1e-3 + 1e-4 * np.abs(want)), i
+        q, s, z = oracle.dynamic_quantize_linear(y)
+        assert np.array_equal(ctx.download(dQ, np.uint8, (1, n)), q)
+        assert ctx.download(dP, np.float32, (1,))[0].tobytes() == np.float32(s).tobytes()
+        step()                              # the same step, eagerly
+        assert np.array_equal(ctx.download(dY, np.float32, (1, n)), y)
+    ns = ctx.measure_graph(graph, 5, 20)
+    assert ns.shape == (5,) and np.all(ns > 0) and np.all(ns < 1e9)
+    ctx.graph_destroy(graph)
+    w.destroy()
+
+
+def test_errors_carry_a_message_and_leave_the_context_usable(ctx, pkg):
+    with pytest.raises(pkg.HipComputeError) as e:
+        ctx.fill(ctx.alloc(16), 0, 6, 0)
+    assert e.value.code == 1 and "multiples of 4" in e.value.message
+    with pytest.raises(pkg.HipComputeError):
+        ctx.capture_end()
+    scratch = ctx.alloc(64)
+    ctx.capture_begin()
+    with pytest.raises(pkg.HipComputeError) as e:
+        ctx.alloc(64)
+    assert e.value.code == 2
+    ctx.fill(scratch, 0, 64, 1)
+    ctx.graph_destroy(ctx.capture_end())
+    d = ctx.upload(np.arange(4, dtype=np.int32))
+    assert np.array_equal(ctx.download(d, np.int32, (4,)), np.arange(4))
+
+
+def test_a_second_context_on_a_caller_stream(pkg, oracle):
+    """Adopting a stream the caller owns (here torch's current one) keeps work ordered with it."""
+    import torch
+    s = torch.cuda.current_stream().cuda_stream
+    with pkg.Context(0, stream=s) as c2:
+        x = pkg.synth.normal_f32(4096, 50)
+        y, sc, z = pkg.ops.dynamic_quantize_linear(c2, x)
+        wy, ws, wz = oracle.dynamic_quantize_linear(x)
+        assert np.array_equal(y, wy) and z == wz
