@@ -1,0 +1,305 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized matrix-product path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line. The headline `value` is the HBM throughput of the int4 MatMulNBits decode
+GEMV over the linears of one gemma3-1b-shaped decode step (26 layers x 7 projections + lm_head,
+block 32 with zero points, M = 1): every weight is distinct and resident in HBM (640 MB per
+step, far beyond the 256 MB last-level cache), a step is replayed from a captured graph, and
+the clock is the host's around K steps with a flush on both sides. `roofline` is the dominant
+kernel (the lm_head GEMV) timed with device events on the library's stream; `extras` carries the
+other configurations (int8 GEMM TOPS, QLinearConv, single-op GEMVs hot and cold);
+`cpu_baseline` is the restated CPU oracle on this box's host cores (ONNX Runtime is not
+installed), on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA, published
+
+# gemma3-1b decoder linears, (K, N, count per layer); lm_head once
+LAYER_LINEARS = [(1152, 1024, 1), (1152, 256, 2), (1024, 1152, 1), (1152, 6912, 2), (6912, 1152, 1)]
+LM_HEAD = (1152, 262144)
+N_LAYERS = 26
+BS = 32
+
+
+def gemv_bytes(K, N, bs=BS, with_zp=True, elt=4):
+    """Compulsory traffic of one MatMulNBits call: packed weight + scales + zero points + A + Y
+    (the reference's convention, crates/onnx-vulkan-core/src/work.rs:263-301)."""
+    nb = -(-K // bs)
+    return N * nb * bs // 2 + N * nb * 4 + (N * ((nb + 1) // 2) if with_zp else 0) + K * elt + N * elt
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class GemvSet:
+    """Prepacked weights + device vectors of a list of (K, N) GEMVs, and a graph replaying them."""
+
+    def __init__(self, pkg, ctx, shapes, seed):
+        self.pkg, self.ctx, self.items = pkg, ctx, []
+        self.bytes = 0
+        for i, (K, N) in enumerate(shapes):
+            B, scales, zp = pkg.synth.fast_nbits_weight(N, K, BS, seed + i)
+            w = pkg.ops.NBitsWeight(ctx, B, scales, zp, K, N, BS)
+            a = ctx.upload(pkg.synth.normal_f32(K, seed + 1000 + i))
+            y = ctx.alloc(4 * N)
+            self.items.append((w, a, y, K, N))
+            self.bytes += gemv_bytes(K, N)
+        self.graph = None
+
+    def enqueue(self):
+        for (w, a, y, K, N) in self.items:
+            self.pkg.ops.matmul_nbits_packed_device(self.ctx, a, self.pkg.F32, w, y, 1)
+
+    def capture(self):
+        self.enqueue()  # warm every launch shape (scratch sizing) before recording
+        self.ctx.flush()
+        self.ctx.capture_begin()
+        self.enqueue()
+        self.graph = self.ctx.capture_end()
+        return self.graph
+
+    def destroy(self):
+        if self.graph:
+            self.ctx.graph_destroy(self.graph)
+        for (w, a, y, _, _) in self.items:
+            w.destroy(), a.free(), y.free()
+        self.ctx.flush()
+
+
+def median_ns(ctx, graph, launches_per_graph=1, samples=20, reps=10):
+    ns = ctx.measure_graph(graph, samples, reps)
+    return float(np.median(ns)) / launches_per_graph, float(ns.min()) / launches_per_graph
+
+
+def bench_decode_linears(pkg, ctx, steps, warmup):
+    shapes = []
+    for _ in range(N_LAYERS):
+        for (K, N, c) in LAYER_LINEARS:
+            shapes += [(K, N)] * c
+    shapes.append(LM_HEAD)
+    t0 = time.time()
+    s = GemvSet(pkg, ctx, shapes, seed=5000)
+    log(f"[bench] decode linears: {len(shapes)} weights, {s.bytes / 1e6:.1f} MB algorithmic, built in {time.time() - t0:.1f}s")
+    g = s.capture()
+    for _ in range(warmup):
+        ctx.graph_launch(g)
+    ctx.flush()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ctx.graph_launch(g)
+    ctx.flush()
+    dt = time.perf_counter() - t0
+    ms = dt / steps * 1e3
+    res = dict(bytes_per_step=s.bytes, launches=len(shapes), ms_per_step=ms, gbs=s.bytes / (ms * 1e-3) / 1e9)
+    s.destroy()
+    return res
+
+
+def bench_lm_head_roofline(pkg, ctx, copies=3):
+    """The dominant kernel: lm_head GEMV rotating over `copies` distinct weights (~200 MB each)."""
+    K, N = LM_HEAD
+    s = GemvSet(pkg, ctx, [LM_HEAD] * copies, seed=7000)
+    g = s.capture()
+    med, mn = median_ns(ctx, g, launches_per_graph=copies, samples=15, reps=5)
+    per = gemv_bytes(K, N)
+    s.destroy()
+    return dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS,
+                traffic=None, kernel="mmnb_gemv_kernel (lm_head 1152->262144, M=1)", bytes_per_launch=per,
+                avg_launch_us=med / 1e3, min_launch_us=mn / 1e3)
+
+
+def bench_single_gemv(pkg, ctx, K, N, cold_copies):
+    per = gemv_bytes(K, N)
+    hot = GemvSet(pkg, ctx, [(K, N)], seed=8000)
+    g = hot.capture()
+    hot_ns, _ = median_ns(ctx, g, 1, samples=20, reps=50)
+    hot.destroy()
+    cold = GemvSet(pkg, ctx, [(K, N)] * cold_copies, seed=8100)
+    g = cold.capture()
+    cold_ns, _ = median_ns(ctx, g, cold_copies, samples=10, reps=2)
+    cold.destroy()
+    return dict(K=K, N=N, bytes=per, hot_us=hot_ns / 1e3, hot_gbs=per / hot_ns, cold_us=cold_ns / 1e3,
+                cold_gbs=per / cold_ns, cold_frac_hbm=per / cold_ns / HBM_PEAK_GBS, cold_ring_mb=cold_copies * per / 1e6)
+
+
+def bench_int8_ffn(pkg, ctx):
+    """DynamicQuantizeLinear [1000,1024] then MatMulInteger x [1024,4096] and x [4096,1024], with the
+    fused fp32 rescale."""
+    ops = pkg.ops
+    out = {}
+    T = 1000
+    x = pkg.synth.normal_f32(T * 1024, 2).reshape(T, 1024)
+    dX = ctx.upload(x)
+    dA, dP = ctx.alloc(T * 4096), ctx.alloc(8)
+    ops.dynamic_quantize_linear_device(ctx, dX, x.size, dA, dP, dP.at(4))
+    ctx.flush()
+    ctx.capture_begin()
+    ops.dynamic_quantize_linear_device(ctx, dX, x.size, dA, dP, dP.at(4))
+    g = ctx.capture_end()
+    ns, _ = median_ns(ctx, g, 1, samples=20, reps=20)
+    ctx.graph_destroy(g)
+    dql_bytes = x.size * 4 + x.size + 5
+    out["dynamic_quantize_linear_1000x1024"] = dict(us=ns / 1e3, gbs=dql_bytes / ns, frac_hbm=dql_bytes / ns / HBM_PEAK_GBS)
+    dS = ctx.upload(np.array([0.01], np.float32))
+    for (K, N) in [(1024, 4096), (4096, 1024)]:
+        w = ops.Int8Weight(ctx, pkg.synth.int8_weight(K, N, 22 + K))
+        a = ctx.upload(pkg.synth.uniform_ints(T * K, 23, 0, 255).astype(np.uint8))
+        y = ctx.alloc(T * N * 4)
+        for name, fn in [("i32", lambda: ops.matmul_integer_device(ctx, a, pkg.U8, w, dP.at(4), None, y, T)),
+                         ("rescale_f32", lambda: ops.matmul_integer_scale_bias_device(
+                             ctx, a, pkg.U8, w, dP.at(4), None, dP, 0, dS, 0, None, 0, False, None, y, T))]:
+            fn()
+            ctx.flush()
+            ctx.capture_begin()
+            fn()
+            g = ctx.capture_end()
+            ns, mn = median_ns(ctx, g, 1, samples=20, reps=20)
+            ctx.graph_destroy(g)
+            opsn = 2.0 * T * K * N
+            byts = T * K + K * N + T * N * 4
+            out[f"matmul_integer_{name}_1000x{K}x{N}"] = dict(
+                us=ns / 1e3, tops=opsn / ns / 1e3, frac_int8_mfma=opsn / ns / 1e3 / INT8_PEAK_TOPS,
+                gbs=byts / ns, frac_hbm=byts / ns / HBM_PEAK_GBS)
+        w.destroy(), a.free(), y.free()
+    # asymptotic shape, to separate the kernel from the launch floor
+    K = N = T2 = 8192
+    w = ops.Int8Weight(ctx, pkg.synth.uniform_ints(K * N, 30, -127, 127).astype(np.int8).reshape(K, N))
+    a = ctx.upload(pkg.synth.uniform_ints(T2 * K, 31, 0, 255).astype(np.uint8))
+    y = ctx.alloc(T2 * N * 4)
+    ops.matmul_integer_device(ctx, a, pkg.U8, w, dP.at(4), None, y, T2)
+    ctx.flush()
+    ctx.capture_begin()
+    ops.matmul_integer_device(ctx, a, pkg.U8, w, dP.at(4), None, y, T2)
+    g = ctx.capture_end()
+    ns, _ = median_ns(ctx, g, 1, samples=5, reps=3)
+    ctx.graph_destroy(g)
+    out["matmul_integer_i32_8192x8192x8192"] = dict(us=ns / 1e3, tops=2.0 * T2 * K * N / ns / 1e3,
+                                                    frac_int8_mfma=2.0 * T2 * K * N / ns / 1e3 / INT8_PEAK_TOPS)
+    w.destroy(), a.free(), y.free()
+    for b in (dX, dA, dP, dS):
+        b.free()
+    ctx.flush()
+    return out
+
+
+def bench_qlinear_conv(pkg, ctx):
+    ops = pkg.ops
+    out = {}
+    for (C, T, dil) in [(192, 4096, 1), (192, 4096, 3), (192, 4096, 5), (512, 4096, 1)]:
+        X = pkg.synth.uniform_ints(C * T, 40, 0, 255).astype(np.uint8).reshape(1, C, 1, T)
+        W = pkg.synth.uniform_ints(C * C * 7, 41, -127, 127).astype(np.int8).reshape(C, C, 1, 7)
+        ws = pkg.synth.uniform_f32(C, 42, 0.001, 0.02)
+        bias = ctx.upload(pkg.synth.uniform_ints(C, 43, -4096, 4096).astype(np.int32))
+        geom = pkg.ConvGeom.make(X.shape, W.shape, dilations=(1, dil), pads=(0, 3 * dil, 0, 3 * dil))
+        w = ops.ConvWeight(ctx, W, geom)
+        dX, dY = ctx.upload(X), ctx.alloc(C * T)
+        # QLinearConv uploads its ratios, so it is timed eagerly between device events via a graph of the
+        # integer convolution + a standalone run for the full operator
+        t = []
+        for _ in range(3):
+            ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, 128, w, ws, 0, 0.5, 128, pkg.U8, bias, geom, dY)
+        ctx.flush()
+        reps = 50
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, 128, w, ws, 0, 0.5, 128, pkg.U8, bias, geom, dY)
+        ctx.flush()
+        wall_us = (time.perf_counter() - t0) / reps * 1e6
+        opsn = 2.0 * C * T * C * 7
+        out[f"qlinear_conv_c{C}_k7_T{T}_d{dil}"] = dict(wall_us=wall_us, tops_wall=opsn / wall_us / 1e6)
+        w.destroy(), dX.free(), dY.free(), bias.free()
+    ctx.flush()
+    return out
+
+
+def cpu_baseline(pkg, budget_s=12.0):
+    """The restated CPU oracle (ONNX Runtime is not installed) on the host cores, on a bounded
+    sample of the headline workload: the largest projection pair of one layer."""
+    import oracle
+    K, N = 1152, 6912
+    B, scales, zp = pkg.synth.fast_nbits_weight(N, K, BS, 99)
+    a = pkg.synth.normal_f32(K, 98).reshape(1, K)
+    oracle.matmul_nbits(a, B, scales, zp, K, N, BS)
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s:
+        oracle.matmul_nbits(a, B, scales, zp, K, N, BS)
+        reps += 1
+    dt = time.perf_counter() - t0
+    per = gemv_bytes(K, N)
+    return dict(value=per * reps / dt / 1e9, unit="GB/s", cores=oracle.threads(), kind="port",
+                sample=f"MatMulNBits M=1 K={K} N={N} bs=32+zp (gate/up projection), {reps} calls in {dt:.1f}s; "
+                       f"restated CPU oracle, ONNX Runtime unavailable")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", default="", help="comma list of sections to run (decode, lm_head, gemv, int8, conv, "
+                    "cpu); default all. Used to profile one kernel at a time.")
+    args = ap.parse_args()
+    only = set(filter(None, args.only.split(",")))
+    want = lambda name: not only or name in only  # noqa: E731
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU; --gpus > 1 is not supported in this build "
+              "(no collectives are part of it). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    pkg = entry.load_package()
+    ctx = pkg.Context(0)
+    head = dict(gbs=None, ms_per_step=None, bytes_per_step=None, launches=None)
+    roof = None
+    if want("decode"):
+        head = bench_decode_linears(pkg, ctx, args.steps, args.warmup)
+        log(f"[bench] decode linears: {head['ms_per_step']:.3f} ms/step, {head['gbs']:.0f} GB/s")
+    if want("lm_head"):
+        roof = bench_lm_head_roofline(pkg, ctx)
+        log(f"[bench] lm_head gemv: {roof['avg_launch_us']:.1f} us, {roof['achieved']:.0f} GB/s")
+    extras = {}
+    if want("gemv"):
+        extras["gemv_up_1152x6912"] = bench_single_gemv(pkg, ctx, 1152, 6912, cold_copies=64)
+        extras["gemv_down_6912x1152"] = bench_single_gemv(pkg, ctx, 6912, 1152, cold_copies=64)
+        log("[bench] single gemv:", json.dumps(extras))
+    if want("int8"):
+        extras.update(bench_int8_ffn(pkg, ctx))
+        log("[bench] int8 ffn done")
+    if want("conv"):
+        extras.update(bench_qlinear_conv(pkg, ctx))
+    cpu = cpu_baseline(pkg) if want("cpu") else None
+    ctx.close()
+
+    line = {
+        "metric": "int4 MatMulNBits HBM GB/s (% peak); int8 GEMM TOPS (% MFMA); tok/s",
+        "value": head["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights x f32 activations (bf16x3 MFMA, f32 accumulate)", "data": "synthetic",
+        "config": {"workload": "int4 MatMulNBits decode GEMVs of one gemma3-1b-shaped token: 26 layers x "
+                               "(q,k,v,o,gate,up,down) + lm_head 1152->262144, block 32 + zero points, M=1, "
+                               "every weight distinct and HBM-resident, graph replay",
+                   "bytes_per_step": head["bytes_per_step"], "launches_per_step": head["launches"],
+                   "frac_hbm_peak": head["gbs"] / HBM_PEAK_GBS if head["gbs"] else None},
+        "roofline": roof, "cpu_baseline": cpu, "extras": extras,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -131,8 +131,11 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
 void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w);
 /* bytes of device memory the prepacked form occupies */
 size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w);
+/* MatMulNBits on a prepacked weight. `accuracy_level` as in the operator: 0 (unset), 2 or 3 let
+ * f32 activations enter the matrix cores as two bf16 terms (16 significant bits, less error than
+ * f32 accumulation over K adds); 1 pins f32 and uses three terms (all 24 bits); 4 is refused. */
 int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w,
-                             void *Y, int64_t M);
+                             void *Y, int64_t M, int accuracy_level);
 
 /* ---------------------------------------------------- DynamicQuantizeLinear */
 

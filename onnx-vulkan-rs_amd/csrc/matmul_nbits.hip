@@ -156,11 +156,8 @@ struct GemvArgs {
     int slice_tiles;   // k tiles (128 k) per workgroup slice
     int ksplit;        // number of slices (gridDim.y)
     int a_f16;
+    uint32_t nib_mask, magic;  // 0x000f000f and 0x43004300 (bf16 128.0 in both halves)
 };
-
-__device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
-    return (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
-}
 
 template <int SG>
 struct ScaleVec;
@@ -168,53 +165,107 @@ template <>
 struct ScaleVec<4> {
     float s[4];
     uint32_t z;
-    __device__ __forceinline__ void load(const float *sc, const uint8_t *zb, size_t at) {
-        const float4 v = *reinterpret_cast<const float4 *>(sc + at * 4);
+    __device__ __forceinline__ void load(const float *sc, const uint8_t *zb, uint32_t at) {
+        const float4 v = *reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(sc) + at * 16u);
         s[0] = v.x, s[1] = v.y, s[2] = v.z, s[3] = v.w;
-        z = *reinterpret_cast<const uint32_t *>(zb + at * 4);
+        z = *reinterpret_cast<const uint32_t *>(zb + at * 4u);
     }
-    __device__ __forceinline__ void clear() { s[0] = s[1] = s[2] = s[3] = 0.f, z = 0; }
 };
 template <>
 struct ScaleVec<2> {
     float s[2];
     uint32_t z;
-    __device__ __forceinline__ void load(const float *sc, const uint8_t *zb, size_t at) {
-        const float2 v = *reinterpret_cast<const float2 *>(sc + at * 2);
+    __device__ __forceinline__ void load(const float *sc, const uint8_t *zb, uint32_t at) {
+        const float2 v = *reinterpret_cast<const float2 *>(reinterpret_cast<const char *>(sc) + at * 8u);
         s[0] = v.x, s[1] = v.y;
-        z = *reinterpret_cast<const uint16_t *>(zb + at * 2);
+        z = *reinterpret_cast<const uint16_t *>(zb + at * 2u);
     }
-    __device__ __forceinline__ void clear() { s[0] = s[1] = 0.f, z = 0; }
 };
 template <>
 struct ScaleVec<1> {
     float s[1];
     uint32_t z;
-    __device__ __forceinline__ void load(const float *sc, const uint8_t *zb, size_t at) {
-        s[0] = sc[at];
+    __device__ __forceinline__ void load(const float *sc, const uint8_t *zb, uint32_t at) {
+        s[0] = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(sc) + at * 4u);
         z = zb[at];
     }
-    __device__ __forceinline__ void clear() { s[0] = 0.f, z = 0; }
 };
 
-// T: 16-column tiles per wavefront; NR: accumulator registers in use (rows m = (lane>>4) + 4r,
-// r < NR, so M <= 4*NR); SG: scale groups per 128-k tile.
-// The workgroup is at most 16 / T wavefronts, which leaves the wide variants their registers.
-template <int T, int NR, int SG>
-__global__ void __launch_bounds__(1024 / T) mmnb_gemv_kernel(const GemvArgs p) {
+// One k tile (128 k) of T column tiles, as it arrives from HBM.
+template <int T, int SG>
+struct GemvStage {
+    uint4 wq[T];
+    ScaleVec<SG> sv[T];
+};
+
+__device__ __forceinline__ uint32_t bf16_rne(float v) {  // bits of the nearest bf16, in the high half
+    const uint32_t u = __float_as_uint(v);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+}
+
+// T:  16-column tiles per wavefront.
+// NR: accumulator registers in use (rows m = (lane>>4) + 4r, r < NR, so M <= 4*NR).
+// SG: scale groups per 128-k tile.
+// MC: M when it is known at compile time (1), else 0 -- with it the LDS offsets of the activation
+//     operands become immediates.
+// NT: bf16 terms an activation is split into. Three terms carry all 24 bits of an f32; two carry
+//     16 (relative error 2^-17 per element after rounding, below what f32 accumulation over K
+//     itself loses) and are exact for f16 activations. The block sums that remove the +128 bias
+//     are taken over the SAME split values, so the bias cancels exactly either way.
+//
+// A workgroup is WK x WN wavefronts: WN column groups side by side, each split WK ways along k.
+// It walks column groups blockIdx.x*WN, += gridDim.x*WN (a persistent grid when N is large), so
+// the activation split is paid once per workgroup, and every wavefront keeps the next tile's
+// loads in flight while it multiplies the current one -- across group boundaries too. Those
+// loads are unconditional (indices are clamped instead), so the wait counters stay exact, and
+// the two stage buffers swap roles by code duplication, not by copies.
+// The workgroup is at most 16 / T wavefronts (8 / T with all four accumulator registers in use),
+// which leaves the wide variants their registers.
+template <int T, int NR, int SG, int MC, int NT>
+__global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel(const GemvArgs p) {
     extern __shared__ uint4 smem[];
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
-    const int M = p.M;
+    const int M = MC > 0 ? MC : p.M;
     const int tile0 = blockIdx.y * p.slice_tiles;
     const int tile1 = min(p.n_cg, tile0 + p.slice_tiles);
     const int nch = (tile1 - tile0) * 4;  // 32-k chunks in this slice
 
-    uint4 *As = smem;                                              // [3][nch][4][M]
-    float *asum = reinterpret_cast<float *>(As + (size_t)3 * nch * 4 * M);  // [nch][M]
-    float *red = asum + ((nch * M + 3) & ~3);                      // [WN][WK][T][NR][64]
+    // LDS: As [nch][NT terms][4 k-groups][M] 16-byte operands | asum [nch][M] | red
+    uint4 *As = smem;
+    float *asum = reinterpret_cast<float *>(As + (size_t)nch * (4 * NT) * M);
+    float *red = asum + ((nch * M + 3) & ~3);  // [WN][WK][T][NR][64]
 
-    // ---- split the activations of this k slice into three bf16 terms, in operand order
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wk = wave % p.WK, wn = wave / p.WK;
+    const int i16 = lane & 15, g4 = lane >> 4;
+    const int groups = (p.n_tiles + T - 1) / T;
+    const int gstride = gridDim.x * p.WN;
+    // the nibble mask and the bf16 bias pattern travel as kernel arguments so that they live in
+    // registers and each unpack step is one v_and_or_b32 instead of an and and an or with literals
+    const uint32_t nib_mask = p.nib_mask;
+    uint32_t magic;  // held in a vector register: only one scalar operand fits the constant bus
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(p.magic));
+
+    // 32-bit byte offsets from uniform bases (the prepacked weight is below 4 GiB)
+    const char *wq_base = reinterpret_cast<const char *>(p.Wq);
+    const uint32_t lane16 = (uint32_t)lane * 16u;
+    auto load_stage = [&](int ng, int tile, GemvStage<T, SG> &st) {
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const uint32_t nt = (uint32_t)min(ng * T + t, p.n_tiles - 1);
+            const uint32_t tl = nt * (uint32_t)p.n_cg + (uint32_t)tile;
+            st.wq[t] = *reinterpret_cast<const uint4 *>(wq_base + (tl * 1024u + lane16));
+            st.sv[t].load(p.Sc, p.Zb, tl * 16u + (uint32_t)i16);
+        }
+    };
+
+    // ---- the first tile's loads go out before anything else
+    GemvStage<T, SG> stA, stB;
+    int ng = blockIdx.x * p.WN + wn;
+    load_stage(min(ng, groups - 1), min(tile0 + wk, tile1 - 1), stA);
+
+    // ---- split the activations of this k slice into NT bf16 terms, in operand order
     {
         const int nitems = M * nch * 4;
         const int kbase = tile0 * 128;
@@ -223,152 +274,190 @@ __global__ void __launch_bounds__(1024 / T) mmnb_gemv_kernel(const GemvArgs p) {
             const int c = (item >> 2) % nch;
             const int m = (item >> 2) / nch;
             const int k0 = kbase + c * 32 + w * 8;
-            float a[8];
+            uint32_t t0[8], t1[8], t2[8];
+            float s = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const int k = k0 + i;
-                float v = 0.f;
-                if (k < p.K) {
-                    v = p.a_f16 ? __half2float(static_cast<const __half *>(p.A)[(size_t)m * p.K + k])
-                                : static_cast<const float *>(p.A)[(size_t)m * p.K + k];
+                const int k = min(k0 + i, p.K - 1);
+                float a = p.a_f16 ? __half2float(static_cast<const __half *>(p.A)[(size_t)m * p.K + k])
+                                  : static_cast<const float *>(p.A)[(size_t)m * p.K + k];
+                if (k0 + i >= p.K) a = 0.f;
+                t0[i] = __float_as_uint(a) & 0xffff0000u;                 // hi: truncated
+                const float r1 = a - __uint_as_float(t0[i]);              // exact
+                float rep;
+                if (NT == 2) {
+                    t1[i] = bf16_rne(r1);
+                    t2[i] = 0;
+                    rep = __uint_as_float(t0[i]) + __uint_as_float(t1[i]);  // exact: 16 significant bits
+                } else {
+                    t1[i] = __float_as_uint(r1) & 0xffff0000u;
+                    t2[i] = bf16_rne(r1 - __uint_as_float(t1[i]));
+                    rep = a;  // the three terms carry every bit of a (up to one rounding in the last)
                 }
-                a[i] = v;
+                s += rep;
             }
-            float s = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
             s += __shfl_xor(s, 1, 64);
             s += __shfl_xor(s, 2, 64);
-            float hi[8], mid[8], lo[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                hi[i] = __uint_as_float(__float_as_uint(a[i]) & 0xffff0000u);
-                const float r1 = a[i] - hi[i];  // exact
-                mid[i] = __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
-                lo[i] = r1 - mid[i];            // exact; truncated to bf16 by the pack
-            }
-            const size_t slot = ((size_t)c * 4 + w) * M + m;
-            const size_t term = (size_t)nch * 4 * M;
-            // slot order (k0,k4,k1,k5,k2,k6,k3,k7) matches the nibble unpack below
-            As[slot] = make_uint4(bf16_pair(hi[0], hi[4]), bf16_pair(hi[1], hi[5]), bf16_pair(hi[2], hi[6]),
-                                  bf16_pair(hi[3], hi[7]));
-            As[term + slot] = make_uint4(bf16_pair(mid[0], mid[4]), bf16_pair(mid[1], mid[5]),
-                                         bf16_pair(mid[2], mid[6]), bf16_pair(mid[3], mid[7]));
-            As[2 * term + slot] = make_uint4(bf16_pair(lo[0], lo[4]), bf16_pair(lo[1], lo[5]),
-                                             bf16_pair(lo[2], lo[6]), bf16_pair(lo[3], lo[7]));
+            const size_t slot = ((size_t)c * (4 * NT) + w) * M + m;
+            // operand slot order (k0,k4,k1,k5,k2,k6,k3,k7) matches the nibble unpack below
+            As[slot] = make_uint4((t0[0] >> 16) | t0[4], (t0[1] >> 16) | t0[5], (t0[2] >> 16) | t0[6], (t0[3] >> 16) | t0[7]);
+            As[slot + 4 * M] = make_uint4((t1[0] >> 16) | t1[4], (t1[1] >> 16) | t1[5], (t1[2] >> 16) | t1[6], (t1[3] >> 16) | t1[7]);
+            if (NT == 3)
+                As[slot + 8 * M] = make_uint4((t2[0] >> 16) | t2[4], (t2[1] >> 16) | t2[5], (t2[2] >> 16) | t2[6], (t2[3] >> 16) | t2[7]);
             if (w == 0) asum[c * M + m] = s;
         }
     }
     __syncthreads();
 
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wk = wave % p.WK, wn = wave / p.WK;
-    const int i16 = lane & 15, g4 = lane >> 4;
-    const int mA = (i16 >> 2) + 4 * (i16 & 3);  // activation row this lane feeds as the A operand
-    const bool a_valid = mA < M;
-    const int nt0 = (blockIdx.x * p.WN + wn) * T;
-    const size_t term = (size_t)nch * 4 * M;
+    // The row of the 16x16 tile this lane feeds as the A operand. Lanes whose row is not one of
+    // the M activations read row 0 instead: the rows of a matrix product are independent, and the
+    // output rows they pollute are never stored.
+    const int mA = (i16 >> 2) + 4 * (i16 & 3);
+    const uint4 *a_lane = As + g4 * M + (mA < M ? mA : 0);
+    const float *s_lane[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) s_lane[r] = asum + (g4 + 4 * r < M ? g4 + 4 * r : 0);
 
     f32x4 acc[T];
 #pragma unroll
     for (int t = 0; t < T; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    if (nt0 < p.n_tiles) {
-        for (int tile = tile0 + wk; tile < tile1; tile += p.WK) {
-            uint4 wq[T];
-            ScaleVec<SG> sv[T];
+    auto compute = [&](const GemvStage<T, SG> &cur, int tile) {
+        const uint4 *a_tile = a_lane + (size_t)(tile - tile0) * (16 * NT) * M;
+        f32x4 c[T];
+        float asg[NR], s_q[T], zb_q[T], as_q[NR];
+        f32x4 d_q[T];
+        constexpr int CPG = 4 / SG;  // chunks per scale group
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            bf16x8 a_op[NT];
+#pragma unroll
+            for (int e = 0; e < NT; e++) a_op[e] = __builtin_bit_cast(bf16x8, a_tile[(j * (4 * NT) + 4 * e) * M]);
+            const bool first = (j % CPG) == 0, last = (j % CPG) == CPG - 1;
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                const float v = s_lane[r][((tile - tile0) * 4 + j) * M];
+                asg[r] = first ? v : asg[r] + v;
+            }
 #pragma unroll
             for (int t = 0; t < T; t++) {
-                if (nt0 + t < p.n_tiles) {
-                    const size_t tl = (size_t)(nt0 + t) * p.n_cg + tile;
-                    wq[t] = p.Wq[tl * 64 + lane];
-                    sv[t].load(p.Sc, p.Zb, tl * 16 + i16);
-                } else {
-                    wq[t] = make_uint4(0, 0, 0, 0);
-                    sv[t].clear();
-                }
+                const uint32_t word = j == 0 ? cur.wq[t].x : j == 1 ? cur.wq[t].y : j == 2 ? cur.wq[t].z : cur.wq[t].w;
+                const uint4 bw = make_uint4((word & nib_mask) | magic, ((word >> 4) & nib_mask) | magic,
+                                            ((word >> 8) & nib_mask) | magic, ((word >> 12) & nib_mask) | magic);
+                const bf16x8 b = __builtin_bit_cast(bf16x8, bw);
+                f32x4 d = first ? f32x4{0.f, 0.f, 0.f, 0.f} : c[t];
+#pragma unroll
+                for (int e = 0; e < NT; e++) d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_op[e], b, d, 0, 0, 0);
+                c[t] = d;
             }
-            f32x4 c[T];
-            float asg[NR];
+            // the epilogue of the scale group that ended one chunk ago runs behind this chunk's MFMAs
+            if (j > 0 && ((j - 1) % CPG) == CPG - 1) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int cl = (tile - tile0) * 4 + j;
-                uint4 ah = make_uint4(0, 0, 0, 0), am = ah, al = ah;
-                if (a_valid) {
-                    const size_t slot = ((size_t)cl * 4 + g4) * M + mA;
-                    ah = As[slot];
-                    am = As[term + slot];
-                    al = As[2 * term + slot];
-                }
-                const bf16x8 a_hi = __builtin_bit_cast(bf16x8, ah);
-                const bf16x8 a_mid = __builtin_bit_cast(bf16x8, am);
-                const bf16x8 a_lo = __builtin_bit_cast(bf16x8, al);
-                constexpr int CPG = 4 / SG;  // chunks per scale group
-                const bool first = (j % CPG) == 0, last = (j % CPG) == CPG - 1;
+                for (int t = 0; t < T; t++)
 #pragma unroll
-                for (int r = 0; r < NR; r++) {
-                    const int m = g4 + 4 * r;
-                    const float v = (m < M) ? asum[cl * M + m] : 0.f;
-                    asg[r] = first ? v : asg[r] + v;
-                }
+                    for (int r = 0; r < NR; r++)
+                        acc[t][r] = fmaf(s_q[t], fmaf(-zb_q[t], as_q[r], d_q[t][r]), acc[t][r]);
+            }
+            if (last) {
+                const int g = j / CPG;
 #pragma unroll
                 for (int t = 0; t < T; t++) {
-                    const uint32_t word = j == 0 ? wq[t].x : j == 1 ? wq[t].y : j == 2 ? wq[t].z : wq[t].w;
-                    const uint4 bw = make_uint4((word & 0x000f000fu) | 0x43004300u,
-                                                ((word >> 4) & 0x000f000fu) | 0x43004300u,
-                                                ((word >> 8) & 0x000f000fu) | 0x43004300u,
-                                                ((word >> 12) & 0x000f000fu) | 0x43004300u);
-                    const bf16x8 b = __builtin_bit_cast(bf16x8, bw);
-                    f32x4 d = first ? f32x4{0.f, 0.f, 0.f, 0.f} : c[t];
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, b, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_mid, b, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, b, d, 0, 0, 0);
-                    c[t] = d;
-                    if (last) {
-                        const int g = j / CPG;
-                        const float s = sv[t].s[g];
-                        const float zb = (float)((sv[t].z >> (8 * g)) & 0xffu);
-#pragma unroll
-                        for (int r = 0; r < NR; r++) acc[t][r] = fmaf(s, fmaf(-zb, asg[r], d[r]), acc[t][r]);
-                    }
+                    d_q[t] = c[t];
+                    s_q[t] = cur.sv[t].s[g];
+                    zb_q[t] = (float)((cur.sv[t].z >> (8 * g)) & 0xffu);
                 }
+#pragma unroll
+                for (int r = 0; r < NR; r++) as_q[r] = asg[r];
             }
         }
-    }
-
-    if (p.WK > 1) {
 #pragma unroll
         for (int t = 0; t < T; t++)
 #pragma unroll
-            for (int r = 0; r < NR; r++) red[((((size_t)wn * p.WK + wk) * T + t) * NR + r) * 64 + lane] = acc[t][r];
-        __syncthreads();
-        if (wk == 0) {
+            for (int r = 0; r < NR; r++) acc[t][r] = fmaf(s_q[t], fmaf(-zb_q[t], as_q[r], d_q[t][r]), acc[t][r]);
+    };
+
+    // one column group is done: reduce over the k wavefronts, store, clear
+    auto group_end = [&](bool more_groups) {
+        if (p.WK > 1) {
 #pragma unroll
             for (int t = 0; t < T; t++)
 #pragma unroll
-                for (int r = 0; r < NR; r++) {
-                    float v = acc[t][r];
-                    for (int k = 1; k < p.WK; k++) v += red[((((size_t)wn * p.WK + k) * T + t) * NR + r) * 64 + lane];
-                    acc[t][r] = v;
-                }
+                for (int r = 0; r < NR; r++)
+                    red[((((size_t)wn * p.WK + wk) * T + t) * NR + r) * 64 + lane] = acc[t][r];
+            __syncthreads();
+            if (wk == 0) {
+#pragma unroll
+                for (int t = 0; t < T; t++)
+#pragma unroll
+                    for (int r = 0; r < NR; r++) {
+                        float v = acc[t][r];
+                        for (int k = 1; k < p.WK; k++)
+                            v += red[((((size_t)wn * p.WK + k) * T + t) * NR + r) * 64 + lane];
+                        acc[t][r] = v;
+                    }
+            }
+            if (more_groups) __syncthreads();  // the buffer is written again next round
         }
-    }
-    if (wk == 0 && nt0 < p.n_tiles) {
+        if (wk == 0 && ng < groups) {
 #pragma unroll
-        for (int t = 0; t < T; t++) {
-            const int n = (nt0 + t) * 16 + i16;
+            for (int t = 0; t < T; t++) {
+                const int n = (ng * T + t) * 16 + i16;
 #pragma unroll
-            for (int r = 0; r < NR; r++) {
-                const int m = g4 + 4 * r;
-                if (m < M && n < p.N) {
-                    if (p.ksplit > 1) {
-                        p.Ypart[((size_t)blockIdx.y * M + m) * p.N + n] = acc[t][r];
-                    } else if (p.a_f16) {
-                        static_cast<__half *>(p.Y)[(size_t)m * p.N + n] = __float2half(acc[t][r]);
-                    } else {
-                        static_cast<float *>(p.Y)[(size_t)m * p.N + n] = acc[t][r];
+                for (int r = 0; r < NR; r++) {
+                    const int m = g4 + 4 * r;
+                    if (m < M && n < p.N) {
+                        if (p.ksplit > 1) {
+                            p.Ypart[((size_t)blockIdx.y * M + m) * p.N + n] = acc[t][r];
+                        } else if (p.a_f16) {
+                            static_cast<__half *>(p.Y)[(size_t)m * p.N + n] = __float2half(acc[t][r]);
+                        } else {
+                            static_cast<float *>(p.Y)[(size_t)m * p.N + n] = acc[t][r];
+                        }
                     }
                 }
             }
         }
+#pragma unroll
+        for (int t = 0; t < T; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    };
+
+    // every wavefront of the workgroup sees the same number of column groups (and so of barriers);
+    // the number of k tiles per group may differ by one between wavefronts, and can be zero
+    const int first_group = blockIdx.x * p.WN;
+    const int my_groups = first_group < groups ? (groups - first_group + gstride - 1) / gstride : 0;
+    const int span = tile1 - tile0;
+    const int my_tiles = wk < span ? (span - wk + p.WK - 1) / p.WK : 0;
+    if (my_tiles == 0) {
+        for (int g = 0; g < my_groups; g++) {
+            group_end(g + 1 < my_groups);
+            ng += gstride;
+        }
+        return;
+    }
+    int tile = tile0 + wk, ti = 0, gi = 0;
+    auto step = [&](const GemvStage<T, SG> &cur, GemvStage<T, SG> &next) {
+        // the tile after this one: same group, or the first tile of this wavefront's next group,
+        // or (at the very end) this one again, which the caches absorb
+        const bool group_done = ti + 1 == my_tiles;
+        const int ntile = group_done ? tile0 + wk : tile + p.WK;
+        const int nng = group_done ? ng + gstride : ng;
+        const bool any_left = nng < groups;
+        load_stage(any_left ? nng : min(ng, groups - 1), any_left ? ntile : tile, next);
+        if (ng < groups) compute(cur, tile);
+        if (group_done) {
+            gi++;
+            group_end(gi < my_groups);
+            ti = 0;
+        } else {
+            ti++;
+        }
+        tile = ntile, ng = nng;
+    };
+    const int total = my_groups * my_tiles;
+    for (int it = 0; it < total; it += 2) {
+        step(stA, stB);
+        if (it + 1 >= total) break;
+        step(stB, stA);
     }
 }
 
@@ -399,13 +488,15 @@ struct hipc_nbits_weight {
 
 namespace {
 
-// Launch-shape overrides for experiments: HIPC_GEMV_T (16-column tiles per
-// wavefront: 1, 2 or 4) and HIPC_GEMV_WAVES (wavefronts to aim for).
+// Launch-shape overrides for experiments: HIPC_GEMV_T (16-column tiles per wavefront: 1, 2 or
+// 4), HIPC_GEMV_WAVES (wavefronts to aim for when k is split inside a workgroup) and
+// HIPC_GEMV_PER_CU (resident wavefronts per CU of the persistent grid).
 struct GemvTune {
-    int T = 0, waves = 0;
+    int T = 0, waves = 0, per_cu = 0;
     GemvTune() {
         if (const char *e = getenv("HIPC_GEMV_T")) T = atoi(e);
         if (const char *e = getenv("HIPC_GEMV_WAVES")) waves = atoi(e);
+        if (const char *e = getenv("HIPC_GEMV_PER_CU")) per_cu = atoi(e);
     }
 };
 const GemvTune g_tune;
@@ -466,55 +557,68 @@ int launch_direct(hipc_ctx *ctx, const void *A, const void *B, const void *scale
     return HIPC_OK;
 }
 
-template <int T, int NR>
+template <int T, int NR, int MC, int NT>
 void launch_gemv_sg(const GemvArgs &a, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
     if (SG == 4)
-        mmnb_gemv_kernel<T, NR, 4><<<grid, block, lds, s>>>(a);
+        mmnb_gemv_kernel<T, NR, 4, MC, NT><<<grid, block, lds, s>>>(a);
     else if (SG == 2)
-        mmnb_gemv_kernel<T, NR, 2><<<grid, block, lds, s>>>(a);
+        mmnb_gemv_kernel<T, NR, 2, MC, NT><<<grid, block, lds, s>>>(a);
     else
-        mmnb_gemv_kernel<T, NR, 1><<<grid, block, lds, s>>>(a);
+        mmnb_gemv_kernel<T, NR, 1, MC, NT><<<grid, block, lds, s>>>(a);
+}
+
+template <int T, int NT>
+void launch_gemv_nr(const GemvArgs &a, int NR, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+    if (a.M == 1)
+        launch_gemv_sg<T, 1, 1, NT>(a, SG, grid, block, lds, s);
+    else if (NR == 1)
+        launch_gemv_sg<T, 1, 0, NT>(a, SG, grid, block, lds, s);
+    else if (NR == 2)
+        launch_gemv_sg<T, 2, 0, NT>(a, SG, grid, block, lds, s);
+    else
+        launch_gemv_sg<T, 4, 0, NT>(a, SG, grid, block, lds, s);
 }
 
 template <int T>
-void launch_gemv_nr(const GemvArgs &a, int NR, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
-    if (NR == 1)
-        launch_gemv_sg<T, 1>(a, SG, grid, block, lds, s);
-    else if (NR == 2)
-        launch_gemv_sg<T, 2>(a, SG, grid, block, lds, s);
+void launch_gemv_nt(const GemvArgs &a, int NT, int NR, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+    if (NT == 3)
+        launch_gemv_nr<T, 3>(a, NR, SG, grid, block, lds, s);
     else
-        launch_gemv_sg<T, 4>(a, SG, grid, block, lds, s);
+        launch_gemv_nr<T, 2>(a, NR, SG, grid, block, lds, s);
 }
 
 // rows [0, M) with M <= 16 of one activation matrix against a prepacked weight
-int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M) {
+int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int NT) {
     GemvArgs a{};
     a.A = A, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = Y, a.Ypart = nullptr;
     a.M = M, a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
     a.a_f16 = a_dtype == HIPC_F16;
+    a.nib_mask = 0x000f000fu, a.magic = 0x43004300u;
     const int NR = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int n_tiles = w->n_tiles, n_cg = w->n_cg;
 
     // columns per wavefront: wide outputs amortise the activation operands over more tiles
     int T = n_tiles >= 8192 ? 4 : (n_tiles >= 2048 ? 2 : 1);
     if (g_tune.T == 1 || g_tune.T == 2 || g_tune.T == 4) T = g_tune.T;
+    if (NR == 4 && T == 4) T = 2;  // four tiles x four accumulator registers do not fit the register file
     const int groups = (int)ceil_div(n_tiles, T);
     // k partition inside a workgroup: enough wavefronts to cover the chip a few times over
     const int want_waves = g_tune.waves > 0 ? g_tune.waves : 8 * ctx->cu_count;
     const int kparts = (int)std::min<int64_t>(n_cg, std::max<int64_t>(1, ceil_div(want_waves, groups)));
-    // the activation slice of a workgroup must fit the LDS budget: 196 bytes per row per 32-k chunk;
-    // only then is k also split across workgroups (partials + a reduce launch)
+    // the activation slice of a workgroup must fit the LDS budget: NT*64 + 4 bytes per row per 32-k
+    // chunk; only then is k also split across workgroups (partials + a reduce launch)
     const int lds_budget = 44 * 1024;
-    const int max_slice_tiles = std::max(1, lds_budget / (196 * 4 * M));
+    const int max_slice_tiles = std::max(1, lds_budget / ((NT * 64 + 4) * 4 * M));
     int ksplit = (int)ceil_div(n_cg, max_slice_tiles);
     const int slice_tiles = (int)ceil_div(n_cg, ksplit);
     ksplit = (int)ceil_div(n_cg, slice_tiles);
-    const int WK = std::max(1, std::min(std::min(16 / T, kparts), slice_tiles));
+    const int max_waves = 16 / T / (NR == 4 ? 2 : 1);
+    const int WK = std::max(1, std::min(std::min(max_waves, kparts), slice_tiles));
     const int WN = std::max(1, std::min(4 / WK, groups));
     a.WK = WK, a.WN = WN, a.slice_tiles = slice_tiles, a.ksplit = ksplit;
 
     const int nch = slice_tiles * 4;
-    size_t lds = (size_t)3 * nch * 4 * M * 16 + (size_t)((nch * M + 3) & ~3) * 4;
+    size_t lds = (size_t)nch * (4 * NT) * M * 16 + (size_t)((nch * M + 3) & ~3) * 4;
     if (WK > 1) lds += (size_t)WN * WK * T * NR * 64 * 4;
     HIPC_REQUIRE(ctx, lds <= 64 * 1024, "MatMulNBits gemv: LDS plan of %zu bytes does not fit", lds);
 
@@ -524,14 +628,18 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
         if (rc != HIPC_OK) return rc;
         a.Ypart = static_cast<float *>(part);
     }
-    const dim3 grid((unsigned)ceil_div(groups, WN), (unsigned)ksplit);
+    // persistent over the column groups once there are more workgroups than the chip holds at the
+    // occupancy aimed for (16 wavefronts per CU unless overridden)
+    const int waves_per_cu = g_tune.per_cu > 0 ? g_tune.per_cu : 16;
+    const int resident = std::max(1, ctx->cu_count * std::max(1, waves_per_cu / (WK * WN)) / ksplit);
+    const dim3 grid((unsigned)std::min<int64_t>(ceil_div(groups, WN), resident), (unsigned)ksplit);
     const dim3 block(64 * WK * WN);
     if (T == 4)
-        launch_gemv_nr<4>(a, NR, w->SG, grid, block, lds, ctx->stream);
+        launch_gemv_nt<4>(a, NT, NR, w->SG, grid, block, lds, ctx->stream);
     else if (T == 2)
-        launch_gemv_nr<2>(a, NR, w->SG, grid, block, lds, ctx->stream);
+        launch_gemv_nt<2>(a, NT, NR, w->SG, grid, block, lds, ctx->stream);
     else
-        launch_gemv_nr<1>(a, NR, w->SG, grid, block, lds, ctx->stream);
+        launch_gemv_nt<1>(a, NT, NR, w->SG, grid, block, lds, ctx->stream);
     HIPC_LAUNCHED(ctx);
     if (ksplit > 1) {
         const long total = (long)M * w->N;
@@ -589,6 +697,10 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
     w->SG = cpb >= 4 ? 1 : 4 / cpb;
     const size_t tiles = (size_t)w->n_tiles * w->n_cg;
     const size_t wq_bytes = tiles * 1024, sc_bytes = tiles * 16 * w->SG * 4, zb_bytes = tiles * 16 * w->SG;
+    if (wq_bytes >= (size_t(1) << 32)) {
+        delete w;
+        return fail(ctx, HIPC_ERR_UNSUPPORTED, "MatMulNBits prepack: a %zu-byte weight exceeds the 4 GiB the kernel addresses", wq_bytes);
+    }
     auto cleanup = [&]() {
         if (w->Wq) (void)hipFree(w->Wq);
         if (w->Sc) (void)hipFree(w->Sc);
@@ -636,19 +748,25 @@ void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w) {
 
 size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w) { return w ? w->bytes : 0; }
 
-int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int64_t M) {
+int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int64_t M,
+                             int accuracy_level) {
     if (!ctx) return HIPC_ERR_INVALID;
     Guard g(ctx);
     HIPC_REQUIRE(ctx, w, "MatMulNBits: null weight");
     HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
+    HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 3,
+                "MatMulNBits: accuracy_level %d asks for quantised activations", accuracy_level);
     HIPC_REQUIRE(ctx, M >= 0 && M < (int64_t(1) << 30), "MatMulNBits: bad M=%ld", (long)M);
     if (M == 0) return HIPC_OK;
     HIPC_REQUIRE(ctx, A && Y, "MatMulNBits: null operand");
     const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
+    // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
+    // terms). Unset, or 2 / 3 (f16 / bf16 are enough): 2 terms. f16 activations are exact in 2.
+    const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int rows = (int)std::min<int64_t>(16, M - m0);
         int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,
-                             static_cast<char *>(Y) + (size_t)m0 * w->N * esz, rows);
+                             static_cast<char *>(Y) + (size_t)m0 * w->N * esz, rows, NT);
         if (rc != HIPC_OK) return rc;
     }
     return HIPC_OK;

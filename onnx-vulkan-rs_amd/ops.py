@@ -53,8 +53,9 @@ def matmul_nbits_device(ctx, A, a_dtype, B, b_len, scales, scale_dtype, scales_l
                                          scales_len, _ptr(zp), zp_len, _ptr(Y), M, K, N, block_size, accuracy_level))
 
 
-def matmul_nbits_packed_device(ctx, A, a_dtype, weight: NBitsWeight, Y, M):
-    ctx._check(ctx.lib.hipc_matmul_nbits_packed(ctx.handle, _ptr(A), a_dtype, weight.handle, _ptr(Y), M))
+def matmul_nbits_packed_device(ctx, A, a_dtype, weight: NBitsWeight, Y, M, accuracy_level=0):
+    ctx._check(ctx.lib.hipc_matmul_nbits_packed(ctx.handle, _ptr(A), a_dtype, weight.handle, _ptr(Y), M,
+                                                accuracy_level))
 
 
 def matmul_nbits(ctx: Context, A, B, scales, zp, K, N, block_size, accuracy_level=0, weight: NBitsWeight = None):
@@ -64,7 +65,7 @@ def matmul_nbits(ctx: Context, A, B, scales, zp, K, N, block_size, accuracy_leve
     dA = ctx.upload(A)
     dY = ctx.alloc(max(M * N * A.dtype.itemsize, 4))
     if weight is not None:
-        matmul_nbits_packed_device(ctx, dA, hipc_dtype(A.dtype), weight, dY, M)
+        matmul_nbits_packed_device(ctx, dA, hipc_dtype(A.dtype), weight, dY, M, accuracy_level)
         tmp = []
     else:
         B = np.ascontiguousarray(B, np.uint8)

@@ -78,7 +78,7 @@ def test_vocoder_resblock_shape(ctx, pkg, oracle, dil):
     assert got.shape == (1, 192, 1, 4096)
     assert np.max(np.abs(got.astype(int) - want.astype(int))) <= 1
     assert np.array_equal(got, want)
-    assert np.count_nonzero((got > 0) & (got < 255)) > 0.9 * got.size
+    assert np.count_nonzero((got > 0) & (got < 255)) > 0.6 * got.size   # the case must not saturate away
 
 
 def test_wide_decoder_variant(ctx, pkg, oracle):

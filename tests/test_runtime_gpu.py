@@ -75,12 +75,18 @@ def test_errors_carry_a_message_and_leave_the_context_usable(ctx, pkg):
     assert np.array_equal(ctx.download(d, np.int32, (4,)), np.arange(4))
 
 
-def test_a_second_context_on_a_caller_stream(pkg, oracle):
-    """Adopting a stream the caller owns (here torch's current one) keeps work ordered with it."""
-    import torch
-    s = torch.cuda.current_stream().cuda_stream
-    with pkg.Context(0, stream=s) as c2:
+def test_a_second_context_on_a_caller_stream(ctx, pkg, oracle):
+    """Adopting a stream the caller owns keeps the library's work on that stream. The stream comes
+    from the HIP runtime the library itself is linked against (a second HIP runtime in the process,
+    such as the one a PyTorch wheel bundles, does not see the device once this one holds it)."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    stream = C.c_void_p()
+    assert hip.hipStreamCreateWithFlags(C.byref(stream), 1) == 0      # hipStreamNonBlocking
+    with pkg.Context(0, stream=stream.value) as c2:
+        assert c2.stream == stream.value
         x = pkg.synth.normal_f32(4096, 50)
         y, sc, z = pkg.ops.dynamic_quantize_linear(c2, x)
         wy, ws, wz = oracle.dynamic_quantize_linear(x)
         assert np.array_equal(y, wy) and z == wz
+    assert hip.hipStreamDestroy(stream) == 0
