@@ -156,6 +156,7 @@ struct GemvArgs {
     int slice_tiles;   // k tiles (128 k) per workgroup slice
     int ksplit;        // number of slices (gridDim.y)
     int a_f16;
+    int a_vec;  // rows of A may be read 8 elements at a time (base 16-byte aligned, K % 8 == 0)
     uint32_t nib_mask, magic;  // 0x000f000f and 0x43004300 (bf16 128.0 in both halves)
 };
 
@@ -260,51 +261,93 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
         }
     };
 
-    // ---- the first tile's loads go out before anything else
+    // ---- Prologue. The activations are split into NT bf16 terms, in operand order, into LDS.
+    // An "item" is 8 consecutive k of one row. On the fast path (aligned rows) a thread's first
+    // item is read with two unconditional 128-bit loads issued BEFORE the first weight tile's
+    // loads, so the split only waits for the activations (an L2 hit) while the weights stream in.
+    const int nitems = M * nch * 4;
+    const int kbase = tile0 * 128;
+    auto item_k0 = [&](int item, int &m, int &c, int &w) {
+        w = item & 3, c = (item >> 2) % nch, m = (item >> 2) / nch;
+        return kbase + c * 32 + w * 8;
+    };
+    auto load_item_vec = [&](int item, float av[8]) {
+        int m, c, w;
+        const int k0 = min(item_k0(item, m, c, w), p.K - 8);  // padding chunks are zeroed by split_item
+        if (p.a_f16) {
+            const uint4 raw = *reinterpret_cast<const uint4 *>(static_cast<const __half *>(p.A) + (size_t)m * p.K + k0);
+            const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+            for (int i = 0; i < 4; i++) av[2 * i] = __low2float(h[i]), av[2 * i + 1] = __high2float(h[i]);
+        } else {
+            const float4 *src = reinterpret_cast<const float4 *>(static_cast<const float *>(p.A) + (size_t)m * p.K + k0);
+            const float4 lo4 = src[0], hi4 = src[1];
+            av[0] = lo4.x, av[1] = lo4.y, av[2] = lo4.z, av[3] = lo4.w;
+            av[4] = hi4.x, av[5] = hi4.y, av[6] = hi4.z, av[7] = hi4.w;
+        }
+    };
+    auto load_item_scalar = [&](int item, float av[8]) {
+        int m, c, w;
+        const int k0 = item_k0(item, m, c, w);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int k = min(k0 + i, p.K - 1);
+            av[i] = p.a_f16 ? __half2float(static_cast<const __half *>(p.A)[(size_t)m * p.K + k])
+                            : static_cast<const float *>(p.A)[(size_t)m * p.K + k];
+        }
+    };
+    // splits one item and writes it (all four lanes of a chunk are active together: items come in fours)
+    auto split_item = [&](int item, const float av[8]) {
+        int m, c, w;
+        const int k0 = item_k0(item, m, c, w);
+        uint32_t t0[8], t1[8], t2[8];
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float a = (k0 + i < p.K) ? av[i] : 0.f;
+            t0[i] = __float_as_uint(a) & 0xffff0000u;                 // hi: truncated
+            const float r1 = a - __uint_as_float(t0[i]);              // exact
+            float rep;
+            if (NT == 2) {
+                t1[i] = bf16_rne(r1);
+                t2[i] = 0;
+                rep = __uint_as_float(t0[i]) + __uint_as_float(t1[i]);  // exact: 16 significant bits
+            } else {
+                t1[i] = __float_as_uint(r1) & 0xffff0000u;
+                t2[i] = bf16_rne(r1 - __uint_as_float(t1[i]));
+                rep = a;  // the three terms carry every bit of a (up to one rounding in the last)
+            }
+            s += rep;
+        }
+        s += __shfl_xor(s, 1, 64);
+        s += __shfl_xor(s, 2, 64);
+        const size_t slot = ((size_t)c * (4 * NT) + w) * M + m;
+        // operand slot order (k0,k4,k1,k5,k2,k6,k3,k7) matches the nibble unpack below
+        As[slot] = make_uint4((t0[0] >> 16) | t0[4], (t0[1] >> 16) | t0[5], (t0[2] >> 16) | t0[6], (t0[3] >> 16) | t0[7]);
+        As[slot + 4 * M] = make_uint4((t1[0] >> 16) | t1[4], (t1[1] >> 16) | t1[5], (t1[2] >> 16) | t1[6], (t1[3] >> 16) | t1[7]);
+        if (NT == 3)
+            As[slot + 8 * M] = make_uint4((t2[0] >> 16) | t2[4], (t2[1] >> 16) | t2[5], (t2[2] >> 16) | t2[6], (t2[3] >> 16) | t2[7]);
+        if (w == 0) asum[c * M + m] = s;
+    };
+
     GemvStage<T, SG> stA, stB;
     int ng = blockIdx.x * p.WN + wn;
-    load_stage(min(ng, groups - 1), min(tile0 + wk, tile1 - 1), stA);
-
-    // ---- split the activations of this k slice into NT bf16 terms, in operand order
-    {
-        const int nitems = M * nch * 4;
-        const int kbase = tile0 * 128;
+    const int first_ng = min(ng, groups - 1), first_tile = min(tile0 + wk, tile1 - 1);
+    if (p.a_vec) {
+        float av[8];
+        load_item_vec(min(tid, nitems - 1), av);
+        load_stage(first_ng, first_tile, stA);
+        if (tid < nitems) split_item(tid, av);
+        for (int item = tid + nthreads; item < nitems; item += nthreads) {
+            load_item_vec(item, av);
+            split_item(item, av);
+        }
+    } else {
+        load_stage(first_ng, first_tile, stA);
         for (int item = tid; item < nitems; item += nthreads) {
-            const int w = item & 3;
-            const int c = (item >> 2) % nch;
-            const int m = (item >> 2) / nch;
-            const int k0 = kbase + c * 32 + w * 8;
-            uint32_t t0[8], t1[8], t2[8];
-            float s = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int k = min(k0 + i, p.K - 1);
-                float a = p.a_f16 ? __half2float(static_cast<const __half *>(p.A)[(size_t)m * p.K + k])
-                                  : static_cast<const float *>(p.A)[(size_t)m * p.K + k];
-                if (k0 + i >= p.K) a = 0.f;
-                t0[i] = __float_as_uint(a) & 0xffff0000u;                 // hi: truncated
-                const float r1 = a - __uint_as_float(t0[i]);              // exact
-                float rep;
-                if (NT == 2) {
-                    t1[i] = bf16_rne(r1);
-                    t2[i] = 0;
-                    rep = __uint_as_float(t0[i]) + __uint_as_float(t1[i]);  // exact: 16 significant bits
-                } else {
-                    t1[i] = __float_as_uint(r1) & 0xffff0000u;
-                    t2[i] = bf16_rne(r1 - __uint_as_float(t1[i]));
-                    rep = a;  // the three terms carry every bit of a (up to one rounding in the last)
-                }
-                s += rep;
-            }
-            s += __shfl_xor(s, 1, 64);
-            s += __shfl_xor(s, 2, 64);
-            const size_t slot = ((size_t)c * (4 * NT) + w) * M + m;
-            // operand slot order (k0,k4,k1,k5,k2,k6,k3,k7) matches the nibble unpack below
-            As[slot] = make_uint4((t0[0] >> 16) | t0[4], (t0[1] >> 16) | t0[5], (t0[2] >> 16) | t0[6], (t0[3] >> 16) | t0[7]);
-            As[slot + 4 * M] = make_uint4((t1[0] >> 16) | t1[4], (t1[1] >> 16) | t1[5], (t1[2] >> 16) | t1[6], (t1[3] >> 16) | t1[7]);
-            if (NT == 3)
-                As[slot + 8 * M] = make_uint4((t2[0] >> 16) | t2[4], (t2[1] >> 16) | t2[5], (t2[2] >> 16) | t2[6], (t2[3] >> 16) | t2[7]);
-            if (w == 0) asum[c * M + m] = s;
+            float av[8];
+            load_item_scalar(item, av);
+            split_item(item, av);
         }
     }
     __syncthreads();
@@ -594,11 +637,12 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
     a.M = M, a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
     a.a_f16 = a_dtype == HIPC_F16;
     a.nib_mask = 0x000f000fu, a.magic = 0x43004300u;
+    a.a_vec = aligned(A, 16) && w->K % 8 == 0;
     const int NR = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int n_tiles = w->n_tiles, n_cg = w->n_cg;
 
     // columns per wavefront: wide outputs amortise the activation operands over more tiles
-    int T = n_tiles >= 8192 ? 4 : (n_tiles >= 2048 ? 2 : 1);
+    int T = n_tiles >= 2048 ? 2 : 1;
     if (g_tune.T == 1 || g_tune.T == 2 || g_tune.T == 4) T = g_tune.T;
     if (NR == 4 && T == 4) T = 2;  // four tiles x four accumulator registers do not fit the register file
     const int groups = (int)ceil_div(n_tiles, T);
