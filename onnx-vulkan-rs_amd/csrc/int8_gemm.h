@@ -5,9 +5,9 @@
 //
 // One 256-thread workgroup owns a 128x128 tile of C; its four wavefronts own
 // 64x64 each as 2x2 v_mfma_i32_32x32x32_i8 accumulators. Each k stage moves a
-// 128x64-byte slab of P and of Q through LDS with 128-bit accesses (row pitch
-// 80 bytes, conflict-free for ds_read_b128), the next slab's global loads
-// being in flight while the current one is multiplied.
+// 128x128-byte slab of P and of Q through LDS with 128-bit accesses (row pitch
+// 144 bytes, conflict-free for ds_read_b128); two further stages are on their
+// way from memory while one is multiplied.
 //
 // gfx950's int8 MFMA is signed x signed, so uint8 operands are shifted by 128
 // (x ^ 0x80), their zero points with them -- the identity the reference uses
@@ -27,7 +27,8 @@ namespace hipc {
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(16))) int i32x16;
 
-constexpr int kBM = 128, kBN = 128, kBK = 64, kPitch = kBK + 16;
+constexpr int kBM = 128, kBN = 128, kBK = 128, kPitch = kBK + 16;
+constexpr size_t kGemmLds = 2 * (kBM + kBN) * kPitch + 4 * 64 * sizeof(int);
 
 enum { EPI_I32 = 0, EPI_SCALE_BIAS = 1, EPI_REQUANT = 2 };
 enum { MODE_MM = 0, MODE_CONV = 1 };
@@ -78,18 +79,36 @@ __device__ __forceinline__ int dot_ones(uint4 v) {
     return __builtin_amdgcn_sdot4((int)v.w, 0x01010101, s, false);
 }
 
-template <int MODE, int EPI>
+// One k stage of both operand slabs as a thread holds it between global memory and LDS.
+struct GemmRegs {
+    uint4 p[4], q[4];
+};
+
+// ALIGNED (MODE_MM only): rows of A start on 16 bytes and K % 16 == 0, so A is read with
+// unconditional 128-bit loads (out-of-range chunks are clamped, then zeroed by a select --
+// no branch, which keeps the load counters exact and two stages in flight).
+template <int MODE, int EPI, bool ALIGNED>
 __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds_p[2][kBM * kPitch];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_q[2][kBN * kPitch];
-    __shared__ int lds_sum[4][64];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint8_t *lds_p = lds_raw;                            // [2][kBM * kPitch]
+    uint8_t *lds_q = lds_raw + 2 * kBM * kPitch;         // [2][kBN * kPitch]
+    int *lds_sum = reinterpret_cast<int *>(lds_raw + 2 * (kBM + kBN) * kPitch);  // [4][64]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int r32 = lane & 31, kg = lane >> 5;
-    const int i0 = blockIdx.y * kBM, j0 = blockIdx.x * kBN;
     const int img = blockIdx.z;
+
+    // Tile order: consecutive workgroup ids land on different XCDs (round robin), each with
+    // its own L2. Give every XCD a contiguous run of tiles, so neighbours that share an
+    // operand slab also share a cache.
+    const int tiles_x = (p.J + kBN - 1) / kBN, tiles_y = (p.I + kBM - 1) / kBM;
+    const int total = tiles_x * tiles_y;
+    const int per_xcd = (total + 7) / 8;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    const int i0 = (logical / tiles_x) * kBM, j0 = (logical % tiles_x) * kBN;
 
     // zero points in the shifted (signed) domain
     const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
@@ -98,22 +117,22 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     const uint32_t flip = p.dyn_shift ? 0x80808080u : 0u;
     const uint32_t pad_word = (uint32_t)(zd & 0xff) * 0x01010101u;
 
-    // the two 16-byte chunks of each operand slab this thread moves
-    int row_[2], kc_[2];
+    // the four 16-byte chunks of each operand slab this thread moves: slab row and k chunk (of 8)
+    int row_[4], kc_[4];
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
+    for (int u = 0; u < 4; u++) {
         const int c = tid + 256 * u;
-        row_[u] = c >> 2;
-        kc_[u] = c & 3;
+        row_[u] = c >> 3;
+        kc_[u] = c & 7;
     }
-    // MODE_CONV: where this thread's two positions sit in the input
-    int base_h[2] = {0, 0}, base_w[2] = {0, 0};
-    bool pos_ok[2] = {false, false};
+    // MODE_CONV: where this thread's positions sit in the input
+    int base_h[4] = {0, 0, 0, 0}, base_w[4] = {0, 0, 0, 0};
+    bool pos_ok[4] = {false, false, false, false};
     const uint8_t *q_img = p.Q;
     if (MODE == MODE_CONV) {
         q_img = p.Q + (size_t)img * p.H * p.W * p.C;
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
+        for (int u = 0; u < 4; u++) {
             const int gj = j0 + row_[u];
             pos_ok[u] = gj < p.J;
             const int oh = gj / p.Wo, ow = gj - oh * p.Wo;
@@ -126,10 +145,14 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
         const int gi = i0 + row_[u], gk = k0 + kc_[u] * 16;
         if (MODE == MODE_CONV) {
             return *reinterpret_cast<const uint4 *>(p.P + (size_t)gi * p.K_pad + gk);
+        } else if (ALIGNED) {
+            const bool ok = gi < p.I && gk < p.K;
+            const uint8_t *src = p.P + (size_t)min(gi, p.I - 1) * p.K + min(gk, p.K - 16);
+            const uint4 v = xor4(*reinterpret_cast<const uint4 *>(src), flip);
+            return make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
         } else {
             if (gi >= p.I || gk >= p.K) return make_uint4(0, 0, 0, 0);
             const uint8_t *src = p.P + (size_t)gi * p.K + gk;
-            if (p.p_aligned) return xor4(*reinterpret_cast<const uint4 *>(src), flip);
             uint32_t w[4] = {0, 0, 0, 0};
             for (int b = 0; b < 16; b++)
                 if (gk + b < p.K) w[b >> 2] |= (uint32_t)(src[b] ^ (flip & 0xff)) << (8 * (b & 3));
@@ -142,12 +165,31 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
             const int gj = j0 + row_[u];
             return *reinterpret_cast<const uint4 *>(p.Q + (size_t)gj * p.K_pad + gk);
         } else {
-            if (!pos_ok[u] || gk >= p.K) return make_uint4(0, 0, 0, 0);
-            const int tap = gk / p.C, c0 = gk - tap * p.C;
+            const int gkc = min(gk, p.K - 16);
+            const int tap = gkc / p.C, c0 = gkc - tap * p.C;
             const int r = tap / p.kw, s = tap - r * p.kw;
             const int ih = base_h[u] + r * p.dh, iw = base_w[u] + s * p.dw;
-            if (ih < 0 || ih >= p.H || iw < 0 || iw >= p.W) return make_uint4(pad_word, pad_word, pad_word, pad_word);
-            return *reinterpret_cast<const uint4 *>(q_img + ((size_t)ih * p.W + iw) * p.C + c0);
+            const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+            const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
+            const uint4 v = *reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + c0);
+            const bool live = pos_ok[u] && gk < p.K;  // beyond the problem: zeros; padding taps: the zero point
+            const uint32_t alt = live ? pad_word : 0u;
+            const bool take = live && inside;
+            return make_uint4(take ? v.x : alt, take ? v.y : alt, take ? v.z : alt, take ? v.w : alt);
+        }
+    };
+    auto load_regs = [&](GemmRegs &r, int stage) {
+        const int k0 = stage * kBK;
+#pragma unroll
+        for (int u = 0; u < 4; u++) r.p[u] = load_p(u, k0);
+#pragma unroll
+        for (int u = 0; u < 4; u++) r.q[u] = load_q(u, k0);
+    };
+    auto store_regs = [&](const GemmRegs &r, int buf) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            *reinterpret_cast<uint4 *>(lds_p + buf * kBM * kPitch + row_[u] * kPitch + kc_[u] * 16) = r.p[u];
+            *reinterpret_cast<uint4 *>(lds_q + buf * kBN * kPitch + row_[u] * kPitch + kc_[u] * 16) = r.q[u];
         }
     };
 
@@ -160,35 +202,16 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
     int dsum[2] = {0, 0};
 
-    const int nk = p.K_pad / kBK;
-    uint4 rp[2], rq[2];
-#pragma unroll
-    for (int u = 0; u < 2; u++) rp[u] = load_p(u, 0), rq[u] = load_q(u, 0);
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        *reinterpret_cast<uint4 *>(&lds_p[0][row_[u] * kPitch + kc_[u] * 16]) = rp[u];
-        *reinterpret_cast<uint4 *>(&lds_q[0][row_[u] * kPitch + kc_[u] * 16]) = rq[u];
-    }
-    __syncthreads();
-
-    for (int ks = 0; ks < nk; ks++) {
-        const int buf = ks & 1;
-        const bool more = ks + 1 < nk;
-        if (more) {
-#pragma unroll
-            for (int u = 0; u < 2; u++) rp[u] = load_p(u, (ks + 1) * kBK), rq[u] = load_q(u, (ks + 1) * kBK);
-        }
+    auto compute = [&](int buf) {
+        const uint8_t *bp = lds_p + buf * kBM * kPitch + (wm * 64 + r32) * kPitch + kg * 16;
+        const uint8_t *bq = lds_q + buf * kBN * kPitch + (wn * 64 + r32) * kPitch + kg * 16;
 #pragma unroll
         for (int step = 0; step < kBK / 32; step++) {
             uint4 pf[2], qf[2];
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-                pf[i] = *reinterpret_cast<const uint4 *>(
-                    &lds_p[buf][(wm * 64 + i * 32 + r32) * kPitch + step * 32 + kg * 16]);
+            for (int i = 0; i < 2; i++) pf[i] = *reinterpret_cast<const uint4 *>(bp + i * 32 * kPitch + step * 32);
 #pragma unroll
-            for (int j = 0; j < 2; j++)
-                qf[j] = *reinterpret_cast<const uint4 *>(
-                    &lds_q[buf][(wn * 64 + j * 32 + r32) * kPitch + step * 32 + kg * 16]);
+            for (int j = 0; j < 2; j++) qf[j] = *reinterpret_cast<const uint4 *>(bq + j * 32 * kPitch + step * 32);
             if (need_dyn_sum) {
 #pragma unroll
                 for (int f = 0; f < 2; f++) dsum[f] += dot_ones(MODE == MODE_MM ? pf[f] : qf[f]);
@@ -200,13 +223,26 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, pf[i]),
                                                                       __builtin_bit_cast(i32x4, qf[j]), acc[i][j], 0, 0, 0);
         }
-        if (more) {
-#pragma unroll
-            for (int u = 0; u < 2; u++) {
-                *reinterpret_cast<uint4 *>(&lds_p[buf ^ 1][row_[u] * kPitch + kc_[u] * 16]) = rp[u];
-                *reinterpret_cast<uint4 *>(&lds_q[buf ^ 1][row_[u] * kPitch + kc_[u] * 16]) = rq[u];
-            }
-        }
+    };
+
+    // Two register sets and two LDS buffers: while stage s is multiplied out of LDS, stage s+1
+    // sits in registers and stage s+2 is in flight. Stage indices past the end are clamped
+    // (a redundant, cached load) rather than branched around.
+    const int nk = p.K_pad / kBK;
+    GemmRegs r0, r1;
+    load_regs(r0, 0);
+    load_regs(r1, min(1, nk - 1));
+    store_regs(r0, 0);
+    __syncthreads();
+    for (int ks = 0; ks < nk; ks += 2) {
+        load_regs(r0, min(ks + 2, nk - 1));
+        compute(0);
+        store_regs(r1, 1);
+        __syncthreads();
+        if (ks + 1 >= nk) break;
+        load_regs(r1, min(ks + 3, nk - 1));
+        compute(1);
+        store_regs(r0, 0);
         __syncthreads();
     }
 
@@ -215,7 +251,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
 #pragma unroll
         for (int f = 0; f < 2; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
         if (MODE == MODE_MM) {
-            if (kg == 0) lds_sum[wave][r32] = dsum[0], lds_sum[wave][32 + r32] = dsum[1];
+            if (kg == 0) lds_sum[wave * 64 + r32] = dsum[0], lds_sum[wave * 64 + 32 + r32] = dsum[1];
         }
     }
     __syncthreads();
@@ -235,7 +271,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
                 int v = acc[i][j][r];
                 const int csum = p.const_sum[MODE == MODE_MM ? gj : gi];
                 v = v - zd * csum + kzz;
-                if (need_dyn_sum) v -= zc * (MODE == MODE_MM ? lds_sum[wave][i * 32 + rf] : dsum[j]);
+                if (need_dyn_sum) v -= zc * (MODE == MODE_MM ? lds_sum[wave * 64 + i * 32 + rf] : dsum[j]);
                 const size_t at = MODE == MODE_MM ? (size_t)gi * p.J + gj : ((size_t)img * p.I + gi) * p.J + gj;
                 if (EPI == EPI_I32) {
                     static_cast<int32_t *>(p.Y)[at] = v;

@@ -125,13 +125,25 @@ int fill_common(hipc_ctx *ctx, const MmOperands &o, GemmArgs &g) {
     return HIPC_OK;
 }
 
+template <int EPI, bool ALIGNED>
+int launch_mm_a(hipc_ctx *ctx, const GemmArgs &g) {
+    static bool lds_set = false;  // the kernel needs more than the default 64 KiB of dynamic LDS
+    if (!lds_set) {
+        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_kernel<MODE_MM, EPI, ALIGNED>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLds));
+        lds_set = true;
+    }
+    const int64_t tiles = ceil_div(g.J, kBN) * ceil_div(g.I, kBM);
+    const dim3 grid((unsigned)(ceil_div(tiles, 8) * 8), 1, 1);
+    int8_gemm_kernel<MODE_MM, EPI, ALIGNED><<<grid, 256, kGemmLds, ctx->stream>>>(g);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
 template <int EPI>
 int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
     if (g.I == 0 || g.J == 0) return HIPC_OK;
-    const dim3 grid((unsigned)ceil_div(g.J, kBN), (unsigned)ceil_div(g.I, kBM), 1);
-    int8_gemm_kernel<MODE_MM, EPI><<<grid, 256, 0, ctx->stream>>>(g);
-    HIPC_LAUNCHED(ctx);
-    return HIPC_OK;
+    return g.p_aligned ? launch_mm_a<EPI, true>(ctx, g) : launch_mm_a<EPI, false>(ctx, g);
 }
 
 }  // namespace
