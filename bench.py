@@ -229,6 +229,49 @@ def bench_qlinear_conv(pkg, ctx):
     return out
 
 
+def bench_decoder(pkg, ctx, steps, warmup, context=2048):
+    """One full int4 decode step of a gemma3-1b-shaped model (random weights) at a context of
+    `context` positions: f16 KV cache filled with random data, greedy sampling on the device, one
+    captured step replayed from a graph. Attention covers the whole context in every layer."""
+    D = pkg.decoder
+    cfg = dict(D.GEMMA3_1B)
+    t0 = time.time()
+    w = D.build_weights(cfg, seed=9)
+    max_seq = context + steps + warmup + 8
+    dec = D.Decoder(ctx, cfg, max_seq)
+    dec.load(w)
+    rng = np.random.default_rng(1)
+    filler = (rng.standard_normal(context * cfg["head_dim"]) * 0.5).astype(np.float16)
+    for li in range(cfg["n_layers"]):
+        k, v = dec.kv_cache(li)
+        for ptr in (k, v):
+            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, filler.ctypes.data, filler.nbytes))
+    log(f"[bench] decoder: weights built and loaded in {time.time() - t0:.1f}s")
+    dec.reset(1234, context - 1)
+    dec.step()
+    ctx.flush()
+    ctx.capture_begin()
+    dec.step()
+    g = ctx.capture_end()
+    for _ in range(warmup):
+        ctx.graph_launch(g)
+    ctx.flush()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ctx.graph_launch(g)
+    ctx.flush()
+    dt = time.perf_counter() - t0
+    tok, pos, _, hist = dec.read(n_history=pos_hist) if (pos_hist := 0) else dec.read()
+    ctx.graph_destroy(g)
+    dec.destroy()
+    ctx.flush()
+    byts = D.bytes_per_token(cfg, context)
+    tok_s = steps / dt
+    return dict(tok_s=tok_s, ms_per_token=dt / steps * 1e3, context=context, bytes_per_token=byts,
+                hbm_bound_tok_s=HBM_PEAK_GBS * 1e9 / byts, frac_of_hbm_bound=tok_s * byts / (HBM_PEAK_GBS * 1e9),
+                launches_per_token=2 + 10 * cfg["n_layers"] + 3, final_position=pos)
+
+
 def cpu_baseline(pkg, budget_s=12.0):
     """The restated CPU oracle (ONNX Runtime is not installed) on the host cores, on a bounded
     sample of the headline workload: the largest projection pair of one layer."""
@@ -254,7 +297,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma list of sections to run (decode, lm_head, gemv, int8, conv, "
-                    "cpu); default all. Used to profile one kernel at a time.")
+                    "decoder, cpu); default all. Used to profile one kernel at a time.")
     args = ap.parse_args()
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only  # noqa: E731
@@ -283,6 +326,9 @@ def main():
         log("[bench] int8 ffn done")
     if want("conv"):
         extras.update(bench_qlinear_conv(pkg, ctx))
+    if want("decoder"):
+        extras["gemma3_1b_int4_decode"] = bench_decoder(pkg, ctx, max(args.steps, 20), args.warmup)
+        log("[bench] decoder:", json.dumps(extras["gemma3_1b_int4_decode"]))
     cpu = cpu_baseline(pkg) if want("cpu") else None
     ctx.close()
 

@@ -256,6 +256,70 @@ int hipc_qlinear_conv(hipc_ctx *ctx, const void *X, int x_dtype, float x_scale, 
                       float y_scale, int32_t y_zp, int y_dtype, const void *bias,
                       const hipc_conv_geom *g, void *Y);
 
+/* ------------------------------------------------------------ decode step */
+
+/*
+ * The glue around the MatMulNBits GEMV that turns it into a decoder-only decode step
+ * (batch 1, greedy), so that its bandwidth can be quoted as tokens per second. It stands in
+ * for these reference operators (crates/onnx-vulkan-core/src): SimplifiedLayerNormalization
+ * (shaders/normalization.rs:109-181), GroupQueryAttention with half-split rotary embedding and
+ * cache append (shaders/attention.rs:128-317), Gelu approximate="tanh" (interp.rs:9020-9027),
+ * GatherBlockQuantized (shaders/gather_block_quantized.rs:26-57), ArgMax
+ * (shaders/reduction.rs:76-191), and for the replayed decode loop of
+ * crates/onnx-vulkan/src/lib.rs:509-623. One layer is
+ *   xn = rmsnorm(x, w_input); qkv = xn W_qkv; q, k = rope(rmsnorm_per_head(q|k, w_q|w_k), pos);
+ *   cache[pos] = (k, v) as f16; a = softmax(scale q K^T) V over positions 0..pos;
+ *   x += rmsnorm(a W_o, w_post_attn); xn = rmsnorm(x, w_pre_ffn);
+ *   h = gelu_tanh(xn W_gate) * (xn W_up); x += rmsnorm(h W_down, w_post_ffn)
+ * followed by logits = rmsnorm(x, w_final) W_lm_head and token = argmax(logits).
+ * The current token and position live in device memory and are advanced by the step itself,
+ * so a captured graph of one step replays without patching.
+ */
+typedef struct hipc_decoder hipc_decoder;
+typedef struct {
+    int32_t n_layers, hidden, ffn, n_q_heads, n_kv_heads, head_dim, vocab, max_seq, block_size;
+    float rms_eps, rope_theta;
+    float attn_scale;  /* 0 => 1 / sqrt(head_dim) */
+    float embed_scale; /* the embedding row is multiplied by this (gemma: sqrt(hidden)) */
+} hipc_decoder_config;
+
+/* linears: all MatMulNBits, 4 bit, f32 scales, ONNX layout. q|k|v and gate|up are given
+ * concatenated along N (they share their input, so each pair is one GEMV). */
+#define HIPC_DEC_QKV 0      /* [hidden -> (n_q + 2 n_kv) * head_dim] */
+#define HIPC_DEC_O 1        /* [n_q * head_dim -> hidden] */
+#define HIPC_DEC_GATE_UP 2  /* [hidden -> 2 * ffn] */
+#define HIPC_DEC_DOWN 3     /* [ffn -> hidden] */
+#define HIPC_DEC_LM_HEAD 4  /* [hidden -> vocab]; `layer` is ignored */
+/* RMS-norm weights, f32 */
+#define HIPC_DEC_NORM_INPUT 0
+#define HIPC_DEC_NORM_POST_ATTN 1
+#define HIPC_DEC_NORM_PRE_FFN 2
+#define HIPC_DEC_NORM_POST_FFN 3
+#define HIPC_DEC_NORM_Q 4     /* [head_dim] */
+#define HIPC_DEC_NORM_K 5     /* [head_dim] */
+#define HIPC_DEC_NORM_FINAL 6 /* `layer` is ignored */
+
+int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_decoder **out);
+void hipc_decoder_destroy(hipc_ctx *ctx, hipc_decoder *dec);
+/* Operands are device pointers (element counts in *_len); they are prepacked / copied and may be
+ * released after the next flush. zp may be NULL (zero point 8). */
+int hipc_decoder_set_linear(hipc_ctx *ctx, hipc_decoder *dec, int layer, int which, const void *B, size_t b_len,
+                            const void *scales, size_t scales_len, const void *zp, size_t zp_len);
+int hipc_decoder_set_norm(hipc_ctx *ctx, hipc_decoder *dec, int layer, int which, const void *w);
+/* the int4 embedding table [vocab, hidden] in the GatherBlockQuantized layout */
+int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *dec, const void *B, size_t b_len, const void *scales,
+                               size_t scales_len, const void *zp, size_t zp_len);
+/* the token the next step consumes and its position (= tokens already in the cache) */
+int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *dec, int32_t token, int32_t pos);
+/* device pointers of one layer's resident f16 cache, [n_kv_heads, max_seq, head_dim] each */
+int hipc_decoder_kv_cache(hipc_ctx *ctx, hipc_decoder *dec, int layer, void **k_cache, void **v_cache);
+/* enqueue one decode step (capturable) */
+int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *dec);
+/* flush, then read the state: next token, next position, the last step's logits [vocab] (or NULL),
+ * and the tokens chosen at positions 0..n_history-1 (or NULL) */
+int hipc_decoder_read(hipc_ctx *ctx, hipc_decoder *dec, int32_t *token, int32_t *pos, float *logits,
+                      int32_t *history, int32_t n_history);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,8 +13,9 @@ from .runtime import (  # noqa: F401
     Buffer,
     HipComputeError,
     ConvGeom,
+    DecoderConfig,
     library_path,
     load_library,
     F32, F16, U8, I8, I32,
 )
-from . import ops, synth, graph  # noqa: F401
+from . import ops, synth, graph, decoder  # noqa: F401

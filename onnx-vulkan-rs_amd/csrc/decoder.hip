@@ -1,0 +1,598 @@
+// A decoder-only decode step (batch 1) around the int4 MatMulNBits GEMV: the glue a
+// gemma3-1b-shaped model needs so that the GEMV's bandwidth becomes a tokens-per-second figure.
+//
+// Reference operators this stands in for (crates/onnx-vulkan-core/src):
+//   SimplifiedLayerNormalization  shaders/normalization.rs:109-181  y = x * rsqrt(mean(x^2) + eps) * w
+//   GroupQueryAttention           shaders/attention.rs:128-317      half-split rotary, cache append,
+//                                                                   scale * q.k^T, causal softmax, p.V
+//   Gelu (approximate = "tanh")   interp.rs:9020-9027               0.5 v (1 + tanh(0.797884 (v + 0.044715 v^3)))
+//   GatherBlockQuantized          shaders/gather_block_quantized.rs:26-57
+//   ArgMax                        shaders/reduction.rs:76-191
+//   the replayed decode loop      crates/onnx-vulkan/src/lib.rs:509-623, core/src/plan.rs
+//
+// The reference replays a recorded command list and patches the scalars that move with the
+// token (plan.rs:52-61). Here nothing needs patching: the position and the current token live in
+// device memory, every kernel reads them there, and the last kernel of a step advances them, so
+// a captured graph of one step replays unchanged. The KV cache is resident and laid out for
+// max_seq (the reference's rule, attention.rs:22-35), in f16.
+#include <hip/hip_fp16.h>
+
+#include <vector>
+
+#include "internal.h"
+
+namespace hipc {
+
+struct DecState {   // device-resident loop state
+    int32_t token;  // the token the next step consumes
+    int32_t pos;    // its position = number of tokens already in the cache
+};
+
+__device__ __forceinline__ float block_sum(float v, float *red) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();  // red may still be read from a previous call
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float s = 0.f;
+    for (int w = 0; w < nw; w++) s += red[w];
+    return s;
+}
+
+// x = embed_scale * dequant(table[token]); xn = rmsnorm(x, w). One workgroup.
+__global__ void __launch_bounds__(256)
+dec_embed_kernel(const DecState *st, const uint8_t *__restrict__ q, const float *__restrict__ scales,
+                 const uint8_t *__restrict__ zp, int hidden, int bs, int n_blocks, float embed_scale,
+                 const float *__restrict__ w, float eps, float *__restrict__ x, float *__restrict__ xn) {
+    __shared__ float red[4];
+    const size_t row = (size_t)st->token;
+    const size_t row_bytes = (size_t)n_blocks * bs / 2, zp_row = (n_blocks + 1) / 2;
+    float sq = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += 256) {
+        const int b = c / bs;
+        const int nib = (q[row * row_bytes + c / 2] >> (4 * (c & 1))) & 15;
+        const int z = zp ? (zp[row * zp_row + b / 2] >> (4 * (b & 1))) & 15 : 8;
+        const float v = ((float)nib - (float)z) * scales[row * n_blocks + b] * embed_scale;
+        x[c] = v;
+        sq += v * v;
+    }
+    const float inv = rsqrtf(block_sum(sq, red) / (float)hidden + eps);
+    for (int c = threadIdx.x; c < hidden; c += 256) xn[c] = x[c] * inv * w[c];
+}
+
+// x += rmsnorm(y, w_post); xn = rmsnorm(x, w_next). One workgroup of 256; every operand is read once,
+// up front (hidden <= 256 * kNormPer), so the kernel costs one memory round trip and two reductions.
+constexpr int kNormPer = 8;
+__global__ void __launch_bounds__(256)
+dec_norm_residual_kernel(const float *__restrict__ y, const float *__restrict__ w_post, const float *__restrict__ w_next,
+                         int hidden, float eps, float *__restrict__ x, float *__restrict__ xn) {
+    __shared__ float red[4];
+    float yv[kNormPer], xv[kNormPer], wp[kNormPer], wn[kNormPer];
+#pragma unroll
+    for (int e = 0; e < kNormPer; e++) {
+        const int c = threadIdx.x + e * 256;
+        const bool ok = c < hidden;
+        yv[e] = ok ? y[c] : 0.f, xv[e] = ok ? x[c] : 0.f, wp[e] = ok ? w_post[c] : 0.f, wn[e] = ok ? w_next[c] : 0.f;
+    }
+    float sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < kNormPer; e++) sq += yv[e] * yv[e];
+    const float inv = rsqrtf(block_sum(sq, red) / (float)hidden + eps);
+    float sq2 = 0.f;
+#pragma unroll
+    for (int e = 0; e < kNormPer; e++) {
+        xv[e] = xv[e] + yv[e] * inv * wp[e];
+        sq2 += xv[e] * xv[e];
+    }
+    const float inv2 = rsqrtf(block_sum(sq2, red) / (float)hidden + eps);
+#pragma unroll
+    for (int e = 0; e < kNormPer; e++) {
+        const int c = threadIdx.x + e * 256;
+        if (c < hidden) x[c] = xv[e], xn[c] = xv[e] * inv2 * wn[e];
+    }
+}
+
+// One workgroup per head of the fused qkv vector: q heads and k heads get a per-head RMS norm and
+// the half-split rotary embedding at `pos`; k and v go to the f16 cache row `pos`; q stays f32.
+__global__ void __launch_bounds__(256)
+dec_qkv_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
+               const float *__restrict__ k_norm, int n_q, int n_kv, int hd, float eps, float theta, int max_seq,
+               float *__restrict__ q_out, __half *__restrict__ k_cache, __half *__restrict__ v_cache) {
+    __shared__ float red[4];
+    __shared__ float buf[512];
+    const int head = blockIdx.x;
+    const int pos = st->pos;
+    const float *src = qkv + (size_t)head * hd;
+    const bool is_q = head < n_q, is_k = !is_q && head < n_q + n_kv;
+    if (!is_q && !is_k) {  // a value head: straight into the cache
+        const int kvh = head - n_q - n_kv;
+        for (int d = threadIdx.x; d < hd; d += 256)
+            v_cache[((size_t)kvh * max_seq + pos) * hd + d] = __float2half(src[d]);
+        return;
+    }
+    const float *w = is_q ? q_norm : k_norm;
+    float sq = 0.f;
+    for (int d = threadIdx.x; d < hd; d += 256) sq += src[d] * src[d];
+    const float inv = rsqrtf(block_sum(sq, red) / (float)hd + eps);
+    for (int d = threadIdx.x; d < hd; d += 256) buf[d] = src[d] * inv * w[d];
+    __syncthreads();
+    const int half = hd / 2;
+    for (int d = threadIdx.x; d < hd; d += 256) {
+        const int j = d < half ? d : d - half;
+        const float ang = (float)pos * powf(theta, -2.f * (float)j / (float)hd);
+        const float c = cosf(ang), s = sinf(ang);
+        const float v = d < half ? buf[d] * c - buf[d + half] * s : buf[d] * c + buf[d - half] * s;
+        if (is_q)
+            q_out[(size_t)head * hd + d] = v;
+        else
+            k_cache[((size_t)(head - n_q) * max_seq + pos) * hd + d] = __float2half(v);
+    }
+}
+
+// Decode attention, split over the context: workgroup `split` of kv head `kvh` owns kAttnChunk
+// positions and serves all G query heads of the group from one read of K and V. Every load of the
+// chunk is independent of every other and is issued up front (one 32-byte piece of a key row per
+// thread; the chunk's values of one channel per thread), so a workgroup costs about two memory
+// round trips. It writes the chunk's running max, sum and unnormalised output;
+// dec_attn_merge_kernel joins them.
+constexpr int kAttnChunk = 16;
+constexpr int kMaxGroup = 8;
+__global__ void __launch_bounds__(256)
+dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const __half *__restrict__ k_cache,
+                        const __half *__restrict__ v_cache, int n_q, int n_kv, int hd, int max_seq, float scale,
+                        float *__restrict__ part_ml, float *__restrict__ part_o) {
+    __shared__ float qs[kMaxGroup * 512];
+    __shared__ float sc[kMaxGroup][kAttnChunk];
+    const int split = blockIdx.x, kvh = blockIdx.y, nsplit = gridDim.x;
+    const int G = n_q / n_kv;
+    const int total = st->pos + 1;  // the step's own key is already in the cache
+    const int t0 = split * kAttnChunk;
+    const int tid = threadIdx.x;
+    const int cnt = min(kAttnChunk, total - t0);
+    float *ml = part_ml + ((size_t)kvh * nsplit + split) * G * 2;
+    if (cnt <= 0) {  // nothing here yet: a neutral partial
+        if (tid < G) ml[tid * 2] = -3.0e38f, ml[tid * 2 + 1] = 0.f;
+        return;
+    }
+    // values first: thread d owns channel d (and d + 256) of every row of the chunk
+    float vreg[2][kAttnChunk];
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int d = tid + c * 256;
+#pragma unroll
+        for (int t = 0; t < kAttnChunk; t++) {
+            const int tt = min(t, cnt - 1);
+            vreg[c][t] = d < hd ? __half2float(v_cache[((size_t)kvh * max_seq + t0 + tt) * hd + d]) : 0.f;
+        }
+    }
+    // keys: 16 threads per position, 16 channels (32 bytes) each per pass over the head
+    const int p = tid >> 4, seg = tid & 15;
+    const int pp = min(p, cnt - 1);
+    float dot[kMaxGroup];
+#pragma unroll
+    for (int g = 0; g < kMaxGroup; g++) dot[g] = 0.f;
+    for (int i = tid; i < G * hd; i += 256) qs[i] = q[(size_t)kvh * G * hd + i];
+    __syncthreads();
+    for (int c0 = seg * 16; c0 < hd; c0 += 256) {
+        const uint4 *kr = reinterpret_cast<const uint4 *>(k_cache + ((size_t)kvh * max_seq + t0 + pp) * hd + c0);
+        const uint4 ka = kr[0], kb = kr[1];
+        const __half2 *h2a = reinterpret_cast<const __half2 *>(&ka), *h2b = reinterpret_cast<const __half2 *>(&kb);
+        float kf[16];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            kf[2 * e] = __low2float(h2a[e]), kf[2 * e + 1] = __high2float(h2a[e]);
+            kf[8 + 2 * e] = __low2float(h2b[e]), kf[8 + 2 * e + 1] = __high2float(h2b[e]);
+        }
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; g++) {
+            if (g < G) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) dot[g] += qs[g * hd + c0 + e] * kf[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < kMaxGroup; g++) {
+        if (g < G) {
+            float v = dot[g];
+            v += __shfl_xor(v, 1, 64);
+            v += __shfl_xor(v, 2, 64);
+            v += __shfl_xor(v, 4, 64);
+            v += __shfl_xor(v, 8, 64);
+            if (seg == 0) sc[g][p] = v * scale;
+        }
+    }
+    __syncthreads();
+    // softmax pieces: thread g handles head g (the chunk is 16 values)
+    if (tid < G) {
+        float m = -3.0e38f;
+        for (int t = 0; t < cnt; t++) m = fmaxf(m, sc[tid][t]);
+        float l = 0.f;
+        for (int t = 0; t < kAttnChunk; t++) {
+            const float pv = t < cnt ? __expf(sc[tid][t] - m) : 0.f;
+            sc[tid][t] = pv;
+            l += pv;
+        }
+        ml[tid * 2] = m, ml[tid * 2 + 1] = l;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int d = tid + c * 256;
+        if (d < hd) {
+            for (int g = 0; g < G; g++) {
+                float o = 0.f;
+#pragma unroll
+                for (int t = 0; t < kAttnChunk; t++) o += sc[g][t] * vreg[c][t];
+                part_o[(((size_t)kvh * nsplit + split) * G + g) * hd + d] = o;
+            }
+        }
+    }
+}
+
+// one workgroup per query head: the weights exp(m_s - m) of the live chunks are formed once,
+// then every thread sums its channel over the chunks
+__global__ void __launch_bounds__(256)
+dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, const float *__restrict__ part_o, int n_q,
+                      int n_kv, int hd, int nsplit, float *__restrict__ out) {
+    extern __shared__ float wgt[];  // [nsplit]
+    __shared__ float red[4];
+    const int head = blockIdx.x;
+    const int G = n_q / n_kv, kvh = head / G, g = head % G;
+    const int live = min(nsplit, (st->pos + kAttnChunk) / kAttnChunk);  // chunks holding at least one position
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float m = -3.0e38f;
+    for (int s = tid; s < live; s += 256) m = fmaxf(m, part_ml[(((size_t)kvh * nsplit + s) * G + g) * 2]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float l = 0.f;
+    for (int s = tid; s < live; s += 256) {
+        const float *p = part_ml + (((size_t)kvh * nsplit + s) * G + g) * 2;
+        const float e = __expf(p[0] - m);
+        wgt[s] = e;
+        l += p[1] * e;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
+    if (lane == 0) red[wave] = l;
+    __syncthreads();
+    l = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = 1.f / l;
+    for (int d = tid; d < hd; d += 256) {
+        float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+        int s = 0;
+        for (; s + 4 <= live; s += 4) {
+            const float *base = part_o + (((size_t)kvh * nsplit + s) * G + g) * hd + d;
+            const size_t step = (size_t)G * hd;
+            o0 += base[0] * wgt[s];
+            o1 += base[step] * wgt[s + 1];
+            o2 += base[2 * step] * wgt[s + 2];
+            o3 += base[3 * step] * wgt[s + 3];
+        }
+        for (; s < live; s++) o0 += part_o[(((size_t)kvh * nsplit + s) * G + g) * hd + d] * wgt[s];
+        out[(size_t)head * hd + d] = ((o0 + o1) + (o2 + o3)) * inv;
+    }
+}
+
+// h[i] = gelu_tanh(gu[i]) * gu[ffn + i]
+__global__ void __launch_bounds__(256) dec_gelu_mul_kernel(const float *__restrict__ gu, int ffn, float *__restrict__ h) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= ffn) return;
+    const float v = gu[i];
+    const float g = 0.5f * v * (1.f + tanhf(0.79788456080286536f * fmaf(0.044715f, v * v * v, v)));
+    h[i] = g * gu[ffn + i];
+}
+
+// argmax, smallest index on ties: per-workgroup candidates, then one workgroup picks and advances the state
+__global__ void __launch_bounds__(256)
+dec_argmax_partial_kernel(const float *__restrict__ logits, int n, float *__restrict__ pv, int *__restrict__ pi) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    float best = -3.4e38f;
+    int bi = 0x7fffffff;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+        const float v = logits[i];
+        if (v > best || (v == best && i < bi)) best = v, bi = i;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (ov > best || (ov == best && oi < bi)) best = ov, bi = oi;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) sv[wave] = best, si[wave] = bi;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++)
+            if (sv[w] > best || (sv[w] == best && si[w] < bi)) best = sv[w], bi = si[w];
+        pv[blockIdx.x] = best, pi[blockIdx.x] = bi;
+    }
+}
+
+__global__ void __launch_bounds__(64)
+dec_argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int nparts, DecState *st,
+                        int32_t *__restrict__ history, int max_hist) {
+    float best = -3.4e38f;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < nparts; i += 64) {
+        if (pv[i] > best || (pv[i] == best && pi[i] < bi)) best = pv[i], bi = pi[i];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (ov > best || (ov == best && oi < bi)) best = ov, bi = oi;
+    }
+    if (threadIdx.x == 0) {
+        const int pos = st->pos;
+        if (pos < max_hist) history[pos] = bi;
+        st->token = bi;
+        st->pos = pos + 1;
+    }
+}
+
+__global__ void dec_set_state_kernel(DecState *st, int token, int pos) {
+    if (threadIdx.x == 0) st->token = token, st->pos = pos;
+}
+
+}  // namespace hipc
+
+using namespace hipc;
+
+struct DecLayer {
+    hipc_nbits_weight *qkv = nullptr, *o = nullptr, *gate_up = nullptr, *down = nullptr;
+    float *norm[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};  // input, post_attn, pre_ffn, post_ffn, q, k
+    __half *k_cache = nullptr, *v_cache = nullptr;
+};
+
+struct hipc_decoder {
+    hipc_decoder_config cfg{};
+    std::vector<DecLayer> layers;
+    hipc_nbits_weight *lm_head = nullptr;
+    float *final_norm = nullptr;
+    uint8_t *emb_q = nullptr, *emb_zp = nullptr;
+    float *emb_scales = nullptr;
+    DecState *state = nullptr;
+    int32_t *history = nullptr;
+    float *x = nullptr, *xn = nullptr, *qkv = nullptr, *q = nullptr, *attn = nullptr, *y = nullptr, *gu = nullptr,
+          *h = nullptr, *logits = nullptr, *part_ml = nullptr, *part_o = nullptr, *am_v = nullptr;
+    int *am_i = nullptr;
+    int nsplit = 0;
+    std::vector<void *> owned;
+};
+
+namespace {
+
+constexpr int kArgmaxParts = 256;
+
+template <typename T>
+int dev_alloc(hipc_ctx *ctx, hipc_decoder *d, T **p, size_t count) {
+    HIPC_TRY(ctx, hipMalloc(reinterpret_cast<void **>(p), std::max<size_t>(count * sizeof(T), 16)));
+    d->owned.push_back(*p);
+    return HIPC_OK;
+}
+
+bool complete(const hipc_decoder *d) {
+    if (!d->lm_head || !d->final_norm || !d->emb_q) return false;
+    for (const DecLayer &l : d->layers) {
+        if (!l.qkv || !l.o || !l.gate_up || !l.down) return false;
+        for (float *n : l.norm)
+            if (!n) return false;
+    }
+    return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_decoder **out) {
+    if (!ctx || !cfg || !out) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    *out = nullptr;
+    HIPC_REFUSE(ctx, ctx->capturing, "decoder create while a capture is open");
+    const hipc_decoder_config &c = *cfg;
+    HIPC_REQUIRE(ctx, c.n_layers > 0 && c.hidden > 0 && c.ffn > 0 && c.n_q_heads > 0 && c.n_kv_heads > 0 && c.head_dim > 0 &&
+                          c.vocab > 0 && c.max_seq > 0, "decoder: non-positive dimension");
+    HIPC_REQUIRE(ctx, c.n_q_heads % c.n_kv_heads == 0 && c.n_q_heads / c.n_kv_heads <= kMaxGroup,
+                 "decoder: %d query heads over %d kv heads (at most %d per group)", c.n_q_heads, c.n_kv_heads, kMaxGroup);
+    HIPC_REQUIRE(ctx, c.head_dim % 64 == 0 && c.head_dim <= 512, "decoder: head_dim %d must be a multiple of 64, at most 512", c.head_dim);
+    HIPC_REQUIRE(ctx, is_pow2(c.block_size) && c.block_size >= 32, "decoder: block_size %d", c.block_size);
+    HIPC_REQUIRE(ctx, c.hidden <= 256 * kNormPer, "decoder: hidden %d exceeds %d", c.hidden, 256 * kNormPer);
+    HIPC_REQUIRE(ctx, c.max_seq <= 8192 * kAttnChunk, "decoder: max_seq %d exceeds %d", c.max_seq, 8192 * kAttnChunk);
+    hipc_decoder *d = new hipc_decoder();
+    d->cfg = c;
+    d->layers.resize(c.n_layers);
+    d->nsplit = (int)ceil_div(c.max_seq, kAttnChunk);
+    const size_t kv = (size_t)c.n_kv_heads * c.max_seq * c.head_dim;
+    const int G = c.n_q_heads / c.n_kv_heads;
+    int rc = HIPC_OK;
+    auto A = [&](auto **p, size_t n) { if (rc == HIPC_OK) rc = dev_alloc(ctx, d, p, n); };
+    for (DecLayer &l : d->layers) {
+        A(&l.k_cache, kv);
+        A(&l.v_cache, kv);
+    }
+    A(&d->state, 1), A(&d->history, (size_t)c.max_seq);
+    A(&d->x, c.hidden), A(&d->xn, c.hidden), A(&d->qkv, (size_t)(c.n_q_heads + 2 * c.n_kv_heads) * c.head_dim);
+    A(&d->q, (size_t)c.n_q_heads * c.head_dim), A(&d->attn, (size_t)c.n_q_heads * c.head_dim), A(&d->y, c.hidden);
+    A(&d->gu, (size_t)2 * c.ffn), A(&d->h, c.ffn), A(&d->logits, c.vocab);
+    A(&d->part_ml, (size_t)c.n_kv_heads * d->nsplit * G * 2), A(&d->part_o, (size_t)c.n_kv_heads * d->nsplit * G * c.head_dim);
+    A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
+    if (rc == HIPC_OK) {
+        for (DecLayer &l : d->layers) {  // an unwritten cache row must not hold NaN bit patterns
+            if (hipMemsetAsync(l.k_cache, 0, kv * 2, ctx->stream) != hipSuccess || hipMemsetAsync(l.v_cache, 0, kv * 2, ctx->stream) != hipSuccess)
+                rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the KV cache");
+        }
+        dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, 0, 0);
+    }
+    if (rc != HIPC_OK) {
+        for (void *p : d->owned) (void)hipFree(p);
+        delete d;
+        return rc;
+    }
+    *out = d;
+    return HIPC_OK;
+}
+
+void hipc_decoder_destroy(hipc_ctx *ctx, hipc_decoder *d) {
+    if (!ctx || !d) return;
+    Guard g(ctx);
+    for (DecLayer &l : d->layers) {
+        nbits_release(ctx, l.qkv), nbits_release(ctx, l.o), nbits_release(ctx, l.gate_up), nbits_release(ctx, l.down);
+    }
+    nbits_release(ctx, d->lm_head);
+    for (void *p : d->owned) ctx->deferred.push_back(p);
+    delete d;
+}
+
+int hipc_decoder_set_linear(hipc_ctx *ctx, hipc_decoder *d, int layer, int which, const void *B, size_t b_len,
+                            const void *scales, size_t scales_len, const void *zp, size_t zp_len) {
+    if (!ctx || !d) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    const hipc_decoder_config &c = d->cfg;
+    const int64_t qd = (int64_t)c.n_q_heads * c.head_dim, kvd = (int64_t)c.n_kv_heads * c.head_dim;
+    int64_t K = 0, N = 0;
+    hipc_nbits_weight **slot = nullptr;
+    if (which == HIPC_DEC_LM_HEAD) {
+        K = c.hidden, N = c.vocab, slot = &d->lm_head;
+    } else {
+        HIPC_REQUIRE(ctx, layer >= 0 && layer < c.n_layers, "decoder: layer %d out of range", layer);
+        DecLayer &l = d->layers[layer];
+        switch (which) {
+            case HIPC_DEC_QKV: K = c.hidden, N = qd + 2 * kvd, slot = &l.qkv; break;
+            case HIPC_DEC_O: K = qd, N = c.hidden, slot = &l.o; break;
+            case HIPC_DEC_GATE_UP: K = c.hidden, N = 2 * (int64_t)c.ffn, slot = &l.gate_up; break;
+            case HIPC_DEC_DOWN: K = c.ffn, N = c.hidden, slot = &l.down; break;
+            default: return fail(ctx, HIPC_ERR_INVALID, "decoder: unknown linear %d", which);
+        }
+    }
+    if (*slot) nbits_release(ctx, *slot), *slot = nullptr;
+    return nbits_prepack(ctx, B, b_len, scales, HIPC_F32, scales_len, zp, zp_len, K, N, c.block_size, slot);
+}
+
+int hipc_decoder_set_norm(hipc_ctx *ctx, hipc_decoder *d, int layer, int which, const void *w) {
+    if (!ctx || !d || !w) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    const hipc_decoder_config &c = d->cfg;
+    float **slot = nullptr;
+    size_t n = c.hidden;
+    if (which == HIPC_DEC_NORM_FINAL) {
+        slot = &d->final_norm;
+    } else {
+        HIPC_REQUIRE(ctx, layer >= 0 && layer < c.n_layers, "decoder: layer %d out of range", layer);
+        HIPC_REQUIRE(ctx, which >= 0 && which < 6, "decoder: unknown norm %d", which);
+        slot = &d->layers[layer].norm[which];
+        if (which == HIPC_DEC_NORM_Q || which == HIPC_DEC_NORM_K) n = c.head_dim;
+    }
+    if (!*slot) {
+        int rc = dev_alloc(ctx, d, slot, n);
+        if (rc != HIPC_OK) return rc;
+    }
+    HIPC_TRY(ctx, hipMemcpyAsync(*slot, w, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+    return HIPC_OK;
+}
+
+int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *d, const void *B, size_t b_len, const void *scales,
+                               size_t scales_len, const void *zp, size_t zp_len) {
+    if (!ctx || !d || !B || !scales) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    const hipc_decoder_config &c = d->cfg;
+    const size_t nb = (size_t)ceil_div(c.hidden, c.block_size);
+    const size_t qb = (size_t)c.vocab * nb * c.block_size / 2, sb = (size_t)c.vocab * nb, zb = (size_t)c.vocab * ((nb + 1) / 2);
+    HIPC_REQUIRE(ctx, b_len >= qb && scales_len >= sb && (!zp || zp_len >= zb), "decoder: embedding table is short");
+    if (!d->emb_q) {
+        int rc = dev_alloc(ctx, d, &d->emb_q, qb);
+        if (rc == HIPC_OK) rc = dev_alloc(ctx, d, &d->emb_scales, sb);
+        if (rc == HIPC_OK && zp) rc = dev_alloc(ctx, d, &d->emb_zp, zb);
+        if (rc != HIPC_OK) return rc;
+    }
+    HIPC_TRY(ctx, hipMemcpyAsync(d->emb_q, B, qb, hipMemcpyDeviceToDevice, ctx->stream));
+    HIPC_TRY(ctx, hipMemcpyAsync(d->emb_scales, scales, sb * 4, hipMemcpyDeviceToDevice, ctx->stream));
+    if (zp) HIPC_TRY(ctx, hipMemcpyAsync(d->emb_zp, zp, zb, hipMemcpyDeviceToDevice, ctx->stream));
+    return HIPC_OK;
+}
+
+int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *d, int32_t token, int32_t pos) {
+    if (!ctx || !d) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, token >= 0 && token < d->cfg.vocab && pos >= 0 && pos < d->cfg.max_seq, "decoder: bad token %d or position %d", token, pos);
+    dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, token, pos);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+int hipc_decoder_kv_cache(hipc_ctx *ctx, hipc_decoder *d, int layer, void **k_cache, void **v_cache) {
+    if (!ctx || !d || !k_cache || !v_cache) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, layer >= 0 && layer < d->cfg.n_layers, "decoder: layer %d out of range", layer);
+    *k_cache = d->layers[layer].k_cache, *v_cache = d->layers[layer].v_cache;
+    return HIPC_OK;
+}
+
+int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
+    if (!ctx || !d) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, complete(d), "decoder: not every weight has been set");
+    const hipc_decoder_config &c = d->cfg;
+    hipStream_t s = ctx->stream;
+    const int nb = (int)ceil_div(c.hidden, c.block_size);
+    const int heads = c.n_q_heads + 2 * c.n_kv_heads;
+    const float scale = c.attn_scale > 0.f ? c.attn_scale : 1.f / sqrtf((float)c.head_dim);
+    const int terms = 2;
+    int rc;
+    dec_embed_kernel<<<1, 256, 0, s>>>(d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
+                                       d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn);
+    HIPC_LAUNCHED(ctx);
+    for (int li = 0; li < c.n_layers; li++) {
+        DecLayer &l = d->layers[li];
+        if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.qkv, d->qkv, 1, terms)) != HIPC_OK) return rc;
+        dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
+                                             c.n_kv_heads, c.head_dim, c.rms_eps, c.rope_theta, c.max_seq, d->q, l.k_cache, l.v_cache);
+        HIPC_LAUNCHED(ctx);
+        dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
+                                                                             c.head_dim, c.max_seq, scale, d->part_ml, d->part_o);
+        HIPC_LAUNCHED(ctx);
+        dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
+                                                                                         c.head_dim, d->nsplit, d->attn);
+        HIPC_LAUNCHED(ctx);
+        if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
+        dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->xn);
+        HIPC_LAUNCHED(ctx);
+        if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.gate_up, d->gu, 1, terms)) != HIPC_OK) return rc;
+        dec_gelu_mul_kernel<<<(unsigned)ceil_div(c.ffn, 256), 256, 0, s>>>(d->gu, c.ffn, d->h);
+        HIPC_LAUNCHED(ctx);
+        if ((rc = nbits_gemv(ctx, d->h, HIPC_F32, l.down, d->y, 1, terms)) != HIPC_OK) return rc;
+        const float *next = li + 1 < c.n_layers ? d->layers[li + 1].norm[HIPC_DEC_NORM_INPUT] : d->final_norm;
+        dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->xn);
+        HIPC_LAUNCHED(ctx);
+    }
+    if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;
+    dec_argmax_partial_kernel<<<kArgmaxParts, 256, 0, s>>>(d->logits, c.vocab, d->am_v, d->am_i);
+    HIPC_LAUNCHED(ctx);
+    dec_argmax_final_kernel<<<1, 64, 0, s>>>(d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+int hipc_decoder_read(hipc_ctx *ctx, hipc_decoder *d, int32_t *token, int32_t *pos, float *logits, int32_t *history, int32_t n_history) {
+    if (!ctx || !d) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REFUSE(ctx, ctx->capturing, "decoder read while a capture is open");
+    HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    DecState st{};
+    HIPC_TRY(ctx, hipMemcpy(&st, d->state, sizeof st, hipMemcpyDeviceToHost));
+    if (token) *token = st.token;
+    if (pos) *pos = st.pos;
+    if (logits) HIPC_TRY(ctx, hipMemcpy(logits, d->logits, (size_t)d->cfg.vocab * 4, hipMemcpyDeviceToHost));
+    if (history && n_history > 0)
+        HIPC_TRY(ctx, hipMemcpy(history, d->history, (size_t)std::min<int32_t>(n_history, d->cfg.max_seq) * 4, hipMemcpyDeviceToHost));
+    return HIPC_OK;
+}
+
+}  // extern "C"

@@ -93,6 +93,15 @@ inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 inline bool is_byte_dtype(int dt) { return dt == HIPC_U8 || dt == HIPC_I8; }
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// MatMulNBits pieces other operators of the library build on (the caller holds the lock)
+int nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype, size_t scales_len,
+                  const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size, hipc_nbits_weight **out);
+void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
+// rows [0, M), M <= 16, of A against a prepacked weight; `terms` = bf16 terms per activation (2 or 3)
+int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms);
+int64_t nbits_cols(const hipc_nbits_weight *w);
+int64_t nbits_depth(const hipc_nbits_weight *w);
+
 // offsets inside ctx->params
 constexpr size_t kParamRange = 0;   // 8 B  {bits(-min), bits(max)}
 constexpr size_t kParamBytes = 256;

@@ -723,6 +723,15 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
                               hipc_nbits_weight **out) {
     if (!ctx || !out) return HIPC_ERR_INVALID;
     Guard g(ctx);
+    return hipc::nbits_prepack(ctx, B, b_len, scales, scale_dtype, scales_len, zp, zp_len, K, N, block_size, out);
+}
+
+}  // extern "C"
+
+// The same operations for callers inside the library that already hold the context's lock.
+int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype,
+                        size_t scales_len, const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size,
+                        hipc_nbits_weight **out) {
     *out = nullptr;
     HIPC_REFUSE(ctx, ctx->capturing, "MatMulNBits prepack while a capture is open");
     int rc = check_nbits_shape(ctx, 1, K, N, block_size, b_len, scales_len, zp, zp_len, scale_dtype);
@@ -780,14 +789,28 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
     return HIPC_OK;
 }
 
-void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w) {
-    if (!ctx || !w) return;
-    Guard g(ctx);
+void hipc::nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w) {
+    if (!w) return;
     // enqueued work may still read the weight: release at the next flush
     if (w->Wq) ctx->deferred.push_back(w->Wq);
     if (w->Sc) ctx->deferred.push_back(w->Sc);
     if (w->Zb) ctx->deferred.push_back(w->Zb);
     delete w;
+}
+
+int hipc::nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms) {
+    return launch_gemv(ctx, A, a_dtype, w, Y, M, terms);
+}
+
+int64_t hipc::nbits_cols(const hipc_nbits_weight *w) { return w->N; }
+int64_t hipc::nbits_depth(const hipc_nbits_weight *w) { return w->K; }
+
+extern "C" {
+
+void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w) {
+    if (!ctx || !w) return;
+    Guard g(ctx);
+    hipc::nbits_release(ctx, w);
 }
 
 size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w) { return w ? w->bytes : 0; }

@@ -44,6 +44,13 @@ def library_path() -> str:
     return os.path.join(_HERE, "libhipcompute.so")
 
 
+class DecoderConfig(C.Structure):
+    """``hipc_decoder_config``."""
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "ffn", "n_q_heads", "n_kv_heads", "head_dim", "vocab",
+                                         "max_seq", "block_size")] + \
+               [(n, C.c_float) for n in ("rms_eps", "rope_theta", "attn_scale", "embed_scale")]
+
+
 _lib = None
 
 # name -> (restype, argtypes); every symbol include/hipcompute.h declares
@@ -91,6 +98,15 @@ SIGNATURES = {
     "hipc_conv_integer": (_int, [_vp, _vp, _int, _vp, _vp, _vp, C.POINTER(ConvGeom), _vp]),
     "hipc_qlinear_conv": (_int, [_vp, _vp, _int, _f, C.c_int32, _vp, C.POINTER(_f), _i64, C.c_int32, _f,
                                  C.c_int32, _int, _vp, C.POINTER(ConvGeom), _vp]),
+    "hipc_decoder_create": (_int, [_vp, C.POINTER(DecoderConfig), C.POINTER(_vp)]),
+    "hipc_decoder_destroy": (None, [_vp, _vp]),
+    "hipc_decoder_set_linear": (_int, [_vp, _vp, _int, _int, _vp, _sz, _vp, _sz, _vp, _sz]),
+    "hipc_decoder_set_norm": (_int, [_vp, _vp, _int, _int, _vp]),
+    "hipc_decoder_set_embedding": (_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz]),
+    "hipc_decoder_reset": (_int, [_vp, _vp, C.c_int32, C.c_int32]),
+    "hipc_decoder_kv_cache": (_int, [_vp, _vp, _int, C.POINTER(_vp), C.POINTER(_vp)]),
+    "hipc_decoder_step": (_int, [_vp, _vp]),
+    "hipc_decoder_read": (_int, [_vp, _vp, C.POINTER(C.c_int32), C.POINTER(C.c_int32), _vp, _vp, C.c_int32]),
 }
 
 

@@ -1,0 +1,108 @@
+"""numpy restatement of one decoder-only decode step -- TEST INFRASTRUCTURE ONLY.
+
+Follows the reference operators a gemma3-1b graph is made of (paths relative to
+crates/onnx-vulkan-core/src in the reference tree):
+  SimplifiedLayerNormalization  shaders/normalization.rs:109-181   x * rsqrt(mean(x^2) + eps) * w
+  GroupQueryAttention           shaders/attention.rs:128-317       half-split rotary (:157-167), cache
+                                                                   append, scale * q.k^T (:264), softmax, p.V
+  Gelu approximate="tanh"       interp.rs:9020-9027
+  GatherBlockQuantized          shaders/gather_block_quantized.rs:26-57
+  MatMulNBits                   oracle.matmul_nbits (the C oracle)
+All arithmetic is float32; the KV cache is rounded to float16 as the configuration asks.
+Pin status: composition of operators pinned elsewhere; the glue itself (norm, rotary, softmax,
+gelu) is checked in tests/test_oracle_pins.py against float64 closed forms.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import matmul_nbits
+
+QKV, O, GATE_UP, DOWN, LM_HEAD = 0, 1, 2, 3, 4
+NORM_INPUT, NORM_POST_ATTN, NORM_PRE_FFN, NORM_POST_FFN, NORM_Q, NORM_K, NORM_FINAL = range(7)
+
+f32 = np.float32
+
+
+def rmsnorm(x, w, eps):
+    x = x.astype(f32)
+    ms = f32(np.sum(x * x, dtype=f32) / f32(x.size))
+    return (x * f32(1.0 / np.sqrt(ms + f32(eps))) * w).astype(f32)
+
+
+def rope_half(x, pos, theta):
+    """Half-split rotary: channel j of the first half pairs with j + half (attention.rs:157-167)."""
+    hd = x.size
+    half = hd // 2
+    j = np.arange(half, dtype=f32)
+    ang = (f32(pos) * np.power(f32(theta), f32(-2.0) * j / f32(hd))).astype(f32)
+    c, s = np.cos(ang).astype(f32), np.sin(ang).astype(f32)
+    out = np.empty(hd, f32)
+    out[:half] = x[:half] * c - x[half:] * s
+    out[half:] = x[half:] * c + x[:half] * s
+    return out
+
+
+def gelu_tanh(v):
+    v = v.astype(f32)
+    return (f32(0.5) * v * (f32(1.0) + np.tanh(f32(0.79788456080286536) * (f32(0.044715) * v * v * v + v)))).astype(f32)
+
+
+def gather_block_quantized(table, row, hidden, bs):
+    B, scales, zp = table
+    nb = -(-hidden // bs)
+    q = B[row].reshape(-1)
+    nib = np.empty(nb * bs, np.int32)
+    nib[0::2], nib[1::2] = q & 15, q >> 4
+    z = np.empty(2 * ((nb + 1) // 2), np.int32)
+    z[0::2], z[1::2] = zp[row] & 15, zp[row] >> 4
+    blk = np.arange(hidden) // bs
+    return ((nib[:hidden] - z[blk]).astype(f32) * scales.reshape(-1, nb)[row][blk]).astype(f32)
+
+
+class Decoder:
+    def __init__(self, weights, max_seq):
+        self.w, self.cfg = weights, weights.cfg
+        c = self.cfg
+        self.k = np.zeros((c["n_layers"], c["n_kv_heads"], max_seq, c["head_dim"]), np.float16)
+        self.v = np.zeros_like(self.k)
+
+    def _lin(self, x, li, which):
+        B, scales, zp = self.w.linears[(li, which)]
+        n_rows = B.shape[0]
+        return matmul_nbits(x.reshape(1, -1).astype(f32), B, scales, zp, x.size, n_rows, self.cfg["block_size"]).reshape(-1)
+
+    def step(self, token, pos):
+        c, w = self.cfg, self.w
+        hd, nq, nkv = c["head_dim"], c["n_q_heads"], c["n_kv_heads"]
+        scale = f32(c["attn_scale"] if c["attn_scale"] > 0 else 1.0 / np.sqrt(hd))
+        x = (gather_block_quantized(w.embedding, token, c["hidden"], c["block_size"]) * f32(c["embed_scale"])).astype(f32)
+        xn = rmsnorm(x, w.norms[(0, NORM_INPUT)], c["rms_eps"])
+        for li in range(c["n_layers"]):
+            qkv = self._lin(xn, li, QKV)
+            q = qkv[: nq * hd].reshape(nq, hd)
+            k = qkv[nq * hd: (nq + nkv) * hd].reshape(nkv, hd)
+            v = qkv[(nq + nkv) * hd:].reshape(nkv, hd)
+            q = np.stack([rope_half(rmsnorm(q[h], w.norms[(li, NORM_Q)], c["rms_eps"]), pos, c["rope_theta"]) for h in range(nq)])
+            for h in range(nkv):
+                self.k[li, h, pos] = rope_half(rmsnorm(k[h], w.norms[(li, NORM_K)], c["rms_eps"]), pos, c["rope_theta"]).astype(np.float16)
+                self.v[li, h, pos] = v[h].astype(np.float16)
+            attn = np.empty((nq, hd), f32)
+            g = nq // nkv
+            for h in range(nq):
+                K = self.k[li, h // g, : pos + 1].astype(f32)
+                V = self.v[li, h // g, : pos + 1].astype(f32)
+                s = (K @ q[h]) * scale
+                p = np.exp(s - s.max()).astype(f32)
+                attn[h] = (p @ V) / f32(p.sum(dtype=f32))
+            y = self._lin(attn.reshape(-1), li, O)
+            x = (x + rmsnorm(y, w.norms[(li, NORM_POST_ATTN)], c["rms_eps"])).astype(f32)
+            xn = rmsnorm(x, w.norms[(li, NORM_PRE_FFN)], c["rms_eps"])
+            gu = self._lin(xn, li, GATE_UP)
+            h_ = (gelu_tanh(gu[: c["ffn"]]) * gu[c["ffn"]:]).astype(f32)
+            y = self._lin(h_, li, DOWN)
+            x = (x + rmsnorm(y, w.norms[(li, NORM_POST_FFN)], c["rms_eps"])).astype(f32)
+            nxt = w.norms[(li + 1, NORM_INPUT)] if li + 1 < c["n_layers"] else w.norms[(0, NORM_FINAL)]
+            xn = rmsnorm(x, nxt, c["rms_eps"])
+        logits = self._lin(xn, 0, LM_HEAD)
+        return logits, int(np.argmax(logits))

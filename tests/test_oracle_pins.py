@@ -303,3 +303,37 @@ def test_conv_geometry_known_answers(oracle):
     assert oracle.same_pads(224, 7, 2, 1, upper=True) == (2, 3)      # odd total: the extra goes last
     assert oracle.same_pads(224, 7, 2, 1, upper=False) == (3, 2)
     assert oracle.same_pads(10, 1, 1, 1) == (0, 0)
+
+
+# ------------------------------------------------------------- decoder glue
+
+def test_decoder_glue_against_float64_closed_forms(oracle):
+    from oracle import decoder as od
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal(96).astype(np.float32) * 3
+    w = rng.standard_normal(96).astype(np.float32)
+    want = x.astype(np.float64) / np.sqrt(np.mean(x.astype(np.float64) ** 2) + 1e-6) * w
+    assert np.allclose(od.rmsnorm(x, w, 1e-6), want, rtol=2e-6, atol=1e-6)
+    assert np.allclose(od.rmsnorm(np.full(8, 2.0, np.float32), np.ones(8, np.float32), 0.0), 1.0)   # known answer
+    # rotary: position 0 is the identity, a rotation keeps the norm of every (j, j + half) pair, and
+    # rotating by p then by q (same frequencies) equals rotating by p + q
+    v = rng.standard_normal(64).astype(np.float32)
+    assert np.array_equal(od.rope_half(v, 0, 10000.0), v)
+    r = od.rope_half(v, 7, 10000.0)
+    assert np.allclose(r[:32] ** 2 + r[32:] ** 2, v[:32] ** 2 + v[32:] ** 2, rtol=1e-5)
+    assert np.allclose(od.rope_half(r, 5, 10000.0), od.rope_half(v, 12, 10000.0), atol=2e-5)
+    assert np.allclose(od.rope_half(np.concatenate([np.ones(1), np.zeros(1)]).astype(np.float32), 1, 10000.0),
+                       [np.cos(1.0), np.sin(1.0)], atol=1e-6)                                       # pair (0, half)
+    g = od.gelu_tanh(np.array([-3.0, -1.0, 0.0, 0.5, 2.0], np.float32))
+    t = np.array([-3.0, -1.0, 0.0, 0.5, 2.0])
+    assert np.allclose(g, 0.5 * t * (1 + np.tanh(np.sqrt(2 / np.pi) * (t + 0.044715 * t ** 3))), atol=1e-6)
+
+
+def test_gather_block_quantized_is_a_row_of_the_dequantised_table(oracle, pkg):
+    from oracle import decoder as od
+    a, nib, zp, scale = rc.matmul_nbits_case(1, 100, 9, 32)
+    table = (pkg.synth.pack_nibbles(nib, 32), scale.reshape(-1), pkg.synth.pack_zero_points(zp))
+    for row in (0, 4, 8):
+        blk = np.arange(100) // 32
+        want = (nib[row].astype(np.float32) - zp[row][blk]) * scale[row][blk]
+        assert np.array_equal(od.gather_block_quantized(table, row, 100, 32), want)
