@@ -35,6 +35,7 @@ LAYER_LINEARS = [(1152, 1024, 1), (1152, 256, 2), (1024, 1152, 1), (1152, 6912, 
 LM_HEAD = (1152, 262144)
 N_LAYERS = 26
 BS = 32
+IN_GRAPH = 16   # instances of a small operator per captured graph: amortises the graph launch
 
 
 def gemv_bytes(K, N, bs=BS, with_zp=True, elt=4):
@@ -116,8 +117,10 @@ def bench_lm_head_roofline(pkg, ctx, copies=3):
     """The dominant kernel: lm_head GEMV rotating over `copies` distinct weights (~200 MB each)."""
     K, N = LM_HEAD
     s = GemvSet(pkg, ctx, [LM_HEAD] * copies, seed=7000)
+    s.items = s.items * 4                     # 4 passes over the ring per graph
     g = s.capture()
-    med, mn = median_ns(ctx, g, launches_per_graph=copies, samples=15, reps=5)
+    med, mn = median_ns(ctx, g, launches_per_graph=copies * 4, samples=15, reps=2)
+    s.items = s.items[:copies]
     per = gemv_bytes(K, N)
     s.destroy()
     return dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS,
@@ -128,8 +131,10 @@ def bench_lm_head_roofline(pkg, ctx, copies=3):
 def bench_single_gemv(pkg, ctx, K, N, cold_copies):
     per = gemv_bytes(K, N)
     hot = GemvSet(pkg, ctx, [(K, N)], seed=8000)
+    hot.items = hot.items * IN_GRAPH          # the same weight again and again: cache-resident
     g = hot.capture()
-    hot_ns, _ = median_ns(ctx, g, 1, samples=20, reps=50)
+    hot_ns, _ = median_ns(ctx, g, IN_GRAPH, samples=20, reps=4)
+    hot.items = hot.items[:1]
     hot.destroy()
     cold = GemvSet(pkg, ctx, [(K, N)] * cold_copies, seed=8100)
     g = cold.capture()
@@ -151,9 +156,10 @@ def bench_int8_ffn(pkg, ctx):
     ops.dynamic_quantize_linear_device(ctx, dX, x.size, dA, dP, dP.at(4))
     ctx.flush()
     ctx.capture_begin()
-    ops.dynamic_quantize_linear_device(ctx, dX, x.size, dA, dP, dP.at(4))
+    for _ in range(IN_GRAPH):
+        ops.dynamic_quantize_linear_device(ctx, dX, x.size, dA, dP, dP.at(4))
     g = ctx.capture_end()
-    ns, _ = median_ns(ctx, g, 1, samples=20, reps=20)
+    ns, _ = median_ns(ctx, g, IN_GRAPH, samples=20, reps=4)
     ctx.graph_destroy(g)
     dql_bytes = x.size * 4 + x.size + 5
     out["dynamic_quantize_linear_1000x1024"] = dict(us=ns / 1e3, gbs=dql_bytes / ns, frac_hbm=dql_bytes / ns / HBM_PEAK_GBS)
@@ -168,9 +174,10 @@ def bench_int8_ffn(pkg, ctx):
             fn()
             ctx.flush()
             ctx.capture_begin()
-            fn()
+            for _ in range(IN_GRAPH):
+                fn()
             g = ctx.capture_end()
-            ns, mn = median_ns(ctx, g, 1, samples=20, reps=20)
+            ns, mn = median_ns(ctx, g, IN_GRAPH, samples=20, reps=4)
             ctx.graph_destroy(g)
             opsn = 2.0 * T * K * N
             byts = T * K + K * N + T * N * 4

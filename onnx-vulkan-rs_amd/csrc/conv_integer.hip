@@ -223,8 +223,7 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLds));
             lds_set = true;
         }
-        const int64_t tiles = ceil_div(ga.J, kBN) * ceil_div(ga.I, kBM);
-        const dim3 grid((unsigned)(ceil_div(tiles, 8) * 8), 1, (unsigned)g->n);
+        const dim3 grid(gemm_grid(ga), 1, (unsigned)g->n);
         if (ep.requant)
             int8_gemm_kernel<MODE_CONV, EPI_REQUANT, true><<<grid, 256, kGemmLds, ctx->stream>>>(ga);
         else

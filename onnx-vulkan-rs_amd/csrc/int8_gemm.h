@@ -49,6 +49,7 @@ struct GemmArgs {
     int dyn_zp_value, const_zp_value;
     int I, J, K, K_pad;
     int p_aligned;  // MODE_MM: rows of A can be read with 128-bit loads
+    int xcd_rows, xcd_cols;  // the 8 XCDs as a grid over the tiles (set by gemm_grid)
 
     // conv geometry (MODE_CONV); Q is [n][H][W][C]
     int C, H, W, Ho, Wo, kh, kw, sh, sw, dh, dw, pt, pl;
@@ -63,6 +64,21 @@ struct GemmArgs {
     const int32_t *qbias;                  // EPI_REQUANT int32 bias (per i in CONV)
     int y_zp, out_signed;
 };
+
+// Chooses how the 8 XCDs tile the grid of output tiles (fewest operand slabs per XCD) and
+// returns the number of workgroups to launch.
+inline unsigned gemm_grid(GemmArgs &g) {
+    const int tiles_x = (g.J + kBN - 1) / kBN, tiles_y = (g.I + kBM - 1) / kBM;
+    int best_a = 8, best_cost = 1 << 30;
+    for (int a = 1; a <= 8; a *= 2) {
+        const int b = 8 / a;
+        const int cost = (tiles_y + a - 1) / a + (tiles_x + b - 1) / b;
+        if (cost < best_cost) best_cost = cost, best_a = a;
+    }
+    g.xcd_rows = best_a, g.xcd_cols = 8 / best_a;
+    const int rows_per = (tiles_y + g.xcd_rows - 1) / g.xcd_rows, cols_per = (tiles_x + g.xcd_cols - 1) / g.xcd_cols;
+    return 8u * (unsigned)(rows_per * cols_per);
+}
 
 __device__ __forceinline__ int zp_byte(const uint8_t *ptr, int is_signed) {
     if (!ptr) return 0;
@@ -84,9 +100,9 @@ struct GemmRegs {
     uint4 p[4], q[4];
 };
 
-// ALIGNED (MODE_MM only): rows of A start on 16 bytes and K % 16 == 0, so A is read with
-// unconditional 128-bit loads (out-of-range chunks are clamped, then zeroed by a select --
-// no branch, which keeps the load counters exact and two stages in flight).
+// ALIGNED (MODE_MM only): rows of A start on 16 bytes and K % 128 == 0, so A is read with
+// unconditional 128-bit loads at base + 32-bit offset (no branch, which keeps the load counters
+// exact and two stages in flight; no per-stage address arithmetic).
 template <int MODE, int EPI, bool ALIGNED>
 __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
@@ -101,14 +117,14 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     const int img = blockIdx.z;
 
     // Tile order: consecutive workgroup ids land on different XCDs (round robin), each with
-    // its own L2. Give every XCD a contiguous run of tiles, so neighbours that share an
-    // operand slab also share a cache.
+    // its own L2. The tile grid is cut into xcd_rows x xcd_cols = 8 rectangles, one per XCD, so
+    // the operand slabs an XCD pulls through its L2 are as few as the shape allows.
     const int tiles_x = (p.J + kBN - 1) / kBN, tiles_y = (p.I + kBM - 1) / kBM;
-    const int total = tiles_x * tiles_y;
-    const int per_xcd = (total + 7) / 8;
-    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= total) return;
-    const int i0 = (logical / tiles_x) * kBM, j0 = (logical % tiles_x) * kBN;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
+    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
+    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
+    const int i0 = ty * kBM, j0 = tx * kBN;
 
     // zero points in the shifted (signed) domain
     const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
@@ -141,16 +157,27 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
         }
     }
 
+    // Byte offsets of this thread's chunks at k = 0, as 32-bit values added to a uniform base
+    // that advances with k: the loads then need no per-stage address arithmetic at all.
+    uint32_t p_off[4], q_off[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int gi = i0 + row_[u], gj = j0 + row_[u];
+        p_off[u] = MODE == MODE_CONV ? (uint32_t)gi * (uint32_t)p.K_pad + kc_[u] * 16
+                                     : (uint32_t)min(gi, p.I - 1) * (uint32_t)p.K + kc_[u] * 16;
+        q_off[u] = (uint32_t)gj * (uint32_t)p.K_pad + kc_[u] * 16;
+    }
     auto load_p = [&](int u, int k0) -> uint4 {
-        const int gi = i0 + row_[u], gk = k0 + kc_[u] * 16;
         if (MODE == MODE_CONV) {
-            return *reinterpret_cast<const uint4 *>(p.P + (size_t)gi * p.K_pad + gk);
+            return *reinterpret_cast<const uint4 *>(p.P + k0 + p_off[u]);
         } else if (ALIGNED) {
-            const bool ok = gi < p.I && gk < p.K;
-            const uint8_t *src = p.P + (size_t)min(gi, p.I - 1) * p.K + min(gk, p.K - 16);
-            const uint4 v = xor4(*reinterpret_cast<const uint4 *>(src), flip);
-            return make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+            // K % 128 == 0: every chunk is inside the row. Rows past I are clamped, not zeroed:
+            // the rows of a product are independent and those outputs are never stored.
+            // (the sign flip of a u8 operand is applied when the chunk is stored to LDS, so the
+            // load has no consumer until then)
+            return *reinterpret_cast<const uint4 *>(p.P + k0 + p_off[u]);
         } else {
+            const int gi = i0 + row_[u], gk = k0 + kc_[u] * 16;
             if (gi >= p.I || gk >= p.K) return make_uint4(0, 0, 0, 0);
             const uint8_t *src = p.P + (size_t)gi * p.K + gk;
             uint32_t w[4] = {0, 0, 0, 0};
@@ -162,8 +189,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     auto load_q = [&](int u, int k0) -> uint4 {
         const int gk = k0 + kc_[u] * 16;
         if (MODE == MODE_MM) {
-            const int gj = j0 + row_[u];
-            return *reinterpret_cast<const uint4 *>(p.Q + (size_t)gj * p.K_pad + gk);
+            return *reinterpret_cast<const uint4 *>(p.Q + k0 + q_off[u]);
         } else {
             const int gkc = min(gk, p.K - 16);
             const int tap = gkc / p.C, c0 = gkc - tap * p.C;
@@ -185,11 +211,18 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
 #pragma unroll
         for (int u = 0; u < 4; u++) r.q[u] = load_q(u, k0);
     };
-    auto store_regs = [&](const GemmRegs &r, int buf) {
+    // `live` false (a stage past the end, only met when the stage count is odd) stores zeros,
+    // which add nothing to the product or to the operand sums.
+    auto store_regs = [&](const GemmRegs &r, int buf, bool live) {
+        const uint32_t keep = live ? 0xffffffffu : 0u;
+        const uint32_t late_flip = (MODE == MODE_MM && ALIGNED) ? flip : 0u;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            *reinterpret_cast<uint4 *>(lds_p + buf * kBM * kPitch + row_[u] * kPitch + kc_[u] * 16) = r.p[u];
-            *reinterpret_cast<uint4 *>(lds_q + buf * kBN * kPitch + row_[u] * kPitch + kc_[u] * 16) = r.q[u];
+            *reinterpret_cast<uint4 *>(lds_p + buf * kBM * kPitch + row_[u] * kPitch + kc_[u] * 16) =
+                make_uint4((r.p[u].x ^ late_flip) & keep, (r.p[u].y ^ late_flip) & keep, (r.p[u].z ^ late_flip) & keep,
+                           (r.p[u].w ^ late_flip) & keep);
+            *reinterpret_cast<uint4 *>(lds_q + buf * kBN * kPitch + row_[u] * kPitch + kc_[u] * 16) =
+                make_uint4(r.q[u].x & keep, r.q[u].y & keep, r.q[u].z & keep, r.q[u].w & keep);
         }
     };
 
@@ -212,10 +245,9 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
             for (int i = 0; i < 2; i++) pf[i] = *reinterpret_cast<const uint4 *>(bp + i * 32 * kPitch + step * 32);
 #pragma unroll
             for (int j = 0; j < 2; j++) qf[j] = *reinterpret_cast<const uint4 *>(bq + j * 32 * kPitch + step * 32);
-            if (need_dyn_sum) {
+            // always taken: a branch here would cost more than the eight dot instructions
 #pragma unroll
-                for (int f = 0; f < 2; f++) dsum[f] += dot_ones(MODE == MODE_MM ? pf[f] : qf[f]);
-            }
+            for (int f = 0; f < 2; f++) dsum[f] += dot_ones(MODE == MODE_MM ? pf[f] : qf[f]);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -232,17 +264,18 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     GemmRegs r0, r1;
     load_regs(r0, 0);
     load_regs(r1, min(1, nk - 1));
-    store_regs(r0, 0);
+    store_regs(r0, 0, true);
     __syncthreads();
+    // Two stages per trip and no exit in between, so the memory counters stay exact. With an
+    // odd stage count the second half of the last trip multiplies a stage of zeros.
     for (int ks = 0; ks < nk; ks += 2) {
         load_regs(r0, min(ks + 2, nk - 1));
         compute(0);
-        store_regs(r1, 1);
+        store_regs(r1, 1, ks + 1 < nk);
         __syncthreads();
-        if (ks + 1 >= nk) break;
         load_regs(r1, min(ks + 3, nk - 1));
         compute(1);
-        store_regs(r0, 0);
+        store_regs(r0, 0, true);
         __syncthreads();
     }
 

@@ -121,20 +121,20 @@ int fill_common(hipc_ctx *ctx, const MmOperands &o, GemmArgs &g) {
     g.dyn_signed = o.a_dtype == HIPC_I8;
     g.const_signed = o.b_dtype == HIPC_I8;
     g.I = (int)o.M, g.J = (int)o.N, g.K = (int)o.K, g.K_pad = o.K_pad;
-    g.p_aligned = (o.K % 16 == 0) && aligned(o.A, 16);
+    // the fast loader: whole 128-byte k stages, 16-byte aligned rows, 32-bit offsets
+    g.p_aligned = (o.K % kBK == 0) && aligned(o.A, 16) && o.M * o.K < (int64_t(1) << 32);
     return HIPC_OK;
 }
 
 template <int EPI, bool ALIGNED>
-int launch_mm_a(hipc_ctx *ctx, const GemmArgs &g) {
+int launch_mm_a(hipc_ctx *ctx, GemmArgs g) {
     static bool lds_set = false;  // the kernel needs more than the default 64 KiB of dynamic LDS
     if (!lds_set) {
         HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_kernel<MODE_MM, EPI, ALIGNED>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLds));
         lds_set = true;
     }
-    const int64_t tiles = ceil_div(g.J, kBN) * ceil_div(g.I, kBM);
-    const dim3 grid((unsigned)(ceil_div(tiles, 8) * 8), 1, 1);
+    const dim3 grid(gemm_grid(g), 1, 1);
     int8_gemm_kernel<MODE_MM, EPI, ALIGNED><<<grid, 256, kGemmLds, ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
@@ -162,6 +162,10 @@ int hipc_prepack_int8_b(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, in
     w->K = K, w->N = N, w->b_dtype = b_dtype;
     w->K_pad = (int)(ceil_div(K, kBK) * kBK);
     w->N_pad = (int)(ceil_div(N, kBN) * kBN);
+    if ((int64_t)w->K_pad * w->N_pad >= (int64_t(1) << 32)) {
+        delete w;
+        return fail(ctx, HIPC_ERR_UNSUPPORTED, "MatMulInteger prepack: a %ld x %ld weight exceeds the 4 GiB the kernel addresses", (long)K, (long)N);
+    }
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->Bp), (size_t)w->K_pad * w->N_pad);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&w->colsum), (size_t)w->N_pad * 4);
     if (e != hipSuccess) {
@@ -214,6 +218,7 @@ int hipc_matmul_integer_raw(hipc_ctx *ctx, const void *A, int a_dtype, const voi
     if (M == 0 || N == 0) return HIPC_OK;
     HIPC_REQUIRE(ctx, A && B && Y, "MatMulInteger: null operand");
     const int K_pad = (int)(ceil_div(K, kBK) * kBK), N_pad = (int)(ceil_div(N, kBN) * kBN);
+    HIPC_REFUSE(ctx, (int64_t)K_pad * N_pad >= (int64_t(1) << 32), "MatMulInteger: a %ld x %ld weight exceeds the 4 GiB the kernel addresses", (long)K, (long)N);
     void *scratch = nullptr;
     const size_t bp_bytes = (size_t)K_pad * N_pad;
     int rc = scratch_get(ctx, 1, bp_bytes + (size_t)N_pad * 4, &scratch);
