@@ -35,6 +35,10 @@ LAYER_LINEARS = [(1152, 1024, 1), (1152, 256, 2), (1024, 1152, 1), (1152, 6912, 
 LM_HEAD = (1152, 262144)
 N_LAYERS = 26
 BS = 32
+# HBM bytes per lm_head GEMV launch as the memory counters see them (FETCH_SIZE + WRITE_SIZE, each
+# scaled by its reading for a 256 MiB copy; profiles/mmnb_gemv_lm_head_1152x262144.txt). A counter
+# run cannot happen inside this program, so the figure is carried over from that profile.
+LM_HEAD_TRAFFIC_BYTES = 200.5e6
 IN_GRAPH = 16   # instances of a small operator per captured graph: amortises the graph launch
 
 
@@ -124,7 +128,7 @@ def bench_lm_head_roofline(pkg, ctx, copies=3):
     per = gemv_bytes(K, N)
     s.destroy()
     return dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS,
-                traffic=None, kernel="mmnb_gemv_kernel (lm_head 1152->262144, M=1)", bytes_per_launch=per,
+                traffic=LM_HEAD_TRAFFIC_BYTES, kernel="mmnb_gemv_kernel (lm_head 1152->262144, M=1)", bytes_per_launch=per,
                 avg_launch_us=med / 1e3, min_launch_us=mn / 1e3)
 
 
@@ -279,6 +283,21 @@ def bench_decoder(pkg, ctx, steps, warmup, context=2048):
                 launches_per_token=2 + 10 * cfg["n_layers"] + 3, final_position=pos)
 
 
+def bench_copy(ctx, mib=256, reps=8):
+    """Calibration for the memory counters: device-to-device copies of a known size (each reads and
+    writes `mib` MiB). Not part of the default run; profile it with --only copy."""
+    n = mib << 20
+    a, b = ctx.alloc(n), ctx.alloc(n)
+    ctx.fill(a, 0, n, 0x01020304)
+    ctx.flush()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        ctx.copy(b, 0, a, 0, n)
+    ctx.flush()
+    dt = (time.perf_counter() - t0) / reps
+    return dict(bytes_read=n, bytes_written=n, us=dt * 1e6, gbs=2 * n / dt / 1e9)
+
+
 def cpu_baseline(pkg, budget_s=12.0):
     """The restated CPU oracle (ONNX Runtime is not installed) on the host cores, on a bounded
     sample of the headline workload: the largest projection pair of one layer."""
@@ -304,7 +323,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma list of sections to run (decode, lm_head, gemv, int8, conv, "
-                    "decoder, cpu); default all. Used to profile one kernel at a time.")
+                    "decoder, cpu; copy = counter calibration, only on request); default all. Used to profile "
+                    "one kernel at a time.")
     args = ap.parse_args()
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only  # noqa: E731
@@ -336,6 +356,9 @@ def main():
     if want("decoder"):
         extras["gemma3_1b_int4_decode"] = bench_decoder(pkg, ctx, max(args.steps, 20), args.warmup)
         log("[bench] decoder:", json.dumps(extras["gemma3_1b_int4_decode"]))
+    if "copy" in only:
+        extras["copy_256MiB"] = bench_copy(ctx)
+        log("[bench] copy:", json.dumps(extras["copy_256MiB"]))
     cpu = cpu_baseline(pkg) if want("cpu") else None
     ctx.close()
 
