@@ -141,8 +141,34 @@ int launch_mm_a(hipc_ctx *ctx, GemmArgs g) {
 }
 
 template <int EPI>
+int launch_mm_big(hipc_ctx *ctx, GemmArgs g) {
+    static bool lds_set = false;
+    if (!lds_set) {
+        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_big_kernel<EPI>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLds));
+        lds_set = true;
+    }
+    const dim3 grid(gemm_grid(g, kBigTile), 1, 1);
+    int8_gemm_big_kernel<EPI><<<grid, kBigThreads, kBigLds, ctx->stream>>>(g);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+// 256x256 tiles once they fill most of the chip's 256 CUs; HIPC_GEMM_BIG=0/1 overrides (tuning, tests)
+bool wants_big_tiles(const GemmArgs &g) {
+    static const int forced = [] {
+        const char *e = getenv("HIPC_GEMM_BIG");
+        return e ? atoi(e) : -1;
+    }();
+    if (!g.p_aligned) return false;
+    if (forced >= 0) return forced != 0;
+    return ceil_div(g.I, kBigTile) * ceil_div(g.J, kBigTile) >= 192;
+}
+
+template <int EPI>
 int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
     if (g.I == 0 || g.J == 0) return HIPC_OK;
+    if (wants_big_tiles(g)) return launch_mm_big<EPI>(ctx, g);
     return g.p_aligned ? launch_mm_a<EPI, true>(ctx, g) : launch_mm_a<EPI, false>(ctx, g);
 }
 

@@ -73,6 +73,26 @@ def test_ffn_pair_shapes(ctx, pkg, oracle, shape):
     weight.destroy()
 
 
+@pytest.mark.parametrize("a_dt,b_dt", [(np.uint8, np.int8), (np.int8, np.uint8)])
+def test_large_products_take_the_256x256_tiles(ctx, pkg, oracle, a_dt, b_dt):
+    """Enough 256x256 tiles to fill the chip switches to the large-tile kernel: ragged edges in
+    both directions, an odd number of k stages, both zero points non-zero, then the same product
+    through the float epilogue."""
+    m, k, n = 3601, 384, 3585
+    a = rc.pseudo_plus1(m * k, 31).view(a_dt).reshape(m, k)
+    b = rc.pseudo_plus1(k * n, 32).view(b_dt).reshape(k, n)
+    za = -9 if a_dt == np.int8 else 200
+    zb = 17 if b_dt == np.int8 else 3
+    want = oracle.matmul_integer(a, b, za, zb)
+    weight = pkg.ops.Int8Weight(ctx, b)
+    assert np.array_equal(pkg.ops.matmul_integer(ctx, a, b, za, zb, weight=weight), want)
+    scale = np.float32(0.003)
+    bias = pkg.synth.uniform_f32(n, 33, -0.5, 0.5)
+    got = pkg.ops.matmul_integer_scale_bias(ctx, a, b, za, zb, scale, bias, weight=weight)
+    assert np.array_equal(got.view(np.uint32), oracle.rescale(want, scale, bias).view(np.uint32))
+    weight.destroy()
+
+
 LAYERS = [  # tests/matmul_integer_epilogue.rs:352-420: (a_shape, N, weight int8?, relu, per-column scale)
     ((2, 50, 64), 200, False, False, False), ((700, 96), 330, True, False, False),
     ((1100, 64), 1040, False, True, False), ((1, 128, 32), 48, True, False, True),
