@@ -215,21 +215,8 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
         ga.ratio = ep.ratio, ga.ratio_step = ep.ratio_step, ga.qbias = ep.qbias, ga.y_zp = ep.y_zp,
         ga.out_signed = ep.out_signed;
         HIPC_REQUIRE(ctx, g->n <= 65535, "Conv: batch %ld too large", (long)g->n);
-        static bool lds_set = false;  // the kernel needs more than the default 64 KiB of dynamic LDS
-        if (!lds_set) {
-            HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_kernel<MODE_CONV, EPI_REQUANT, true>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLds));
-            HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_kernel<MODE_CONV, EPI_I32, true>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLds));
-            lds_set = true;
-        }
-        const dim3 grid(gemm_grid(ga), 1, (unsigned)g->n);
-        if (ep.requant)
-            int8_gemm_kernel<MODE_CONV, EPI_REQUANT, true><<<grid, 256, kGemmLds, ctx->stream>>>(ga);
-        else
-            int8_gemm_kernel<MODE_CONV, EPI_I32, true><<<grid, 256, kGemmLds, ctx->stream>>>(ga);
-        HIPC_LAUNCHED(ctx);
-        return HIPC_OK;
+        return ep.requant ? gemm_launch<MODE_CONV, EPI_REQUANT, true>(ctx, ga, (unsigned)g->n)
+                          : gemm_launch<MODE_CONV, EPI_I32, true>(ctx, ga, (unsigned)g->n);
     }
 
     DirectConvArgs d{};

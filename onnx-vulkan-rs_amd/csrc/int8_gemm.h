@@ -20,6 +20,8 @@
 // point is not 0.
 #pragma once
 
+#include <cstdlib>
+
 #include "internal.h"
 
 namespace hipc {
@@ -29,7 +31,7 @@ typedef __attribute__((ext_vector_type(16))) int i32x16;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 constexpr int kBM = 128, kBN = 128, kBK = 128, kPitch = kBK + 16;
-constexpr size_t kGemmLds = 2 * (kBM + kBN) * kPitch + 4 * 64 * sizeof(int);
+constexpr size_t gemm_lds(int tile) { return 4 * (size_t)tile * kPitch + 4 * (tile / 2) * sizeof(int); }
 
 enum { EPI_I32 = 0, EPI_SCALE_BIAS = 1, EPI_REQUANT = 2 };
 enum { MODE_MM = 0, MODE_CONV = 1 };
@@ -143,19 +145,25 @@ __device__ __forceinline__ void gemm_emit_range(const GemmArgs &p, int lane, flo
 }
 
 // One k stage of both operand slabs as a thread holds it between global memory and LDS.
+template <int N>
 struct GemmRegs {
-    uint4 p[4], q[4];
+    uint4 p[N], q[N];
 };
 
 // ALIGNED (MODE_MM only): rows of A start on 16 bytes and K % 128 == 0, so A is read with
 // unconditional 128-bit loads at base + 32-bit offset (no branch, which keeps the load counters
 // exact and two stages in flight; no per-stage address arithmetic).
-template <int MODE, int EPI, bool ALIGNED>
+// T is the tile edge: 128, or 64 when 128x128 tiles would leave most CUs idle or alone with one
+// workgroup (several small workgroups per CU then overlap each other's memory and LDS latency).
+template <int MODE, int EPI, bool ALIGNED, int T>
 __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
+    constexpr int kChunks = T / 32;  // 16-byte chunks of a slab per thread
+    constexpr int kF = T / 64;       // 32x32 accumulators per wavefront, per direction
+    constexpr int kWT = T / 2;       // edge of a wavefront's part of the tile
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    uint8_t *lds_p = lds_raw;                            // [2][kBM * kPitch]
-    uint8_t *lds_q = lds_raw + 2 * kBM * kPitch;         // [2][kBN * kPitch]
-    int *lds_sum = reinterpret_cast<int *>(lds_raw + 2 * (kBM + kBN) * kPitch);  // [4][64]
+    uint8_t *lds_p = lds_raw;                       // [2][T * kPitch]
+    uint8_t *lds_q = lds_raw + 2 * T * kPitch;      // [2][T * kPitch]
+    int *lds_sum = reinterpret_cast<int *>(lds_raw + 4 * T * kPitch);  // [4][kWT]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -166,12 +174,12 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     // Tile order: consecutive workgroup ids land on different XCDs (round robin), each with
     // its own L2. The tile grid is cut into xcd_rows x xcd_cols = 8 rectangles, one per XCD, so
     // the operand slabs an XCD pulls through its L2 are as few as the shape allows.
-    const int tiles_x = (p.J + kBN - 1) / kBN, tiles_y = (p.I + kBM - 1) / kBM;
+    const int tiles_x = (p.J + T - 1) / T, tiles_y = (p.I + T - 1) / T;
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
     const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
     const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
     if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
-    const int i0 = ty * kBM, j0 = tx * kBN;
+    const int i0 = ty * T, j0 = tx * T;
 
     // zero points in the shifted (signed) domain
     const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
@@ -181,21 +189,21 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     const uint32_t pad_word = (uint32_t)(zd & 0xff) * 0x01010101u;
 
     // the four 16-byte chunks of each operand slab this thread moves: slab row and k chunk (of 8)
-    int row_[4], kc_[4];
+    int row_[kChunks], kc_[kChunks];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
+    for (int u = 0; u < kChunks; u++) {
         const int c = tid + 256 * u;
         row_[u] = c >> 3;
         kc_[u] = c & 7;
     }
     // MODE_CONV: where this thread's positions sit in the input
-    int base_h[4] = {0, 0, 0, 0}, base_w[4] = {0, 0, 0, 0};
-    bool pos_ok[4] = {false, false, false, false};
+    int base_h[kChunks] = {}, base_w[kChunks] = {};
+    bool pos_ok[kChunks] = {};
     const uint8_t *q_img = p.Q;
     if (MODE == MODE_CONV) {
         q_img = p.Q + (size_t)img * p.H * p.W * p.C;
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kChunks; u++) {
             const int gj = j0 + row_[u];
             pos_ok[u] = gj < p.J;
             const int oh = gj / p.Wo, ow = gj - oh * p.Wo;
@@ -206,9 +214,9 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
 
     // Byte offsets of this thread's chunks at k = 0, as 32-bit values added to a uniform base
     // that advances with k: the loads then need no per-stage address arithmetic at all.
-    uint32_t p_off[4], q_off[4];
+    uint32_t p_off[kChunks], q_off[kChunks];
 #pragma unroll
-    for (int u = 0; u < 4; u++) {
+    for (int u = 0; u < kChunks; u++) {
         const int gi = i0 + row_[u], gj = j0 + row_[u];
         p_off[u] = MODE == MODE_CONV ? (uint32_t)gi * (uint32_t)p.K_pad + kc_[u] * 16
                                      : (uint32_t)min(gi, p.I - 1) * (uint32_t)p.K + kc_[u] * 16;
@@ -251,54 +259,54 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
             return make_uint4(take ? v.x : alt, take ? v.y : alt, take ? v.z : alt, take ? v.w : alt);
         }
     };
-    auto load_regs = [&](GemmRegs &r, int stage) {
+    auto load_regs = [&](GemmRegs<kChunks> &r, int stage) {
         const int k0 = stage * kBK;
 #pragma unroll
-        for (int u = 0; u < 4; u++) r.p[u] = load_p(u, k0);
+        for (int u = 0; u < kChunks; u++) r.p[u] = load_p(u, k0);
 #pragma unroll
-        for (int u = 0; u < 4; u++) r.q[u] = load_q(u, k0);
+        for (int u = 0; u < kChunks; u++) r.q[u] = load_q(u, k0);
     };
     // `live` false (a stage past the end, only met when the stage count is odd) stores zeros,
     // which add nothing to the product or to the operand sums.
-    auto store_regs = [&](const GemmRegs &r, int buf, bool live) {
+    auto store_regs = [&](const GemmRegs<kChunks> &r, int buf, bool live) {
         const uint32_t keep = live ? 0xffffffffu : 0u;
         const uint32_t late_flip = (MODE == MODE_MM && ALIGNED) ? flip : 0u;
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            *reinterpret_cast<uint4 *>(lds_p + buf * kBM * kPitch + row_[u] * kPitch + kc_[u] * 16) =
+        for (int u = 0; u < kChunks; u++) {
+            *reinterpret_cast<uint4 *>(lds_p + buf * T * kPitch + row_[u] * kPitch + kc_[u] * 16) =
                 make_uint4((r.p[u].x ^ late_flip) & keep, (r.p[u].y ^ late_flip) & keep, (r.p[u].z ^ late_flip) & keep,
                            (r.p[u].w ^ late_flip) & keep);
-            *reinterpret_cast<uint4 *>(lds_q + buf * kBN * kPitch + row_[u] * kPitch + kc_[u] * 16) =
+            *reinterpret_cast<uint4 *>(lds_q + buf * T * kPitch + row_[u] * kPitch + kc_[u] * 16) =
                 make_uint4(r.q[u].x & keep, r.q[u].y & keep, r.q[u].z & keep, r.q[u].w & keep);
         }
     };
 
-    i32x16 acc[2][2];
+    i32x16 acc[kF][kF];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < kF; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < kF; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
-    int dsum[2] = {0, 0};
+    int dsum[kF] = {};
 
     auto compute = [&](int buf) {
-        const uint8_t *bp = lds_p + buf * kBM * kPitch + (wm * 64 + r32) * kPitch + kg * 16;
-        const uint8_t *bq = lds_q + buf * kBN * kPitch + (wn * 64 + r32) * kPitch + kg * 16;
+        const uint8_t *bp = lds_p + buf * T * kPitch + (wm * kWT + r32) * kPitch + kg * 16;
+        const uint8_t *bq = lds_q + buf * T * kPitch + (wn * kWT + r32) * kPitch + kg * 16;
 #pragma unroll
         for (int step = 0; step < kBK / 32; step++) {
-            uint4 pf[2], qf[2];
+            uint4 pf[kF], qf[kF];
 #pragma unroll
-            for (int i = 0; i < 2; i++) pf[i] = *reinterpret_cast<const uint4 *>(bp + i * 32 * kPitch + step * 32);
+            for (int i = 0; i < kF; i++) pf[i] = *reinterpret_cast<const uint4 *>(bp + i * 32 * kPitch + step * 32);
 #pragma unroll
-            for (int j = 0; j < 2; j++) qf[j] = *reinterpret_cast<const uint4 *>(bq + j * 32 * kPitch + step * 32);
+            for (int j = 0; j < kF; j++) qf[j] = *reinterpret_cast<const uint4 *>(bq + j * 32 * kPitch + step * 32);
             // always taken: a branch here would cost more than the eight dot instructions
 #pragma unroll
-            for (int f = 0; f < 2; f++) dsum[f] += dot_ones(MODE == MODE_MM ? pf[f] : qf[f]);
+            for (int f = 0; f < kF; f++) dsum[f] += dot_ones(MODE == MODE_MM ? pf[f] : qf[f]);
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < kF; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < kF; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, pf[i]),
                                                                       __builtin_bit_cast(i32x4, qf[j]), acc[i][j], 0, 0, 0);
         }
@@ -308,7 +316,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     // sits in registers and stage s+2 is in flight. Stage indices past the end are clamped
     // (a redundant, cached load) rather than branched around.
     const int nk = p.K_pad / kBK;
-    GemmRegs r0, r1;
+    GemmRegs<kChunks> r0, r1;
     load_regs(r0, 0);
     load_regs(r1, min(1, nk - 1));
     store_regs(r0, 0, true);
@@ -329,9 +337,12 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     // sums of the dynamic operand over k: the two k halves of a row live in lanes l and l+32
     if (need_dyn_sum) {
 #pragma unroll
-        for (int f = 0; f < 2; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
+        for (int f = 0; f < kF; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
         if (MODE == MODE_MM) {
-            if (kg == 0) lds_sum[wave * 64 + r32] = dsum[0], lds_sum[wave * 64 + 32 + r32] = dsum[1];
+            if (kg == 0) {
+#pragma unroll
+                for (int f = 0; f < kF; f++) lds_sum[wave * kWT + f * 32 + r32] = dsum[f];
+            }
         }
     }
     __syncthreads();
@@ -339,24 +350,57 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     const int kzz = p.K * zd * zc;
     float fmn = 0.f, fmx = 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (int i = 0; i < kF; i++) {
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int gj = j0 + wn * 64 + j * 32 + r32;
+        for (int j = 0; j < kF; j++) {
+            const int gj = j0 + wn * kWT + j * 32 + r32;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);  // row inside the 32x32 fragment
-                const int gi = i0 + wm * 64 + i * 32 + rf;
+                const int gi = i0 + wm * kWT + i * 32 + rf;
                 if (gi >= p.I || gj >= p.J) continue;
                 int v = acc[i][j][r];
                 const int csum = p.const_sum[MODE == MODE_MM ? gj : gi];
                 v = v - zd * csum + kzz;
-                if (need_dyn_sum) v -= zc * (MODE == MODE_MM ? lds_sum[wave * 64 + i * 32 + rf] : dsum[j]);
+                if (need_dyn_sum) v -= zc * (MODE == MODE_MM ? lds_sum[wave * kWT + i * 32 + rf] : dsum[j]);
                 gemm_emit<MODE, EPI>(p, img, gi, gj, v, fmn, fmx);
             }
         }
     }
     if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
+}
+
+// ---- host side: tile choice and launch of the kernel above ---------------------------------
+// 64x64 tiles until 128x128 ones would give every CU at least two workgroups;
+// HIPC_GEMM_TILE=64/128 overrides (tuning, tests).
+inline int gemm_tile(const GemmArgs &g, unsigned batch) {
+    static const int forced = [] {
+        const char *e = getenv("HIPC_GEMM_TILE");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced == 64 || forced == 128) return forced;
+    const int64_t tiles = ceil_div(g.I, kBM) * ceil_div(g.J, kBN) * (int64_t)batch;
+    return tiles >= 512 ? 128 : 64;
+}
+
+template <int MODE, int EPI, bool ALIGNED, int T>
+int gemm_launch_tile(hipc_ctx *ctx, GemmArgs g, unsigned batch) {
+    static bool lds_set = false;  // 128-tiles need more than the default 64 KiB of dynamic LDS
+    if (!lds_set) {
+        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_kernel<MODE, EPI, ALIGNED, T>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds(T)));
+        lds_set = true;
+    }
+    const dim3 grid(gemm_grid(g, T), 1, batch);
+    int8_gemm_kernel<MODE, EPI, ALIGNED, T><<<grid, 256, gemm_lds(T), ctx->stream>>>(g);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+template <int MODE, int EPI, bool ALIGNED>
+int gemm_launch(hipc_ctx *ctx, const GemmArgs &g, unsigned batch) {
+    return gemm_tile(g, batch) == 64 ? gemm_launch_tile<MODE, EPI, ALIGNED, 64>(ctx, g, batch)
+                                     : gemm_launch_tile<MODE, EPI, ALIGNED, 128>(ctx, g, batch);
 }
 
 // ---- the large-problem variant (MODE_MM, aligned A) --------------------------------------

@@ -126,20 +126,6 @@ int fill_common(hipc_ctx *ctx, const MmOperands &o, GemmArgs &g) {
     return HIPC_OK;
 }
 
-template <int EPI, bool ALIGNED>
-int launch_mm_a(hipc_ctx *ctx, GemmArgs g) {
-    static bool lds_set = false;  // the kernel needs more than the default 64 KiB of dynamic LDS
-    if (!lds_set) {
-        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_kernel<MODE_MM, EPI, ALIGNED>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLds));
-        lds_set = true;
-    }
-    const dim3 grid(gemm_grid(g), 1, 1);
-    int8_gemm_kernel<MODE_MM, EPI, ALIGNED><<<grid, 256, kGemmLds, ctx->stream>>>(g);
-    HIPC_LAUNCHED(ctx);
-    return HIPC_OK;
-}
-
 template <int EPI>
 int launch_mm_big(hipc_ctx *ctx, GemmArgs g) {
     static bool lds_set = false;
@@ -169,7 +155,7 @@ template <int EPI>
 int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
     if (g.I == 0 || g.J == 0) return HIPC_OK;
     if (wants_big_tiles(g)) return launch_mm_big<EPI>(ctx, g);
-    return g.p_aligned ? launch_mm_a<EPI, true>(ctx, g) : launch_mm_a<EPI, false>(ctx, g);
+    return g.p_aligned ? gemm_launch<MODE_MM, EPI, true>(ctx, g, 1) : gemm_launch<MODE_MM, EPI, false>(ctx, g, 1);
 }
 
 }  // namespace
