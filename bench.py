@@ -283,6 +283,39 @@ def bench_decoder(pkg, ctx, steps, warmup, context=2048):
                 launches_per_token=2 + 10 * cfg["n_layers"] + 3, final_position=pos)
 
 
+F16_PEAK_TFLOPS = 2500.0    # MI355X dense f16 MFMA, published
+
+
+def bench_prefill(pkg, ctx, M=512, bs=128):
+    """MatMulNBits with 512 rows of f16 activations (block 128, f16 scales, no zero points): the
+    gate/up, down and fused q/k/v linears of a 2048-wide model, eight instances per graph."""
+    out = {}
+    reps = 8
+    for name, (K, N) in {"gate_up_2048x11008": (2048, 11008), "down_11008x2048": (11008, 2048),
+                         "qkv_2048x2560": (2048, 2560)}.items():
+        B, scales, _ = pkg.synth.fast_nbits_weight(N, K, bs, seed=4, with_zp=False, scale_dtype=np.float16)
+        w = pkg.ops.NBitsWeight(ctx, B, scales, None, K, N, bs)
+        a = ctx.upload(pkg.synth.normal_f32(M * K, 40).reshape(M, K).astype(np.float16))
+        y = ctx.alloc(2 * M * N)
+        run = lambda: pkg.ops.matmul_nbits_packed_device(ctx, a, pkg.F16, w, y, M)  # noqa: E731
+        run()
+        ctx.flush()
+        ctx.capture_begin()
+        for _ in range(reps):
+            run()
+        g = ctx.capture_end()
+        ns, _ = median_ns(ctx, g, reps, samples=10, reps=4)
+        ctx.graph_destroy(g)
+        flops = 2.0 * M * K * N
+        byts = K * N // 2 + (K // bs) * N * 2 + M * K * 2 + M * N * 2
+        out["matmul_nbits_f16_M512_" + name] = dict(us=ns / 1e3, tflops=flops / ns / 1e3,
+                                                    frac_f16_mfma=flops / ns / 1e3 / F16_PEAK_TFLOPS,
+                                                    gbs=byts / ns, frac_hbm=byts / ns / HBM_PEAK_GBS)
+        w.destroy(), a.free(), y.free()
+        ctx.flush()
+    return out
+
+
 def bench_copy(ctx, mib=256, reps=8):
     """Calibration for the memory counters: device-to-device copies of a known size (each reads and
     writes `mib` MiB). Not part of the default run; profile it with --only copy."""
@@ -322,7 +355,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", default="", help="comma list of sections to run (decode, lm_head, gemv, int8, conv, "
+    ap.add_argument("--only", default="", help="comma list of sections to run (decode, lm_head, gemv, int8, conv, prefill, "
                     "decoder, cpu; copy = counter calibration, only on request); default all. Used to profile "
                     "one kernel at a time.")
     args = ap.parse_args()
@@ -353,6 +386,9 @@ def main():
         log("[bench] int8 ffn done")
     if want("conv"):
         extras.update(bench_qlinear_conv(pkg, ctx))
+    if want("prefill"):
+        extras.update(bench_prefill(pkg, ctx))
+        log("[bench] prefill done")
     if want("decoder"):
         extras["gemma3_1b_int4_decode"] = bench_decoder(pkg, ctx, max(args.steps, 20), args.warmup)
         log("[bench] decoder:", json.dumps(extras["gemma3_1b_int4_decode"]))

@@ -45,6 +45,19 @@ struct hipc_graph {
     hipGraphExec_t exec = nullptr;
 };
 
+// A MatMulNBits weight repacked for the matrix cores: 1 KiB tiles of 16 columns x 128 k. Lane l
+// of tile (nt, cg) = Wq[(nt * n_cg + cg) * 64 + l] holds, in word j, the eight nibbles (natural
+// order) k = 128 cg + 32 j + 8 (l >> 4) .. + 8 of column 16 nt + (l & 15). Sc / Zb hold SG scales
+// and (128 + zero point) bytes per tile column, SG = 4, 2, 1 for block sizes 32, 64, >= 128.
+struct hipc_nbits_weight {
+    int64_t K = 0, N = 0, block_size = 0;
+    int n_tiles = 0, n_cg = 0, SG = 0;
+    uint4 *Wq = nullptr;
+    float *Sc = nullptr;
+    uint8_t *Zb = nullptr;
+    size_t bytes = 0;
+};
+
 namespace hipc {
 
 inline int fail(hipc_ctx *ctx, int code, const char *fmt, ...) {
@@ -101,6 +114,10 @@ void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
 int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms);
 int64_t nbits_cols(const hipc_nbits_weight *w);
 int64_t nbits_depth(const hipc_nbits_weight *w);
+// f16 activations, any M: tiled matrix-core kernel that dequantises the weight on its way to LDS.
+// Returns HIPC_ERR_UNSUPPORTED (and launches nothing) for shapes it does not take.
+bool nbits_prefill_takes(const void *A, const hipc_nbits_weight *w, int64_t M);
+int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M);
 
 // offsets inside ctx->params
 constexpr size_t kParamRange = 0;   // 8 B  {bits(-min), bits(max)}

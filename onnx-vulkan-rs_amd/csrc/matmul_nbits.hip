@@ -520,15 +520,6 @@ mmnb_ksplit_reduce_kernel(const float *__restrict__ part, void *__restrict__ Y, 
 
 using namespace hipc;
 
-struct hipc_nbits_weight {
-    int64_t K = 0, N = 0, block_size = 0;
-    int n_tiles = 0, n_cg = 0, SG = 0;
-    uint4 *Wq = nullptr;
-    float *Sc = nullptr;
-    uint8_t *Zb = nullptr;
-    size_t bytes = 0;
-};
-
 namespace {
 
 // Launch-shape overrides for experiments: HIPC_GEMV_T (16-column tiles per wavefront: 1, 2 or
@@ -830,6 +821,8 @@ int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hi
     // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
     // terms). Unset, or 2 / 3 (f16 / bf16 are enough): 2 terms. f16 activations are exact in 2.
     const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
+    // many rows of f16: the tiled kernel reads the weight once per row tile instead of once per 16 rows
+    if (a_dtype == HIPC_F16 && nbits_prefill_takes(A, w, M)) return nbits_prefill(ctx, A, w, Y, M);
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int rows = (int)std::min<int64_t>(16, M - m0);
         int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,

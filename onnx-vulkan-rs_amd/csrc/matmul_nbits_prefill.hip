@@ -1,0 +1,294 @@
+// MatMulNBits for many rows of f16 activations (prefill): Y[M, N] = A[M, K] x dequant(W)[K, N].
+//
+// The reference has no tiled path for this shape: its kernels re-read the weight once per row
+// (crates/onnx-vulkan-core/src/shaders/matmul_nbits.rs:21-25). Here the weight is read once per
+// 64- or 128-row tile of A and the products run on the matrix cores:
+//
+//   * a 256-thread workgroup owns a T x T tile of Y (T = 128, or 64 when that would leave CUs
+//     idle), four wavefronts as 2 x 2, each T/2 x T/2 as 32x32 accumulators of
+//     v_mfma_f32_32x32x16_f16 (f16 x f16 products are exact in the f32 accumulator);
+//   * a k stage is 64 values: 128-byte LDS rows (pitch 144, conflict-free 128-bit reads) for
+//     both operands. A goes memory -> registers -> LDS as it is. The weight comes from the
+//     prepacked tiles as 32-bit words of eight nibbles and becomes f16 on the way into LDS:
+//     nibble bytes are spread with v_perm_b32, or-ed with 0x6400 (f16 1024 + q, exact) and the
+//     f16 value 1024 + zero_point is subtracted, so LDS holds the exact integers q - zp;
+//   * scales stay out of the f16 operands (folding them in would round every weight): the
+//     accumulators of one quantisation block are multiplied by the block's scale and added to
+//     the running total in f32, once per block (per 32, 64 or 128 k).
+//
+// Two register sets and two LDS buffers keep two stages in flight, as in the int8 kernel.
+#include <hip/hip_fp16.h>
+
+#include <algorithm>
+#include <cstdlib>
+
+#include "internal.h"
+
+namespace hipc {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kPK = 64;          // k values per stage
+constexpr int kPPitch = 144;     // bytes between LDS rows (128 of data)
+constexpr size_t prefill_lds(int tile) { return 4 * (size_t)tile * kPPitch; }
+
+struct PrefillArgs {
+    const __half *A;
+    const uint4 *Wq;
+    const float *Sc;
+    const uint8_t *Zb;
+    __half *Y;
+    int M, K, N;
+    int n_tiles, n_cg;
+    int xcd_rows, xcd_cols;
+};
+
+// eight nibbles (natural k order) -> eight f16 values q - zp, as four 32-bit words of pairs
+__device__ __forceinline__ uint4 dequant8(uint32_t w, uint32_t zb) {
+    const uint32_t even = w & 0x0f0f0f0fu;         // k0 k2 k4 k6, one per byte
+    const uint32_t odd = (w >> 4) & 0x0f0f0f0fu;   // k1 k3 k5 k7
+    // 1024 + zp in both halves; zb carries 128 + zp
+    const uint32_t zh = 0x6400u + (zb - 128u);
+    const f16x2 z2 = __builtin_bit_cast(f16x2, zh | (zh << 16));
+    uint32_t out[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        // bytes: [even.b_i, 0, odd.b_i, 0], then the exponent of 1024 into both halves
+        const uint32_t pair = __builtin_amdgcn_perm(odd, even, 0x0c040c00u + 0x00010001u * i) | 0x64006400u;
+        out[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, pair) - z2);
+    }
+    return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+template <int SG, int T>
+__global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) {
+    constexpr int kChunks = T / 32;  // 16-byte chunks of the A slab per thread
+    constexpr int kPairs = T / 64;   // (weight tile, lane) pairs per thread, two words each
+    constexpr int kF = T / 64;       // 32x32 accumulators per wavefront, per direction
+    constexpr int kWT = T / 2;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint8_t *lds_a = lds_raw;                    // [2][T * kPPitch]
+    uint8_t *lds_w = lds_raw + 2 * T * kPPitch;  // [2][T * kPPitch], row = column of W
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r32 = lane & 31, kg = lane >> 5;
+
+    // one rectangle of the tile grid per XCD (round-robin workgroup ids), as in the int8 kernel
+    const int tiles_x = (p.N + T - 1) / T, tiles_y = (p.M + T - 1) / T;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
+    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
+    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
+    const int i0 = ty * T, j0 = tx * T;
+
+    // A: chunk c = tid + 256 u -> slab row c / 8, 16-byte column c % 8 (8 halves)
+    uint32_t a_off[kChunks], a_lds[kChunks];
+    int a_k[kChunks];
+#pragma unroll
+    for (int u = 0; u < kChunks; u++) {
+        const int c = tid + 256 * u, row = c >> 3, kc = c & 7;
+        a_off[u] = ((uint32_t)min(i0 + row, p.M - 1) * (uint32_t)p.K + kc * 8) * 2;  // rows past M: clamped, never stored
+        a_lds[u] = row * kPPitch + kc * 16;
+        a_k[u] = kc * 8;
+    }
+    // W: pair q = tid + 256 u -> weight tile q / 64 of this column range, lane q % 64 of that tile
+    uint32_t w_tile[kPairs], w_lds[kPairs], w_sz[kPairs];
+#pragma unroll
+    for (int u = 0; u < kPairs; u++) {
+        const int q = tid + 256 * u, t = q >> 6, l = q & 63;
+        const int nt = min(j0 / 16 + t, p.n_tiles - 1);  // tiles past N: clamped, never stored
+        w_tile[u] = (uint32_t)nt * (uint32_t)p.n_cg;
+        w_lds[u] = (t * 16 + (l & 15)) * kPPitch + (l >> 4) * 16;
+        w_sz[u] = (l & 15);
+    }
+    struct Regs {
+        uint4 a[kChunks];
+        uint2 w[kPairs];
+        uint32_t z[kPairs];  // two (128 + zp) bytes: for word 0 and word 1 of the stage
+    };
+    const char *a_base = reinterpret_cast<const char *>(p.A);
+    auto load_regs = [&](Regs &r, int stage) {
+        const int k0 = stage * kPK;
+#pragma unroll
+        for (int u = 0; u < kChunks; u++) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(a_base + a_off[u] + (size_t)k0 * 2);
+            const bool in = k0 + a_k[u] < p.K;  // K is a multiple of 8: a chunk is inside or outside as a whole
+            r.a[u] = make_uint4(in ? v.x : 0u, in ? v.y : 0u, in ? v.z : 0u, in ? v.w : 0u);
+        }
+        const int cg = stage >> 1, half = stage & 1;
+#pragma unroll
+        for (int u = 0; u < kPairs; u++) {
+            const uint32_t tile = w_tile[u] + cg;
+            const int l = (tid + 256 * u) & 63;
+            r.w[u] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(p.Wq + (size_t)tile * 64 + l) + half * 8);
+            const uint8_t *zb = p.Zb + ((size_t)tile * 16 + w_sz[u]) * SG;
+            // the scale group of word j (0..3) of a tile: j for SG 4, j / 2 for SG 2, 0 for SG 1
+            const int g0 = SG == 4 ? half * 2 : (SG == 2 ? half : 0), g1 = SG == 4 ? g0 + 1 : g0;
+            r.z[u] = (uint32_t)zb[g0] | ((uint32_t)zb[g1] << 8);
+        }
+    };
+    // a stage past the end reads clamped addresses and stores zeros for A: it adds nothing
+    auto store_regs = [&](const Regs &r, int buf, bool live) {
+        const uint32_t keep = live ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int u = 0; u < kChunks; u++)
+            *reinterpret_cast<uint4 *>(lds_a + buf * T * kPPitch + a_lds[u]) =
+                make_uint4(r.a[u].x & keep, r.a[u].y & keep, r.a[u].z & keep, r.a[u].w & keep);
+#pragma unroll
+        for (int u = 0; u < kPairs; u++) {
+            uint8_t *dst = lds_w + buf * T * kPPitch + w_lds[u];
+            *reinterpret_cast<uint4 *>(dst) = dequant8(r.w[u].x, r.z[u] & 0xffu);        // k = 8 (l >> 4) .. + 8
+            *reinterpret_cast<uint4 *>(dst + 64) = dequant8(r.w[u].y, r.z[u] >> 8);     // k + 32
+        }
+    };
+
+    f32x16 total[kF][kF], raw[kF][kF];
+#pragma unroll
+    for (int i = 0; i < kF; i++)
+#pragma unroll
+        for (int j = 0; j < kF; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) total[i][j][r] = 0.f, raw[i][j][r] = 0.f;
+
+    // scales of the lane's columns (one per accumulator column block)
+    uint32_t sc_at[kF];
+#pragma unroll
+    for (int j = 0; j < kF; j++) {
+        const int col = wn * kWT + j * 32 + r32;
+        const int nt = min((j0 + col) / 16, p.n_tiles - 1);
+        sc_at[j] = ((uint32_t)nt * (uint32_t)p.n_cg * 16 + (col & 15)) * SG;
+    }
+    auto scale_of = [&](int j, int cg, int g) { return p.Sc[sc_at[j] + (uint32_t)cg * 16 * SG + g]; };
+    auto fold = [&](const float (&s)[kF]) {
+#pragma unroll
+        for (int i = 0; i < kF; i++)
+#pragma unroll
+            for (int j = 0; j < kF; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    total[i][j][r] = fmaf(raw[i][j][r], s[j], total[i][j][r]);
+                    raw[i][j][r] = 0.f;
+                }
+    };
+
+    // One stage = four k steps of 16. `half` is the stage's parity inside its 128-k weight tile;
+    // scale groups end after every second step (SG 4), every stage (SG 2) or every odd stage (SG 1).
+    auto compute = [&](int buf, int stage, int half) {
+        const int cg = stage >> 1;
+        float s0[kF], s1[kF];
+#pragma unroll
+        for (int j = 0; j < kF; j++) {
+            if (SG == 4) s0[j] = scale_of(j, cg, half * 2), s1[j] = scale_of(j, cg, half * 2 + 1);
+            else if (SG == 2) s1[j] = scale_of(j, cg, half);
+            else s1[j] = scale_of(j, cg, 0);
+        }
+        const uint8_t *ba = lds_a + buf * T * kPPitch + (wm * kWT + r32) * kPPitch + kg * 16;
+        const uint8_t *bw = lds_w + buf * T * kPPitch + (wn * kWT + r32) * kPPitch + kg * 16;
+#pragma unroll
+        for (int step = 0; step < 4; step++) {
+            f16x8 af[kF], wf[kF];
+#pragma unroll
+            for (int i = 0; i < kF; i++) af[i] = *reinterpret_cast<const f16x8 *>(ba + i * 32 * kPPitch + step * 32);
+#pragma unroll
+            for (int j = 0; j < kF; j++) wf[j] = *reinterpret_cast<const f16x8 *>(bw + j * 32 * kPPitch + step * 32);
+#pragma unroll
+            for (int i = 0; i < kF; i++)
+#pragma unroll
+                for (int j = 0; j < kF; j++)
+                    raw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], raw[i][j], 0, 0, 0);
+            if (SG == 4 && step == 1) fold(s0);
+            if (step == 3 && (SG != 1 || half == 1)) fold(s1);
+        }
+    };
+
+    const int nk = (p.K + kPK - 1) / kPK;
+    Regs r0, r1;
+    load_regs(r0, 0);
+    load_regs(r1, min(1, nk - 1));
+    store_regs(r0, 0, true);
+    __syncthreads();
+    // two stages per trip and no exit in between, so the memory counters stay exact; with an odd
+    // stage count the second half of the last trip multiplies a stage whose A is all zeros
+    for (int ks = 0; ks < nk; ks += 2) {
+        load_regs(r0, min(ks + 2, nk - 1));
+        compute(0, ks, 0);
+        store_regs(r1, 1, ks + 1 < nk);
+        __syncthreads();
+        load_regs(r1, min(ks + 3, nk - 1));
+        compute(1, min(ks + 1, nk - 1), 1);
+        store_regs(r0, 0, true);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < kF; i++) {
+#pragma unroll
+        for (int j = 0; j < kF; j++) {
+            const int gj = j0 + wn * kWT + j * 32 + r32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);
+                const int gi = i0 + wm * kWT + i * 32 + rf;
+                if (gi < p.M && gj < p.N) p.Y[(size_t)gi * p.N + gj] = __float2half(total[i][j][r]);
+            }
+        }
+    }
+}
+
+namespace {
+
+template <int SG, int T>
+int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
+    static bool lds_set = false;  // 128-tiles need more than the default 64 KiB of dynamic LDS
+    if (!lds_set) {
+        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(mmnb_prefill_kernel<SG, T>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)prefill_lds(T)));
+        lds_set = true;
+    }
+    const int tiles_x = (int)ceil_div(a.N, T), tiles_y = (int)ceil_div(a.M, T);
+    int best = 8, best_cost = 1 << 30;
+    for (int r = 1; r <= 8; r *= 2) {
+        const int cost = (int)(ceil_div(tiles_y, r) + ceil_div(tiles_x, 8 / r));
+        if (cost < best_cost) best_cost = cost, best = r;
+    }
+    a.xcd_rows = best, a.xcd_cols = 8 / best;
+    const unsigned grid = 8u * (unsigned)(ceil_div(tiles_y, a.xcd_rows) * ceil_div(tiles_x, a.xcd_cols));
+    mmnb_prefill_kernel<SG, T><<<dim3(grid), dim3(256), prefill_lds(T), ctx->stream>>>(a);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+template <int SG>
+int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
+    static const int forced = [] {
+        const char *e = getenv("HIPC_PREFILL_TILE");
+        return e ? atoi(e) : 0;
+    }();
+    int tile = ceil_div(a.M, 128) * ceil_div(a.N, 128) >= 512 ? 128 : 64;
+    if (forced == 64 || forced == 128) tile = forced;
+    return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_tile<SG, 128>(ctx, a);
+}
+
+}  // namespace
+
+bool nbits_prefill_takes(const void *A, const hipc_nbits_weight *w, int64_t M) {
+    return M > 16 && w->K % 8 == 0 && aligned(A, 16) && M * w->K < (int64_t(1) << 31);
+}
+
+int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M) {
+    HIPC_REFUSE(ctx, !nbits_prefill_takes(A, w, M), "MatMulNBits prefill: shape or alignment not taken by the tiled kernel");
+    PrefillArgs a{};
+    a.A = static_cast<const __half *>(A), a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = static_cast<__half *>(Y);
+    a.M = (int)M, a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
+    switch (w->SG) {
+        case 4: return prefill_launch<4>(ctx, a);
+        case 2: return prefill_launch<2>(ctx, a);
+        default: return prefill_launch<1>(ctx, a);
+    }
+}
+
+}  // namespace hipc

@@ -102,13 +102,13 @@ def nbits_weight(N: int, K: int, block_size: int, seed: int, with_zp: bool = Tru
     return B, scales, zp
 
 
-def fast_nbits_weight(N: int, K: int, block_size: int, seed: int, with_zp: bool = True):
+def fast_nbits_weight(N: int, K: int, block_size: int, seed: int, with_zp: bool = True, scale_dtype=np.float32):
     """Same distributions from numpy's PCG64, for weights too large for the LCG to be worth it
     (hundreds of MB); still seeded and reproducible."""
     rng = np.random.default_rng(seed)
     n_blocks = -(-K // block_size)
     B = rng.integers(0, 256, size=(N, n_blocks, block_size // 2), dtype=np.uint8)
-    scales = rng.uniform(0.005, 0.05, size=N * n_blocks).astype(np.float32)
+    scales = rng.uniform(0.005, 0.05, size=N * n_blocks).astype(np.float32).astype(scale_dtype)
     zp = rng.integers(0, 256, size=(N, (n_blocks + 1) // 2), dtype=np.uint8) if with_zp else None
     return B, scales, zp
 

@@ -109,6 +109,40 @@ def test_f16_tensors(ctx, pkg, oracle, shape):
     assert got.dtype == np.float16 and close(got, want, RTOL16), ("gemv", worst(got, want))
 
 
+PREFILL = [  # (M, K, N, block_size, zero points): ragged tiles, partial last stage, every scale grouping
+    (100, 1000, 200, 32, True), (130, 384, 131, 64, True), (257, 640, 96, 128, True), (64, 256, 1024, 256, False),
+    (17, 72, 16, 32, True),
+]
+
+
+@pytest.mark.parametrize("shape", PREFILL, ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_f16_rows_beyond_sixteen_run_the_tiled_kernel(ctx, pkg, oracle, shape):
+    """A and the scales share one element type in MatMulNBits, so the scales are f16 here too."""
+    m, k, n, bs, with_zp = shape
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=41, with_zp=with_zp, scale_dtype=np.float16)
+    a = pkg.synth.normal_f32(m * k, 42).reshape(m, k).astype(np.float16)
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    assert got.dtype == np.float16 and close(got, want, RTOL16), worst(got, want)
+
+
+@pytest.mark.parametrize("kn", [(2048, 11008), (11008, 2048), (2048, 2560)], ids=lambda s: "K%d_N%d" % s)
+def test_prefill_configuration_full_size(ctx, pkg, oracle, kn):
+    """512 rows of f16 activations against block-128 symmetric weights with f16 scales (no zero
+    points: 8 is implied), the three linears of the prefill configuration at full size."""
+    k, n = kn
+    m, bs = 512, 128
+    B, scales, _ = pkg.synth.fast_nbits_weight(n, k, bs, seed=43, with_zp=False, scale_dtype=np.float16)
+    a = pkg.synth.normal_f32(m * k, 44).reshape(m, k).astype(np.float16)
+    want = oracle.matmul_nbits(a, B, scales, None, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, None, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    assert close(got, want, RTOL16), worst(got, want)
+
+
 def test_unembedding_width_full_size(ctx, pkg, oracle):
     """lm_head of the decoder configuration: K = 1152, N = 262144, every column checked."""
     k, n, bs = 1152, 262144, 32
