@@ -17,11 +17,14 @@
 // max_seq (the reference's rule, attention.rs:22-35), in f16.
 #include <hip/hip_fp16.h>
 
+#include <cstdlib>
 #include <vector>
 
 #include "internal.h"
 
 namespace hipc {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 struct DecState {   // device-resident loop state
     int32_t token;  // the token the next step consumes
@@ -40,12 +43,19 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
     return s;
 }
 
-// x = embed_scale * dequant(table[token]); xn = rmsnorm(x, w). One workgroup.
+// x = embed_scale * dequant(table[token]); xn = rmsnorm(x, w). One workgroup. It also leaves the
+// step's rotary table behind: rope[j] = cos(pos * theta^(-2j/hd)), rope[hd/2 + j] = the sine, which
+// every layer's attention reads instead of evaluating the functions again.
 __global__ void __launch_bounds__(256)
 dec_embed_kernel(const DecState *st, const uint8_t *__restrict__ q, const float *__restrict__ scales,
                  const uint8_t *__restrict__ zp, int hidden, int bs, int n_blocks, float embed_scale,
-                 const float *__restrict__ w, float eps, float *__restrict__ x, float *__restrict__ xn) {
+                 const float *__restrict__ w, float eps, float *__restrict__ x, float *__restrict__ xn, int hd, float theta,
+                 float *__restrict__ rope) {
     __shared__ float red[4];
+    for (int j = threadIdx.x; j < hd / 2; j += 256) {
+        const float ang = (float)st->pos * powf(theta, -2.f * (float)j / (float)hd);
+        rope[j] = cosf(ang), rope[hd / 2 + j] = sinf(ang);
+    }
     const size_t row = (size_t)st->token;
     const size_t row_bytes = (size_t)n_blocks * bs / 2, zp_row = (n_blocks + 1) / 2;
     float sq = 0.f;
@@ -279,6 +289,292 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
     }
 }
 
+// ---- attention of one decode step in one launch (head_dim <= 256, group x head_dim <= 1024) ----
+// Workgroup (split, kvh) owns kFusedChunk positions of kv head kvh and serves all G query heads of
+// the group. It
+//   1. issues every load of its K and V rows at once (16-byte pieces),
+//   2. meanwhile prepares the step's own q, k, v from the fused qkv vector: per-head RMS norm and
+//      half-split rotary embedding for q and k (every workgroup does this redundantly: 1.3 k
+//      values), k and v rounded to f16 as the cache holds them; the workgroup whose chunk holds
+//      position `pos` writes them into the cache and all use the LDS copy for that position,
+//   3. forms its chunk's scores, running max / sum and unnormalised output (the flash-decoding
+//      partial), and
+//   4. takes a ticket; the workgroup that finds all other live chunks done merges the partials.
+//      Nobody waits for anybody: every workgroup runs straight to its end.
+constexpr int kFusedChunk = 64;
+constexpr int kFusedKP = kFusedChunk / 32;  // passes of 32 positions over the keys
+constexpr int kFusedVP = kFusedChunk / 8;   // positions per thread for the values
+
+__global__ void __launch_bounds__(256)
+dec_attn_fused_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
+                      const float *__restrict__ k_norm, int n_q, int n_kv, int hd, float eps, const float *__restrict__ rope,
+                      int max_seq, float scale, __half *__restrict__ k_cache, __half *__restrict__ v_cache, float *part_ml,
+                      float *part_o, unsigned int *tickets, float *__restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int G = n_q / n_kv, GH = G * hd;
+    const int split = blockIdx.x, kvh = blockIdx.y, nsplit = gridDim.x;
+    float *qs = lds;                       // [G][hd] query heads, normed and rotated
+    float *kn = qs + GH;                   // [hd] the step's key, as the cache will hold it
+    float *vn = kn + hd;                   // [hd] the step's value
+    float *sc = vn + hd;                   // [G][kFusedChunk]
+    float *ored = sc + G * kFusedChunk;    // [4][G][hd]; the merge reuses it for its weights
+    __shared__ int last_flag;
+
+    const int pos = st->pos, total = pos + 1;
+    const int t0 = split * kFusedChunk;
+    const int cnt = min(kFusedChunk, total - t0);
+    if (cnt <= 0) return;  // no position of this chunk exists yet
+    const int live = (total + kFusedChunk - 1) / kFusedChunk;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // 1. K: 8 threads per position, each the 16-byte piece `seg` of every 128-byte run of the row
+    //    (so a position's row is read in whole cache lines); V: thread (pg, cb) reads 8 channels
+    //    of positions pg, pg + 8, pg + 16, ...
+    const int kp = tid >> 3, seg = tid & 7, nk = hd >> 6;
+    uint4 kreg[kFusedKP][4];
+#pragma unroll
+    for (int ps = 0; ps < kFusedKP; ps++) {
+        const __half *krow = k_cache + ((size_t)kvh * max_seq + t0 + min(kp + 32 * ps, cnt - 1)) * hd + seg * 8;
+#pragma unroll
+        for (int u = 0; u < 4; u++) kreg[ps][u] = u < nk ? *reinterpret_cast<const uint4 *>(krow + u * 64) : make_uint4(0, 0, 0, 0);
+    }
+    const int pg = tid >> 5, cb = tid & 31;
+    const bool v_on = cb * 8 < hd;
+    uint4 vreg[kFusedVP];
+#pragma unroll
+    for (int i = 0; i < kFusedVP; i++) {
+        const int tp = min(pg + 8 * i, cnt - 1);
+        vreg[i] = v_on ? *reinterpret_cast<const uint4 *>(v_cache + ((size_t)kvh * max_seq + t0 + tp) * hd + cb * 8)
+                       : make_uint4(0, 0, 0, 0);
+    }
+    // ... and everything the step's own q, k, v need: rows 0..G-1 are the query heads, row G the
+    // key head; wavefront w prepares rows w, w + 4, w + 8; lane l holds elements l + 64 i of a row
+    const int half = hd >> 1;
+    constexpr int kRowsPerWave = (kMaxGroup + 1 + 3) / 4;
+    float px[kRowsPerWave][4], pw[kRowsPerWave][4], pc[4], psn[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int j = (lane + 64 * i) % half;
+        pc[i] = i < nk ? rope[j] : 0.f, psn[i] = i < nk ? rope[half + j] : 0.f;
+    }
+#pragma unroll
+    for (int rr = 0; rr < kRowsPerWave; rr++) {
+        const int row = wave + 4 * rr;
+        const float *src = row < G ? qkv + (size_t)(kvh * G + row) * hd : qkv + (size_t)(n_q + kvh) * hd;
+        const float *w = row < G ? q_norm : k_norm;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const bool on = row <= G && i < nk;
+            px[rr][i] = on ? src[lane + 64 * i] : 0.f, pw[rr][i] = on ? w[lane + 64 * i] : 0.f;
+        }
+    }
+    const float pv_own = tid < hd ? qkv[(size_t)(n_q + n_kv + kvh) * hd + tid] : 0.f;
+    // 2. per-head RMS norm and half-split rotary embedding (pairs d, d + hd/2), one wavefront per
+    //    row and no workgroup barrier: with hd = 128 or 256 both members of a pair sit in one lane
+    //    (elements i and i + nk/2), with hd = 64 in lanes l and l + 32
+#pragma unroll
+    for (int rr = 0; rr < kRowsPerWave; rr++) {
+        const int row = wave + 4 * rr;
+        if (row > G) break;
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) sq += px[rr][i] * px[rr][i];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) sq += __shfl_xor(sq, off, 64);
+        const float inv = rsqrtf(sq / (float)hd + eps);
+        float x[4], r[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = px[rr][i] * inv * pw[rr][i], r[i] = 0.f;
+        if (nk == 1) {
+            const float other = __shfl_xor(x[0], 32, 64);
+            r[0] = lane < 32 ? x[0] * pc[0] - other * psn[0] : x[0] * pc[0] + other * psn[0];
+        } else {
+            const int hk = nk >> 1;
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                if (i < hk) {
+                    r[i] = x[i] * pc[i] - x[i + hk] * psn[i];
+                    r[i + hk] = x[i + hk] * pc[i] + x[i] * psn[i];
+                }
+            }
+        }
+        float *dst = row < G ? qs + row * hd : kn;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (i < nk) dst[lane + 64 * i] = row < G ? r[i] : __half2float(__float2half(r[i]));
+    }
+    if (tid < hd) vn[tid] = __half2float(__float2half(pv_own));
+    __syncthreads();
+    const bool owner = pos >= t0 && pos < t0 + kFusedChunk;
+    if (owner && tid < hd) {
+        k_cache[((size_t)kvh * max_seq + pos) * hd + tid] = __float2half(kn[tid]);
+        v_cache[((size_t)kvh * max_seq + pos) * hd + tid] = __float2half(vn[tid]);
+    }
+    // 3a. scores
+#pragma unroll
+    for (int ps = 0; ps < kFusedKP; ps++) {
+        const int tp = kp + 32 * ps;
+        const bool fresh = t0 + tp == pos;
+        float dot[kMaxGroup];
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; g++) dot[g] = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (u < nk) {
+                const __half2 *h2 = reinterpret_cast<const __half2 *>(&kreg[ps][u]);
+                float kf[8];
+#pragma unroll
+                for (int e = 0; e < 4; e++) kf[2 * e] = __low2float(h2[e]), kf[2 * e + 1] = __high2float(h2[e]);
+                const int c0 = u * 64 + seg * 8;
+                if (fresh) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) kf[e] = kn[c0 + e];
+                }
+#pragma unroll
+                for (int g = 0; g < kMaxGroup; g++) {
+                    if (g < G) {
+                        const float4 qa = *reinterpret_cast<const float4 *>(qs + g * hd + c0);
+                        const float4 qb = *reinterpret_cast<const float4 *>(qs + g * hd + c0 + 4);
+                        dot[g] += (qa.x * kf[0] + qa.y * kf[1]) + (qa.z * kf[2] + qa.w * kf[3]) +
+                                  (qb.x * kf[4] + qb.y * kf[5]) + (qb.z * kf[6] + qb.w * kf[7]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; g++) {
+            if (g < G) {
+                float v = dot[g];
+                v += __shfl_xor(v, 1, 64);
+                v += __shfl_xor(v, 2, 64);
+                v += __shfl_xor(v, 4, 64);
+                if (seg == 0) sc[g * kFusedChunk + tp] = v * scale;
+            }
+        }
+    }
+    __syncthreads();
+    float *ml = part_ml + ((size_t)kvh * nsplit + split) * G * 2;
+    static_assert(kFusedChunk == 64, "one lane per position of the chunk");
+    for (int g = wave; g < G; g += 4) {
+        const float x = lane < cnt ? sc[g * kFusedChunk + lane] : -3.0e38f;
+        float m = x;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        const float pv = lane < cnt ? __expf(x - m) : 0.f;
+        float l = pv;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
+        sc[g * kFusedChunk + lane] = pv;
+        if (lane == 0) ml[g * 2] = m, ml[g * 2 + 1] = l;
+    }
+    __syncthreads();
+    // 3b. unnormalised output: 8 channels x G heads per thread over its positions
+    {
+        float o[kMaxGroup][8];
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; g++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[g][e] = 0.f;
+#pragma unroll
+        for (int i = 0; i < kFusedVP; i++) {
+            const int tp = pg + 8 * i;
+            if (tp < cnt && v_on) {
+                const __half2 *h2 = reinterpret_cast<const __half2 *>(&vreg[i]);
+                float vf[8];
+#pragma unroll
+                for (int e = 0; e < 4; e++) vf[2 * e] = __low2float(h2[e]), vf[2 * e + 1] = __high2float(h2[e]);
+                if (t0 + tp == pos) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) vf[e] = vn[cb * 8 + e];
+                }
+#pragma unroll
+                for (int g = 0; g < kMaxGroup; g++) {
+                    if (g < G) {
+                        const float w = sc[g * kFusedChunk + tp];
+#pragma unroll
+                        for (int e = 0; e < 8; e++) o[g][e] += w * vf[e];
+                    }
+                }
+            }
+        }
+        // lanes l and l + 32 hold the same channels of neighbouring position groups
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; g++) {
+            if (g < G) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[g][e] += __shfl_xor(o[g][e], 32, 64);
+                if (lane < 32 && v_on) {
+                    float4 *dst = reinterpret_cast<float4 *>(ored + (wave * G + g) * hd + cb * 8);
+                    dst[0] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
+                    dst[1] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    float *po = part_o + ((size_t)kvh * nsplit + split) * GH;
+    for (int idx = tid; idx < GH; idx += 256)
+        po[idx] = (ored[idx] + ored[GH + idx]) + (ored[2 * GH + idx] + ored[3 * GH + idx]);
+    // 4. the last workgroup of this kv head to get here merges
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned int t = atomicAdd(&tickets[kvh], 1u);
+        last_flag = t == (unsigned int)(live - 1);
+        if (last_flag) tickets[kvh] = 0u;  // everyone else has already taken theirs
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    __threadfence();
+    // The partials were written by other CUs during this launch: read them at device scope (past
+    // this CU's vector cache), as buffer loads so that many are in flight at once.
+    const __amdgpu_buffer_rsrc_t r_ml = __builtin_amdgcn_make_buffer_rsrc(
+        part_ml + (size_t)kvh * nsplit * G * 2, 0, nsplit * G * 2 * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t r_po = __builtin_amdgcn_make_buffer_rsrc(
+        part_o + (size_t)kvh * nsplit * GH, 0, nsplit * GH * 4, 0x00020000);
+    constexpr int kDev = 16;  // cache policy: device scope
+    // (max, sum) of every (chunk, head) in one round trip, then the heads' maxima, the chunk
+    // weights exp(m_s - m) and the normalisers out of LDS: [live * G] each, pair index s * G + g
+    float *mm = ored, *lw = ored + live * G, *wgt = ored + 2 * live * G;  // 3 * live * G <= 4 * G * hd floats
+    for (int i = tid; i < live * G; i += 256) {
+        const uint2 v = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r_ml, i * 8, 0, kDev));
+        mm[i] = __uint_as_float(v.x), lw[i] = __uint_as_float(v.y);
+    }
+    __syncthreads();
+    for (int i = tid; i < live * G; i += 256) {
+        const int g = i % G;
+        float m = -3.0e38f;
+        for (int s = 0; s < live; s++) m = fmaxf(m, mm[s * G + g]);
+        const float e = __expf(mm[i] - m);
+        wgt[i] = e;
+        lw[i] *= e;
+    }
+    __syncthreads();
+    // thread -> four channels of one head; eight chunks' loads in flight at a time
+    if (tid * 4 < GH) {
+        const int g = tid * 4 / hd;
+        float l = 0.f;
+        for (int s = 0; s < live; s++) l += lw[s * G + g];
+        const float inv = 1.f / l;
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+        constexpr int kAhead = 8;
+        for (int s0 = 0; s0 < live; s0 += kAhead) {
+            u32x4 v[kAhead];
+#pragma unroll
+            for (int u = 0; u < kAhead; u++)
+                v[u] = __builtin_amdgcn_raw_buffer_load_b128(r_po, (min(s0 + u, live - 1) * GH + tid * 4) * 4, 0, kDev);
+#pragma unroll
+            for (int u = 0; u < kAhead; u++) {
+                const float ws = s0 + u < live ? wgt[(s0 + u) * G + g] : 0.f;
+                const float4 f = __builtin_bit_cast(float4, v[u]);
+                o[0] += f.x * ws, o[1] += f.y * ws, o[2] += f.z * ws, o[3] += f.w * ws;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) out[(size_t)kvh * GH + tid * 4 + e] = o[e] * inv;
+    }
+}
+
 // h[i] = gelu_tanh(gu[i]) * gu[ffn + i]
 __global__ void __launch_bounds__(256) dec_gelu_mul_kernel(const float *__restrict__ gu, int ffn, float *__restrict__ h) {
     const int i = blockIdx.x * 256 + threadIdx.x;
@@ -363,7 +659,11 @@ struct hipc_decoder {
     float *x = nullptr, *xn = nullptr, *qkv = nullptr, *q = nullptr, *attn = nullptr, *y = nullptr, *gu = nullptr,
           *h = nullptr, *logits = nullptr, *part_ml = nullptr, *part_o = nullptr, *am_v = nullptr;
     int *am_i = nullptr;
+    unsigned int *tickets = nullptr;
+    float *rope = nullptr;      // [head_dim] cosines then sines of the current position
     int nsplit = 0;
+    int nsplit_fused = 0;       // chunks of the one-launch attention; 0: the shape takes the three-kernel path
+    size_t fused_lds = 0;
     std::vector<void *> owned;
 };
 
@@ -424,7 +724,18 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
     A(&d->gu, (size_t)2 * c.ffn), A(&d->h, c.ffn), A(&d->logits, c.vocab);
     A(&d->part_ml, (size_t)c.n_kv_heads * d->nsplit * G * 2), A(&d->part_o, (size_t)c.n_kv_heads * d->nsplit * G * c.head_dim);
     A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
+    A(&d->tickets, (size_t)c.n_kv_heads), A(&d->rope, (size_t)c.head_dim);
+    {
+        const int GH = G * c.head_dim, chunks = (int)ceil_div(c.max_seq, kFusedChunk);
+        const char *e = getenv("HIPC_DEC_FUSED_ATTN");  // 0: keep the three-kernel attention (tests of that path)
+        if ((c.head_dim == 64 || c.head_dim == 128 || c.head_dim == 256) && GH <= 1024 && 3 * chunks <= 4 * c.head_dim && chunks <= 65535 && !(e && atoi(e) == 0)) {
+            d->nsplit_fused = chunks;
+            d->fused_lds = (size_t)(GH + 2 * c.head_dim + G * kFusedChunk + 4 * GH) * sizeof(float);
+        }
+    }
     if (rc == HIPC_OK) {
+        if (hipMemsetAsync(d->tickets, 0, (size_t)c.n_kv_heads * sizeof(unsigned int), ctx->stream) != hipSuccess)
+            rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the attention tickets");
         for (DecLayer &l : d->layers) {  // an unwritten cache row must not hold NaN bit patterns
             if (hipMemsetAsync(l.k_cache, 0, kv * 2, ctx->stream) != hipSuccess || hipMemsetAsync(l.v_cache, 0, kv * 2, ctx->stream) != hipSuccess)
                 rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the KV cache");
@@ -547,11 +858,18 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
     const int terms = 2;
     int rc;
     dec_embed_kernel<<<1, 256, 0, s>>>(d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
-                                       d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn);
+                                       d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn, c.head_dim, c.rope_theta,
+                                       d->rope);
     HIPC_LAUNCHED(ctx);
     for (int li = 0; li < c.n_layers; li++) {
         DecLayer &l = d->layers[li];
         if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.qkv, d->qkv, 1, terms)) != HIPC_OK) return rc;
+        if (d->nsplit_fused) {
+            dec_attn_fused_kernel<<<dim3(d->nsplit_fused, c.n_kv_heads), 256, d->fused_lds, s>>>(
+                d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.head_dim,
+                c.rms_eps, d->rope, c.max_seq, scale, l.k_cache, l.v_cache, d->part_ml, d->part_o, d->tickets, d->attn);
+            HIPC_LAUNCHED(ctx);
+        } else {
         dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
                                              c.n_kv_heads, c.head_dim, c.rms_eps, c.rope_theta, c.max_seq, d->q, l.k_cache, l.v_cache);
         HIPC_LAUNCHED(ctx);
@@ -561,6 +879,7 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
                                                                                          c.head_dim, d->nsplit, d->attn);
         HIPC_LAUNCHED(ctx);
+        }
         if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
         dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->xn);
         HIPC_LAUNCHED(ctx);

@@ -127,8 +127,12 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
             r.w[u] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(p.Wq + (size_t)tile * 64 + l) + half * 8);
             const uint8_t *zb = p.Zb + ((size_t)tile * 16 + w_sz[u]) * SG;
             // the scale group of word j (0..3) of a tile: j for SG 4, j / 2 for SG 2, 0 for SG 1
-            const int g0 = SG == 4 ? half * 2 : (SG == 2 ? half : 0), g1 = SG == 4 ? g0 + 1 : g0;
-            r.z[u] = (uint32_t)zb[g0] | ((uint32_t)zb[g1] << 8);
+            if (SG == 4) {
+                r.z[u] = *reinterpret_cast<const uint16_t *>(zb + half * 2);  // groups 2 half and 2 half + 1
+            } else {
+                const uint32_t z = zb[SG == 2 ? half : 0];
+                r.z[u] = z | (z << 8);
+            }
         }
     };
     // a stage past the end reads clamped addresses and stores zeros for A: it adds nothing
@@ -177,15 +181,19 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
 
     // One stage = four k steps of 16. `half` is the stage's parity inside its 128-k weight tile;
     // scale groups end after every second step (SG 4), every stage (SG 2) or every odd stage (SG 1).
-    auto compute = [&](int buf, int stage, int half) {
+    // The scales of a stage are requested before the operand loads of the stage after next, so
+    // that waiting for them (loads retire in order) never waits for those.
+    float s0[kF], s1[kF];
+    auto fetch_scales = [&](int stage, int half) {
         const int cg = stage >> 1;
-        float s0[kF], s1[kF];
 #pragma unroll
         for (int j = 0; j < kF; j++) {
             if (SG == 4) s0[j] = scale_of(j, cg, half * 2), s1[j] = scale_of(j, cg, half * 2 + 1);
             else if (SG == 2) s1[j] = scale_of(j, cg, half);
-            else s1[j] = scale_of(j, cg, 0);
+            else if (half == 1) s1[j] = scale_of(j, cg, 0);
         }
+    };
+    auto compute = [&](int buf, int half) {
         const uint8_t *ba = lds_a + buf * T * kPPitch + (wm * kWT + r32) * kPPitch + kg * 16;
         const uint8_t *bw = lds_w + buf * T * kPPitch + (wn * kWT + r32) * kPPitch + kg * 16;
 #pragma unroll
@@ -214,12 +222,14 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
     // two stages per trip and no exit in between, so the memory counters stay exact; with an odd
     // stage count the second half of the last trip multiplies a stage whose A is all zeros
     for (int ks = 0; ks < nk; ks += 2) {
+        fetch_scales(ks, 0);
         load_regs(r0, min(ks + 2, nk - 1));
-        compute(0, ks, 0);
+        compute(0, 0);
         store_regs(r1, 1, ks + 1 < nk);
         __syncthreads();
+        fetch_scales(min(ks + 1, nk - 1), 1);
         load_regs(r1, min(ks + 3, nk - 1));
-        compute(1, min(ks + 1, nk - 1), 1);
+        compute(1, 1);
         store_regs(r0, 0, true);
         __syncthreads();
     }
