@@ -280,7 +280,7 @@ def bench_decoder(pkg, ctx, steps, warmup, context=2048):
     tok_s = steps / dt
     return dict(tok_s=tok_s, ms_per_token=dt / steps * 1e3, context=context, bytes_per_token=byts,
                 hbm_bound_tok_s=HBM_PEAK_GBS * 1e9 / byts, frac_of_hbm_bound=tok_s * byts / (HBM_PEAK_GBS * 1e9),
-                launches_per_token=1 + 8 * cfg["n_layers"] + 3, final_position=pos)
+                launches_per_token=1 + 5 * cfg["n_layers"] + 4, final_position=pos)
 
 
 F16_PEAK_TFLOPS = 2500.0    # MI355X dense f16 MFMA, published

@@ -18,6 +18,7 @@
 #include <hip/hip_fp16.h>
 
 #include <cstdlib>
+#include <utility>
 #include <vector>
 
 #include "internal.h"
@@ -661,6 +662,8 @@ struct hipc_decoder {
     int *am_i = nullptr;
     unsigned int *tickets = nullptr;
     float *rope = nullptr;      // [head_dim] cosines then sines of the current position
+    float *x2 = nullptr;        // second buffer of the residual stream
+    bool fused_glue = false;    // norms, residual adds and the gated GELU run inside the GEMV prologues
     int nsplit = 0;
     int nsplit_fused = 0;       // chunks of the one-launch attention; 0: the shape takes the three-kernel path
     size_t fused_lds = 0;
@@ -724,7 +727,11 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
     A(&d->gu, (size_t)2 * c.ffn), A(&d->h, c.ffn), A(&d->logits, c.vocab);
     A(&d->part_ml, (size_t)c.n_kv_heads * d->nsplit * G * 2), A(&d->part_o, (size_t)c.n_kv_heads * d->nsplit * G * c.head_dim);
     A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
-    A(&d->tickets, (size_t)c.n_kv_heads), A(&d->rope, (size_t)c.head_dim);
+    A(&d->tickets, (size_t)c.n_kv_heads), A(&d->rope, (size_t)c.head_dim), A(&d->x2, c.hidden);
+    {
+        const char *e = getenv("HIPC_DEC_FUSED_GLUE");  // 0: keep the separate norm / GELU kernels (tests of that path)
+        d->fused_glue = c.hidden % 8 == 0 && c.ffn % 8 == 0 && !(e && atoi(e) == 0);
+    }
     {
         const int GH = G * c.head_dim, chunks = (int)ceil_div(c.max_seq, kFusedChunk);
         const char *e = getenv("HIPC_DEC_FUSED_ATTN");  // 0: keep the three-kernel attention (tests of that path)
@@ -861,9 +868,20 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                                        d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn, c.head_dim, c.rope_theta,
                                        d->rope);
     HIPC_LAUNCHED(ctx);
+    // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
+    // branch into the stream reads one and (its first workgroup) writes the other.
+    float *xc = d->x, *xo = d->x2;
     for (int li = 0; li < c.n_layers; li++) {
         DecLayer &l = d->layers[li];
-        if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.qkv, d->qkv, 1, terms)) != HIPC_OK) return rc;
+        if (d->fused_glue && li > 0) {
+            GemvPrologue pro;
+            pro.mode = 2, pro.x = xc, pro.y = d->y, pro.w_post = d->layers[li - 1].norm[HIPC_DEC_NORM_POST_FFN];
+            pro.w_in = l.norm[HIPC_DEC_NORM_INPUT], pro.x_out = xo, pro.eps = c.rms_eps;
+            if ((rc = nbits_gemv(ctx, xc, HIPC_F32, l.qkv, d->qkv, 1, terms, &pro)) != HIPC_OK) return rc;
+            std::swap(xc, xo);
+        } else {
+            if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.qkv, d->qkv, 1, terms)) != HIPC_OK) return rc;
+        }
         if (d->nsplit_fused) {
             dec_attn_fused_kernel<<<dim3(d->nsplit_fused, c.n_kv_heads), 256, d->fused_lds, s>>>(
                 d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.head_dim,
@@ -881,14 +899,32 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         HIPC_LAUNCHED(ctx);
         }
         if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
-        dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->xn);
-        HIPC_LAUNCHED(ctx);
-        if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.gate_up, d->gu, 1, terms)) != HIPC_OK) return rc;
-        dec_gelu_mul_kernel<<<(unsigned)ceil_div(c.ffn, 256), 256, 0, s>>>(d->gu, c.ffn, d->h);
-        HIPC_LAUNCHED(ctx);
-        if ((rc = nbits_gemv(ctx, d->h, HIPC_F32, l.down, d->y, 1, terms)) != HIPC_OK) return rc;
-        const float *next = li + 1 < c.n_layers ? d->layers[li + 1].norm[HIPC_DEC_NORM_INPUT] : d->final_norm;
-        dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->xn);
+        if (d->fused_glue) {
+            GemvPrologue pro;
+            pro.mode = 2, pro.x = xc, pro.y = d->y, pro.w_post = l.norm[HIPC_DEC_NORM_POST_ATTN];
+            pro.w_in = l.norm[HIPC_DEC_NORM_PRE_FFN], pro.x_out = xo, pro.eps = c.rms_eps;
+            if ((rc = nbits_gemv(ctx, xc, HIPC_F32, l.gate_up, d->gu, 1, terms, &pro)) != HIPC_OK) return rc;
+            std::swap(xc, xo);
+            GemvPrologue gelu;
+            gelu.mode = 1;
+            if ((rc = nbits_gemv(ctx, d->gu, HIPC_F32, l.down, d->y, 1, terms, &gelu)) != HIPC_OK) return rc;
+        } else {
+            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->xn);
+            HIPC_LAUNCHED(ctx);
+            if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.gate_up, d->gu, 1, terms)) != HIPC_OK) return rc;
+            dec_gelu_mul_kernel<<<(unsigned)ceil_div(c.ffn, 256), 256, 0, s>>>(d->gu, c.ffn, d->h);
+            HIPC_LAUNCHED(ctx);
+            if ((rc = nbits_gemv(ctx, d->h, HIPC_F32, l.down, d->y, 1, terms)) != HIPC_OK) return rc;
+            const float *next = li + 1 < c.n_layers ? d->layers[li + 1].norm[HIPC_DEC_NORM_INPUT] : d->final_norm;
+            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->xn);
+            HIPC_LAUNCHED(ctx);
+        }
+    }
+    if (d->fused_glue) {
+        // the unembedding streams ~200 MB: its workgroups start on the weights at once and the
+        // final norm stays a launch of its own
+        dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], d->final_norm, c.hidden,
+                                                   c.rms_eps, xc, d->xn);
         HIPC_LAUNCHED(ctx);
     }
     if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;

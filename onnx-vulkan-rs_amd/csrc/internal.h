@@ -111,7 +111,18 @@ int nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales
                   const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size, hipc_nbits_weight **out);
 void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
 // rows [0, M), M <= 16, of A against a prepacked weight; `terms` = bf16 terms per activation (2 or 3)
-int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms);
+// What the single activation row of a decode GEMV is computed from (mode 0 / null: A as given):
+//   mode 1  A = [gate | up] (2K floats): the row is gelu_tanh(gate) * up
+//   mode 2  the row is rmsnorm(x', w_in), x' = x + rmsnorm(y, w_post) (x' = x when y is null);
+//           x' is also written to x_out (not x itself) when x_out is set. A is ignored.
+struct GemvPrologue {
+    int mode = 0;
+    const float *x = nullptr, *y = nullptr, *w_post = nullptr, *w_in = nullptr;
+    float *x_out = nullptr;
+    float eps = 0.f;
+};
+int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
+               const GemvPrologue *pro = nullptr);
 int64_t nbits_cols(const hipc_nbits_weight *w);
 int64_t nbits_depth(const hipc_nbits_weight *w);
 // f16 activations, any M: tiled matrix-core kernel that dequantises the weight on its way to LDS.

@@ -158,6 +158,10 @@ struct GemvArgs {
     int a_f16;
     int a_vec;  // rows of A may be read 8 elements at a time (base 16-byte aligned, K % 8 == 0)
     uint32_t nib_mask, magic;  // 0x000f000f and 0x43004300 (bf16 128.0 in both halves)
+    // activation prologues of the decoder (one row of f32): see GemvPrologue
+    const float *nx, *ny, *nw_post, *nw_in;
+    float *nx_out;
+    float eps;
 };
 
 template <int SG>
@@ -222,7 +226,13 @@ __device__ __forceinline__ uint32_t bf16_rne(float v) {  // bits of the nearest 
 // the two stage buffers swap roles by code duplication, not by copies.
 // The workgroup is at most 16 / T wavefronts (8 / T with all four accumulator registers in use),
 // which leaves the wide variants their registers.
-template <int T, int NR, int SG, int MC, int NT>
+// PRO selects what the one activation row is (decoder glue folded into the prologue, M == 1, f32):
+//   0  A as given
+//   1  gelu_tanh(A[k]) * A[K + k]                      (gated FFN: A = [gate | up])
+//   2  rmsnorm(x', nw_in) with x' = nx + rmsnorm(ny, nw_post) (x' = nx when ny is null); every
+//      workgroup forms the two sums of squares over the whole row itself, workgroup (0, 0) also
+//      writes x' to nx_out (a different buffer than nx: others may still be reading nx)
+template <int T, int NR, int SG, int MC, int NT, int PRO>
 __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel(const GemvArgs p) {
     extern __shared__ uint4 smem[];
     const int tid = threadIdx.x;
@@ -271,10 +281,66 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
         w = item & 3, c = (item >> 2) % nch, m = (item >> 2) / nch;
         return kbase + c * 32 + w * 8;
     };
+    GemvStage<T, SG> stA, stB;
+    int ng = blockIdx.x * p.WN + wn;
+    const int first_ng = min(ng, groups - 1), first_tile = min(tile0 + wk, tile1 - 1);
+    float inv1 = 0.f, inv2 = 0.f;
+    if (PRO == 2) {
+        load_stage(first_ng, first_tile, stA);  // the first weight tile travels while the row is normalised
+        __shared__ float nred[16];
+        const int nw = nthreads >> 6;
+        auto block_total = [&](float v) {
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+            __syncthreads();
+            if ((tid & 63) == 0) nred[tid >> 6] = v;
+            __syncthreads();
+            float t = 0.f;
+            for (int i = 0; i < nw; i++) t += nred[i];
+            return t;
+        };
+        if (p.ny) {
+            float sq = 0.f;
+            for (int c = tid; c < p.K; c += nthreads) sq += p.ny[c] * p.ny[c];
+            inv1 = rsqrtf(block_total(sq) / (float)p.K + p.eps);
+        }
+        float sq2 = 0.f;
+        const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && p.nx_out;
+        for (int c = tid; c < p.K; c += nthreads) {
+            const float xp = p.ny ? p.nx[c] + p.ny[c] * inv1 * p.nw_post[c] : p.nx[c];
+            sq2 += xp * xp;
+            if (writer) p.nx_out[c] = xp;
+        }
+        inv2 = rsqrtf(block_total(sq2) / (float)p.K + p.eps);
+    }
     auto load_item_vec = [&](int item, float av[8]) {
         int m, c, w;
         const int k0 = min(item_k0(item, m, c, w), p.K - 8);  // padding chunks are zeroed by split_item
-        if (p.a_f16) {
+        if (PRO == 1) {
+            const float4 *g = reinterpret_cast<const float4 *>(static_cast<const float *>(p.A) + k0);
+            const float4 *u = reinterpret_cast<const float4 *>(static_cast<const float *>(p.A) + p.K + k0);
+            const float4 g0 = g[0], g1 = g[1], u0 = u[0], u1 = u[1];
+            const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+            const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float v = gv[i];
+                av[i] = 0.5f * v * (1.f + tanhf(0.79788456080286536f * fmaf(0.044715f, v * v * v, v))) * uv[i];
+            }
+        } else if (PRO == 2) {
+            auto ld8 = [&](const float *src, float o[8]) {
+                const float4 a = reinterpret_cast<const float4 *>(src + k0)[0], b = reinterpret_cast<const float4 *>(src + k0)[1];
+                o[0] = a.x, o[1] = a.y, o[2] = a.z, o[3] = a.w, o[4] = b.x, o[5] = b.y, o[6] = b.z, o[7] = b.w;
+            };
+            float x8[8], y8[8], p8[8], w8[8];
+            ld8(p.nx, x8), ld8(p.nw_in, w8);
+            if (p.ny) ld8(p.ny, y8), ld8(p.nw_post, p8);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float xp = p.ny ? x8[i] + y8[i] * inv1 * p8[i] : x8[i];
+                av[i] = xp * inv2 * w8[i];
+            }
+        } else if (p.a_f16) {
             const uint4 raw = *reinterpret_cast<const uint4 *>(static_cast<const __half *>(p.A) + (size_t)m * p.K + k0);
             const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
 #pragma unroll
@@ -330,13 +396,10 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
         if (w == 0) asum[c * M + m] = s;
     };
 
-    GemvStage<T, SG> stA, stB;
-    int ng = blockIdx.x * p.WN + wn;
-    const int first_ng = min(ng, groups - 1), first_tile = min(tile0 + wk, tile1 - 1);
     if (p.a_vec) {
         float av[8];
         load_item_vec(min(tid, nitems - 1), av);
-        load_stage(first_ng, first_tile, stA);
+        if (PRO != 2) load_stage(first_ng, first_tile, stA);
         if (tid < nitems) split_item(tid, av);
         for (int item = tid + nthreads; item < nitems; item += nthreads) {
             load_item_vec(item, av);
@@ -591,19 +654,23 @@ int launch_direct(hipc_ctx *ctx, const void *A, const void *B, const void *scale
     return HIPC_OK;
 }
 
-template <int T, int NR, int MC, int NT>
+template <int T, int NR, int MC, int NT, int PRO = 0>
 void launch_gemv_sg(const GemvArgs &a, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
     if (SG == 4)
-        mmnb_gemv_kernel<T, NR, 4, MC, NT><<<grid, block, lds, s>>>(a);
+        mmnb_gemv_kernel<T, NR, 4, MC, NT, PRO><<<grid, block, lds, s>>>(a);
     else if (SG == 2)
-        mmnb_gemv_kernel<T, NR, 2, MC, NT><<<grid, block, lds, s>>>(a);
+        mmnb_gemv_kernel<T, NR, 2, MC, NT, PRO><<<grid, block, lds, s>>>(a);
     else
-        mmnb_gemv_kernel<T, NR, 1, MC, NT><<<grid, block, lds, s>>>(a);
+        mmnb_gemv_kernel<T, NR, 1, MC, NT, PRO><<<grid, block, lds, s>>>(a);
 }
 
 template <int T, int NT>
-void launch_gemv_nr(const GemvArgs &a, int NR, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
-    if (a.M == 1)
+void launch_gemv_nr(const GemvArgs &a, int pro, int NR, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+    if (a.M == 1 && pro == 1 && NT == 2)
+        launch_gemv_sg<T, 1, 1, 2, 1>(a, SG, grid, block, lds, s);
+    else if (a.M == 1 && pro == 2 && NT == 2)
+        launch_gemv_sg<T, 1, 1, 2, 2>(a, SG, grid, block, lds, s);
+    else if (a.M == 1)
         launch_gemv_sg<T, 1, 1, NT>(a, SG, grid, block, lds, s);
     else if (NR == 1)
         launch_gemv_sg<T, 1, 0, NT>(a, SG, grid, block, lds, s);
@@ -614,15 +681,16 @@ void launch_gemv_nr(const GemvArgs &a, int NR, int SG, dim3 grid, dim3 block, si
 }
 
 template <int T>
-void launch_gemv_nt(const GemvArgs &a, int NT, int NR, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+void launch_gemv_nt(const GemvArgs &a, int pro, int NT, int NR, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
     if (NT == 3)
-        launch_gemv_nr<T, 3>(a, NR, SG, grid, block, lds, s);
+        launch_gemv_nr<T, 3>(a, 0, NR, SG, grid, block, lds, s);
     else
-        launch_gemv_nr<T, 2>(a, NR, SG, grid, block, lds, s);
+        launch_gemv_nr<T, 2>(a, pro, NR, SG, grid, block, lds, s);
 }
 
 // rows [0, M) with M <= 16 of one activation matrix against a prepacked weight
-int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int NT) {
+int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int NT,
+                const GemvPrologue *pro = nullptr) {
     GemvArgs a{};
     a.A = A, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = Y, a.Ypart = nullptr;
     a.M = M, a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
@@ -669,12 +737,24 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
     const int resident = std::max(1, ctx->cu_count * std::max(1, waves_per_cu / (WK * WN)) / ksplit);
     const dim3 grid((unsigned)std::min<int64_t>(ceil_div(groups, WN), resident), (unsigned)ksplit);
     const dim3 block(64 * WK * WN);
+    int mode = 0;
+    if (pro && pro->mode != 0) {
+        mode = pro->mode;
+        HIPC_REQUIRE(ctx, M == 1 && a_dtype == HIPC_F32 && NT == 2 && a.a_vec, "MatMulNBits gemv: a prologue needs one aligned f32 row");
+        if (mode == 2) {
+            HIPC_REQUIRE(ctx, pro->x && pro->w_in && (!pro->y || pro->w_post), "MatMulNBits gemv: norm prologue operands missing");
+            HIPC_REQUIRE(ctx, aligned(pro->x, 16) && aligned(pro->w_in, 16) && (!pro->y || (aligned(pro->y, 16) && aligned(pro->w_post, 16))),
+                         "MatMulNBits gemv: norm prologue operands must be 16-byte aligned");
+            a.nx = pro->x, a.ny = pro->y, a.nw_post = pro->w_post, a.nw_in = pro->w_in, a.nx_out = pro->x_out, a.eps = pro->eps;
+            a.a_vec = 1;
+        }
+    }
     if (T == 4)
-        launch_gemv_nt<4>(a, NT, NR, w->SG, grid, block, lds, ctx->stream);
+        launch_gemv_nt<4>(a, mode, NT, NR, w->SG, grid, block, lds, ctx->stream);
     else if (T == 2)
-        launch_gemv_nt<2>(a, NT, NR, w->SG, grid, block, lds, ctx->stream);
+        launch_gemv_nt<2>(a, mode, NT, NR, w->SG, grid, block, lds, ctx->stream);
     else
-        launch_gemv_nt<1>(a, NT, NR, w->SG, grid, block, lds, ctx->stream);
+        launch_gemv_nt<1>(a, mode, NT, NR, w->SG, grid, block, lds, ctx->stream);
     HIPC_LAUNCHED(ctx);
     if (ksplit > 1) {
         const long total = (long)M * w->N;
@@ -789,8 +869,9 @@ void hipc::nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w) {
     delete w;
 }
 
-int hipc::nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms) {
-    return launch_gemv(ctx, A, a_dtype, w, Y, M, terms);
+int hipc::nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
+                     const GemvPrologue *pro) {
+    return launch_gemv(ctx, A, a_dtype, w, Y, M, terms, pro);
 }
 
 int64_t hipc::nbits_cols(const hipc_nbits_weight *w) { return w->N; }
