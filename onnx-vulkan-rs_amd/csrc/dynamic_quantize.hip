@@ -19,14 +19,22 @@ __global__ void dql_clear_range_kernel(uint32_t *range) {
 }
 
 __global__ void __launch_bounds__(256)
-dql_range_kernel(const float *__restrict__ x, long n, uint32_t *__restrict__ range, int vec_ok) {
+dql_range_kernel(const float *__restrict__ x, long n, uint32_t *__restrict__ range, int vec_ok, int per_block) {
     float mn = 0.f, mx = 0.f;
     const long tid = (long)blockIdx.x * 256 + threadIdx.x;
     const long nthreads = (long)gridDim.x * 256;
     if (vec_ok) {
         const long n4 = n >> 2;
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
-        for (long i = tid; i < n4; i += nthreads) {
+        long i = tid;
+        for (; i + 3 * nthreads < n4; i += 4 * nthreads) {  // four independent loads in flight
+            const float4 a = x4[i], b = x4[i + nthreads], c = x4[i + 2 * nthreads], d = x4[i + 3 * nthreads];
+            mn = fminf(mn, fminf(fminf(fminf(a.x, a.y), fminf(a.z, a.w)), fminf(fminf(b.x, b.y), fminf(b.z, b.w))));
+            mn = fminf(mn, fminf(fminf(fminf(c.x, c.y), fminf(c.z, c.w)), fminf(fminf(d.x, d.y), fminf(d.z, d.w))));
+            mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)), fmaxf(fmaxf(b.x, b.y), fmaxf(b.z, b.w))));
+            mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(c.x, c.y), fmaxf(c.z, c.w)), fmaxf(fmaxf(d.x, d.y), fmaxf(d.z, d.w))));
+        }
+        for (; i < n4; i += nthreads) {
             const float4 v = x4[i];
             mn = fminf(mn, fminf(fminf(v.x, v.y), fminf(v.z, v.w)));
             mx = fmaxf(mx, fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
@@ -54,8 +62,13 @@ dql_range_kernel(const float *__restrict__ x, long n, uint32_t *__restrict__ ran
         mn = fminf(fminf(smn[0], smn[1]), fminf(smn[2], smn[3]));
         mx = fmaxf(fmaxf(smx[0], smx[1]), fmaxf(smx[2], smx[3]));
         // -0.0 counts as 0: drop the sign bit
-        atomicMax(&range[0], __float_as_uint(-mn) & 0x7fffffffu);
-        atomicMax(&range[1], __float_as_uint(mx) & 0x7fffffffu);
+        if (per_block) {  // one {bits(-min), bits(max)} pair per workgroup, joined by the quantize pass
+            range[2 * blockIdx.x] = __float_as_uint(-mn) & 0x7fffffffu;
+            range[2 * blockIdx.x + 1] = __float_as_uint(mx) & 0x7fffffffu;
+        } else {
+            atomicMax(&range[0], __float_as_uint(-mn) & 0x7fffffffu);
+            atomicMax(&range[1], __float_as_uint(mx) & 0x7fffffffu);
+        }
     }
 }
 
@@ -75,10 +88,32 @@ __device__ __forceinline__ uint32_t dql_one(float v, float scale, float zp) {
 
 // four values per thread, packed into one 32-bit store where the output allows it
 __global__ void __launch_bounds__(256)
-dql_quantize_kernel(const float *__restrict__ x, long n, const uint32_t *__restrict__ range,
+dql_quantize_kernel(const float *__restrict__ x, long n, const uint32_t *__restrict__ range, int nparts,
                     uint8_t *__restrict__ y, float *__restrict__ scale_out, uint8_t *__restrict__ zp_out, int vec_ok) {
     float scale, zp;
-    dql_params(range, scale, zp);
+    if (nparts > 0) {
+        // range holds nparts pairs (nparts <= 256): every workgroup joins them itself; the maximum of
+        // non-negative floats is the maximum of their bit patterns
+        __shared__ uint32_t joined[2];
+        __shared__ uint32_t wave_max[4][2];
+        uint32_t a = 0, b = 0;
+        if ((int)threadIdx.x < nparts) a = range[2 * threadIdx.x], b = range[2 * threadIdx.x + 1];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            a = max(a, (uint32_t)__shfl_xor((int)a, off, 64));
+            b = max(b, (uint32_t)__shfl_xor((int)b, off, 64));
+        }
+        if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6][0] = a, wave_max[threadIdx.x >> 6][1] = b;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            joined[0] = max(max(wave_max[0][0], wave_max[1][0]), max(wave_max[2][0], wave_max[3][0]));
+            joined[1] = max(max(wave_max[0][1], wave_max[1][1]), max(wave_max[2][1], wave_max[3][1]));
+        }
+        __syncthreads();
+        dql_params(joined, scale, zp);
+    } else {
+        dql_params(range, scale, zp);
+    }
     const long i4 = (long)blockIdx.x * 256 + threadIdx.x;
     if (i4 == 0) {
         *scale_out = scale;
@@ -126,19 +161,27 @@ extern "C" int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_
     HIPC_REQUIRE(ctx, !(range_ready && !range), "DynamicQuantizeLinear: range_ready needs a caller-owned range slot");
     const int vec_ok = aligned(X, 16) && aligned(Y, 4);
     const float *x = static_cast<const float *>(X);
-    if (!range_ready) {
+    int nparts = 0;
+    if (!range_ready && !range) {
+        // no slot of the caller's to fill: per-workgroup pairs in the context's block, joined by the
+        // second pass -- no clearing launch and no atomics
+        slot = reinterpret_cast<uint32_t *>(static_cast<char *>(ctx->params) + kParamParts);
+        nparts = (int)std::min<long>(std::max<long>(ceil_div(n, 256 * 16), 1), kParamPartsMax);
+        dql_range_kernel<<<(unsigned)nparts, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 1);
+        HIPC_LAUNCHED(ctx);
+    } else if (!range_ready) {
         dql_clear_range_kernel<<<1, 64, 0, ctx->stream>>>(slot);
         HIPC_LAUNCHED(ctx);
         // enough workgroups to pull from every HBM channel, few enough that the atomics are noise
         const long want = ceil_div(n, 256 * 16);
         const unsigned grid = (unsigned)std::min<long>(std::max<long>(want, 1), 8L * ctx->cu_count);
-        dql_range_kernel<<<grid, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok);
+        dql_range_kernel<<<grid, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 0);
         HIPC_LAUNCHED(ctx);
     }
     const long quads = ceil_div(n, 4);
     HIPC_REQUIRE(ctx, ceil_div(quads, 256) < (int64_t(1) << 31), "DynamicQuantizeLinear: tensor too large");
     dql_quantize_kernel<<<(unsigned)ceil_div(quads, 256), 256, 0, ctx->stream>>>(
-        x, (long)n, slot, static_cast<uint8_t *>(Y), static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out),
+        x, (long)n, slot, nparts, static_cast<uint8_t *>(Y), static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out),
         vec_ok);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;

@@ -36,7 +36,7 @@ struct hipc_ctx {
     std::string err;
     std::vector<void *> deferred;        // released at the next flush
     hipc::Scratch scratch[hipc::kScratchSlots];
-    void *params = nullptr;              // small device block: range slot + scalars (256 B)
+    void *params = nullptr;              // small device block: range slot, scalars, range partials
     int cu_count = 256;
 };
 
@@ -132,6 +132,8 @@ int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void
 
 // offsets inside ctx->params
 constexpr size_t kParamRange = 0;   // 8 B  {bits(-min), bits(max)}
-constexpr size_t kParamBytes = 256;
+constexpr size_t kParamParts = 256; // 2 KiB: per-workgroup {bits(-min), bits(max)} pairs of DynamicQuantizeLinear
+constexpr int kParamPartsMax = 256;
+constexpr size_t kParamBytes = 256 + 8 * kParamPartsMax;
 
 }  // namespace hipc

@@ -30,20 +30,19 @@ pack_b_kernel(const uint8_t *__restrict__ B, uint32_t *__restrict__ Bp, int K, i
     Bp[(size_t)n * (K_pad / 4) + kw] = word;
 }
 
-// per-column sums of the shifted weight
+// per-column sums of the shifted weight, from the packed form: one wavefront per column, 16 bytes
+// per lane and step (the padding is zero, so whole rows can be summed)
 __global__ void __launch_bounds__(256)
-col_sum_kernel(const uint8_t *__restrict__ B, int32_t *__restrict__ sums, int K, int N, int N_pad, int is_signed,
-               int shift) {
-    const int n = blockIdx.x * 256 + threadIdx.x;
+col_sum_kernel(const uint8_t *__restrict__ Bp, int32_t *__restrict__ sums, int K_pad, int N_pad) {
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n >= N_pad) return;
+    const uint4 *row = reinterpret_cast<const uint4 *>(Bp + (size_t)n * K_pad);
     int s = 0;
-    if (n < N) {
-        for (int k = 0; k < K; k++) {
-            const uint8_t v = B[(size_t)k * N + n];
-            s += (is_signed ? (int)(int8_t)v : (int)v) - shift;
-        }
-    }
-    sums[n] = s;
+    for (int c = lane; c < K_pad / 16; c += 64) s += dot_ones(row[c]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == 0) sums[n] = s;
 }
 
 __global__ void __launch_bounds__(256)
@@ -93,8 +92,7 @@ int pack_into(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, int64_t N, i
     pack_b_kernel<<<dim3((unsigned)ceil_div(N_pad, 64), (unsigned)ceil_div(K_pad / 4, 4)), 256, 0, ctx->stream>>>(
         static_cast<const uint8_t *>(B), reinterpret_cast<uint32_t *>(Bp), (int)K, (int)N, K_pad, N_pad, flip);
     HIPC_LAUNCHED(ctx);
-    col_sum_kernel<<<dim3((unsigned)ceil_div(N_pad, 256)), 256, 0, ctx->stream>>>(
-        static_cast<const uint8_t *>(B), colsum, (int)K, (int)N, N_pad, b_dtype == HIPC_I8, b_dtype == HIPC_U8 ? 128 : 0);
+    col_sum_kernel<<<dim3((unsigned)ceil_div(N_pad, 4)), 256, 0, ctx->stream>>>(Bp, colsum, K_pad, N_pad);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }
