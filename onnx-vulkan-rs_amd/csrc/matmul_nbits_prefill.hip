@@ -278,7 +278,7 @@ int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
         const char *e = getenv("HIPC_PREFILL_TILE");
         return e ? atoi(e) : 0;
     }();
-    int tile = ceil_div(a.M, 128) * ceil_div(a.N, 128) >= 512 ? 128 : 64;
+    int tile = ceil_div(a.M, 128) * ceil_div(a.N, 128) >= 256 ? 128 : 64;  // at least one 128-tile per CU
     if (forced == 64 || forced == 128) tile = forced;
     return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_tile<SG, 128>(ctx, a);
 }
