@@ -384,6 +384,12 @@ def main():
     if want("int8"):
         extras.update(bench_int8_ffn(pkg, ctx))
         log("[bench] int8 ffn done")
+    if want("int8"):
+        # what the matrix cores sustain with nothing else going on (register-only MFMA loop, ~3 ms each)
+        extras["int8_mfma_register_loop_tops"] = {
+            "random_bytes_2_waves_per_simd": ctx.probe_int8_mfma(True, 2), "random_bytes_1_wave_per_simd": ctx.probe_int8_mfma(True, 1),
+            "constant_bytes_2_waves_per_simd": ctx.probe_int8_mfma(False, 2), "published_peak": INT8_PEAK_TOPS}
+        log("[bench] int8 mfma loop:", json.dumps(extras["int8_mfma_register_loop_tops"]))
     if want("conv"):
         extras.update(bench_qlinear_conv(pkg, ctx))
     if want("prefill"):

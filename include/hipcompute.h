@@ -100,6 +100,15 @@ void hipc_graph_destroy(hipc_ctx *ctx, hipc_graph *graph);
  * events on the context's stream; writes nanoseconds PER LAUNCH to ns_out[samples]. */
 int hipc_measure_graph(hipc_ctx *ctx, hipc_graph *graph, int samples, int launches_per_sample, double *ns_out);
 
+/* Measurement aid with no counterpart in the reference: what the matrix cores of this device
+ * sustain on int8 when nothing else happens. Every CU runs `waves_per_simd` (1 or 2) wavefronts
+ * per SIMD, each issuing `iterations` x 8 independent v_mfma_i32_32x32x32_i8 on operands that stay
+ * in registers (uniformly random bytes when random_operands != 0, constants otherwise: the clock
+ * the device holds depends on how many bits toggle). Writes tera-operations per second, measured
+ * with device events on the context's stream, to *tops. The int8 GEMM figures are read against
+ * this ceiling as well as against the published peak. */
+int hipc_probe_int8_mfma(hipc_ctx *ctx, int random_operands, int waves_per_simd, int iterations, double *tops);
+
 /* -------------------------------------------------------------- MatMulNBits */
 
 /*

@@ -45,6 +45,42 @@ col_sum_kernel(const uint8_t *__restrict__ Bp, int32_t *__restrict__ sums, int K
     if (lane == 0) sums[n] = s;
 }
 
+// register-only MFMA loop: 8 independent accumulators per wavefront (128 registers, so two wavefronts fit a SIMD), operands never reloaded
+__global__ void __launch_bounds__(256) int8_mfma_probe_kernel(int iterations, uint32_t seed, int random_operands, int *sink) {
+    uint32_t x = seed ^ (blockIdx.x * 256u + threadIdx.x) * 2654435761u;
+    auto next = [&]() {
+        x = x * 1664525u + 1013904223u;
+        return random_operands ? (int)(x ^ (x >> 15)) : 0x01010101;
+    };
+    i32x4 a[2], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (i < 2) a[i] = i32x4{next(), next(), next(), next()};
+        b[i] = i32x4{next(), next(), next(), next()};
+    }
+    i32x16 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    for (int it = 0; it < iterations; it++) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) s ^= acc[i][j][r];
+    if (s == 0x7fffffff) sink[0] = s;  // keeps the loop alive; practically never true
+}
+
 __global__ void __launch_bounds__(256)
 requantize_kernel(const int32_t *__restrict__ acc, const int32_t *__restrict__ bias, const float *__restrict__ ratio,
                   long n, long inner, long axis_len, int y_zp, int out_signed, uint8_t *__restrict__ out) {
@@ -159,6 +195,33 @@ int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
 }  // namespace
 
 extern "C" {
+
+int hipc_probe_int8_mfma(hipc_ctx *ctx, int random_operands, int waves_per_simd, int iterations, double *tops) {
+    if (!ctx || !tops) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, (waves_per_simd == 1 || waves_per_simd == 2) && iterations > 0 && iterations <= (1 << 20),
+                 "hipc_probe_int8_mfma: waves_per_simd must be 1 or 2, iterations in 1..2^20");
+    HIPC_REFUSE(ctx, ctx->capturing, "hipc_probe_int8_mfma while a capture is open");
+    hipEvent_t t0, t1;
+    HIPC_TRY(ctx, hipEventCreate(&t0));
+    HIPC_TRY(ctx, hipEventCreate(&t1));
+    int *sink = reinterpret_cast<int *>(static_cast<char *>(ctx->params) + 128);
+    const unsigned grid = (unsigned)(ctx->cu_count * waves_per_simd);  // 4 wavefronts per workgroup, one per SIMD
+    int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(64, 1u, random_operands, sink);  // warm the clocks and the code
+    hipError_t e = hipEventRecord(t0, ctx->stream);
+    int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(iterations, 7u, random_operands, sink);
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e == hipSuccess) e = hipEventRecord(t1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (e != hipSuccess) return fail(ctx, HIPC_ERR_BACKEND, "hipc_probe_int8_mfma: %s", hipGetErrorString(e));
+    const double ops = 2.0 * 32 * 32 * 32 * 8.0 * iterations * 4.0 * grid;
+    *tops = ops / (ms * 1e-3) / 1e12;
+    return HIPC_OK;
+}
 
 int hipc_prepack_int8_b(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, int64_t N, hipc_int8_weight **out) {
     if (!ctx || !out) return HIPC_ERR_INVALID;

@@ -74,6 +74,7 @@ SIGNATURES = {
     "hipc_graph_launch": (_int, [_vp, _vp]),
     "hipc_graph_destroy": (None, [_vp, _vp]),
     "hipc_measure_graph": (_int, [_vp, _vp, _int, _int, C.POINTER(C.c_double)]),
+    "hipc_probe_int8_mfma": (_int, [_vp, _int, _int, _int, C.POINTER(C.c_double)]),
     "hipc_matmul_nbits": (_int, [_vp, _vp, _int, _vp, _sz, _vp, _int, _sz, _vp, _sz, _vp, _i64, _i64, _i64,
                                  _i64, _int]),
     "hipc_prepack_matmul_nbits": (_int, [_vp, _vp, _sz, _vp, _int, _sz, _vp, _sz, _i64, _i64, _i64,
@@ -223,6 +224,12 @@ class Context:
 
     def graph_destroy(self, graph):
         self.lib.hipc_graph_destroy(self.handle, graph)
+
+    def probe_int8_mfma(self, random_operands: bool, waves_per_simd: int = 2, iterations: int = 4096) -> float:
+        """Sustained int8 matrix-core rate (TOPS) of a register-only MFMA loop."""
+        out = C.c_double()
+        self._check(self.lib.hipc_probe_int8_mfma(self.handle, int(random_operands), waves_per_simd, iterations, C.byref(out)))
+        return out.value
 
     def measure_graph(self, graph, samples: int, launches_per_sample: int) -> np.ndarray:
         """Nanoseconds per launch for each sample (``measure_dispatch_gpu``)."""
