@@ -46,8 +46,8 @@ struct hipc_graph {
 };
 
 // A MatMulNBits weight repacked for the matrix cores: 1 KiB tiles of 16 columns x 128 k. Lane l
-// of tile (nt, cg) = Wq[(nt * n_cg + cg) * 64 + l] holds, in word j, the eight nibbles (natural
-// order) k = 128 cg + 32 j + 8 (l >> 4) .. + 8 of column 16 nt + (l & 15). Sc / Zb hold SG scales
+// of tile (nt, cg) = Wq[(nt * n_cg + cg) * 64 + l] holds, in word j, the eight nibbles
+// k = 128 cg + 32 j + 8 (l >> 4) .. + 8 of column 16 nt + (l & 15), in the order k0 k2 k4 k6 k1 k3 k5 k7. Sc / Zb hold SG scales
 // and (128 + zero point) bytes per tile column, SG = 4, 2, 1 for block sizes 32, 64, >= 128.
 struct hipc_nbits_weight {
     int64_t K = 0, N = 0, block_size = 0;

@@ -104,7 +104,8 @@ mmnb_direct_kernel(const AT *__restrict__ A, const uint32_t *__restrict__ B, con
 
 // Tile (nt, cg): 16 columns n = 16*nt + (lane & 15), four 32-k chunks c = 4*cg + j.
 // Lane l's 128-bit element holds, in word j, the 8 nibbles k = 32*c + 8*(l >> 4) .. +8
-// of column n -- exactly the B operand of one 16x16x32 MFMA per word.
+// of column n -- exactly the B operand of one 16x16x32 MFMA per word -- in the nibble order
+// k0 k2 k4 k6 k1 k3 k5 k7, so that (word >> 4 i) & 0x000f000f is the pair (k_2i, k_2i+1).
 // SG scale groups per tile (4 when block_size == 32, 2 for 64, 1 for >= 128).
 template <typename ST>
 __global__ void __launch_bounds__(256)
@@ -122,7 +123,11 @@ mmnb_prepack_kernel(const uint32_t *__restrict__ B, const ST *__restrict__ scale
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int widx = (cg * 4 + j) * 4 + w;
-        v[j] = (n < N && widx < row_words) ? B[(size_t)n * row_words + widx] : 0u;
+        const uint32_t raw = (n < N && widx < row_words) ? B[(size_t)n * row_words + widx] : 0u;
+        // nibble order k0 k2 k4 k6 k1 k3 k5 k7: then (word >> 4 i) & 0x000f000f is the pair (k_2i, k_2i+1)
+        const uint32_t even = raw & 0x0f0f0f0fu, odd = (raw >> 4) & 0x0f0f0f0fu;
+        auto squeeze = [](uint32_t e) { return (e & 0xfu) | ((e >> 4) & 0xf0u) | ((e >> 8) & 0xf00u) | ((e >> 12) & 0xf000u); };
+        v[j] = squeeze(even) | (squeeze(odd) << 16);
     }
     Wq[idx] = make_uint4(v[0], v[1], v[2], v[3]);
     if (w == 0) {
@@ -388,11 +393,11 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
         s += __shfl_xor(s, 1, 64);
         s += __shfl_xor(s, 2, 64);
         const size_t slot = ((size_t)c * (4 * NT) + w) * M + m;
-        // operand slot order (k0,k4,k1,k5,k2,k6,k3,k7) matches the nibble unpack below
-        As[slot] = make_uint4((t0[0] >> 16) | t0[4], (t0[1] >> 16) | t0[5], (t0[2] >> 16) | t0[6], (t0[3] >> 16) | t0[7]);
-        As[slot + 4 * M] = make_uint4((t1[0] >> 16) | t1[4], (t1[1] >> 16) | t1[5], (t1[2] >> 16) | t1[6], (t1[3] >> 16) | t1[7]);
+        // k order, two bf16 per word: the nibble unpack below yields the pairs (k0,k1) (k2,k3) (k4,k5) (k6,k7)
+        As[slot] = make_uint4((t0[0] >> 16) | t0[1], (t0[2] >> 16) | t0[3], (t0[4] >> 16) | t0[5], (t0[6] >> 16) | t0[7]);
+        As[slot + 4 * M] = make_uint4((t1[0] >> 16) | t1[1], (t1[2] >> 16) | t1[3], (t1[4] >> 16) | t1[5], (t1[6] >> 16) | t1[7]);
         if (NT == 3)
-            As[slot + 8 * M] = make_uint4((t2[0] >> 16) | t2[4], (t2[1] >> 16) | t2[5], (t2[2] >> 16) | t2[6], (t2[3] >> 16) | t2[7]);
+            As[slot + 8 * M] = make_uint4((t2[0] >> 16) | t2[1], (t2[2] >> 16) | t2[3], (t2[4] >> 16) | t2[5], (t2[6] >> 16) | t2[7]);
         if (w == 0) asum[c * M + m] = s;
     };
 

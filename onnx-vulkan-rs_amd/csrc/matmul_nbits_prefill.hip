@@ -10,8 +10,9 @@
 //   * a k stage is 64 values: 128-byte LDS rows (pitch 144, conflict-free 128-bit reads) for
 //     both operands. A goes memory -> registers -> LDS as it is. The weight comes from the
 //     prepacked tiles as 32-bit words of eight nibbles and becomes f16 on the way into LDS:
-//     nibble bytes are spread with v_perm_b32, or-ed with 0x6400 (f16 1024 + q, exact) and the
-//     f16 value 1024 + zero_point is subtracted, so LDS holds the exact integers q - zp;
+//     the prepacked nibble order makes (word >> 4 i) & 0x000f000f the pair (k_2i, k_2i+1); or-ed with
+//     0x6400 that is f16 1024 + q (exact), and the f16 value 1024 + zero_point is subtracted, so LDS
+//     holds the exact integers q - zp;
 //   * scales stay out of the f16 operands (folding them in would round every weight): the
 //     accumulators of one quantisation block are multiplied by the block's scale and added to
 //     the running total in f32, once per block (per 32, 64 or 128 k).
@@ -45,18 +46,16 @@ struct PrefillArgs {
     int xcd_rows, xcd_cols;
 };
 
-// eight nibbles (natural k order) -> eight f16 values q - zp, as four 32-bit words of pairs
+// eight nibbles (order k0 k2 k4 k6 k1 k3 k5 k7) -> eight f16 values q - zp in k order, as four words of pairs
 __device__ __forceinline__ uint4 dequant8(uint32_t w, uint32_t zb) {
-    const uint32_t even = w & 0x0f0f0f0fu;         // k0 k2 k4 k6, one per byte
-    const uint32_t odd = (w >> 4) & 0x0f0f0f0fu;   // k1 k3 k5 k7
     // 1024 + zp in both halves; zb carries 128 + zp
     const uint32_t zh = 0x6400u + (zb - 128u);
     const f16x2 z2 = __builtin_bit_cast(f16x2, zh | (zh << 16));
     uint32_t out[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        // bytes: [even.b_i, 0, odd.b_i, 0], then the exponent of 1024 into both halves
-        const uint32_t pair = __builtin_amdgcn_perm(odd, even, 0x0c040c00u + 0x00010001u * i) | 0x64006400u;
+        // nibbles i and i + 4 into the two halves, then the exponent of 1024: f16 (1024 + q), exact
+        const uint32_t pair = ((w >> (4 * i)) & 0x000f000fu) | 0x64006400u;
         out[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, pair) - z2);
     }
     return make_uint4(out[0], out[1], out[2], out[3]);
