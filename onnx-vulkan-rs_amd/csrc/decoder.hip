@@ -537,9 +537,17 @@ dec_attn_fused_kernel(const DecState *st, const float *__restrict__ qkv, const f
     // (max, sum) of every (chunk, head) in one round trip, then the heads' maxima, the chunk
     // weights exp(m_s - m) and the normalisers out of LDS: [live * G] each, pair index s * G + g
     float *mm = ored, *lw = ored + live * G, *wgt = ored + 2 * live * G;  // 3 * live * G <= 4 * G * hd floats
+    // thread -> four channels of one head. The first kAhead chunks' outputs are requested together
+    // with the statistics, so the two round trips overlap.
+    constexpr int kAhead = 16;
+    const bool owns = tid * 4 < GH;
+    u32x4 v[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; u++)
+        v[u] = owns ? __builtin_amdgcn_raw_buffer_load_b128(r_po, (min(u, live - 1) * GH + tid * 4) * 4, 0, kDev) : u32x4{0, 0, 0, 0};
     for (int i = tid; i < live * G; i += 256) {
-        const uint2 v = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r_ml, i * 8, 0, kDev));
-        mm[i] = __uint_as_float(v.x), lw[i] = __uint_as_float(v.y);
+        const uint2 st2 = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r_ml, i * 8, 0, kDev));
+        mm[i] = __uint_as_float(st2.x), lw[i] = __uint_as_float(st2.y);
     }
     __syncthreads();
     for (int i = tid; i < live * G; i += 256) {
@@ -551,19 +559,18 @@ dec_attn_fused_kernel(const DecState *st, const float *__restrict__ qkv, const f
         lw[i] *= e;
     }
     __syncthreads();
-    // thread -> four channels of one head; eight chunks' loads in flight at a time
-    if (tid * 4 < GH) {
+    if (owns) {
         const int g = tid * 4 / hd;
         float l = 0.f;
         for (int s = 0; s < live; s++) l += lw[s * G + g];
         const float inv = 1.f / l;
         float o[4] = {0.f, 0.f, 0.f, 0.f};
-        constexpr int kAhead = 8;
         for (int s0 = 0; s0 < live; s0 += kAhead) {
-            u32x4 v[kAhead];
+            if (s0 > 0) {
 #pragma unroll
-            for (int u = 0; u < kAhead; u++)
-                v[u] = __builtin_amdgcn_raw_buffer_load_b128(r_po, (min(s0 + u, live - 1) * GH + tid * 4) * 4, 0, kDev);
+                for (int u = 0; u < kAhead; u++)
+                    v[u] = __builtin_amdgcn_raw_buffer_load_b128(r_po, (min(s0 + u, live - 1) * GH + tid * 4) * 4, 0, kDev);
+            }
 #pragma unroll
             for (int u = 0; u < kAhead; u++) {
                 const float ws = s0 + u < live ? wgt[(s0 + u) * G + g] : 0.f;
