@@ -88,6 +88,11 @@ class GemvSet:
         self.ctx.flush()
 
 
+def min_bound_us(byts, ops, peak_tops):
+    """The roofline time of an operator: the larger of its HBM time and its matrix-core time."""
+    return max(byts / (HBM_PEAK_GBS * 1e3), ops / (peak_tops * 1e6))
+
+
 def median_ns(ctx, graph, launches_per_graph=1, samples=20, reps=10):
     ns = ctx.measure_graph(graph, samples, reps)
     return float(np.median(ns)) / launches_per_graph, float(ns.min()) / launches_per_graph
@@ -186,8 +191,9 @@ def bench_int8_ffn(pkg, ctx):
             opsn = 2.0 * T * K * N
             byts = T * K + K * N + T * N * 4
             out[f"matmul_integer_{name}_1000x{K}x{N}"] = dict(
-                us=ns / 1e3, tops=opsn / ns / 1e3, frac_int8_mfma=opsn / ns / 1e3 / INT8_PEAK_TOPS,
-                gbs=byts / ns, frac_hbm=byts / ns / HBM_PEAK_GBS)
+                us=ns / 1e3, us_min=mn / 1e3, tops=opsn / ns / 1e3, frac_int8_mfma=opsn / ns / 1e3 / INT8_PEAK_TOPS,
+                gbs=byts / ns, frac_hbm=byts / ns / HBM_PEAK_GBS,
+                frac_of_min_bound=min_bound_us(byts, opsn, INT8_PEAK_TOPS) / (ns / 1e3))
         w.destroy(), a.free(), y.free()
     # asymptotic shape, to separate the kernel from the launch floor
     K = N = T2 = 8192
@@ -221,20 +227,20 @@ def bench_qlinear_conv(pkg, ctx):
         geom = pkg.ConvGeom.make(X.shape, W.shape, dilations=(1, dil), pads=(0, 3 * dil, 0, 3 * dil))
         w = ops.ConvWeight(ctx, W, geom)
         dX, dY = ctx.upload(X), ctx.alloc(C * T)
-        # QLinearConv uploads its ratios, so it is timed eagerly between device events via a graph of the
-        # integer convolution + a standalone run for the full operator
-        t = []
-        for _ in range(3):
-            ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, 128, w, ws, 0, 0.5, 128, pkg.U8, bias, geom, dY)
+        run = lambda: ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, 128, w, ws, 0, 0.5, 128, pkg.U8, bias, geom, dY)  # noqa: E731
+        run()   # the first call uploads the requantisation ratios; later ones reuse them and can be captured
         ctx.flush()
-        reps = 50
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, 128, w, ws, 0, 0.5, 128, pkg.U8, bias, geom, dY)
-        ctx.flush()
-        wall_us = (time.perf_counter() - t0) / reps * 1e6
+        ctx.capture_begin()
+        for _ in range(IN_GRAPH):
+            run()
+        g = ctx.capture_end()
+        ns, mn = median_ns(ctx, g, IN_GRAPH, samples=20, reps=4)
+        ctx.graph_destroy(g)
         opsn = 2.0 * C * T * C * 7
-        out[f"qlinear_conv_c{C}_k7_T{T}_d{dil}"] = dict(wall_us=wall_us, tops_wall=opsn / wall_us / 1e6)
+        byts = C * T + C * C * 7 + C * T + C * 8
+        out[f"qlinear_conv_c{C}_k7_T{T}_d{dil}"] = dict(
+            us=ns / 1e3, us_min=mn / 1e3, tops=opsn / ns / 1e3, frac_int8_mfma=opsn / ns / 1e3 / INT8_PEAK_TOPS,
+            frac_of_min_bound=min_bound_us(byts, opsn, INT8_PEAK_TOPS) / (ns / 1e3))
         w.destroy(), dX.free(), dY.free(), bias.free()
     ctx.flush()
     return out
@@ -304,13 +310,14 @@ def bench_prefill(pkg, ctx, M=512, bs=128):
         for _ in range(reps):
             run()
         g = ctx.capture_end()
-        ns, _ = median_ns(ctx, g, reps, samples=10, reps=4)
+        ns, mn = median_ns(ctx, g, reps, samples=10, reps=4)
         ctx.graph_destroy(g)
         flops = 2.0 * M * K * N
         byts = K * N // 2 + (K // bs) * N * 2 + M * K * 2 + M * N * 2
-        out["matmul_nbits_f16_M512_" + name] = dict(us=ns / 1e3, tflops=flops / ns / 1e3,
+        out["matmul_nbits_f16_M512_" + name] = dict(us=ns / 1e3, us_min=mn / 1e3, tflops=flops / ns / 1e3,
                                                     frac_f16_mfma=flops / ns / 1e3 / F16_PEAK_TFLOPS,
-                                                    gbs=byts / ns, frac_hbm=byts / ns / HBM_PEAK_GBS)
+                                                    gbs=byts / ns, frac_hbm=byts / ns / HBM_PEAK_GBS,
+                                                    frac_of_min_bound=min_bound_us(byts, flops, F16_PEAK_TFLOPS) / (ns / 1e3))
         w.destroy(), a.free(), y.free()
         ctx.flush()
     return out
@@ -378,8 +385,8 @@ def main():
         log(f"[bench] lm_head gemv: {roof['avg_launch_us']:.1f} us, {roof['achieved']:.0f} GB/s")
     extras = {}
     if want("gemv"):
-        extras["gemv_up_1152x6912"] = bench_single_gemv(pkg, ctx, 1152, 6912, cold_copies=64)
-        extras["gemv_down_6912x1152"] = bench_single_gemv(pkg, ctx, 6912, 1152, cold_copies=64)
+        extras["gemv_up_1152x6912"] = bench_single_gemv(pkg, ctx, 1152, 6912, cold_copies=104)
+        extras["gemv_down_6912x1152"] = bench_single_gemv(pkg, ctx, 6912, 1152, cold_copies=104)
         log("[bench] single gemv:", json.dumps(extras))
     if want("int8"):
         extras.update(bench_int8_ffn(pkg, ctx))

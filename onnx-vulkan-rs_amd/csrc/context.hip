@@ -3,6 +3,9 @@
 // (crates/vk-compute/src/{buffer,stream,pipeline}.rs). One in-order HIP stream
 // gives the reference's "every command waits for everything before it"
 // semantics (stream.rs:11-14) by construction; a HIP graph is its capture/replay.
+#include <algorithm>
+#include <cstring>
+
 #include "internal.h"
 
 namespace hipc {
@@ -65,6 +68,34 @@ static int create(int device, void *stream, bool adopt, hipc_ctx **out) {
         ctx->cu_count = prop.multiProcessorCount;
     *out = ctx;
     return HIPC_OK;
+}
+
+int ratio_resident(hipc_ctx *ctx, RatioCache &cache, const std::vector<float> &ratio, const float **out) {
+    if (cache.dev && cache.host.size() == ratio.size() &&
+        memcmp(cache.host.data(), ratio.data(), ratio.size() * sizeof(float)) == 0) {
+        *out = cache.dev;
+        return HIPC_OK;
+    }
+    HIPC_REFUSE(ctx, ctx->capturing, "QLinear: the requantisation ratios changed and would have to be uploaded inside a capture; run the operator once before capturing");
+    if (cache.host.size() != ratio.size() || !cache.dev) {
+        // earlier launches may still read the old buffer: it goes with the next flush
+        if (cache.dev) ctx->deferred.push_back(cache.dev);
+        cache.dev = nullptr;
+        HIPC_TRY(ctx, hipMalloc(reinterpret_cast<void **>(&cache.dev), std::max<size_t>(ratio.size() * sizeof(float), 16)));
+    } else {
+        HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));  // nobody reads the buffer while it is rewritten
+    }
+    HIPC_TRY(ctx, hipMemcpyAsync(cache.dev, ratio.data(), ratio.size() * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    cache.host = ratio;
+    *out = cache.dev;
+    return HIPC_OK;
+}
+
+void ratio_release(hipc_ctx *ctx, RatioCache &cache) {
+    if (cache.dev) ctx->deferred.push_back(cache.dev);
+    cache.dev = nullptr;
+    cache.host.clear();
 }
 
 }  // namespace hipc

@@ -135,6 +135,7 @@ struct hipc_conv_weight {
     uint8_t *Wp = nullptr;   // [O_pad, K_pad], (kh, kw, c) order; null when the MFMA path does not apply
     int32_t *rowsum = nullptr;
     int O_pad = 0, K_pad = 0;
+    mutable hipc::RatioCache ratios;  // QLinearConv's requantisation ratios as last used
 };
 
 namespace {
@@ -306,6 +307,7 @@ void hipc_conv_weight_destroy(hipc_ctx *ctx, hipc_conv_weight *w) {
     if (w->raw) ctx->deferred.push_back(w->raw);
     if (w->Wp) ctx->deferred.push_back(w->Wp);
     if (w->rowsum) ctx->deferred.push_back(w->rowsum);
+    ratio_release(ctx, w->ratios);
     delete w;
 }
 
@@ -328,7 +330,7 @@ int hipc_qlinear_conv(hipc_ctx *ctx, const void *X, int x_dtype, float x_scale, 
                  (long)n_w_scale, (long)g->c_out);
     HIPC_REFUSE(ctx, n_w_scale > 1 && w_zp != 0, "QLinearConv: w per-channel zero point is not zero (asymmetric weights)");
     HIPC_REQUIRE(ctx, y_scale != 0.f, "QLinear: y_scale is zero");
-    HIPC_REFUSE(ctx, ctx->capturing, "QLinearConv uploads its requantisation ratios: not capturable");
+    HIPC_REQUIRE(ctx, W, "QLinearConv: null weight");
     // ratio[c] = x_scale * w_scale[c] / y_scale (interp.rs:4693); a per-tensor scale is
     // broadcast to c_out so the bias stays per channel (interp.rs:4815-4823)
     std::vector<float> ratio((size_t)g->c_out);
@@ -336,14 +338,12 @@ int hipc_qlinear_conv(hipc_ctx *ctx, const void *X, int x_dtype, float x_scale, 
         volatile float t = x_scale * w_scale[n_w_scale == 1 ? 0 : c];
         ratio[(size_t)c] = t / y_scale;
     }
-    void *dratio = nullptr;
-    int rc = scratch_get(ctx, 2, ratio.size() * 4, &dratio);
+    const float *dratio = nullptr;
+    int rc = ratio_resident(ctx, W->ratios, ratio, &dratio);
     if (rc != HIPC_OK) return rc;
-    HIPC_TRY(ctx, hipMemcpyAsync(dratio, ratio.data(), ratio.size() * 4, hipMemcpyHostToDevice, ctx->stream));
-    HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));
     ConvEpilogue ep;
     ep.requant = 1;
-    ep.ratio = static_cast<const float *>(dratio), ep.ratio_step = 1;
+    ep.ratio = dratio, ep.ratio_step = 1;
     ep.qbias = static_cast<const int32_t *>(bias);
     ep.y_zp = y_zp, ep.out_signed = y_dtype == HIPC_I8;
     return run_conv(ctx, X, x_dtype, W, nullptr, nullptr, 1, x_zp, w_zp, g, Y, ep);

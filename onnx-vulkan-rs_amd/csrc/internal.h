@@ -97,6 +97,18 @@ struct Guard {
 // status of the launch just made (configuration errors surface here, not at the next sync)
 #define HIPC_LAUNCHED(ctx) HIPC_TRY((ctx), hipGetLastError())
 
+// Requantisation ratios of a QLinear operator, kept with the weight handle. They are formed on the
+// host from the operator's scale attributes; as long as those do not change between calls the
+// device copy is reused, so a call neither uploads nor synchronises and can be captured.
+struct RatioCache {
+    float *dev = nullptr;
+    std::vector<float> host;
+};
+// *out = device pointer holding `ratio` (uploading it first when it differs from the cached copy;
+// that upload is refused while a capture is open)
+int ratio_resident(hipc_ctx *ctx, RatioCache &cache, const std::vector<float> &ratio, const float **out);
+void ratio_release(hipc_ctx *ctx, RatioCache &cache);
+
 // Returns ctx->scratch[slot] grown to at least `bytes`. Growth allocates, so it is
 // refused while a capture is open.
 int scratch_get(hipc_ctx *ctx, int slot, size_t bytes, void **out);

@@ -118,6 +118,7 @@ struct hipc_int8_weight {
     int b_dtype = HIPC_I8;
     uint8_t *Bp = nullptr;
     int32_t *colsum = nullptr;
+    mutable hipc::RatioCache ratios;  // QLinearMatMul's requantisation ratios as last used
 };
 
 namespace {
@@ -262,6 +263,7 @@ void hipc_int8_weight_destroy(hipc_ctx *ctx, hipc_int8_weight *w) {
     Guard g(ctx);
     if (w->Bp) ctx->deferred.push_back(w->Bp);
     if (w->colsum) ctx->deferred.push_back(w->colsum);
+    ratio_release(ctx, w->ratios);
     delete w;
 }
 
@@ -375,15 +377,12 @@ int hipc_qlinear_matmul(hipc_ctx *ctx, const void *A, int a_dtype, float a_scale
         volatile float t = a_scale * b_scale[c];
         ratio[(size_t)c] = t / y_scale;
     }
-    void *dratio = nullptr;
-    rc = scratch_get(ctx, 2, ratio.size() * 4, &dratio);
+    const float *dratio = nullptr;
+    rc = ratio_resident(ctx, B->ratios, ratio, &dratio);
     if (rc != HIPC_OK) return rc;
-    HIPC_REFUSE(ctx, ctx->capturing, "QLinearMatMul uploads its requantisation ratios: not capturable");
-    HIPC_TRY(ctx, hipMemcpyAsync(dratio, ratio.data(), ratio.size() * 4, hipMemcpyHostToDevice, ctx->stream));
-    HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));
     ga.host_zp = 1, ga.dyn_zp_value = a_zp, ga.const_zp_value = b_zp;
     ga.Y = Y;
-    ga.ratio = static_cast<const float *>(dratio), ga.ratio_step = n_b_scale > 1 ? 1 : 0;
+    ga.ratio = dratio, ga.ratio_step = n_b_scale > 1 ? 1 : 0;
     ga.y_zp = y_zp, ga.out_signed = y_dtype == HIPC_I8;
     return launch_mm<EPI_REQUANT>(ctx, ga);
 }

@@ -81,6 +81,36 @@ def test_vocoder_resblock_shape(ctx, pkg, oracle, dil):
     assert np.count_nonzero((got > 0) & (got < 255)) > 0.6 * got.size   # the case must not saturate away
 
 
+def test_replays_from_a_graph_once_its_ratios_are_resident(ctx, pkg, oracle):
+    """The requantisation ratios are uploaded by the first call with given scales and kept with the
+    weight: the same call is then captured, and each replay requantises a new input correctly. A
+    call whose scales differ would have to upload inside the capture and is refused."""
+    X, W, w_scale, bias, kw = _qconv_case(pkg, 64, 64, 512, 7, 3, seed=77)
+    geom, og = pkg.ConvGeom.make(X.shape, W.shape, **kw), oracle.conv_geom(X.shape, W.shape, **kw)
+    ys = _y_scale(0.02, w_scale, 64 * 7)
+    weight = pkg.ops.ConvWeight(ctx, W, geom)
+    dX, dY, dB = ctx.upload(X), ctx.alloc(X.size), ctx.upload(bias.astype(np.int32))
+    run = lambda s: pkg.ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, 128, weight, w_scale, 0, s, 128, pkg.U8, dB, geom, dY)
+    run(ys)
+    ctx.flush()
+    ctx.capture_begin()
+    run(ys)
+    with pytest.raises(pkg.HipComputeError) as e:
+        run(2 * ys)
+    assert e.value.code == 2
+    graph = ctx.capture_end()
+    for seed in (78, 79):
+        X2 = pkg.synth.uniform_ints(X.size, seed, 0, 255).astype(np.uint8).reshape(X.shape)
+        ctx.upload(X2, dX)
+        ctx.graph_launch(graph)
+        got = ctx.download(dY, np.uint8, X.shape)
+        assert np.array_equal(got, oracle.qlinear_conv(X2, 0.02, 128, W, w_scale, 0, ys, 128, bias, og))
+    ctx.graph_destroy(graph)
+    weight.destroy()
+    for b in (dX, dY, dB):
+        b.free()
+
+
 def test_wide_decoder_variant(ctx, pkg, oracle):
     """512 -> 512 channels, kernel 7, stride 1; T shortened to keep the oracle in seconds."""
     X, W, w_scale, bias, kw = _qconv_case(pkg, 512, 512, 1024, 7, 1, seed=60)
