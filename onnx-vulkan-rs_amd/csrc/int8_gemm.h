@@ -385,12 +385,8 @@ inline int gemm_tile(const GemmArgs &g, unsigned batch) {
 
 template <int MODE, int EPI, bool ALIGNED, int T>
 int gemm_launch_tile(hipc_ctx *ctx, GemmArgs g, unsigned batch) {
-    static bool lds_set = false;  // 128-tiles need more than the default 64 KiB of dynamic LDS
-    if (!lds_set) {
-        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_kernel<MODE, EPI, ALIGNED, T>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds(T)));
-        lds_set = true;
-    }
+    static bool lds_allowed[kMaxDevices] = {};
+    if (int rc = allow_dynamic_lds(ctx, int8_gemm_kernel<MODE, EPI, ALIGNED, T>, gemm_lds(T), lds_allowed)) return rc;
     const dim3 grid(gemm_grid(g, T), 1, batch);
     int8_gemm_kernel<MODE, EPI, ALIGNED, T><<<grid, 256, gemm_lds(T), ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);

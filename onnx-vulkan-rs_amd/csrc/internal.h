@@ -109,6 +109,19 @@ struct RatioCache {
 int ratio_resident(hipc_ctx *ctx, RatioCache &cache, const std::vector<float> &ratio, const float **out);
 void ratio_release(hipc_ctx *ctx, RatioCache &cache);
 
+// Kernels that use more than the default 64 KiB of dynamic LDS must say so once per device. `done` is
+// the launcher's own flag array (one per kernel instantiation); a race between two contexts merely
+// sets the attribute twice.
+constexpr int kMaxDevices = 64;
+template <typename K>
+int allow_dynamic_lds(hipc_ctx *ctx, K kernel, size_t bytes, bool (&done)[kMaxDevices]) {
+    const int d = ctx->device >= 0 && ctx->device < kMaxDevices ? ctx->device : 0;
+    if (done[d] && ctx->device == d) return HIPC_OK;
+    HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    done[d] = true;
+    return HIPC_OK;
+}
+
 // Returns ctx->scratch[slot] grown to at least `bytes`. Growth allocates, so it is
 // refused while a capture is open.
 int scratch_get(hipc_ctx *ctx, int slot, size_t bytes, void **out);

@@ -163,12 +163,8 @@ int fill_common(hipc_ctx *ctx, const MmOperands &o, GemmArgs &g) {
 
 template <int EPI>
 int launch_mm_big(hipc_ctx *ctx, GemmArgs g) {
-    static bool lds_set = false;
-    if (!lds_set) {
-        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(int8_gemm_big_kernel<EPI>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLds));
-        lds_set = true;
-    }
+    static bool lds_allowed[kMaxDevices] = {};
+    if (int rc = allow_dynamic_lds(ctx, int8_gemm_big_kernel<EPI>, kBigLds, lds_allowed)) return rc;
     const dim3 grid(gemm_grid(g, kBigTile), 1, 1);
     int8_gemm_big_kernel<EPI><<<grid, kBigThreads, kBigLds, ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);

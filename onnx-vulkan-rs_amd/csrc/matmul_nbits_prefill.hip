@@ -252,12 +252,8 @@ namespace {
 
 template <int SG, int T>
 int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
-    static bool lds_set = false;  // 128-tiles need more than the default 64 KiB of dynamic LDS
-    if (!lds_set) {
-        HIPC_TRY(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(mmnb_prefill_kernel<SG, T>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)prefill_lds(T)));
-        lds_set = true;
-    }
+    static bool lds_allowed[kMaxDevices] = {};
+    if (int rc = allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T>, prefill_lds(T), lds_allowed)) return rc;
     const int tiles_x = (int)ceil_div(a.N, T), tiles_y = (int)ceil_div(a.M, T);
     int best = 8, best_cost = 1 << 30;
     for (int r = 1; r <= 8; r *= 2) {
