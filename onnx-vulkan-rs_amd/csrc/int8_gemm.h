@@ -419,7 +419,8 @@ constexpr int kBigFI = kBigTile / kBigWM / 32, kBigFJ = kBigTile / kBigWN / 32; 
 constexpr int kBigChunks = kBigTile * (kBK / 16) / kBigThreads;  // 16-byte chunks of a slab per thread
 constexpr size_t kBigLds = 2 * (2 * kBigTile) * kPitch + kBigTile * sizeof(int);
 
-template <int EPI>
+// DYN: the row sums of A are needed (the constant operand's zero point, in the signed domain, is not 0)
+template <int EPI, bool DYN>
 __global__ void __launch_bounds__(kBigThreads) int8_gemm_big_kernel(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     uint8_t *lds_p = lds_raw;                                 // [2][256 * kPitch]
@@ -508,7 +509,8 @@ __global__ void __launch_bounds__(kBigThreads) int8_gemm_big_kernel(const GemmAr
     // reads, buffer loads and LDS writes share the step.
     auto multiply = [&](const Frags &f, int reads, int loads, int writes) {
 #pragma unroll
-        for (int i = 0; i < kBigFI; i++) dsum[i] += dot_ones(f.pf[i]);
+        for (int i = 0; i < kBigFI; i++)
+            if (DYN) dsum[i] += dot_ones(f.pf[i]);
 #pragma unroll
         for (int i = 0; i < kBigFI; i++)
 #pragma unroll

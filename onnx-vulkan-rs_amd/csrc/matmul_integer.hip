@@ -161,14 +161,22 @@ int fill_common(hipc_ctx *ctx, const MmOperands &o, GemmArgs &g) {
     return HIPC_OK;
 }
 
-template <int EPI>
-int launch_mm_big(hipc_ctx *ctx, GemmArgs g) {
+template <int EPI, bool DYN>
+int launch_mm_big_dyn(hipc_ctx *ctx, GemmArgs g) {
     static bool lds_allowed[kMaxDevices] = {};
-    if (int rc = allow_dynamic_lds(ctx, int8_gemm_big_kernel<EPI>, kBigLds, lds_allowed)) return rc;
+    if (int rc = allow_dynamic_lds(ctx, int8_gemm_big_kernel<EPI, DYN>, kBigLds, lds_allowed)) return rc;
     const dim3 grid(gemm_grid(g, kBigTile), 1, 1);
-    int8_gemm_big_kernel<EPI><<<grid, kBigThreads, kBigLds, ctx->stream>>>(g);
+    int8_gemm_big_kernel<EPI, DYN><<<grid, kBigThreads, kBigLds, ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
+}
+
+template <int EPI>
+int launch_mm_big(hipc_ctx *ctx, const GemmArgs &g) {
+    // the row sums of A only matter when the weight's zero point, shifted to the signed domain, is
+    // not zero; the host knows that it is zero when the weight is int8 and carries no zero point
+    const bool zero_known = g.const_shift == 0 && (g.host_zp ? g.const_zp_value == 0 : g.const_zp == nullptr);
+    return zero_known ? launch_mm_big_dyn<EPI, false>(ctx, g) : launch_mm_big_dyn<EPI, true>(ctx, g);
 }
 
 // 256x256 tiles once they fill most of the chip's 256 CUs; HIPC_GEMM_BIG=0/1 overrides (tuning, tests)
