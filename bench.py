@@ -30,8 +30,9 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA, published
 
-# gemma3-1b decoder linears, (K, N, count per layer); lm_head once
-LAYER_LINEARS = [(1152, 1024, 1), (1152, 256, 2), (1024, 1152, 1), (1152, 6912, 2), (6912, 1152, 1)]
+# gemma3-1b decoder linears as the decoder prepacks them, (K, N, count per layer): q|k|v in one
+# weight (1024 + 256 + 256 columns), o, gate|up in one weight (2 x 6912 columns), down; lm_head once
+LAYER_LINEARS = [(1152, 1536, 1), (1024, 1152, 1), (1152, 13824, 1), (6912, 1152, 1)]
 LM_HEAD = (1152, 262144)
 N_LAYERS = 26
 BS = 32
@@ -417,8 +418,8 @@ def main():
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights x f32 activations (bf16x3 MFMA, f32 accumulate)", "data": "synthetic",
         "config": {"workload": "int4 MatMulNBits decode GEMVs of one gemma3-1b-shaped token: 26 layers x "
-                               "(q,k,v,o,gate,up,down) + lm_head 1152->262144, block 32 + zero points, M=1, "
-                               "every weight distinct and HBM-resident, graph replay",
+                               "(q|k|v fused, o, gate|up fused, down) + lm_head 1152->262144, block 32 + zero points, "
+                               "M=1, every weight distinct and HBM-resident, graph replay",
                    "bytes_per_step": head["bytes_per_step"], "launches_per_step": head["launches"],
                    "frac_hbm_peak": head["gbs"] / HBM_PEAK_GBS if head["gbs"] else None},
         "roofline": roof, "cpu_baseline": cpu, "extras": extras,
