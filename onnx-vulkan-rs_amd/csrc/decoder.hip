@@ -246,12 +246,13 @@ dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const _
 // then every thread sums its channel over the chunks
 __global__ void __launch_bounds__(256)
 dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, const float *__restrict__ part_o, int n_q,
-                      int n_kv, int hd, int nsplit, float *__restrict__ out) {
+                      int n_kv, int hd, int nsplit, int even_chunks, float *__restrict__ out) {
     extern __shared__ float wgt[];  // [nsplit]
     __shared__ float red[4];
     const int head = blockIdx.x;
     const int G = n_q / n_kv, kvh = head / G, g = head % G;
-    const int live = min(nsplit, (st->pos + kAttnChunk) / kAttnChunk);  // chunks holding at least one position
+    // chunks holding at least one position: kAttnChunk each, or the context dealt evenly to kAttnSplits
+    const int live = even_chunks ? attn_live_chunks(st->pos + 1) : min(nsplit, (st->pos + kAttnChunk) / kAttnChunk);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float m = -3.0e38f;
     for (int s = tid; s < live; s += 256) m = fmaxf(m, part_ml[(((size_t)kvh * nsplit + s) * G + g) * 2]);
@@ -290,297 +291,268 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
     }
 }
 
-// ---- attention of one decode step in one launch (head_dim <= 256, group x head_dim <= 1024) ----
-// Workgroup (split, kvh) owns kFusedChunk positions of kv head kvh and serves all G query heads of
-// the group. It
-//   1. issues every load of its K and V rows at once (16-byte pieces),
-//   2. meanwhile prepares the step's own q, k, v from the fused qkv vector: per-head RMS norm and
-//      half-split rotary embedding for q and k (every workgroup does this redundantly: 1.3 k
-//      values), k and v rounded to f16 as the cache holds them; the workgroup whose chunk holds
-//      position `pos` writes them into the cache and all use the LDS copy for that position,
-//   3. forms its chunk's scores, running max / sum and unnormalised output (the flash-decoding
-//      partial), and
-//   4. takes a ticket; the workgroup that finds all other live chunks done merges the partials.
-//      Nobody waits for anybody: every workgroup runs straight to its end.
-constexpr int kFusedChunk = 64;
-constexpr int kFusedKP = kFusedChunk / 32;  // passes of 32 positions over the keys
-constexpr int kFusedVP = kFusedChunk / 8;   // positions per thread for the values
-
+// ---- the context chunks of one decode step's attention in one launch (head_dim 64 / 128 / 256) ----
+// Workgroup (split, kvh) owns attn_chunk(total) consecutive positions of kv head kvh, walks them
+// kAttnPass at a time and serves all G query heads of the group. It
+//   1. asks for the fused qkv vector's pieces it needs and for the K and V rows of its first pass
+//      (16-byte pieces, every load of a pass independent of every other),
+//   2. prepares the step's own q, k, v: per-head RMS norm and half-split rotary embedding for q
+//      and k (every workgroup does this redundantly: 1.3 k values), k and v rounded to f16 as the
+//      cache holds them; the workgroup whose chunk holds position `pos` writes them into the cache,
+//      and every use of that position takes the LDS copy,
+//   3. per pass: scores, running max / sum (rescaling what it has), unnormalised output, and
+//   4. writes the chunk's (max, sum) pairs and unnormalised output: the flash-decoding partial.
+// The partials of the live chunks are joined by the consumer (the output projection's prologue,
+// or dec_attn_merge_kernel). HD and G are template parameters so that the body is straight-line
+// code: with them as run-time values it was several times as long, and a workgroup that runs its
+// code once pays for every instruction-cache line it touches.
+template <int HD, int G>
 __global__ void __launch_bounds__(256)
-dec_attn_fused_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
-                      const float *__restrict__ k_norm, int n_q, int n_kv, int hd, float eps, const float *__restrict__ rope,
-                      int max_seq, float scale, __half *__restrict__ k_cache, __half *__restrict__ v_cache, float *part_ml,
-                      float *part_o, unsigned int *tickets, float *__restrict__ out) {
-    extern __shared__ __attribute__((aligned(16))) float lds[];
-    const int G = n_q / n_kv, GH = G * hd;
-    const int split = blockIdx.x, kvh = blockIdx.y, nsplit = gridDim.x;
-    float *qs = lds;                       // [G][hd] query heads, normed and rotated
-    float *kn = qs + GH;                   // [hd] the step's key, as the cache will hold it
-    float *vn = kn + hd;                   // [hd] the step's value
-    float *sc = vn + hd;                   // [G][kFusedChunk]
-    float *ored = sc + G * kFusedChunk;    // [4][G][hd]; the merge reuses it for its weights
-    __shared__ int last_flag;
+dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
+                       const float *__restrict__ k_norm, int n_q, int n_kv, float eps, const float *__restrict__ rope,
+                       int max_seq, float scale, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
+                       float *__restrict__ part_ml, float *__restrict__ part_o) {
+    constexpr int GH = G * HD, NK = HD / 64, HALF = HD / 2;
+    constexpr int KP = kAttnPass / 32;         // passes of 32 positions over the keys (8 threads per position)
+    constexpr int VT = HD / 8;                 // threads per value row (8 channels each)
+    constexpr int VPP = 256 / VT;              // value rows in flight per pass of the workgroup
+    constexpr int VI = kAttnPass / VPP;        // value rows per thread
+    constexpr int ROWS = (G + 1 + 3) / 4;      // q heads and the k head, dealt to four wavefronts
+    static_assert(kAttnPass == 64, "one lane per position of a pass");
+    __shared__ __attribute__((aligned(16))) float qs[GH];      // query heads, normed and rotated
+    __shared__ __attribute__((aligned(16))) float kn[HD];      // the step's key, as the cache will hold it
+    __shared__ __attribute__((aligned(16))) float vn[HD];      // the step's value
+    __shared__ __attribute__((aligned(16))) float sc[G * kAttnPass];
+    __shared__ __attribute__((aligned(16))) float ored[4 * GH];
+    __shared__ float mrun[G], lrun[G], fac[G];
 
+    const int split = blockIdx.x, kvh = blockIdx.y;
     const int pos = st->pos, total = pos + 1;
-    const int t0 = split * kFusedChunk;
-    const int cnt = min(kFusedChunk, total - t0);
-    if (cnt <= 0) return;  // no position of this chunk exists yet
-    const int live = (total + kFusedChunk - 1) / kFusedChunk;
+    const int chunk = attn_chunk(total);
+    const int t_begin = split * chunk;
+    if (t_begin >= total) return;  // no position of this chunk exists yet
+    const int t_end = min(total, t_begin + chunk);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    // 1. K: 8 threads per position, each the 16-byte piece `seg` of every 128-byte run of the row
-    //    (so a position's row is read in whole cache lines); V: thread (pg, cb) reads 8 channels
-    //    of positions pg, pg + 8, pg + 16, ...
-    const int kp = tid >> 3, seg = tid & 7, nk = hd >> 6;
-    uint4 kreg[kFusedKP][4];
+    // 1. the step's own rows first (they come out of L2 and are needed first): rows 0..G-1 are the
+    //    query heads, row G the key head; wavefront w prepares rows w, w + 4, ...; lane l holds
+    //    elements l + 64 i of a row
+    float px[ROWS][NK], pw[ROWS][NK], pc[NK], psn[NK];
 #pragma unroll
-    for (int ps = 0; ps < kFusedKP; ps++) {
-        const __half *krow = k_cache + ((size_t)kvh * max_seq + t0 + min(kp + 32 * ps, cnt - 1)) * hd + seg * 8;
-#pragma unroll
-        for (int u = 0; u < 4; u++) kreg[ps][u] = u < nk ? *reinterpret_cast<const uint4 *>(krow + u * 64) : make_uint4(0, 0, 0, 0);
-    }
-    const int pg = tid >> 5, cb = tid & 31;
-    const bool v_on = cb * 8 < hd;
-    uint4 vreg[kFusedVP];
-#pragma unroll
-    for (int i = 0; i < kFusedVP; i++) {
-        const int tp = min(pg + 8 * i, cnt - 1);
-        vreg[i] = v_on ? *reinterpret_cast<const uint4 *>(v_cache + ((size_t)kvh * max_seq + t0 + tp) * hd + cb * 8)
-                       : make_uint4(0, 0, 0, 0);
-    }
-    // ... and everything the step's own q, k, v need: rows 0..G-1 are the query heads, row G the
-    // key head; wavefront w prepares rows w, w + 4, w + 8; lane l holds elements l + 64 i of a row
-    const int half = hd >> 1;
-    constexpr int kRowsPerWave = (kMaxGroup + 1 + 3) / 4;
-    float px[kRowsPerWave][4], pw[kRowsPerWave][4], pc[4], psn[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int j = (lane + 64 * i) % half;
-        pc[i] = i < nk ? rope[j] : 0.f, psn[i] = i < nk ? rope[half + j] : 0.f;
+    for (int i = 0; i < NK; i++) {
+        const int j = (lane + 64 * i) % HALF;
+        pc[i] = rope[j], psn[i] = rope[HALF + j];
     }
 #pragma unroll
-    for (int rr = 0; rr < kRowsPerWave; rr++) {
-        const int row = wave + 4 * rr;
-        const float *src = row < G ? qkv + (size_t)(kvh * G + row) * hd : qkv + (size_t)(n_q + kvh) * hd;
+    for (int rr = 0; rr < ROWS; rr++) {
+        const int row = min(wave + 4 * rr, G);
+        const float *src = row < G ? qkv + (size_t)(kvh * G + row) * HD : qkv + (size_t)(n_q + kvh) * HD;
         const float *w = row < G ? q_norm : k_norm;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const bool on = row <= G && i < nk;
-            px[rr][i] = on ? src[lane + 64 * i] : 0.f, pw[rr][i] = on ? w[lane + 64 * i] : 0.f;
-        }
+        for (int i = 0; i < NK; i++) px[rr][i] = src[lane + 64 * i], pw[rr][i] = w[lane + 64 * i];
     }
-    const float pv_own = tid < hd ? qkv[(size_t)(n_q + n_kv + kvh) * hd + tid] : 0.f;
-    // 2. per-head RMS norm and half-split rotary embedding (pairs d, d + hd/2), one wavefront per
-    //    row and no workgroup barrier: with hd = 128 or 256 both members of a pair sit in one lane
-    //    (elements i and i + nk/2), with hd = 64 in lanes l and l + 32
+    const float pv_own = qkv[(size_t)(n_q + n_kv + kvh) * HD + min(tid, HD - 1)];
+    //    K: thread (kp, seg) reads the 16-byte piece `seg` of every 128-byte run of rows kp and
+    //    kp + 32 (a row is read in whole cache lines); V: thread (pg, cb) reads 8 channels of rows
+    //    pg, pg + VPP, ...  Rows past the end repeat the last one (their weights are zero).
+    const int kp = tid >> 3, seg = tid & 7;
+    const int pg = tid / VT, cb = tid % VT;
+    const __half *k_head = k_cache + (size_t)kvh * max_seq * HD + seg * 8;
+    const __half *v_head = v_cache + (size_t)kvh * max_seq * HD + cb * 8;
+    uint4 kreg[KP][NK], vreg[VI];
+    auto load_k = [&](int t0) {
 #pragma unroll
-    for (int rr = 0; rr < kRowsPerWave; rr++) {
+        for (int ps = 0; ps < KP; ps++) {
+            const __half *krow = k_head + (size_t)min(t0 + kp + 32 * ps, t_end - 1) * HD;
+#pragma unroll
+            for (int u = 0; u < NK; u++) kreg[ps][u] = *reinterpret_cast<const uint4 *>(krow + u * 64);
+        }
+    };
+    auto load_v = [&](int t0) {
+#pragma unroll
+        for (int i = 0; i < VI; i++)
+            vreg[i] = *reinterpret_cast<const uint4 *>(v_head + (size_t)min(t0 + pg + VPP * i, t_end - 1) * HD);
+    };
+    load_k(t_begin);
+    load_v(t_begin);
+
+    // 2. per-head RMS norm and half-split rotary embedding (pairs d, d + HD/2), one wavefront per
+    //    row and no workgroup barrier: with HD = 128 or 256 both members of a pair sit in one lane
+    //    (elements i and i + NK/2), with HD = 64 in lanes l and l + 32
+#pragma unroll
+    for (int rr = 0; rr < ROWS; rr++) {
         const int row = wave + 4 * rr;
-        if (row > G) break;
-        float sq = 0.f;
+        if (row <= G) {
+            float sq = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; i++) sq += px[rr][i] * px[rr][i];
+            for (int i = 0; i < NK; i++) sq += px[rr][i] * px[rr][i];
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) sq += __shfl_xor(sq, off, 64);
-        const float inv = rsqrtf(sq / (float)hd + eps);
-        float x[4], r[4];
+            for (int off = 32; off >= 1; off >>= 1) sq += __shfl_xor(sq, off, 64);
+            const float inv = rsqrtf(sq / (float)HD + eps);
+            float x[NK], r[NK];
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = px[rr][i] * inv * pw[rr][i], r[i] = 0.f;
-        if (nk == 1) {
-            const float other = __shfl_xor(x[0], 32, 64);
-            r[0] = lane < 32 ? x[0] * pc[0] - other * psn[0] : x[0] * pc[0] + other * psn[0];
-        } else {
-            const int hk = nk >> 1;
+            for (int i = 0; i < NK; i++) x[i] = px[rr][i] * inv * pw[rr][i];
+            if (NK == 1) {
+                const float other = __shfl_xor(x[0], 32, 64);
+                r[0] = lane < 32 ? x[0] * pc[0] - other * psn[0] : x[0] * pc[0] + other * psn[0];
+            } else {
+                constexpr int HK = NK / 2 > 0 ? NK / 2 : 1;
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                if (i < hk) {
-                    r[i] = x[i] * pc[i] - x[i + hk] * psn[i];
-                    r[i + hk] = x[i + hk] * pc[i] + x[i] * psn[i];
+                for (int i = 0; i < HK; i++) {
+                    r[i] = x[i] * pc[i] - x[(i + HK) % NK] * psn[i];
+                    r[(i + HK) % NK] = x[(i + HK) % NK] * pc[i] + x[i] * psn[i];
                 }
             }
+            float *dst = row < G ? qs + row * HD : kn;
+#pragma unroll
+            for (int i = 0; i < NK; i++) dst[lane + 64 * i] = row < G ? r[i] : __half2float(__float2half(r[i]));
         }
-        float *dst = row < G ? qs + row * hd : kn;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (i < nk) dst[lane + 64 * i] = row < G ? r[i] : __half2float(__float2half(r[i]));
     }
-    if (tid < hd) vn[tid] = __half2float(__float2half(pv_own));
+    if (tid < HD) vn[tid] = __half2float(__float2half(pv_own));
+    if (tid < G) mrun[tid] = -3.0e38f, lrun[tid] = 0.f;
     __syncthreads();
-    const bool owner = pos >= t0 && pos < t0 + kFusedChunk;
-    if (owner && tid < hd) {
-        k_cache[((size_t)kvh * max_seq + pos) * hd + tid] = __float2half(kn[tid]);
-        v_cache[((size_t)kvh * max_seq + pos) * hd + tid] = __float2half(vn[tid]);
+    if (pos >= t_begin && tid < HD) {  // pos = total - 1 lies in the last live chunk
+        k_cache[((size_t)kvh * max_seq + pos) * HD + tid] = __float2half(kn[tid]);
+        v_cache[((size_t)kvh * max_seq + pos) * HD + tid] = __float2half(vn[tid]);
     }
-    // 3a. scores
+
+    float o[G][8];
 #pragma unroll
-    for (int ps = 0; ps < kFusedKP; ps++) {
-        const int tp = kp + 32 * ps;
-        const bool fresh = t0 + tp == pos;
-        float dot[kMaxGroup];
+    for (int g = 0; g < G; g++)
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; g++) dot[g] = 0.f;
+        for (int e = 0; e < 8; e++) o[g][e] = 0.f;
+
+    for (int t0 = t_begin; t0 < t_end; t0 += kAttnPass) {
+        const int cnt = min(kAttnPass, t_end - t0);
+        const bool more = t0 + kAttnPass < t_end;
+        // 3a. scores. The row of `pos` as loaded is not the step's key: it counts as zero here and
+        //     the thread that owns it takes the key from LDS below.
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            if (u < nk) {
-                const __half2 *h2 = reinterpret_cast<const __half2 *>(&kreg[ps][u]);
+        for (int ps = 0; ps < KP; ps++) {
+            const int tp = kp + 32 * ps;
+            const bool stale = min(t0 + tp, t_end - 1) == pos;
+            float dot[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) dot[g] = 0.f;
+#pragma unroll
+            for (int u = 0; u < NK; u++) {
+                const uint4 raw = stale ? make_uint4(0, 0, 0, 0) : kreg[ps][u];
+                const __half2 *h2 = reinterpret_cast<const __half2 *>(&raw);
                 float kf[8];
 #pragma unroll
                 for (int e = 0; e < 4; e++) kf[2 * e] = __low2float(h2[e]), kf[2 * e + 1] = __high2float(h2[e]);
                 const int c0 = u * 64 + seg * 8;
-                if (fresh) {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) kf[e] = kn[c0 + e];
+                for (int g = 0; g < G; g++) {
+                    const float4 qa = *reinterpret_cast<const float4 *>(qs + g * HD + c0);
+                    const float4 qb = *reinterpret_cast<const float4 *>(qs + g * HD + c0 + 4);
+                    dot[g] += (qa.x * kf[0] + qa.y * kf[1]) + (qa.z * kf[2] + qa.w * kf[3]) +
+                              (qb.x * kf[4] + qb.y * kf[5]) + (qb.z * kf[6] + qb.w * kf[7]);
                 }
+            }
+            if (t0 + tp == pos) {
+#pragma unroll 1
+                for (int u = 0; u < NK; u++) {
+                    const int c0 = u * 64 + seg * 8;
+                    const float4 ka = *reinterpret_cast<const float4 *>(kn + c0), kb = *reinterpret_cast<const float4 *>(kn + c0 + 4);
 #pragma unroll
-                for (int g = 0; g < kMaxGroup; g++) {
-                    if (g < G) {
-                        const float4 qa = *reinterpret_cast<const float4 *>(qs + g * hd + c0);
-                        const float4 qb = *reinterpret_cast<const float4 *>(qs + g * hd + c0 + 4);
-                        dot[g] += (qa.x * kf[0] + qa.y * kf[1]) + (qa.z * kf[2] + qa.w * kf[3]) +
-                                  (qb.x * kf[4] + qb.y * kf[5]) + (qb.z * kf[6] + qb.w * kf[7]);
+                    for (int g = 0; g < G; g++) {
+                        const float4 qa = *reinterpret_cast<const float4 *>(qs + g * HD + c0);
+                        const float4 qb = *reinterpret_cast<const float4 *>(qs + g * HD + c0 + 4);
+                        dot[g] += (qa.x * ka.x + qa.y * ka.y) + (qa.z * ka.z + qa.w * ka.w) +
+                                  (qb.x * kb.x + qb.y * kb.y) + (qb.z * kb.z + qb.w * kb.w);
                     }
                 }
             }
-        }
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; g++) {
-            if (g < G) {
+            for (int g = 0; g < G; g++) {
                 float v = dot[g];
                 v += __shfl_xor(v, 1, 64);
                 v += __shfl_xor(v, 2, 64);
                 v += __shfl_xor(v, 4, 64);
-                if (seg == 0) sc[g * kFusedChunk + tp] = v * scale;
+                if (seg == 0) sc[g * kAttnPass + tp] = v * scale;
             }
         }
-    }
-    __syncthreads();
-    float *ml = part_ml + ((size_t)kvh * nsplit + split) * G * 2;
-    static_assert(kFusedChunk == 64, "one lane per position of the chunk");
-    for (int g = wave; g < G; g += 4) {
-        const float x = lane < cnt ? sc[g * kFusedChunk + lane] : -3.0e38f;
-        float m = x;
+        if (more) load_k(t0 + kAttnPass);
+        __syncthreads();
+        // 3b. one wavefront per head: the pass's max and sum join the running pair
+        for (int g = wave; g < G; g += 4) {
+            const float x = lane < cnt ? sc[g * kAttnPass + lane] : -3.0e38f;
+            const float m_old = mrun[g], l_old = lrun[g];
+            float m = x;
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-        const float pv = lane < cnt ? __expf(x - m) : 0.f;
-        float l = pv;
+            for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+            m = fmaxf(m, m_old);
+            const float pv = lane < cnt ? __expf(x - m) : 0.f;
+            float l = pv;
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
-        sc[g * kFusedChunk + lane] = pv;
-        if (lane == 0) ml[g * 2] = m, ml[g * 2 + 1] = l;
-    }
-    __syncthreads();
-    // 3b. unnormalised output: 8 channels x G heads per thread over its positions
-    {
-        float o[kMaxGroup][8];
+            for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
+            const float f = __expf(m_old - m);
+            sc[g * kAttnPass + lane] = pv;
+            if (lane == 0) mrun[g] = m, lrun[g] = l_old * f + l, fac[g] = f;
+        }
+        __syncthreads();
+        // 3c. unnormalised output: 8 channels x G heads per thread over its rows
+        {
+            float fg[G];
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; g++)
+            for (int g = 0; g < G; g++) fg[g] = fac[g];
 #pragma unroll
-            for (int e = 0; e < 8; e++) o[g][e] = 0.f;
+            for (int g = 0; g < G; g++)
 #pragma unroll
-        for (int i = 0; i < kFusedVP; i++) {
-            const int tp = pg + 8 * i;
-            if (tp < cnt && v_on) {
-                const __half2 *h2 = reinterpret_cast<const __half2 *>(&vreg[i]);
+                for (int e = 0; e < 8; e++) o[g][e] *= fg[g];
+#pragma unroll
+            for (int i = 0; i < VI; i++) {
+                const int tp = pg + VPP * i;
+                const bool stale = min(t0 + tp, t_end - 1) == pos;
+                const uint4 raw = stale ? make_uint4(0, 0, 0, 0) : vreg[i];
+                const __half2 *h2 = reinterpret_cast<const __half2 *>(&raw);
                 float vf[8];
 #pragma unroll
                 for (int e = 0; e < 4; e++) vf[2 * e] = __low2float(h2[e]), vf[2 * e + 1] = __high2float(h2[e]);
-                if (t0 + tp == pos) {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) vf[e] = vn[cb * 8 + e];
+                for (int g = 0; g < G; g++) {
+                    const float w = sc[g * kAttnPass + tp];  // zero past the end of the pass
+#pragma unroll
+                    for (int e = 0; e < 8; e++) o[g][e] += w * vf[e];
                 }
+            }
+            const int own = pos - t0;  // the step's own position, if this pass holds it
+            if (own >= 0 && own < kAttnPass && (own % VPP) == pg) {
+                const float4 va = *reinterpret_cast<const float4 *>(vn + cb * 8), vb = *reinterpret_cast<const float4 *>(vn + cb * 8 + 4);
 #pragma unroll
-                for (int g = 0; g < kMaxGroup; g++) {
-                    if (g < G) {
-                        const float w = sc[g * kFusedChunk + tp];
-#pragma unroll
-                        for (int e = 0; e < 8; e++) o[g][e] += w * vf[e];
-                    }
+                for (int g = 0; g < G; g++) {
+                    const float w = sc[g * kAttnPass + own];
+                    o[g][0] += w * va.x, o[g][1] += w * va.y, o[g][2] += w * va.z, o[g][3] += w * va.w;
+                    o[g][4] += w * vb.x, o[g][5] += w * vb.y, o[g][6] += w * vb.z, o[g][7] += w * vb.w;
                 }
             }
         }
-        // lanes l and l + 32 hold the same channels of neighbouring position groups
+        if (more) load_v(t0 + kAttnPass);
+        // the next pass rewrites sc only after the barrier that follows its scores' LDS reads of qs;
+        // its writes to sc must not overtake this pass's reads of sc
+        __syncthreads();
+    }
+    // 4. lanes VT apart hold the same channels of neighbouring rows; then the four wavefronts
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; g++) {
-            if (g < G) {
+    for (int g = 0; g < G; g++) {
 #pragma unroll
-                for (int e = 0; e < 8; e++) o[g][e] += __shfl_xor(o[g][e], 32, 64);
-                if (lane < 32 && v_on) {
-                    float4 *dst = reinterpret_cast<float4 *>(ored + (wave * G + g) * hd + cb * 8);
-                    dst[0] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
-                    dst[1] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
-                }
-            }
+        for (int e = 0; e < 8; e++) {
+#pragma unroll
+            for (int off = VT; off < 64; off <<= 1) o[g][e] += __shfl_xor(o[g][e], off, 64);
+        }
+        if (lane < VT) {
+            float4 *dst = reinterpret_cast<float4 *>(ored + (wave * G + g) * HD + cb * 8);
+            dst[0] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
+            dst[1] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
         }
     }
     __syncthreads();
-    float *po = part_o + ((size_t)kvh * nsplit + split) * GH;
+    float *po = part_o + ((size_t)kvh * kAttnSplits + split) * GH;
     for (int idx = tid; idx < GH; idx += 256)
         po[idx] = (ored[idx] + ored[GH + idx]) + (ored[2 * GH + idx] + ored[3 * GH + idx]);
-    // 4. the last workgroup of this kv head to get here merges
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = atomicAdd(&tickets[kvh], 1u);
-        last_flag = t == (unsigned int)(live - 1);
-        if (last_flag) tickets[kvh] = 0u;  // everyone else has already taken theirs
-    }
-    __syncthreads();
-    if (!last_flag) return;
-    __threadfence();
-    // The partials were written by other CUs during this launch: read them at device scope (past
-    // this CU's vector cache), as buffer loads so that many are in flight at once.
-    const __amdgpu_buffer_rsrc_t r_ml = __builtin_amdgcn_make_buffer_rsrc(
-        part_ml + (size_t)kvh * nsplit * G * 2, 0, nsplit * G * 2 * 4, 0x00020000);
-    const __amdgpu_buffer_rsrc_t r_po = __builtin_amdgcn_make_buffer_rsrc(
-        part_o + (size_t)kvh * nsplit * GH, 0, nsplit * GH * 4, 0x00020000);
-    constexpr int kDev = 16;  // cache policy: device scope
-    // (max, sum) of every (chunk, head) in one round trip, then the heads' maxima, the chunk
-    // weights exp(m_s - m) and the normalisers out of LDS: [live * G] each, pair index s * G + g
-    float *mm = ored, *lw = ored + live * G, *wgt = ored + 2 * live * G;  // 3 * live * G <= 4 * G * hd floats
-    // thread -> four channels of one head. The first kAhead chunks' outputs are requested together
-    // with the statistics, so the two round trips overlap.
-    constexpr int kAhead = 16;
-    const bool owns = tid * 4 < GH;
-    u32x4 v[kAhead];
-#pragma unroll
-    for (int u = 0; u < kAhead; u++)
-        v[u] = owns ? __builtin_amdgcn_raw_buffer_load_b128(r_po, (min(u, live - 1) * GH + tid * 4) * 4, 0, kDev) : u32x4{0, 0, 0, 0};
-    for (int i = tid; i < live * G; i += 256) {
-        const uint2 st2 = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r_ml, i * 8, 0, kDev));
-        mm[i] = __uint_as_float(st2.x), lw[i] = __uint_as_float(st2.y);
-    }
-    __syncthreads();
-    for (int i = tid; i < live * G; i += 256) {
-        const int g = i % G;
-        float m = -3.0e38f;
-        for (int s = 0; s < live; s++) m = fmaxf(m, mm[s * G + g]);
-        const float e = __expf(mm[i] - m);
-        wgt[i] = e;
-        lw[i] *= e;
-    }
-    __syncthreads();
-    if (owns) {
-        const int g = tid * 4 / hd;
-        float l = 0.f;
-        for (int s = 0; s < live; s++) l += lw[s * G + g];
-        const float inv = 1.f / l;
-        float o[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int s0 = 0; s0 < live; s0 += kAhead) {
-            if (s0 > 0) {
-#pragma unroll
-                for (int u = 0; u < kAhead; u++)
-                    v[u] = __builtin_amdgcn_raw_buffer_load_b128(r_po, (min(s0 + u, live - 1) * GH + tid * 4) * 4, 0, kDev);
-            }
-#pragma unroll
-            for (int u = 0; u < kAhead; u++) {
-                const float ws = s0 + u < live ? wgt[(s0 + u) * G + g] : 0.f;
-                const float4 f = __builtin_bit_cast(float4, v[u]);
-                o[0] += f.x * ws, o[1] += f.y * ws, o[2] += f.z * ws, o[3] += f.w * ws;
-            }
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++) out[(size_t)kvh * GH + tid * 4 + e] = o[e] * inv;
-    }
+    float *ml = part_ml + ((size_t)kvh * kAttnSplits + split) * G * 2;
+    if (tid < G) ml[tid * 2] = mrun[tid], ml[tid * 2 + 1] = lrun[tid];
 }
 
 // h[i] = gelu_tanh(gu[i]) * gu[ffn + i]
@@ -667,13 +639,11 @@ struct hipc_decoder {
     float *x = nullptr, *xn = nullptr, *qkv = nullptr, *q = nullptr, *attn = nullptr, *y = nullptr, *gu = nullptr,
           *h = nullptr, *logits = nullptr, *part_ml = nullptr, *part_o = nullptr, *am_v = nullptr;
     int *am_i = nullptr;
-    unsigned int *tickets = nullptr;
     float *rope = nullptr;      // [head_dim] cosines then sines of the current position
     float *x2 = nullptr;        // second buffer of the residual stream
     bool fused_glue = false;    // norms, residual adds and the gated GELU run inside the GEMV prologues
     int nsplit = 0;
-    int nsplit_fused = 0;       // chunks of the one-launch attention; 0: the shape takes the three-kernel path
-    size_t fused_lds = 0;
+    bool one_launch_attn = false;  // head_dim and group size have an instance of dec_attn_chunks_kernel
     std::vector<void *> owned;
 };
 
@@ -685,6 +655,35 @@ template <typename T>
 int dev_alloc(hipc_ctx *ctx, hipc_decoder *d, T **p, size_t count) {
     HIPC_TRY(ctx, hipMalloc(reinterpret_cast<void **>(p), std::max<size_t>(count * sizeof(T), 16)));
     d->owned.push_back(*p);
+    return HIPC_OK;
+}
+
+template <int HD, int G>
+void attn_chunks_launch(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale) {
+    const hipc_decoder_config &c = d->cfg;
+    dec_attn_chunks_kernel<HD, G><<<dim3(kAttnSplits, c.n_kv_heads), 256, 0, ctx->stream>>>(
+        d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.rms_eps, d->rope, c.max_seq,
+        scale, l.k_cache, l.v_cache, d->part_ml, d->part_o);
+}
+
+template <int HD>
+void attn_chunks_launch_g(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale, int G) {
+    switch (G) {
+        case 1: attn_chunks_launch<HD, 1>(ctx, d, l, scale); break;
+        case 2: attn_chunks_launch<HD, 2>(ctx, d, l, scale); break;
+        case 4: attn_chunks_launch<HD, 4>(ctx, d, l, scale); break;
+        default: attn_chunks_launch<HD, 8>(ctx, d, l, scale); break;
+    }
+}
+
+int launch_attn_chunks(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale) {
+    const int G = d->cfg.n_q_heads / d->cfg.n_kv_heads;
+    switch (d->cfg.head_dim) {
+        case 64: attn_chunks_launch_g<64>(ctx, d, l, scale, G); break;
+        case 128: attn_chunks_launch_g<128>(ctx, d, l, scale, G); break;
+        default: attn_chunks_launch_g<256>(ctx, d, l, scale, G); break;
+    }
+    HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }
 
@@ -732,24 +731,20 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
     A(&d->x, c.hidden), A(&d->xn, c.hidden), A(&d->qkv, (size_t)(c.n_q_heads + 2 * c.n_kv_heads) * c.head_dim);
     A(&d->q, (size_t)c.n_q_heads * c.head_dim), A(&d->attn, (size_t)c.n_q_heads * c.head_dim), A(&d->y, c.hidden);
     A(&d->gu, (size_t)2 * c.ffn), A(&d->h, c.ffn), A(&d->logits, c.vocab);
-    A(&d->part_ml, (size_t)c.n_kv_heads * d->nsplit * G * 2), A(&d->part_o, (size_t)c.n_kv_heads * d->nsplit * G * c.head_dim);
+    const size_t parts = (size_t)c.n_kv_heads * std::max(d->nsplit, kAttnSplits) * G;
+    A(&d->part_ml, parts * 2), A(&d->part_o, parts * c.head_dim);
     A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
-    A(&d->tickets, (size_t)c.n_kv_heads), A(&d->rope, (size_t)c.head_dim), A(&d->x2, c.hidden);
+    A(&d->rope, (size_t)c.head_dim), A(&d->x2, c.hidden);
     {
         const char *e = getenv("HIPC_DEC_FUSED_GLUE");  // 0: keep the separate norm / GELU kernels (tests of that path)
         d->fused_glue = c.hidden % 8 == 0 && c.ffn % 8 == 0 && !(e && atoi(e) == 0);
     }
     {
-        const int GH = G * c.head_dim, chunks = (int)ceil_div(c.max_seq, kFusedChunk);
         const char *e = getenv("HIPC_DEC_FUSED_ATTN");  // 0: keep the three-kernel attention (tests of that path)
-        if ((c.head_dim == 64 || c.head_dim == 128 || c.head_dim == 256) && GH <= 1024 && 3 * chunks <= 4 * c.head_dim && chunks <= 65535 && !(e && atoi(e) == 0)) {
-            d->nsplit_fused = chunks;
-            d->fused_lds = (size_t)(GH + 2 * c.head_dim + G * kFusedChunk + 4 * GH) * sizeof(float);
-        }
+        d->one_launch_attn = (c.head_dim == 64 || c.head_dim == 128 || c.head_dim == 256) && (G == 1 || G == 2 || G == 4 || G == 8) &&
+                             !(e && atoi(e) == 0);
     }
     if (rc == HIPC_OK) {
-        if (hipMemsetAsync(d->tickets, 0, (size_t)c.n_kv_heads * sizeof(unsigned int), ctx->stream) != hipSuccess)
-            rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the attention tickets");
         for (DecLayer &l : d->layers) {  // an unwritten cache row must not hold NaN bit patterns
             if (hipMemsetAsync(l.k_cache, 0, kv * 2, ctx->stream) != hipSuccess || hipMemsetAsync(l.v_cache, 0, kv * 2, ctx->stream) != hipSuccess)
                 rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the KV cache");
@@ -889,23 +884,31 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         } else {
             if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.qkv, d->qkv, 1, terms)) != HIPC_OK) return rc;
         }
-        if (d->nsplit_fused) {
-            dec_attn_fused_kernel<<<dim3(d->nsplit_fused, c.n_kv_heads), 256, d->fused_lds, s>>>(
-                d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.head_dim,
-                c.rms_eps, d->rope, c.max_seq, scale, l.k_cache, l.v_cache, d->part_ml, d->part_o, d->tickets, d->attn);
-            HIPC_LAUNCHED(ctx);
+        if (d->one_launch_attn) {
+            if ((rc = launch_attn_chunks(ctx, d, l, scale)) != HIPC_OK) return rc;
+            if (d->fused_glue) {  // the output projection joins the chunks' partials in its prologue
+                GemvPrologue merge;
+                merge.mode = 3, merge.part_o = d->part_o, merge.part_ml = d->part_ml, merge.pos = &d->state->pos;
+                merge.group = c.n_q_heads / c.n_kv_heads, merge.head_dim = c.head_dim;
+                if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms, &merge)) != HIPC_OK) return rc;
+            } else {
+                dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)kAttnSplits * sizeof(float), s>>>(
+                    d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads, c.head_dim, kAttnSplits, 1, d->attn);
+                HIPC_LAUNCHED(ctx);
+                if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
+            }
         } else {
-        dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
-                                             c.n_kv_heads, c.head_dim, c.rms_eps, c.rope_theta, c.max_seq, d->q, l.k_cache, l.v_cache);
-        HIPC_LAUNCHED(ctx);
-        dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
-                                                                             c.head_dim, c.max_seq, scale, d->part_ml, d->part_o);
-        HIPC_LAUNCHED(ctx);
-        dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
-                                                                                         c.head_dim, d->nsplit, d->attn);
-        HIPC_LAUNCHED(ctx);
+            dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
+                                                 c.n_kv_heads, c.head_dim, c.rms_eps, c.rope_theta, c.max_seq, d->q, l.k_cache, l.v_cache);
+            HIPC_LAUNCHED(ctx);
+            dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
+                                                                                 c.head_dim, c.max_seq, scale, d->part_ml, d->part_o);
+            HIPC_LAUNCHED(ctx);
+            dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
+                                                                                             c.head_dim, d->nsplit, 0, d->attn);
+            HIPC_LAUNCHED(ctx);
+            if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
         }
-        if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
         if (d->fused_glue) {
             GemvPrologue pro;
             pro.mode = 2, pro.x = xc, pro.y = d->y, pro.w_post = l.norm[HIPC_DEC_NORM_POST_ATTN];

@@ -140,12 +140,32 @@ void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
 //   mode 1  A = [gate | up] (2K floats): the row is gelu_tanh(gate) * up
 //   mode 2  the row is rmsnorm(x', w_in), x' = x + rmsnorm(y, w_post) (x' = x when y is null);
 //           x' is also written to x_out (not x itself) when x_out is set. A is ignored.
+//   mode 3  the row is the attention output of the step, joined from the flash-decoding partials
+//           of its kAttnSplits context chunks: part_o [kv head][split][group * head_dim]
+//           unnormalised outputs, part_ml [kv head][split][group] (max, sum) pairs; the number of
+//           live chunks follows from *pos (see attn_live_chunks). A is ignored.
 struct GemvPrologue {
     int mode = 0;
     const float *x = nullptr, *y = nullptr, *w_post = nullptr, *w_in = nullptr;
     float *x_out = nullptr;
     float eps = 0.f;
+    const float *part_o = nullptr, *part_ml = nullptr;
+    const int *pos = nullptr;
+    int group = 0, head_dim = 0;
 };
+// Decode attention splits the context of a kv head over kAttnSplits workgroups. Each takes
+// `attn_chunk(total)` consecutive positions, a multiple of kAttnPass, so that all splits together
+// cover `total` positions; the first attn_live_chunks(total) splits hold at least one position
+// and only those write a partial.
+constexpr int kAttnPass = 64;
+constexpr int kAttnSplits = 32;
+__host__ __device__ inline int attn_chunk(int total) {
+    return kAttnPass * ((total + kAttnPass * kAttnSplits - 1) / (kAttnPass * kAttnSplits));
+}
+__host__ __device__ inline int attn_live_chunks(int total) {
+    const int c = attn_chunk(total);
+    return (total + c - 1) / c;
+}
 int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
                const GemvPrologue *pro = nullptr);
 int64_t nbits_cols(const hipc_nbits_weight *w);

@@ -167,6 +167,11 @@ struct GemvArgs {
     const float *nx, *ny, *nw_post, *nw_in;
     float *nx_out;
     float eps;
+    // attention-merge prologue: nx = partial outputs, ny = (max, sum) pairs
+    const int *npos;
+    int ngroup, nhd;
+    int nparts;   // ways the live chunks are divided among threads that share four channels
+    int pro_off;  // byte offset of the prologue's own LDS area
 };
 
 template <int SG>
@@ -237,6 +242,9 @@ __device__ __forceinline__ uint32_t bf16_rne(float v) {  // bits of the nearest 
 //   2  rmsnorm(x', nw_in) with x' = nx + rmsnorm(ny, nw_post) (x' = nx when ny is null); every
 //      workgroup forms the two sums of squares over the whole row itself, workgroup (0, 0) also
 //      writes x' to nx_out (a different buffer than nx: others may still be reading nx)
+//   3  the attention output of the step: sum_s exp(m_s - m) o_s / sum_s exp(m_s - m) l_s over the
+//      live context chunks s of each head (flash-decoding merge); every workgroup forms the whole
+//      row itself out of L2
 template <int T, int NR, int SG, int MC, int NT, int PRO>
 __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel(const GemvArgs p) {
     extern __shared__ uint4 smem[];
@@ -318,6 +326,58 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
         }
         inv2 = rsqrtf(block_total(sq2) / (float)p.K + p.eps);
     }
+    float *mrow = nullptr;  // PRO 3: [nparts][K] partial sums of the merged row, then inv per head
+    float *minv = nullptr;
+    if (PRO == 3) {
+        const int live = attn_live_chunks(*p.npos + 1);
+        const int G = p.ngroup, hd = p.nhd, GH = G * hd, n_q = p.K / hd;
+        float *wgt = reinterpret_cast<float *>(reinterpret_cast<char *>(smem) + p.pro_off);  // [n_q][kAttnSplits]
+        minv = wgt + n_q * kAttnSplits;                                                     // [n_q]
+        mrow = minv + ((n_q + 3) & ~3);
+        const int nw = nthreads >> 6, ln = tid & 63, wv = tid >> 6;
+        static_assert(kAttnSplits <= 64, "one lane per chunk");
+        auto stat_at = [&](int h) {
+            const int hh = min(h, n_q - 1), kvh = hh / G, g = hh % G;
+            return *reinterpret_cast<const float2 *>(p.ny + (((size_t)kvh * kAttnSplits + min(ln, live - 1)) * G + g) * 2);
+        };
+        float2 ml = stat_at(wv);                 // the statistics are asked for first ...
+        load_stage(first_ng, first_tile, stA);   // ... the first weight tile travels meanwhile
+        for (int h = wv; h < n_q; h += nw) {
+            if (h != wv) ml = stat_at(h);
+            const bool on = ln < live;
+            float m = on ? ml.x : -3.0e38f;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+            const float e = on ? __expf(ml.x - m) : 0.f;
+            float l = on ? ml.y * e : 0.f;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
+            if (ln < kAttnSplits) wgt[h * kAttnSplits + ln] = e;
+            if (ln == 0) minv[h] = 1.f / l;
+        }
+        __syncthreads();
+        const int groups4 = p.K >> 2;
+        for (int u = tid; u < groups4 * p.nparts; u += nthreads) {
+            const int c4 = u % groups4, part = u / groups4;
+            const int e0 = c4 * 4, h = e0 / hd, kvh = h / G;
+            const int s0 = part * live / p.nparts, s1 = (part + 1) * live / p.nparts;
+            const float *src = p.nx + (size_t)kvh * kAttnSplits * GH + (e0 - kvh * GH);
+            const float *wh = wgt + h * kAttnSplits;
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int s = s0; s < s1; s += 8) {
+                float4 f[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) f[j] = *reinterpret_cast<const float4 *>(src + (size_t)min(s + j, s1 - 1) * GH);
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float ws = s + j < s1 ? wh[s + j] : 0.f;
+                    o.x += f[j].x * ws, o.y += f[j].y * ws, o.z += f[j].z * ws, o.w += f[j].w * ws;
+                }
+            }
+            *reinterpret_cast<float4 *>(mrow + (size_t)part * p.K + e0) = o;
+        }
+        __syncthreads();
+    }
     auto load_item_vec = [&](int item, float av[8]) {
         int m, c, w;
         const int k0 = min(item_k0(item, m, c, w), p.K - 8);  // padding chunks are zeroed by split_item
@@ -345,6 +405,17 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
                 const float xp = p.ny ? x8[i] + y8[i] * inv1 * p8[i] : x8[i];
                 av[i] = xp * inv2 * w8[i];
             }
+        } else if (PRO == 3) {
+            const float inv = minv[k0 / p.nhd];
+#pragma unroll
+            for (int i = 0; i < 8; i++) av[i] = 0.f;
+            for (int part = 0; part < p.nparts; part++) {
+                const float4 a = *reinterpret_cast<const float4 *>(mrow + (size_t)part * p.K + k0);
+                const float4 b = *reinterpret_cast<const float4 *>(mrow + (size_t)part * p.K + k0 + 4);
+                av[0] += a.x, av[1] += a.y, av[2] += a.z, av[3] += a.w, av[4] += b.x, av[5] += b.y, av[6] += b.z, av[7] += b.w;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) av[i] *= inv;
         } else if (p.a_f16) {
             const uint4 raw = *reinterpret_cast<const uint4 *>(static_cast<const __half *>(p.A) + (size_t)m * p.K + k0);
             const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
@@ -404,7 +475,7 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     if (p.a_vec) {
         float av[8];
         load_item_vec(min(tid, nitems - 1), av);
-        if (PRO != 2) load_stage(first_ng, first_tile, stA);
+        if (PRO != 2 && PRO != 3) load_stage(first_ng, first_tile, stA);
         if (tid < nitems) split_item(tid, av);
         for (int item = tid + nthreads; item < nitems; item += nthreads) {
             load_item_vec(item, av);
@@ -675,6 +746,8 @@ void launch_gemv_nr(const GemvArgs &a, int pro, int NR, int SG, dim3 grid, dim3 
         launch_gemv_sg<T, 1, 1, 2, 1>(a, SG, grid, block, lds, s);
     else if (a.M == 1 && pro == 2 && NT == 2)
         launch_gemv_sg<T, 1, 1, 2, 2>(a, SG, grid, block, lds, s);
+    else if (a.M == 1 && pro == 3 && NT == 2)
+        launch_gemv_sg<T, 1, 1, 2, 3>(a, SG, grid, block, lds, s);
     else if (a.M == 1)
         launch_gemv_sg<T, 1, 1, NT>(a, SG, grid, block, lds, s);
     else if (NR == 1)
@@ -751,6 +824,20 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
             HIPC_REQUIRE(ctx, aligned(pro->x, 16) && aligned(pro->w_in, 16) && (!pro->y || (aligned(pro->y, 16) && aligned(pro->w_post, 16))),
                          "MatMulNBits gemv: norm prologue operands must be 16-byte aligned");
             a.nx = pro->x, a.ny = pro->y, a.nw_post = pro->w_post, a.nw_in = pro->w_in, a.nx_out = pro->x_out, a.eps = pro->eps;
+            a.a_vec = 1;
+        }
+        if (mode == 3) {
+            HIPC_REQUIRE(ctx, pro->part_o && pro->part_ml && pro->pos && pro->group > 0 && pro->head_dim > 0 &&
+                                  pro->head_dim % 8 == 0 && w->K % ((int64_t)pro->group * pro->head_dim) == 0,
+                         "MatMulNBits gemv: attention prologue operands missing or K not a whole number of head groups");
+            HIPC_REQUIRE(ctx, aligned(pro->part_o, 16) && aligned(pro->part_ml, 8), "MatMulNBits gemv: attention partials must be 16-byte aligned");
+            HIPC_REQUIRE(ctx, ksplit == 1, "MatMulNBits gemv: the attention prologue needs the whole row in one workgroup");
+            a.nx = pro->part_o, a.ny = pro->part_ml, a.npos = pro->pos, a.ngroup = pro->group, a.nhd = pro->head_dim;
+            const int groups4 = (int)(w->K / 4), n_q = (int)(w->K / pro->head_dim);
+            a.nparts = std::max(1, std::min(4, (int)block.x / groups4));
+            a.pro_off = (int)((lds + 15) & ~(size_t)15);
+            lds = (size_t)a.pro_off + ((size_t)n_q * kAttnSplits + ((n_q + 3) & ~3) + (size_t)a.nparts * w->K) * 4;
+            HIPC_REQUIRE(ctx, lds <= 64 * 1024, "MatMulNBits gemv: LDS plan of %zu bytes does not fit", lds);
             a.a_vec = 1;
         }
     }

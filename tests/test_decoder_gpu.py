@@ -40,6 +40,53 @@ def test_decode_steps_match_the_oracle(ctx, pkg, oracle):
     dec.destroy()
 
 
+DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / group size the chunk kernel is built for
+    (256, 4, 1, 2046),   # crosses from 64 to 128 positions per workgroup at 2048
+    (128, 8, 1, 4290),   # three passes per workgroup, the last one ragged
+    (64, 2, 2, 2300),    # one query head per kv head
+    (128, 4, 2, 130),    # three live chunks only
+    (192, 2, 1, 100),    # no instance for this head_dim: the three-kernel path
+]
+PATHS = [{}, {"HIPC_DEC_FUSED_GLUE": "0"}, {"HIPC_DEC_FUSED_ATTN": "0"}]
+
+
+@pytest.mark.parametrize("env", PATHS, ids=["default", "separate-glue", "three-kernel-attention"])
+@pytest.mark.parametrize("hd,nq,nkv,p0", DEEP)
+def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, monkeypatch, hd, nq, nkv, p0, env):
+    """Steps taken deep into a context whose cache rows hold random f16 values on both sides: the
+    chunked attention (several passes per workgroup, the join in the output projection's prologue
+    or in the merge kernel) against the oracle's softmax over the whole context."""
+    from oracle import decoder as od
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)   # read when the decoder is created
+    cfg = dict(SMALL, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd)
+    steps, max_seq = 3, p0 + 8
+    w = pkg.decoder.build_weights(cfg, seed=11)
+    dec = pkg.decoder.Decoder(ctx, cfg, max_seq)
+    dec.load(w)
+    ref = od.Decoder(w, max_seq)
+    rng = np.random.default_rng(hd + p0)
+    for li in range(cfg["n_layers"]):
+        kptr, vptr = dec.kv_cache(li)
+        for ptr, dst in ((kptr, ref.k), (vptr, ref.v)):
+            rows = (rng.standard_normal((nkv, max_seq, hd)) * 0.7).astype(np.float16)
+            dst[li] = rows
+            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, rows.ctypes.data, rows.nbytes))
+    token = 23
+    dec.reset(token, p0)
+    for pos in range(p0, p0 + steps):
+        dec.step()
+        got_tok, got_pos, logits, _ = dec.read(want_logits=True)
+        want_logits, _ = ref.step(token, pos)
+        assert got_pos == pos + 1
+        err = np.abs(logits - want_logits)
+        assert np.all(err <= 2e-3 + 2e-3 * np.abs(want_logits)), (pos, float(err.max()))
+        k_row = ctx.download(dec.kv_cache(1)[0], np.float16, (hd,), offset=((nkv - 1) * max_seq + pos) * hd * 2)
+        assert np.allclose(k_row.astype(np.float32), ref.k[1, nkv - 1, pos].astype(np.float32), atol=2e-3, rtol=2e-3), pos
+        token = got_tok
+    dec.destroy()
+
+
 def test_a_captured_step_replays_without_patching(ctx, pkg):
     """Position and token live on the device: replaying one captured step N times must give the
     same tokens as N eager steps."""
