@@ -158,7 +158,7 @@ struct GemvPrologue {
 // cover `total` positions; the first attn_live_chunks(total) splits hold at least one position
 // and only those write a partial.
 constexpr int kAttnPass = 64;
-constexpr int kAttnSplits = 32;
+constexpr int kAttnSplits = 64;
 __host__ __device__ inline int attn_chunk(int total) {
     return kAttnPass * ((total + kAttnPass * kAttnSplits - 1) / (kAttnPass * kAttnSplits));
 }
