@@ -318,6 +318,13 @@ int hipc_decoder_set_norm(hipc_ctx *ctx, hipc_decoder *dec, int layer, int which
 /* the int4 embedding table [vocab, hidden] in the GatherBlockQuantized layout */
 int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *dec, const void *B, size_t b_len, const void *scales,
                                size_t scales_len, const void *zp, size_t zp_len);
+/* Attention of one layer: `window` > 0 limits it to the last `window` positions, the step's own
+ * included (GroupQueryAttention's local_window_size, interp.rs:7528; the bound is the reference's,
+ * shaders/attention.rs:202-214 and :250: key t is masked when pos - t >= window); window <= 0 is
+ * the default, the whole context. `rope_theta` > 0 replaces the configuration's base for this layer
+ * (gemma3's local layers rotate with another base than its global ones; the reference gets the
+ * tables as the operator's cos / sin cache inputs); at most two distinct bases per decoder. */
+int hipc_decoder_set_layer_attention(hipc_ctx *ctx, hipc_decoder *dec, int layer, int32_t window, float rope_theta);
 /* the token the next step consumes and its position (= tokens already in the cache) */
 int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *dec, int32_t token, int32_t pos);
 /* device pointers of one layer's resident f16 cache, [n_kv_heads, max_seq, head_dim] each */

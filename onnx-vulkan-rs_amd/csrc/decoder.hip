@@ -46,16 +46,21 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 
 // x = embed_scale * dequant(table[token]); xn = rmsnorm(x, w). One workgroup. It also leaves the
 // step's rotary table behind: rope[j] = cos(pos * theta^(-2j/hd)), rope[hd/2 + j] = the sine, which
-// every layer's attention reads instead of evaluating the functions again.
+// every layer's attention reads instead of evaluating the functions again; a second table for the
+// layers that rotate with another base follows at rope[hd...] when theta2 > 0.
 __global__ void __launch_bounds__(256)
 dec_embed_kernel(const DecState *st, const uint8_t *__restrict__ q, const float *__restrict__ scales,
                  const uint8_t *__restrict__ zp, int hidden, int bs, int n_blocks, float embed_scale,
                  const float *__restrict__ w, float eps, float *__restrict__ x, float *__restrict__ xn, int hd, float theta,
-                 float *__restrict__ rope) {
+                 float theta2, float *__restrict__ rope) {
     __shared__ float red[4];
     for (int j = threadIdx.x; j < hd / 2; j += 256) {
         const float ang = (float)st->pos * powf(theta, -2.f * (float)j / (float)hd);
         rope[j] = cosf(ang), rope[hd / 2 + j] = sinf(ang);
+        if (theta2 > 0.f) {
+            const float ang2 = (float)st->pos * powf(theta2, -2.f * (float)j / (float)hd);
+            rope[hd + j] = cosf(ang2), rope[hd + hd / 2 + j] = sinf(ang2);
+        }
     }
     const size_t row = (size_t)st->token;
     const size_t row_bytes = (size_t)n_blocks * bs / 2, zp_row = (n_blocks + 1) / 2;
@@ -151,7 +156,7 @@ constexpr int kAttnChunk = 16;
 constexpr int kMaxGroup = 8;
 __global__ void __launch_bounds__(256)
 dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const __half *__restrict__ k_cache,
-                        const __half *__restrict__ v_cache, int n_q, int n_kv, int hd, int max_seq, float scale,
+                        const __half *__restrict__ v_cache, int n_q, int n_kv, int hd, int max_seq, float scale, int window,
                         float *__restrict__ part_ml, float *__restrict__ part_o) {
     __shared__ float qs[kMaxGroup * 512];
     __shared__ float sc[kMaxGroup][kAttnChunk];
@@ -162,8 +167,11 @@ dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const _
     const int tid = threadIdx.x;
     const int cnt = min(kAttnChunk, total - t0);
     float *ml = part_ml + ((size_t)kvh * nsplit + split) * G * 2;
-    if (cnt <= 0) {  // nothing here yet: a neutral partial
+    const int t_first = attn_first(total, window);  // positions before it are outside the layer's window
+    if (cnt <= 0 || t0 + cnt <= t_first) {  // nothing here yet, or nothing visible any more: a neutral partial
         if (tid < G) ml[tid * 2] = -3.0e38f, ml[tid * 2 + 1] = 0.f;
+        if (cnt > 0)
+            for (int i = tid; i < G * hd; i += 256) part_o[((size_t)kvh * nsplit + split) * G * hd + i] = 0.f;
         return;
     }
     // values first: thread d owns channel d (and d + 256) of every row of the chunk
@@ -217,11 +225,12 @@ dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const _
     __syncthreads();
     // softmax pieces: thread g handles head g (the chunk is 16 values)
     if (tid < G) {
+        const int lo = max(0, t_first - t0);  // first visible position of the chunk
         float m = -3.0e38f;
-        for (int t = 0; t < cnt; t++) m = fmaxf(m, sc[tid][t]);
+        for (int t = lo; t < cnt; t++) m = fmaxf(m, sc[tid][t]);
         float l = 0.f;
         for (int t = 0; t < kAttnChunk; t++) {
-            const float pv = t < cnt ? __expf(sc[tid][t] - m) : 0.f;
+            const float pv = t >= lo && t < cnt ? __expf(sc[tid][t] - m) : 0.f;
             sc[tid][t] = pv;
             l += pv;
         }
@@ -246,13 +255,14 @@ dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const _
 // then every thread sums its channel over the chunks
 __global__ void __launch_bounds__(256)
 dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, const float *__restrict__ part_o, int n_q,
-                      int n_kv, int hd, int nsplit, int even_chunks, float *__restrict__ out) {
+                      int n_kv, int hd, int nsplit, int even_chunks, int window, float *__restrict__ out) {
     extern __shared__ float wgt[];  // [nsplit]
     __shared__ float red[4];
     const int head = blockIdx.x;
     const int G = n_q / n_kv, kvh = head / G, g = head % G;
     // chunks holding at least one position: kAttnChunk each, or the context dealt evenly to kAttnSplits
-    const int live = even_chunks ? attn_live_chunks(st->pos + 1) : min(nsplit, (st->pos + kAttnChunk) / kAttnChunk);
+    const int total = st->pos + 1;
+    const int live = even_chunks ? attn_live_chunks(total - attn_first(total, window)) : min(nsplit, (st->pos + kAttnChunk) / kAttnChunk);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float m = -3.0e38f;
     for (int s = tid; s < live; s += 256) m = fmaxf(m, part_ml[(((size_t)kvh * nsplit + s) * G + g) * 2]);
@@ -292,7 +302,7 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
 }
 
 // ---- the context chunks of one decode step's attention in one launch (head_dim 64 / 128 / 256) ----
-// Workgroup (split, kvh) owns attn_chunk(total) consecutive positions of kv head kvh, walks them
+// Workgroup (split, kvh) owns attn_chunk(span) consecutive visible positions of kv head kvh, walks them
 // kAttnPass at a time and serves all G query heads of the group. It
 //   1. asks for the fused qkv vector's pieces it needs and for the K and V rows of its first pass
 //      (16-byte pieces, every load of a pass independent of every other),
@@ -310,7 +320,7 @@ template <int HD, int G>
 __global__ void __launch_bounds__(256)
 dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
                        const float *__restrict__ k_norm, int n_q, int n_kv, float eps, const float *__restrict__ rope,
-                       int max_seq, float scale, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
+                       int max_seq, float scale, int window, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
                        float *__restrict__ part_ml, float *__restrict__ part_o) {
     constexpr int GH = G * HD, NK = HD / 64, HALF = HD / 2;
     constexpr int KP = kAttnPass / 32;         // passes of 32 positions over the keys (8 threads per position)
@@ -328,8 +338,9 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int pos = st->pos, total = pos + 1;
-    const int chunk = attn_chunk(total);
-    const int t_begin = split * chunk;
+    const int t_first = attn_first(total, window);  // a local layer sees the last `window` positions only
+    const int chunk = attn_chunk(total - t_first);
+    const int t_begin = t_first + split * chunk;
     if (t_begin >= total) return;  // no position of this chunk exists yet
     const int t_end = min(total, t_begin + chunk);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -625,6 +636,8 @@ struct DecLayer {
     hipc_nbits_weight *qkv = nullptr, *o = nullptr, *gate_up = nullptr, *down = nullptr;
     float *norm[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};  // input, post_attn, pre_ffn, post_ffn, q, k
     __half *k_cache = nullptr, *v_cache = nullptr;
+    int window = 0;      // > 0: attention sees the last `window` positions only
+    int rope_table = 0;  // 0: the configuration's rotary base, 1: the decoder's second base
 };
 
 struct hipc_decoder {
@@ -639,7 +652,8 @@ struct hipc_decoder {
     float *x = nullptr, *xn = nullptr, *qkv = nullptr, *q = nullptr, *attn = nullptr, *y = nullptr, *gu = nullptr,
           *h = nullptr, *logits = nullptr, *part_ml = nullptr, *part_o = nullptr, *am_v = nullptr;
     int *am_i = nullptr;
-    float *rope = nullptr;      // [head_dim] cosines then sines of the current position
+    float *rope = nullptr;      // 2 x [head_dim]: cosines then sines of the current position, per rotary base
+    float theta2 = 0.f;         // the second rotary base (0: none in use)
     float *x2 = nullptr;        // second buffer of the residual stream
     bool fused_glue = false;    // norms, residual adds and the gated GELU run inside the GEMV prologues
     int nsplit = 0;
@@ -662,8 +676,8 @@ template <int HD, int G>
 void attn_chunks_launch(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale) {
     const hipc_decoder_config &c = d->cfg;
     dec_attn_chunks_kernel<HD, G><<<dim3(kAttnSplits, c.n_kv_heads), 256, 0, ctx->stream>>>(
-        d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.rms_eps, d->rope, c.max_seq,
-        scale, l.k_cache, l.v_cache, d->part_ml, d->part_o);
+        d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.rms_eps,
+        d->rope + (size_t)l.rope_table * c.head_dim, c.max_seq, scale, l.window, l.k_cache, l.v_cache, d->part_ml, d->part_o);
 }
 
 template <int HD>
@@ -734,7 +748,7 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
     const size_t parts = (size_t)c.n_kv_heads * std::max(d->nsplit, kAttnSplits) * G;
     A(&d->part_ml, parts * 2), A(&d->part_o, parts * c.head_dim);
     A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
-    A(&d->rope, (size_t)c.head_dim), A(&d->x2, c.hidden);
+    A(&d->rope, (size_t)2 * c.head_dim), A(&d->x2, c.hidden);
     {
         const char *e = getenv("HIPC_DEC_FUSED_GLUE");  // 0: keep the separate norm / GELU kernels (tests of that path)
         d->fused_glue = c.hidden % 8 == 0 && c.ffn % 8 == 0 && !(e && atoi(e) == 0);
@@ -838,6 +852,25 @@ int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *d, const void *B, si
     return HIPC_OK;
 }
 
+int hipc_decoder_set_layer_attention(hipc_ctx *ctx, hipc_decoder *d, int layer, int32_t window, float rope_theta) {
+    if (!ctx || !d) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REFUSE(ctx, ctx->capturing, "decoder: layer attention changed while a capture is open");
+    HIPC_REQUIRE(ctx, layer >= 0 && layer < d->cfg.n_layers, "decoder: layer %d out of range", layer);
+    HIPC_REQUIRE(ctx, !(rope_theta < 0.f) && rope_theta == rope_theta, "decoder: bad rotary base");
+    DecLayer &l = d->layers[layer];
+    int table = 0;
+    if (rope_theta > 0.f && rope_theta != d->cfg.rope_theta) {
+        HIPC_REQUIRE(ctx, d->theta2 == 0.f || d->theta2 == rope_theta,
+                     "decoder: a third rotary base (%g beside %g and %g)", rope_theta, d->cfg.rope_theta, d->theta2);
+        d->theta2 = rope_theta;
+        table = 1;
+    }
+    l.window = window > 0 ? window : 0;
+    l.rope_table = table;
+    return HIPC_OK;
+}
+
 int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *d, int32_t token, int32_t pos) {
     if (!ctx || !d) return HIPC_ERR_INVALID;
     Guard g(ctx);
@@ -868,7 +901,7 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
     int rc;
     dec_embed_kernel<<<1, 256, 0, s>>>(d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
                                        d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn, c.head_dim, c.rope_theta,
-                                       d->rope);
+                                       d->theta2, d->rope);
     HIPC_LAUNCHED(ctx);
     // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
     // branch into the stream reads one and (its first workgroup) writes the other.
@@ -889,23 +922,24 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
             if (d->fused_glue) {  // the output projection joins the chunks' partials in its prologue
                 GemvPrologue merge;
                 merge.mode = 3, merge.part_o = d->part_o, merge.part_ml = d->part_ml, merge.pos = &d->state->pos;
-                merge.group = c.n_q_heads / c.n_kv_heads, merge.head_dim = c.head_dim;
+                merge.group = c.n_q_heads / c.n_kv_heads, merge.head_dim = c.head_dim, merge.window = l.window;
                 if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms, &merge)) != HIPC_OK) return rc;
             } else {
                 dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)kAttnSplits * sizeof(float), s>>>(
-                    d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads, c.head_dim, kAttnSplits, 1, d->attn);
+                    d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads, c.head_dim, kAttnSplits, 1, l.window, d->attn);
                 HIPC_LAUNCHED(ctx);
                 if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
             }
         } else {
             dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
-                                                 c.n_kv_heads, c.head_dim, c.rms_eps, c.rope_theta, c.max_seq, d->q, l.k_cache, l.v_cache);
+                                                 c.n_kv_heads, c.head_dim, c.rms_eps, l.rope_table ? d->theta2 : c.rope_theta, c.max_seq, d->q,
+                                                 l.k_cache, l.v_cache);
             HIPC_LAUNCHED(ctx);
             dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
-                                                                                 c.head_dim, c.max_seq, scale, d->part_ml, d->part_o);
+                                                                                 c.head_dim, c.max_seq, scale, l.window, d->part_ml, d->part_o);
             HIPC_LAUNCHED(ctx);
             dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
-                                                                                             c.head_dim, d->nsplit, 0, d->attn);
+                                                                                             c.head_dim, d->nsplit, 0, l.window, d->attn);
             HIPC_LAUNCHED(ctx);
             if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
         }

@@ -143,7 +143,7 @@ void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
 //   mode 3  the row is the attention output of the step, joined from the flash-decoding partials
 //           of its kAttnSplits context chunks: part_o [kv head][split][group * head_dim]
 //           unnormalised outputs, part_ml [kv head][split][group] (max, sum) pairs; the number of
-//           live chunks follows from *pos (see attn_live_chunks). A is ignored.
+//           live chunks follows from *pos and the layer's window (see attn_live_chunks). A is ignored.
 struct GemvPrologue {
     int mode = 0;
     const float *x = nullptr, *y = nullptr, *w_post = nullptr, *w_in = nullptr;
@@ -151,12 +151,12 @@ struct GemvPrologue {
     float eps = 0.f;
     const float *part_o = nullptr, *part_ml = nullptr;
     const int *pos = nullptr;
-    int group = 0, head_dim = 0;
+    int group = 0, head_dim = 0, window = 0;
 };
-// Decode attention splits the context of a kv head over kAttnSplits workgroups. Each takes
-// `attn_chunk(total)` consecutive positions, a multiple of kAttnPass, so that all splits together
-// cover `total` positions; the first attn_live_chunks(total) splits hold at least one position
-// and only those write a partial.
+// Decode attention splits the visible context of a kv head (`span` positions: all of them, or the
+// last `window`) over kAttnSplits workgroups. Each takes `attn_chunk(span)` consecutive positions,
+// a multiple of kAttnPass, so that all splits together cover the span; the first
+// attn_live_chunks(span) splits hold at least one position and only those write a partial.
 constexpr int kAttnPass = 64;
 constexpr int kAttnSplits = 64;
 __host__ __device__ inline int attn_chunk(int total) {
@@ -166,6 +166,8 @@ __host__ __device__ inline int attn_live_chunks(int total) {
     const int c = attn_chunk(total);
     return (total + c - 1) / c;
 }
+// first visible position of a step that sees `total` positions through a window (<= 0: no window)
+__host__ __device__ inline int attn_first(int total, int window) { return window > 0 && total > window ? total - window : 0; }
 int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
                const GemvPrologue *pro = nullptr);
 int64_t nbits_cols(const hipc_nbits_weight *w);

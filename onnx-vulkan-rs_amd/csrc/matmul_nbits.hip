@@ -169,7 +169,7 @@ struct GemvArgs {
     float eps;
     // attention-merge prologue: nx = partial outputs, ny = (max, sum) pairs
     const int *npos;
-    int ngroup, nhd;
+    int ngroup, nhd, nwindow;
     int nparts;   // ways the live chunks are divided among threads that share four channels
     int pro_off;  // byte offset of the prologue's own LDS area
 };
@@ -392,7 +392,8 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     float *mrow = nullptr;  // PRO 3: [nparts][K] partial sums of the merged row, then inv per head
     float *minv = nullptr;
     if (PRO == 3) {
-        const int live = attn_live_chunks(*p.npos + 1);
+        const int total = *p.npos + 1;
+        const int live = attn_live_chunks(total - attn_first(total, p.nwindow));
         const int G = p.ngroup, hd = p.nhd, GH = G * hd, n_q = p.K / hd;
         float *wgt = reinterpret_cast<float *>(reinterpret_cast<char *>(smem) + p.pro_off);  // [n_q][kAttnSplits]
         minv = wgt + n_q * kAttnSplits;                                                     // [n_q]
@@ -891,7 +892,7 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
                          "MatMulNBits gemv: attention prologue operands missing or K not a whole number of head groups");
             HIPC_REQUIRE(ctx, aligned(pro->part_o, 16) && aligned(pro->part_ml, 8), "MatMulNBits gemv: attention partials must be 16-byte aligned");
             HIPC_REQUIRE(ctx, ksplit == 1, "MatMulNBits gemv: the attention prologue needs the whole row in one workgroup");
-            a.nx = pro->part_o, a.ny = pro->part_ml, a.npos = pro->pos, a.ngroup = pro->group, a.nhd = pro->head_dim;
+            a.nx = pro->part_o, a.ny = pro->part_ml, a.npos = pro->pos, a.ngroup = pro->group, a.nhd = pro->head_dim, a.nwindow = pro->window;
             const int groups4 = (int)(w->K / 4), n_q = (int)(w->K / pro->head_dim);
             a.nparts = std::max(1, std::min(4, (int)block.x / groups4));
             a.pro_off = (int)((lds + 15) & ~(size_t)15);

@@ -99,6 +99,11 @@ class Decoder:
     def reset(self, token: int, pos: int = 0):
         self.ctx._check(self.ctx.lib.hipc_decoder_reset(self.ctx.handle, self.handle, token, pos))
 
+    def set_layer_attention(self, layer: int, window: int = 0, rope_theta: float = 0.0):
+        """``window`` > 0: the layer sees its last ``window`` positions only (GroupQueryAttention's
+        local_window_size); ``rope_theta`` > 0: this layer's rotary base."""
+        self.ctx._check(self.ctx.lib.hipc_decoder_set_layer_attention(self.ctx.handle, self.handle, layer, window, rope_theta))
+
     def kv_cache(self, layer: int):
         k, v = C.c_void_p(), C.c_void_p()
         self.ctx._check(self.ctx.lib.hipc_decoder_kv_cache(self.ctx.handle, self.handle, layer, C.byref(k), C.byref(v)))

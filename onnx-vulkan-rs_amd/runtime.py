@@ -105,6 +105,7 @@ SIGNATURES = {
     "hipc_decoder_set_norm": (_int, [_vp, _vp, _int, _int, _vp]),
     "hipc_decoder_set_embedding": (_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz]),
     "hipc_decoder_reset": (_int, [_vp, _vp, C.c_int32, C.c_int32]),
+    "hipc_decoder_set_layer_attention": (_int, [_vp, _vp, _int, C.c_int32, _f]),
     "hipc_decoder_kv_cache": (_int, [_vp, _vp, _int, C.POINTER(_vp), C.POINTER(_vp)]),
     "hipc_decoder_step": (_int, [_vp, _vp]),
     "hipc_decoder_read": (_int, [_vp, _vp, C.POINTER(C.c_int32), C.POINTER(C.c_int32), _vp, _vp, C.c_int32]),

@@ -60,12 +60,32 @@ def gather_block_quantized(table, row, hidden, bs):
     return ((nib[:hidden] - z[blk]).astype(f32) * scales.reshape(-1, nb)[row][blk]).astype(f32)
 
 
+def attend(q, K, V, pos, window, scale):
+    """One query head at position `pos` over the cache rows K, V [>= pos + 1, hd] (float16):
+    softmax(scale * K q) V over the visible keys. Key t is visible iff t <= pos and, with a window,
+    pos - t < window (attention.rs:202-214, :250)."""
+    first = max(0, pos + 1 - window) if window > 0 else 0
+    Kf, Vf = K[first: pos + 1].astype(f32), V[first: pos + 1].astype(f32)
+    s = (Kf @ q) * f32(scale)
+    p = np.exp(s - s.max()).astype(f32)
+    return (p @ Vf) / f32(p.sum(dtype=f32))
+
+
 class Decoder:
     def __init__(self, weights, max_seq):
         self.w, self.cfg = weights, weights.cfg
         c = self.cfg
         self.k = np.zeros((c["n_layers"], c["n_kv_heads"], max_seq, c["head_dim"]), np.float16)
         self.v = np.zeros_like(self.k)
+        # per layer: sliding window (0 = the whole context) and rotary base. Key t is visible from
+        # position pos iff t <= pos and pos - t < window (attention.rs:202-214, :250): `window`
+        # keys, the step's own included.
+        self.window = [0] * c["n_layers"]
+        self.theta = [c["rope_theta"]] * c["n_layers"]
+
+    def set_layer_attention(self, li, window=0, rope_theta=0.0):
+        self.window[li] = window if window > 0 else 0
+        self.theta[li] = rope_theta if rope_theta > 0 else self.cfg["rope_theta"]
 
     def _lin(self, x, li, which):
         B, scales, zp = self.w.linears[(li, which)]
@@ -83,18 +103,15 @@ class Decoder:
             q = qkv[: nq * hd].reshape(nq, hd)
             k = qkv[nq * hd: (nq + nkv) * hd].reshape(nkv, hd)
             v = qkv[(nq + nkv) * hd:].reshape(nkv, hd)
-            q = np.stack([rope_half(rmsnorm(q[h], w.norms[(li, NORM_Q)], c["rms_eps"]), pos, c["rope_theta"]) for h in range(nq)])
+            theta = self.theta[li]
+            q = np.stack([rope_half(rmsnorm(q[h], w.norms[(li, NORM_Q)], c["rms_eps"]), pos, theta) for h in range(nq)])
             for h in range(nkv):
-                self.k[li, h, pos] = rope_half(rmsnorm(k[h], w.norms[(li, NORM_K)], c["rms_eps"]), pos, c["rope_theta"]).astype(np.float16)
+                self.k[li, h, pos] = rope_half(rmsnorm(k[h], w.norms[(li, NORM_K)], c["rms_eps"]), pos, theta).astype(np.float16)
                 self.v[li, h, pos] = v[h].astype(np.float16)
             attn = np.empty((nq, hd), f32)
             g = nq // nkv
             for h in range(nq):
-                K = self.k[li, h // g, : pos + 1].astype(f32)
-                V = self.v[li, h // g, : pos + 1].astype(f32)
-                s = (K @ q[h]) * scale
-                p = np.exp(s - s.max()).astype(f32)
-                attn[h] = (p @ V) / f32(p.sum(dtype=f32))
+                attn[h] = attend(q[h], self.k[li, h // g], self.v[li, h // g], pos, self.window[li], scale)
             y = self._lin(attn.reshape(-1), li, O)
             x = (x + rmsnorm(y, w.norms[(li, NORM_POST_ATTN)], c["rms_eps"])).astype(f32)
             xn = rmsnorm(x, w.norms[(li, NORM_PRE_FFN)], c["rms_eps"])

@@ -87,6 +87,65 @@ def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, monkeypatch, hd, n
     dec.destroy()
 
 
+WINDOWS = [  # (head_dim, query heads, kv heads, first position, window of layer 0, window of layer 1)
+    (256, 4, 1, 2300, 512, 0),     # gemma3's local window beside a global layer
+    (128, 4, 2, 509, 512, 100),    # the window starts to mask at 512 positions, i.e. during these steps
+    (64, 2, 2, 4400, 4200, 70),    # a window longer than one pass of all chunks; one shorter than a chunk
+    (192, 2, 1, 100, 40, 16),      # the three-kernel path: whole 16-position chunks fall out of the window
+]
+
+
+@pytest.mark.parametrize("env", PATHS, ids=["default", "separate-glue", "three-kernel-attention"])
+@pytest.mark.parametrize("hd,nq,nkv,p0,w0,w1", WINDOWS)
+def test_sliding_windows_and_a_second_rotary_base(ctx, pkg, oracle, monkeypatch, hd, nq, nkv, p0, w0, w1, env):
+    """Local layers: the last `window` positions only, the step's own included (the reference's
+    bound, shaders/attention.rs:202-214), rotating with their own base; against the oracle over a
+    filled cache, across the step at which the window starts to cut."""
+    from oracle import decoder as od
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    cfg = dict(SMALL, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd, rope_theta=1.0e6)
+    steps, max_seq = 5, p0 + 8
+    w = pkg.decoder.build_weights(cfg, seed=12)
+    dec = pkg.decoder.Decoder(ctx, cfg, max_seq)
+    dec.load(w)
+    ref = od.Decoder(w, max_seq)
+    for li, win in enumerate((w0, w1)):
+        theta = 10000.0 if win else 0.0          # local layers use the second base
+        dec.set_layer_attention(li, win, theta)
+        ref.set_layer_attention(li, win, theta)
+    rng = np.random.default_rng(hd + p0)
+    for li in range(cfg["n_layers"]):
+        kptr, vptr = dec.kv_cache(li)
+        for ptr, dst in ((kptr, ref.k), (vptr, ref.v)):
+            rows = (rng.standard_normal((nkv, max_seq, hd)) * 0.7).astype(np.float16)
+            dst[li] = rows
+            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, rows.ctypes.data, rows.nbytes))
+    token = 31
+    dec.reset(token, p0)
+    for pos in range(p0, p0 + steps):
+        dec.step()
+        got_tok, got_pos, logits, _ = dec.read(want_logits=True)
+        want_logits, _ = ref.step(token, pos)
+        assert got_pos == pos + 1
+        err = np.abs(logits - want_logits)
+        assert np.all(err <= 2e-3 + 2e-3 * np.abs(want_logits)), (pos, float(err.max()))
+        token = got_tok
+    dec.destroy()
+
+
+def test_a_third_rotary_base_is_refused(ctx, pkg):
+    dec = pkg.decoder.Decoder(ctx, SMALL, 16)
+    dec.set_layer_attention(0, 8, 500.0)
+    dec.set_layer_attention(1, 0, 500.0)
+    with pytest.raises(pkg.HipComputeError) as e:
+        dec.set_layer_attention(1, 0, 700.0)
+    assert "third rotary base" in e.value.message
+    with pytest.raises(pkg.HipComputeError):
+        dec.set_layer_attention(2, 0, 0.0)
+    dec.destroy()
+
+
 def test_a_captured_step_replays_without_patching(ctx, pkg):
     """Position and token live on the device: replaying one captured step N times must give the
     same tokens as N eager steps."""

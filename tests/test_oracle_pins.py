@@ -329,6 +329,30 @@ def test_decoder_glue_against_float64_closed_forms(oracle):
     assert np.allclose(g, 0.5 * t * (1 + np.tanh(np.sqrt(2 / np.pi) * (t + 0.044715 * t ** 3))), atol=1e-6)
 
 
+def test_attention_window_is_the_reference_mask(oracle):
+    """The oracle slices the visible keys; the reference writes -3.4028235e38 into the masked scores
+    of the whole row (`t > pq`, and with a window `pq - t >= window`, shaders/attention.rs:249-254)
+    and takes a softmax over all of it. Same result, in float64, for windows around every boundary."""
+    from oracle import decoder as od
+    rng = np.random.default_rng(5)
+    hd, rows = 16, 40
+    K = rng.standard_normal((rows, hd)).astype(np.float16)
+    V = rng.standard_normal((rows, hd)).astype(np.float16)
+    q = rng.standard_normal(hd).astype(np.float32)
+    for pq in (0, 1, 7, 31):
+        for window in (-1, 0, 1, 2, 7, 8, 9, 32, 100):
+            t = np.arange(rows)
+            masked = t > pq
+            if window > 0:                       # the operator's attribute defaults to -1: no window
+                masked |= (pq - t) >= window
+            scores = np.where(masked, -3.4028235e38, 0.25 * (K.astype(np.float64) @ q.astype(np.float64)))
+            p = np.exp(scores - scores.max())
+            want = (p / p.sum()) @ V.astype(np.float64)
+            assert int((~masked).sum()) == (min(window, pq + 1) if window > 0 else pq + 1)
+            got = od.attend(q, K, V, pq, window, 0.25)
+            assert np.allclose(got, want, rtol=2e-5, atol=2e-6), (pq, window)
+
+
 def test_gather_block_quantized_is_a_row_of_the_dequantised_table(oracle, pkg):
     from oracle import decoder as od
     a, nib, zp, scale = rc.matmul_nbits_case(1, 100, 9, 32)
