@@ -40,7 +40,7 @@ struct GemmArgs {
     // P operand: MODE_MM  -> the activation matrix A [I, K] (u8 / i8, pitch K)
     //            MODE_CONV -> prepacked weight [I_pad, K_pad] signed
     const uint8_t *P;
-    // Q operand: MODE_MM  -> prepacked B [J_pad, K_pad] signed
+    // Q operand: MODE_MM  -> prepacked B, J_pad x K_pad signed bytes, fragment-major (qfrag_offset)
     //            MODE_CONV -> NHWC activations, already signed
     const uint8_t *Q;
     const int32_t *const_sum;  // sums over k of the prepacked operand (per j in MM, per i in CONV)
@@ -81,6 +81,17 @@ inline unsigned gemm_grid(GemmArgs &g, int tile = kBM) {
     g.xcd_rows = best_a, g.xcd_cols = 8 / best_a;
     const int rows_per = (tiles_y + g.xcd_rows - 1) / g.xcd_rows, cols_per = (tiles_x + g.xcd_cols - 1) / g.xcd_cols;
     return 8u * (unsigned)(rows_per * cols_per);
+}
+
+// Where byte (n, k) of the prepacked constant operand of a matrix product lives. The operand is kept
+// fragment-major: a fragment is 32 columns n x 32 bytes of k, stored as the matrix core takes it --
+// lane (n % 32, h = (k / 16) % 2) holds 16 bytes, lanes in order, 1 KB per fragment -- and the
+// fragments of 32 columns follow each other along k. A kernel that stages the operand through LDS
+// still reads whole 128-byte lines (eight consecutive columns of one k half), and a kernel that
+// feeds the matrix cores straight from memory reads a fragment with one fully coalesced load.
+__host__ __device__ __forceinline__ uint32_t qfrag_offset(int n, int k, int K_pad) {
+    return ((uint32_t)(n >> 5) * (uint32_t)(K_pad >> 5) + (uint32_t)(k >> 5)) * 1024u +
+           ((uint32_t)(((k >> 4) & 1) << 5) + (uint32_t)(n & 31)) * 16u + (uint32_t)(k & 15);
 }
 
 __device__ __forceinline__ int zp_byte(const uint8_t *ptr, int is_signed) {
@@ -190,11 +201,16 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
 
     // the four 16-byte chunks of each operand slab this thread moves: slab row and k chunk (of 8)
     int row_[kChunks], kc_[kChunks];
+    // the fragment-major constant operand of a matrix product is read with consecutive lanes on
+    // consecutive columns (16 bytes apart in memory), its k chunk changing with the chunk index
+    int qrow_[kChunks], qkc_[kChunks];
 #pragma unroll
     for (int u = 0; u < kChunks; u++) {
         const int c = tid + 256 * u;
         row_[u] = c >> 3;
         kc_[u] = c & 7;
+        qrow_[u] = MODE == MODE_MM ? c % T : row_[u];
+        qkc_[u] = MODE == MODE_MM ? c / T : kc_[u];
     }
     // MODE_CONV: where this thread's positions sit in the input
     int base_h[kChunks] = {}, base_w[kChunks] = {};
@@ -217,10 +233,10 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     uint32_t p_off[kChunks], q_off[kChunks];
 #pragma unroll
     for (int u = 0; u < kChunks; u++) {
-        const int gi = i0 + row_[u], gj = j0 + row_[u];
+        const int gi = i0 + row_[u], gj = j0 + qrow_[u];
         p_off[u] = MODE == MODE_CONV ? (uint32_t)gi * (uint32_t)p.K_pad + kc_[u] * 16
                                      : (uint32_t)min(gi, p.I - 1) * (uint32_t)p.K + kc_[u] * 16;
-        q_off[u] = (uint32_t)gj * (uint32_t)p.K_pad + kc_[u] * 16;
+        q_off[u] = MODE == MODE_MM ? qfrag_offset(gj, qkc_[u] * 16, p.K_pad) : 0u;  // a stage of 128 k is 4 KB further on
     }
     auto load_p = [&](int u, int k0) -> uint4 {
         if (MODE == MODE_CONV) {
@@ -244,7 +260,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     auto load_q = [&](int u, int k0) -> uint4 {
         const int gk = k0 + kc_[u] * 16;
         if (MODE == MODE_MM) {
-            return *reinterpret_cast<const uint4 *>(p.Q + k0 + q_off[u]);
+            return *reinterpret_cast<const uint4 *>(p.Q + (size_t)k0 * 32 + q_off[u]);
         } else {
             const int gkc = min(gk, p.K - 16);
             const int tap = gkc / p.C, c0 = gkc - tap * p.C;
@@ -276,7 +292,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
             *reinterpret_cast<uint4 *>(lds_p + buf * T * kPitch + row_[u] * kPitch + kc_[u] * 16) =
                 make_uint4((r.p[u].x ^ late_flip) & keep, (r.p[u].y ^ late_flip) & keep, (r.p[u].z ^ late_flip) & keep,
                            (r.p[u].w ^ late_flip) & keep);
-            *reinterpret_cast<uint4 *>(lds_q + buf * T * kPitch + row_[u] * kPitch + kc_[u] * 16) =
+            *reinterpret_cast<uint4 *>(lds_q + buf * T * kPitch + qrow_[u] * kPitch + qkc_[u] * 16) =
                 make_uint4(r.q[u].x & keep, r.q[u].y & keep, r.q[u].z & keep, r.q[u].w & keep);
         }
     };
@@ -399,6 +415,195 @@ int gemm_launch(hipc_ctx *ctx, const GemmArgs &g, unsigned batch) {
                                      : gemm_launch_tile<MODE, EPI, ALIGNED, 128>(ctx, g, batch);
 }
 
+// ---- the small-problem variant (MODE_MM, aligned A) ---------------------------------------
+// A product of a few hundred 64x64 tiles. The LDS-staged kernel above is bound by LDS bandwidth
+// there: per 128-k stage a 64x64 tile stores 16 KB and its four 32x32 wavefronts read 32 KB, 384
+// clocks of LDS for 128 clocks of products. Here
+//   * the four wavefronts of a workgroup split the four 32-k product steps of a stage between them
+//     and each owns the whole 64x64 tile (2x2 accumulators), so every byte in LDS is read once;
+//   * only A goes through LDS (8 KB stored, 8 KB read per stage); the fragments of the prepacked,
+//     fragment-major B come straight from memory into the matrix-core layout, one fully coalesced
+//     1 KB load each, four stages ahead;
+//   * the four partial tiles are added through LDS at the end, wavefront w finishing fragment w.
+// Measured against the LDS-staged 64x64 tiles: 12.8 against 17.3 us for 1000 x 4096 x 1024, 7.8
+// against 8.5 us at k = 1024; from about four tiles per CU on, or with very short k, the reduction
+// at the end costs more than the loop saves. (The same kernel with 128x128 tiles, wavefronts 2x2
+// and no k split was slower than either: 16 products per stage issued back to back keep the
+// wavefront from issuing the stage's memory instructions, as in the 128x128 LDS-staged kernel.)
+constexpr int kSmallSets = 4;  // register sets of A chunks and of B fragments: stages in flight
+// the hand-over of three fragments per wavefront reuses the two A buffers (18 KB of its 48 KB)
+constexpr size_t kSmallLds = 4 * 3 * 16 * 64 * sizeof(int) + 4 * 64 * sizeof(int);
+
+template <int EPI, bool DYN>
+__global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) {
+    constexpr int T = 64;                       // edge of the workgroup's tile
+    constexpr int kCh = T / 32;                 // 16-byte chunks of an A slab per thread
+    constexpr int kSteps = 1;                   // product steps of a stage per wavefront
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint8_t *lds_a = lds_raw;                                              // [2][T * kPitch]
+    int *lds_acc = reinterpret_cast<int *>(lds_raw);                       // after the loop: [owner][source 0..2][16][64]
+    int *lds_sum = lds_acc + 4 * 3 * 16 * 64;                              // [4 wavefronts][64 rows]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r32 = lane & 31, kg = lane >> 5;
+    auto handed = [&](int owner, int slot, int r) -> int & { return lds_acc[((owner * 3 + slot) * 16 + r) * 64 + lane]; };
+
+    const int tiles_x = (p.J + T - 1) / T, tiles_y = (p.I + T - 1) / T;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
+    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
+    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
+    const int i0 = ty * T, j0 = tx * T;
+    const int nk = p.K / kBK;
+
+    const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
+    const int zc = (p.host_zp ? p.const_zp_value : zp_byte(p.const_zp, p.const_signed)) - p.const_shift;
+    const uint32_t flip = p.dyn_shift ? 0x80808080u : 0u;
+
+    // A: chunk c = tid + 256 u of a T-row slab: row c / 8, 16-byte column c % 8 (whole lines per row)
+    uint32_t p_off[kCh], l_off[kCh];
+#pragma unroll
+    for (int u = 0; u < kCh; u++) {
+        const int c = tid + 256 * u, row = c >> 3, kc = c & 7;
+        p_off[u] = (uint32_t)min(i0 + row, p.I - 1) * (uint32_t)p.K + kc * 16;  // rows past I: clamped, never stored
+        l_off[u] = row * kPitch + kc * 16;
+    }
+    // B: fragments j0 / 32 and j0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
+    const int j_last = (p.J + kBN - 1) / kBN * kBN - 1;  // B is packed in whole 128-column tiles
+    uint32_t q_off[2];
+#pragma unroll
+    for (int f = 0; f < 2; f++)
+        q_off[f] = qfrag_offset(min(j0 + f * 32, j_last - 31), wave * 32, p.K_pad) + lane * 16;
+    const __amdgpu_buffer_rsrc_t rsrc_p = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t *>(p.P), 0, (int)((uint32_t)p.I * (uint32_t)p.K), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t *>(p.Q), 0, (int)((uint32_t)(j_last + 1) * (uint32_t)p.K_pad), 0x00020000);
+
+    u32x4 ra[kSmallSets][kCh], rb[kSmallSets][kSteps][2];
+    auto load_a = [&](int set, int stage) {
+#pragma unroll
+        for (int u = 0; u < kCh; u++) ra[set][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, p_off[u], min(stage, nk - 1) * kBK, 0);
+    };
+    auto load_b = [&](int set, int stage) {
+#pragma unroll
+        for (int step = 0; step < kSteps; step++)
+#pragma unroll
+            for (int f = 0; f < 2; f++)
+                rb[set][step][f] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, q_off[f] + step * 1024, min(stage, nk - 1) * kBK * 32, 0);
+    };
+    // a stage past the end is stored as zeros: its products add nothing whatever B holds
+    auto store_a = [&](int set, int buf, bool live) {
+        const uint32_t keep = live ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int u = 0; u < kCh; u++)
+            *reinterpret_cast<u32x4 *>(lds_a + buf * T * kPitch + l_off[u]) = (ra[set][u] ^ flip) & keep;
+    };
+
+    i32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    int dsum[2] = {0, 0};
+    const uint32_t frag_a = r32 * kPitch + wave * 32 + kg * 16;
+    auto compute = [&](int buf, int set) {
+        uint4 av[kSteps][2];
+#pragma unroll
+        for (int step = 0; step < kSteps; step++)
+#pragma unroll
+            for (int f = 0; f < 2; f++)
+                av[step][f] = *reinterpret_cast<const uint4 *>(lds_a + buf * T * kPitch + frag_a + f * 32 * kPitch + step * 32);
+#pragma unroll
+        for (int step = 0; step < kSteps; step++) {
+            if (DYN) {
+#pragma unroll
+                for (int f = 0; f < 2; f++) dsum[f] += dot_ones(av[step][f]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, av[step][i]),
+                                                                      __builtin_bit_cast(i32x4, rb[set][step][j]), acc[i][j], 0, 0, 0);
+        }
+    };
+
+#pragma unroll
+    for (int d = 0; d < kSmallSets; d++) load_a(d, d), load_b(d, d);
+    store_a(0, 0, true);
+    load_a(0, kSmallSets);
+    __syncthreads();
+    // Stage s: multiply it out of LDS buffer s & 1 with B set s % 4, refill that B set with stage
+    // s + 4, move stage s + 1 from its A set into the other LDS buffer (last read during stage s - 1,
+    // before the previous barrier) and refill that A set with stage s + 5. Nothing in the loop is
+    // conditional, so the memory counters stay exact.
+    for (int s = 0; s < nk; s += kSmallSets) {
+#pragma unroll
+        for (int d = 0; d < kSmallSets; d++) {
+            compute(d & 1, d);
+            load_b(d, s + d + kSmallSets);
+            store_a((d + 1) % kSmallSets, (d + 1) & 1, s + d + 1 < nk);
+            load_a((d + 1) % kSmallSets, s + d + 1 + kSmallSets);
+            __syncthreads();
+        }
+    }
+
+    // row sums of A over this wavefront's product steps: the two k halves of a row live in lanes l and l + 32
+    if (DYN) {
+#pragma unroll
+        for (int f = 0; f < 2; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
+        if (kg == 0) {
+#pragma unroll
+            for (int f = 0; f < 2; f++) lds_sum[wave * 64 + f * 32 + r32] = dsum[f];
+        }
+    }
+    // wavefront w finishes fragment (w >> 1, w & 1); the other three it hands over (the A buffers
+    // are free: the loop ended with a barrier)
+    {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int owner = i * 2 + j;
+                if (owner == wave) continue;
+                const int slot = wave < owner ? wave : wave - 1;  // 0..2 among the three sources
+#pragma unroll
+                for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[i][j][r];
+            }
+    }
+    __syncthreads();
+
+    const int kzz = p.K * zd * zc;
+    float fmn = 0.f, fmx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if (i * 2 + j != wave) continue;
+            const int gj = j0 + j * 32 + r32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);  // row inside the 32x32 fragment
+                const int gi = i0 + i * 32 + rf;
+                int v = acc[i][j][r];
+#pragma unroll
+                for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
+                if (gi >= p.I || gj >= p.J) continue;
+                v = v - zd * p.const_sum[gj] + kzz;
+                if (DYN) {
+                    int rs = 0;
+#pragma unroll
+                    for (int w = 0; w < 4; w++) rs += lds_sum[w * 64 + i * 32 + rf];
+                    v -= zc * rs;
+                }
+                gemm_emit<MODE_MM, EPI>(p, 0, gi, gj, v, fmn, fmx);
+            }
+        }
+    }
+    if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
+}
+
 // ---- the large-problem variant (MODE_MM, aligned A) --------------------------------------
 // A 128x128 tile needs 64 bytes of operand per clock per CU to keep the matrix cores busy,
 // which is all the vector memory path delivers. Large products therefore run on 256x256 tiles:
@@ -445,13 +650,16 @@ __global__ void __launch_bounds__(kBigThreads) int8_gemm_big_kernel(const GemmAr
 
     // chunk c = tid + kBigThreads u of a 256-row slab: row c / 8, 16-byte column c % 8
     const int j_last = (p.J + kBN - 1) / kBN * kBN - 1;  // B is packed in whole 128-column tiles
-    uint32_t p_off[kBigChunks], q_off[kBigChunks], l_off[kBigChunks];
+    // (the fragment-major B is read with consecutive lanes on consecutive columns instead: 16 bytes apart)
+    uint32_t p_off[kBigChunks], q_off[kBigChunks], l_off[kBigChunks], lq_off[kBigChunks];
 #pragma unroll
     for (int u = 0; u < kBigChunks; u++) {
         const int c = tid + kBigThreads * u, row = c >> 3, kc = c & 7;
+        const int qrow = c % kBigTile, qkc = c / kBigTile;
         p_off[u] = (uint32_t)min(i0 + row, p.I - 1) * (uint32_t)p.K + kc * 16;  // rows past I: clamped, never stored
-        q_off[u] = (uint32_t)min(j0 + row, j_last) * (uint32_t)p.K_pad + kc * 16;
+        q_off[u] = qfrag_offset(min(j0 + qrow, j_last), qkc * 16, p.K_pad);
         l_off[u] = row * kPitch + kc * 16;
+        lq_off[u] = qrow * kPitch + qkc * 16;
     }
     // Buffer loads: a uniform descriptor, the k offset in a scalar register and a fixed 32-bit
     // offset per chunk, so a stage costs no address arithmetic. The descriptors carry the true
@@ -467,13 +675,13 @@ __global__ void __launch_bounds__(kBigThreads) int8_gemm_big_kernel(const GemmAr
     };
     auto load_q = [&](int stage) {
 #pragma unroll
-        for (int u = 0; u < kBigChunks; u++) rq[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, q_off[u], stage * kBK, 0);
+        for (int u = 0; u < kBigChunks; u++) rq[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, q_off[u], stage * kBK * 32, 0);
     };
     auto store_regs = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < kBigChunks; u++) {
             *reinterpret_cast<u32x4 *>(lds_p + buf * kBigTile * kPitch + l_off[u]) = rp[u] ^ flip;
-            *reinterpret_cast<u32x4 *>(lds_q + buf * kBigTile * kPitch + l_off[u]) = rq[u];
+            *reinterpret_cast<u32x4 *>(lds_q + buf * kBigTile * kPitch + lq_off[u]) = rq[u];
         }
     };
 

@@ -10,9 +10,9 @@
 
 namespace hipc {
 
-// B [K, N] (N contiguous) -> Bp [N_pad, K_pad] (k contiguous), signed domain, zero padded.
-// One thread writes one 32-bit word (4 consecutive k of one column); reads are
-// coalesced along n.
+// B [K, N] (N contiguous) -> Bp, N_pad x K_pad bytes in the fragment-major order of qfrag_offset,
+// signed domain, zero padded. One thread writes one 32-bit word (4 consecutive k of one column);
+// reads are coalesced along n, and so are the writes (16 bytes apart).
 __global__ void __launch_bounds__(256)
 pack_b_kernel(const uint8_t *__restrict__ B, uint32_t *__restrict__ Bp, int K, int N, int K_pad, int N_pad,
               uint32_t flip) {
@@ -27,7 +27,7 @@ pack_b_kernel(const uint8_t *__restrict__ B, uint32_t *__restrict__ Bp, int K, i
             if (k < K) word |= (uint32_t)(B[(size_t)k * N + n] ^ (flip & 0xff)) << (8 * b);
         }
     }
-    Bp[(size_t)n * (K_pad / 4) + kw] = word;
+    Bp[qfrag_offset(n, kw * 4, K_pad) / 4] = word;
 }
 
 // per-column sums of the shifted weight, from the packed form: one wavefront per column, 16 bytes
@@ -37,9 +37,8 @@ col_sum_kernel(const uint8_t *__restrict__ Bp, int32_t *__restrict__ sums, int K
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n >= N_pad) return;
-    const uint4 *row = reinterpret_cast<const uint4 *>(Bp + (size_t)n * K_pad);
     int s = 0;
-    for (int c = lane; c < K_pad / 16; c += 64) s += dot_ones(row[c]);
+    for (int c = lane; c < K_pad / 16; c += 64) s += dot_ones(*reinterpret_cast<const uint4 *>(Bp + qfrag_offset(n, c * 16, K_pad)));
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
     if (lane == 0) sums[n] = s;
@@ -190,10 +189,34 @@ bool wants_big_tiles(const GemmArgs &g) {
     return ceil_div(g.I, kBigTile) * ceil_div(g.J, kBigTile) >= 192;
 }
 
+// Products of at most two 64x64 tiles per CU run on the kernel that keeps B out of LDS and splits
+// k over the wavefronts of a workgroup. HIPC_GEMM_SMALL=0/1 overrides (tuning, tests).
+bool wants_small_tiles(hipc_ctx *ctx, const GemmArgs &g) {
+    static const int forced = [] {
+        const char *e = getenv("HIPC_GEMM_SMALL");
+        return e ? atoi(e) : -1;
+    }();
+    if (!g.p_aligned) return false;
+    if (forced >= 0) return forced != 0;
+    return ceil_div(g.I, 64) * ceil_div(g.J, 64) <= 2 * (int64_t)ctx->cu_count && g.K >= 4 * kBK;
+}
+template <int EPI, bool DYN>
+int launch_mm_small_dyn(hipc_ctx *ctx, GemmArgs g) {
+    const dim3 grid(gemm_grid(g, 64));
+    int8_gemm_small_kernel<EPI, DYN><<<grid, 256, kSmallLds, ctx->stream>>>(g);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+template <int EPI>
+int launch_mm_small(hipc_ctx *ctx, const GemmArgs &g) {
+    const bool zero_known = g.const_shift == 0 && (g.host_zp ? g.const_zp_value == 0 : g.const_zp == nullptr);
+    return zero_known ? launch_mm_small_dyn<EPI, false>(ctx, g) : launch_mm_small_dyn<EPI, true>(ctx, g);
+}
 template <int EPI>
 int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
     if (g.I == 0 || g.J == 0) return HIPC_OK;
     if (wants_big_tiles(g)) return launch_mm_big<EPI>(ctx, g);
+    if (wants_small_tiles(ctx, g)) return launch_mm_small<EPI>(ctx, g);
     return g.p_aligned ? gemm_launch<MODE_MM, EPI, true>(ctx, g, 1) : gemm_launch<MODE_MM, EPI, false>(ctx, g, 1);
 }
 

@@ -93,6 +93,29 @@ def test_large_products_take_the_256x256_tiles(ctx, pkg, oracle, a_dt, b_dt):
     weight.destroy()
 
 
+@pytest.mark.parametrize("a_dt,b_dt", [(np.uint8, np.int8), (np.uint8, np.uint8), (np.int8, np.int8), (np.int8, np.uint8)])
+@pytest.mark.parametrize("shape", [(130, 640, 257), (70, 1536, 64), (1, 512, 1), (333, 4096, 200)], ids=lambda s: "M%d_K%d_N%d" % s)
+def test_few_tiles_and_long_k_take_the_k_split_kernel(ctx, pkg, oracle, shape, a_dt, b_dt):
+    """Up to two 64x64 tiles per CU with k a multiple of 128 and at least 512: the workgroup's
+    wavefronts split k, A alone passes through LDS, B comes fragment by fragment from the
+    fragment-major prepacked weight. Stage counts that are not a multiple of the four in flight
+    (5, 12, 4, 32), ragged edges, zero points on both sides or none, and the float epilogue."""
+    m, k, n = shape
+    a = rc.pseudo_plus1(m * k, 51).view(a_dt).reshape(m, k)
+    b = rc.pseudo_plus1(k * n, 52).view(b_dt).reshape(k, n)
+    za = -9 if a_dt == np.int8 else 200
+    zb = 17 if b_dt == np.int8 else 3
+    want = oracle.matmul_integer(a, b, za, zb)
+    weight = pkg.ops.Int8Weight(ctx, b)
+    assert np.array_equal(pkg.ops.matmul_integer(ctx, a, b, za, zb, weight=weight), want)
+    assert np.array_equal(pkg.ops.matmul_integer(ctx, a, b, None, None, weight=weight), oracle.matmul_integer(a, b, 0, 0))
+    scale = np.float32(0.002)
+    bias = pkg.synth.uniform_f32(n, 53, -0.5, 0.5)
+    got = pkg.ops.matmul_integer_scale_bias(ctx, a, b, za, zb, scale, bias, weight=weight)
+    assert np.array_equal(got.view(np.uint32), oracle.rescale(want, scale, bias).view(np.uint32))
+    weight.destroy()
+
+
 LAYERS = [  # tests/matmul_integer_epilogue.rs:352-420: (a_shape, N, weight int8?, relu, per-column scale)
     ((2, 50, 64), 200, False, False, False), ((700, 96), 330, True, False, False),
     ((1100, 64), 1040, False, True, False), ((1, 128, 32), 48, True, False, True),
