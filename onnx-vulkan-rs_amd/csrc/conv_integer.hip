@@ -41,7 +41,8 @@ nchw_to_nhwc_kernel(const uint8_t *__restrict__ X, uint8_t *__restrict__ Xt, int
     }
 }
 
-// W [O, C, kh, kw] -> Wp [O_pad, K_pad], k = (r*kw + s)*C + c, signed domain, zero padded;
+// W [O, C, kh, kw] -> Wp, O_pad x K_pad bytes in the fragment-major order of qfrag_offset,
+// k = (r*kw + s)*C + c, signed domain, zero padded;
 // rowsum[o] = sum_k Wp[o][k].
 __global__ void __launch_bounds__(256)
 pack_conv_w_kernel(const uint8_t *__restrict__ W, uint8_t *__restrict__ Wp, int32_t *__restrict__ rowsum, int O, int C,
@@ -58,7 +59,7 @@ pack_conv_w_kernel(const uint8_t *__restrict__ W, uint8_t *__restrict__ Wp, int3
             local += sv;
             out = (uint8_t)sv;
         }
-        Wp[(size_t)o * K_pad + k] = out;
+        Wp[qfrag_offset(o, k, K_pad)] = out;
     }
     __shared__ int part[256];
     part[threadIdx.x] = local;
@@ -216,6 +217,28 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
         ga.ratio = ep.ratio, ga.ratio_step = ep.ratio_step, ga.qbias = ep.qbias, ga.y_zp = ep.y_zp,
         ga.out_signed = ep.out_signed;
         HIPC_REQUIRE(ctx, g->n <= 65535, "Conv: batch %ld too large", (long)g->n);
+        // few 64x64 tiles and a long k: the wavefronts of a workgroup split k and the weight stays out of LDS
+        // (HIPC_GEMM_SMALL=0/1 overrides: tuning, tests)
+        static const int forced = [] {
+            const char *e = getenv("HIPC_GEMM_SMALL");
+            return e ? atoi(e) : -1;
+        }();
+        const int64_t tiles64 = ceil_div(ga.I, 64) * ceil_div(ga.J, 64) * g->n;
+        const bool small = forced >= 0 ? forced != 0 : (tiles64 <= 2 * (int64_t)ctx->cu_count && ga.K_pad >= 4 * kBK);
+        if (small) {
+            // the row sums of the activations only matter when the weight's zero point, in the signed domain, is not zero
+            const bool zero_known = ga.const_shift == 0 && (host_zp ? w_zp_value == 0 : w_zp == nullptr);
+            const dim3 grid(gemm_grid(ga, 64), 1, (unsigned)g->n);
+            if (ep.requant) {
+                if (zero_known) int8_conv_small_kernel<EPI_REQUANT, false><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
+                else int8_conv_small_kernel<EPI_REQUANT, true><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
+            } else {
+                if (zero_known) int8_conv_small_kernel<EPI_I32, false><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
+                else int8_conv_small_kernel<EPI_I32, true><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
+            }
+            HIPC_LAUNCHED(ctx);
+            return HIPC_OK;
+        }
         return ep.requant ? gemm_launch<MODE_CONV, EPI_REQUANT, true>(ctx, ga, (unsigned)g->n)
                           : gemm_launch<MODE_CONV, EPI_I32, true>(ctx, ga, (unsigned)g->n);
     }

@@ -38,7 +38,7 @@ enum { MODE_MM = 0, MODE_CONV = 1 };
 
 struct GemmArgs {
     // P operand: MODE_MM  -> the activation matrix A [I, K] (u8 / i8, pitch K)
-    //            MODE_CONV -> prepacked weight [I_pad, K_pad] signed
+    //            MODE_CONV -> prepacked weight, I_pad x K_pad signed bytes, fragment-major (qfrag_offset)
     const uint8_t *P;
     // Q operand: MODE_MM  -> prepacked B, J_pad x K_pad signed bytes, fragment-major (qfrag_offset)
     //            MODE_CONV -> NHWC activations, already signed
@@ -212,6 +212,14 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
         qrow_[u] = MODE == MODE_MM ? c % T : row_[u];
         qkc_[u] = MODE == MODE_MM ? c / T : kc_[u];
     }
+    // (a convolution's constant operand is P, the prepacked weight, and it is read the same way)
+    int prow_[kChunks], pkc_[kChunks];
+#pragma unroll
+    for (int u = 0; u < kChunks; u++) {
+        const int c = tid + 256 * u;
+        prow_[u] = MODE == MODE_CONV ? c % T : row_[u];
+        pkc_[u] = MODE == MODE_CONV ? c / T : kc_[u];
+    }
     // MODE_CONV: where this thread's positions sit in the input
     int base_h[kChunks] = {}, base_w[kChunks] = {};
     bool pos_ok[kChunks] = {};
@@ -233,14 +241,14 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     uint32_t p_off[kChunks], q_off[kChunks];
 #pragma unroll
     for (int u = 0; u < kChunks; u++) {
-        const int gi = i0 + row_[u], gj = j0 + qrow_[u];
-        p_off[u] = MODE == MODE_CONV ? (uint32_t)gi * (uint32_t)p.K_pad + kc_[u] * 16
+        const int gi = i0 + prow_[u], gj = j0 + qrow_[u];
+        p_off[u] = MODE == MODE_CONV ? qfrag_offset(gi, pkc_[u] * 16, p.K_pad)  // a stage of 128 k is 4 KB further on
                                      : (uint32_t)min(gi, p.I - 1) * (uint32_t)p.K + kc_[u] * 16;
         q_off[u] = MODE == MODE_MM ? qfrag_offset(gj, qkc_[u] * 16, p.K_pad) : 0u;  // a stage of 128 k is 4 KB further on
     }
     auto load_p = [&](int u, int k0) -> uint4 {
         if (MODE == MODE_CONV) {
-            return *reinterpret_cast<const uint4 *>(p.P + k0 + p_off[u]);
+            return *reinterpret_cast<const uint4 *>(p.P + (size_t)k0 * 32 + p_off[u]);
         } else if (ALIGNED) {
             // K % 128 == 0: every chunk is inside the row. Rows past I are clamped, not zeroed:
             // the rows of a product are independent and those outputs are never stored.
@@ -289,7 +297,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
         const uint32_t late_flip = (MODE == MODE_MM && ALIGNED) ? flip : 0u;
 #pragma unroll
         for (int u = 0; u < kChunks; u++) {
-            *reinterpret_cast<uint4 *>(lds_p + buf * T * kPitch + row_[u] * kPitch + kc_[u] * 16) =
+            *reinterpret_cast<uint4 *>(lds_p + buf * T * kPitch + prow_[u] * kPitch + pkc_[u] * 16) =
                 make_uint4((r.p[u].x ^ late_flip) & keep, (r.p[u].y ^ late_flip) & keep, (r.p[u].z ^ late_flip) & keep,
                            (r.p[u].w ^ late_flip) & keep);
             *reinterpret_cast<uint4 *>(lds_q + buf * T * kPitch + qrow_[u] * kPitch + qkc_[u] * 16) =
@@ -602,6 +610,178 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
         }
     }
     if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
+}
+
+// The same arrangement for a convolution with few 64x64 tiles (MODE_CONV): the gathered activation
+// chunks (the Q operand: 64 output positions x 128 bytes of (kh, kw, c) per stage) go through LDS,
+// the fragments of the prepacked, fragment-major weight (the P operand) come straight from memory,
+// and the four wavefronts split the product steps of a stage and add up at the end.
+template <int EPI, bool DYN>
+__global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) {
+    constexpr int T = 64;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint8_t *lds_q = lds_raw;                                              // [2][T * kPitch]
+    int *lds_acc = reinterpret_cast<int *>(lds_raw);                       // after the loop: [owner][source 0..2][16][64]
+    int *lds_sum = lds_acc + 4 * 3 * 16 * 64;                              // [4 wavefronts][64 positions]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r32 = lane & 31, kg = lane >> 5;
+    const int img = blockIdx.z;
+    auto handed = [&](int owner, int slot, int r) -> int & { return lds_acc[((owner * 3 + slot) * 16 + r) * 64 + lane]; };
+
+    const int tiles_x = (p.J + T - 1) / T, tiles_y = (p.I + T - 1) / T;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
+    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
+    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
+    const int i0 = ty * T, j0 = tx * T;
+    const int nk = p.K_pad / kBK;
+
+    const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
+    const int zc = (p.host_zp ? p.const_zp_value : zp_byte(p.const_zp, p.const_signed)) - p.const_shift;
+    const uint32_t pad_word = (uint32_t)(zd & 0xff) * 0x01010101u;
+
+    // Q: chunk c = tid + 256 u of a 64-position slab: position c / 8, 16-byte k chunk c % 8
+    int kc_[2], base_h[2], base_w[2];
+    bool pos_ok[2];
+    uint32_t l_off[2];
+    const uint8_t *q_img = p.Q + (size_t)img * p.H * p.W * p.C;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int c = tid + 256 * u, row = c >> 3;
+        kc_[u] = c & 7;
+        const int gj = j0 + row;
+        pos_ok[u] = gj < p.J;
+        const int oh = gj / p.Wo, ow = gj - oh * p.Wo;
+        base_h[u] = oh * p.sh - p.pt;
+        base_w[u] = ow * p.sw - p.pl;
+        l_off[u] = row * kPitch + kc_[u] * 16;
+    }
+    // P: fragments i0 / 32 and i0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
+    const uint8_t *p_frag[2];
+#pragma unroll
+    for (int f = 0; f < 2; f++) p_frag[f] = p.P + qfrag_offset(i0 + f * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
+
+    uint4 rq[kSmallSets][2], rp[kSmallSets][2];
+    // beyond the problem: zeros; padding taps: the zero point (which contributes nothing)
+    auto load_q = [&](int set, int stage) {
+        const int k0 = min(stage, nk - 1) * kBK;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int gk = k0 + kc_[u] * 16;
+            const int gkc = min(gk, p.K - 16);
+            const int tap = gkc / p.C, c0 = gkc - tap * p.C;
+            const int r = tap / p.kw, s = tap - r * p.kw;
+            const int ih = base_h[u] + r * p.dh, iw = base_w[u] + s * p.dw;
+            const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+            const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
+            const uint4 v = *reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + c0);
+            const bool live = pos_ok[u] && gk < p.K;
+            const uint32_t alt = live ? pad_word : 0u;
+            const bool take = live && inside;
+            rq[set][u] = make_uint4(take ? v.x : alt, take ? v.y : alt, take ? v.z : alt, take ? v.w : alt);
+        }
+    };
+    auto load_p = [&](int set, int stage) {
+#pragma unroll
+        for (int f = 0; f < 2; f++) rp[set][f] = *reinterpret_cast<const uint4 *>(p_frag[f] + (size_t)min(stage, nk - 1) * kBK * 32);
+    };
+    // a stage past the end is stored as zeros: its products add nothing whatever the weight holds
+    auto store_q = [&](int set, int buf, bool live) {
+        const uint32_t keep = live ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            *reinterpret_cast<uint4 *>(lds_q + buf * T * kPitch + l_off[u]) =
+                make_uint4(rq[set][u].x & keep, rq[set][u].y & keep, rq[set][u].z & keep, rq[set][u].w & keep);
+    };
+
+    i32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    int dsum[2] = {0, 0};
+    const uint32_t frag_q = r32 * kPitch + wave * 32 + kg * 16;
+    auto compute = [&](int buf, int set) {
+        i32x4 b[2];
+#pragma unroll
+        for (int f = 0; f < 2; f++) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(lds_q + buf * T * kPitch + frag_q + f * 32 * kPitch);
+            b[f] = __builtin_bit_cast(i32x4, v);
+            if (DYN) dsum[f] += dot_ones(v);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, rp[set][i]), b[j], acc[i][j], 0, 0, 0);
+    };
+
+#pragma unroll
+    for (int d = 0; d < kSmallSets; d++) load_q(d, d), load_p(d, d);
+    store_q(0, 0, true);
+    load_q(0, kSmallSets);
+    __syncthreads();
+    for (int s = 0; s < nk; s += kSmallSets) {
+#pragma unroll
+        for (int d = 0; d < kSmallSets; d++) {
+            compute(d & 1, d);
+            load_p(d, s + d + kSmallSets);
+            store_q((d + 1) % kSmallSets, (d + 1) & 1, s + d + 1 < nk);
+            load_q((d + 1) % kSmallSets, s + d + 1 + kSmallSets);
+            __syncthreads();
+        }
+    }
+
+    // sums of the activations over this wavefront's product steps, per position: the two k halves live in lanes l and l + 32
+    if (DYN) {
+#pragma unroll
+        for (int f = 0; f < 2; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
+        if (kg == 0) {
+#pragma unroll
+            for (int f = 0; f < 2; f++) lds_sum[wave * 64 + f * 32 + r32] = dsum[f];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int owner = i * 2 + j;
+            if (owner == wave) continue;
+            const int slot = wave < owner ? wave : wave - 1;
+#pragma unroll
+            for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[i][j][r];
+        }
+    __syncthreads();
+
+    const int kzz = p.K * zd * zc;
+    float fmn = 0.f, fmx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if (i * 2 + j != wave) continue;
+            const int gj = j0 + j * 32 + r32;
+            int qs = 0;
+            if (DYN) {
+#pragma unroll
+                for (int w = 0; w < 4; w++) qs += lds_sum[w * 64 + j * 32 + r32];
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);  // row inside the 32x32 fragment
+                const int gi = i0 + i * 32 + rf;
+                int v = acc[i][j][r];
+#pragma unroll
+                for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
+                if (gi >= p.I || gj >= p.J) continue;
+                v = v - zd * p.const_sum[gi] + kzz;
+                if (DYN) v -= zc * qs;
+                gemm_emit<MODE_CONV, EPI>(p, img, gi, gj, v, fmn, fmx);
+            }
+        }
+    }
 }
 
 // ---- the large-problem variant (MODE_MM, aligned A) --------------------------------------
