@@ -121,6 +121,9 @@ __device__ __forceinline__ void gemm_emit(const GemmArgs &p, int img, int gi, in
         float s = p.scale[(size_t)gj * p.scale_step];
         if (p.product) s = __fmul_rn(s, p.product[(size_t)gj * p.product_step]);
         float o = __fmul_rn((float)v, s);
+        // the product and the sum round separately, as the unfused Cast, Mul, Add do; the _rn
+        // functions are plain operators to the compiler, which may otherwise fuse them
+        asm volatile("" : "+v"(o));
         if (p.bias) o = __fadd_rn(o, p.bias[(size_t)gj * p.bias_step]);
         if (p.relu) o = o > 0.f ? o : 0.f;
         static_cast<float *>(p.Y)[at] = o;
@@ -130,6 +133,51 @@ __device__ __forceinline__ void gemm_emit(const GemmArgs &p, int img, int gi, in
         const int c = MODE == MODE_MM ? gj : gi;
         if (p.qbias) v += p.qbias[c];
         const float t = __fmul_rn((float)v, p.ratio[(size_t)c * p.ratio_step]);
+        int q = (int)rintf(t) + p.y_zp;
+        if (p.out_signed) {
+            q = min(max(q, -128), 127);
+            static_cast<int8_t *>(p.Y)[at] = (int8_t)q;
+        } else {
+            q = min(max(q, 0), 255);
+            static_cast<uint8_t *>(p.Y)[at] = (uint8_t)q;
+        }
+    }
+}
+
+// The same for a kernel all of whose outputs in a lane share the column: what the column
+// contributes is loaded once, ahead of time, and the stores then wait for nothing.
+struct EmitColumn {
+    float s = 0.f, b = 0.f;  // scale (times product) or requantisation ratio; float bias
+    int qb = 0;              // requantisation's int32 bias
+};
+template <int EPI>
+__device__ __forceinline__ EmitColumn gemm_emit_column(const GemmArgs &p, int gj) {
+    EmitColumn e;
+    if (EPI == EPI_SCALE_BIAS) {
+        e.s = p.scale[(size_t)gj * p.scale_step];
+        if (p.product) e.s = __fmul_rn(e.s, p.product[(size_t)gj * p.product_step]);
+        if (p.bias) e.b = p.bias[(size_t)gj * p.bias_step];
+    } else if (EPI == EPI_REQUANT) {
+        e.s = p.ratio[(size_t)gj * p.ratio_step];
+        if (p.qbias) e.qb = p.qbias[gj];
+    }
+    return e;
+}
+template <int EPI>
+__device__ __forceinline__ void gemm_emit_mm(const GemmArgs &p, const EmitColumn &e, int gi, int gj, int v, float &fmn, float &fmx) {
+    const size_t at = (size_t)gi * p.J + gj;
+    if (EPI == EPI_I32) {
+        static_cast<int32_t *>(p.Y)[at] = v;
+    } else if (EPI == EPI_SCALE_BIAS) {
+        float o = __fmul_rn((float)v, e.s);
+        asm volatile("" : "+v"(o));  // two roundings, as in gemm_emit
+        if (p.bias) o = __fadd_rn(o, e.b);
+        if (p.relu) o = o > 0.f ? o : 0.f;
+        static_cast<float *>(p.Y)[at] = o;
+        fmn = fminf(fmn, o);
+        fmx = fmaxf(fmx, o);
+    } else {
+        const float t = __fmul_rn((float)(v + e.qb), e.s);
         int q = (int)rintf(t) + p.y_zp;
         if (p.out_signed) {
             q = min(max(q, -128), 127);
@@ -506,6 +554,12 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
             *reinterpret_cast<u32x4 *>(lds_a + buf * T * kPitch + l_off[u]) = (ra[set][u] ^ flip) & keep;
     };
 
+    // what this lane's outputs need of their column (fragment (wave >> 1, wave & 1), column r32): asked
+    // for now, so that the epilogue does not start with a memory round trip
+    const int my_col = min(j0 + (wave & 1) * 32 + r32, p.J - 1);
+    const int my_csum = p.const_sum[my_col];
+    const EmitColumn my_emit = gemm_emit_column<EPI>(p, my_col);
+
     i32x16 acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; i++)
@@ -598,14 +652,14 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
 #pragma unroll
                 for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
                 if (gi >= p.I || gj >= p.J) continue;
-                v = v - zd * p.const_sum[gj] + kzz;
+                v = v - zd * my_csum + kzz;
                 if (DYN) {
                     int rs = 0;
 #pragma unroll
                     for (int w = 0; w < 4; w++) rs += lds_sum[w * 64 + i * 32 + rf];
                     v -= zc * rs;
                 }
-                gemm_emit<MODE_MM, EPI>(p, 0, gi, gj, v, fmn, fmx);
+                gemm_emit_mm<EPI>(p, my_emit, gi, gj, v, fmn, fmx);
             }
         }
     }
