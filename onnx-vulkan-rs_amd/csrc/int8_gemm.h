@@ -788,6 +788,11 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
         }
     }
 
+    // the weight sums of the rows this lane will finish (fragment (wave >> 1, wave & 1)): asked for
+    // before the hand-over, so that the epilogue does not start with a memory round trip
+    int my_csum[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) my_csum[r] = p.const_sum[i0 + (wave >> 1) * 32 + (r >> 2) * 8 + kg * 4 + (r & 3)];  // I_pad rows exist
     // sums of the activations over this wavefront's product steps, per position: the two k halves live in lanes l and l + 32
     if (DYN) {
 #pragma unroll
@@ -830,7 +835,7 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
 #pragma unroll
                 for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
                 if (gi >= p.I || gj >= p.J) continue;
-                v = v - zd * p.const_sum[gi] + kzz;
+                v = v - zd * my_csum[r] + kzz;
                 if (DYN) v -= zc * qs;
                 gemm_emit<MODE_CONV, EPI>(p, img, gi, gj, v, fmn, fmx);
             }
