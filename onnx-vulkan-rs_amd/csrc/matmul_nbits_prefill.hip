@@ -61,7 +61,8 @@ __device__ __forceinline__ uint4 dequant8(uint32_t w, uint32_t zb) {
     return make_uint4(out[0], out[1], out[2], out[3]);
 }
 
-template <int SG, int T>
+// FULL: K is a multiple of 128, so no stage is partial or missing and nothing needs masking.
+template <int SG, int T, bool FULL>
 __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) {
     constexpr int kChunks = T / 32;  // 16-byte chunks of the A slab per thread
     constexpr int kPairs = T / 64;   // (weight tile, lane) pairs per thread, two words each
@@ -115,7 +116,7 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
 #pragma unroll
         for (int u = 0; u < kChunks; u++) {
             const uint4 v = *reinterpret_cast<const uint4 *>(a_base + a_off[u] + (size_t)k0 * 2);
-            const bool in = k0 + a_k[u] < p.K;  // K is a multiple of 8: a chunk is inside or outside as a whole
+            const bool in = FULL || k0 + a_k[u] < p.K;  // K is a multiple of 8: a chunk is inside or outside as a whole
             r.a[u] = make_uint4(in ? v.x : 0u, in ? v.y : 0u, in ? v.z : 0u, in ? v.w : 0u);
         }
         const int cg = stage >> 1, half = stage & 1;
@@ -136,7 +137,7 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
     };
     // a stage past the end reads clamped addresses and stores zeros for A: it adds nothing
     auto store_regs = [&](const Regs &r, int buf, bool live) {
-        const uint32_t keep = live ? 0xffffffffu : 0u;
+        const uint32_t keep = FULL || live ? 0xffffffffu : 0u;
 #pragma unroll
         for (int u = 0; u < kChunks; u++)
             *reinterpret_cast<uint4 *>(lds_a + buf * T * kPPitch + a_lds[u]) =
@@ -252,8 +253,11 @@ namespace {
 
 template <int SG, int T>
 int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
-    static bool lds_allowed[kMaxDevices] = {};
-    if (int rc = allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T>, prefill_lds(T), lds_allowed)) return rc;
+    const bool full = a.K % (2 * kPK) == 0;
+    static bool lds_allowed[2][kMaxDevices] = {};
+    if (int rc = full ? allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, true>, prefill_lds(T), lds_allowed[1])
+                      : allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, false>, prefill_lds(T), lds_allowed[0]))
+        return rc;
     const int tiles_x = (int)ceil_div(a.N, T), tiles_y = (int)ceil_div(a.M, T);
     int best = 8, best_cost = 1 << 30;
     for (int r = 1; r <= 8; r *= 2) {
@@ -262,10 +266,36 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
     }
     a.xcd_rows = best, a.xcd_cols = 8 / best;
     const unsigned grid = 8u * (unsigned)(ceil_div(tiles_y, a.xcd_rows) * ceil_div(tiles_x, a.xcd_cols));
-    mmnb_prefill_kernel<SG, T><<<dim3(grid), dim3(256), prefill_lds(T), ctx->stream>>>(a);
+    if (full)
+        mmnb_prefill_kernel<SG, T, true><<<dim3(grid), dim3(256), prefill_lds(T), ctx->stream>>>(a);
+    else
+        mmnb_prefill_kernel<SG, T, false><<<dim3(grid), dim3(256), prefill_lds(T), ctx->stream>>>(a);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }
+
+}  // namespace
+
+// This file is compiled twice. The 128x128 instances live in an object of their own, built with
+// HIPC_PREFILL_WIDE and with the matrix-core accumulators in ordinary vector registers (the block
+// scales then multiply them without copies out of the accumulation file: 48.5 -> 44.7 us for
+// 512 x 2048 x 11008); the 64x64 instances are faster with the accumulation file (80.6 against
+// 87.9 us for 512 x 11008 x 2048), and that is a switch of the whole compilation.
+int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG);
+
+#ifdef HIPC_PREFILL_WIDE
+
+int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG) {
+    switch (SG) {
+        case 4: return prefill_launch_tile<4, 128>(ctx, a);
+        case 2: return prefill_launch_tile<2, 128>(ctx, a);
+        default: return prefill_launch_tile<1, 128>(ctx, a);
+    }
+}
+
+#else
+
+namespace {
 
 template <int SG>
 int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
@@ -275,7 +305,7 @@ int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
     }();
     int tile = ceil_div(a.M, 128) * ceil_div(a.N, 128) >= 256 ? 128 : 64;  // at least one 128-tile per CU
     if (forced == 64 || forced == 128) tile = forced;
-    return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_tile<SG, 128>(ctx, a);
+    return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_wide(ctx, a, SG);
 }
 
 }  // namespace
@@ -295,5 +325,7 @@ int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void
         default: return prefill_launch<1>(ctx, a);
     }
 }
+
+#endif  // HIPC_PREFILL_WIDE
 
 }  // namespace hipc
