@@ -44,6 +44,10 @@ struct PrefillArgs {
     int M, K, N;
     int n_tiles, n_cg;
     int xcd_rows, xcd_cols;
+    // k split over workgroups (gridDim.y): each takes `split_stages` stages (an even number, so that
+    // weight tiles are not cut) and writes f32 partials [split][M][N] that a second launch adds up
+    int ksplit, split_stages;
+    float *Ypart;
 };
 
 // eight nibbles (order k0 k2 k4 k6 k1 k3 k5 k7) -> eight f16 values q - zp in k order, as four words of pairs
@@ -213,15 +217,16 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
         }
     };
 
-    const int nk = (p.K + kPK - 1) / kPK;
+    const int nk_all = (p.K + kPK - 1) / kPK;
+    const int ks0 = blockIdx.y * p.split_stages, nk = min(nk_all, ks0 + p.split_stages);  // this workgroup's stages
     Regs r0, r1;
-    load_regs(r0, 0);
-    load_regs(r1, min(1, nk - 1));
+    load_regs(r0, ks0);
+    load_regs(r1, min(ks0 + 1, nk - 1));
     store_regs(r0, 0, true);
     __syncthreads();
     // two stages per trip and no exit in between, so the memory counters stay exact; with an odd
     // stage count the second half of the last trip multiplies a stage whose A is all zeros
-    for (int ks = 0; ks < nk; ks += 2) {
+    for (int ks = ks0; ks < nk; ks += 2) {
         fetch_scales(ks, 0);
         load_regs(r0, min(ks + 2, nk - 1));
         compute(0, 0);
@@ -243,13 +248,45 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
             for (int r = 0; r < 16; r++) {
                 const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);
                 const int gi = i0 + wm * kWT + i * 32 + rf;
-                if (gi < p.M && gj < p.N) p.Y[(size_t)gi * p.N + gj] = __float2half(total[i][j][r]);
+                if (gi < p.M && gj < p.N) {
+                    if (p.ksplit > 1)
+                        p.Ypart[((size_t)blockIdx.y * p.M + gi) * p.N + gj] = total[i][j][r];
+                    else
+                        p.Y[(size_t)gi * p.N + gj] = __float2half(total[i][j][r]);
+                }
             }
         }
     }
 }
 
+// Y = f16(sum over splits of the f32 partials), in split order (static: this file is compiled twice)
+static __global__ void __launch_bounds__(256)
+mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ Y, long total, int ksplit) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= total) return;
+    if (i + 4 <= total && (total & 3) == 0) {
+        float4 v = *reinterpret_cast<const float4 *>(part + i);
+        for (int s = 1; s < ksplit; s++) {
+            const float4 w = *reinterpret_cast<const float4 *>(part + (size_t)s * total + i);
+            v.x += w.x, v.y += w.y, v.z += w.z, v.w += w.w;
+        }
+        Y[i] = __float2half(v.x), Y[i + 1] = __float2half(v.y), Y[i + 2] = __float2half(v.z), Y[i + 3] = __float2half(v.w);
+    } else {
+        for (long j = i; j < min(i + 4, total); j++) {
+            float v = part[j];
+            for (int s = 1; s < ksplit; s++) v += part[(size_t)s * total + j];
+            Y[j] = __float2half(v);
+        }
+    }
+}
+
 namespace {
+
+// HIPC_PREFILL_SPLIT: 0 never splits k, n > 0 forces n ways (tuning, tests); unset: chosen by shape
+const int g_prefill_split = [] {
+    const char *e = getenv("HIPC_PREFILL_SPLIT");
+    return e ? atoi(e) : -1;
+}();
 
 template <int SG, int T>
 int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
@@ -266,11 +303,36 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
     }
     a.xcd_rows = best, a.xcd_cols = 8 / best;
     const unsigned grid = 8u * (unsigned)(ceil_div(tiles_y, a.xcd_rows) * ceil_div(tiles_x, a.xcd_cols));
+    // Too few tiles for the chip: split k over workgroups, as many ways as gives every CU a
+    // workgroup, at least 32 stages each (with fewer, the second launch and the partials cost more
+    // than the idle CUs: 512 x 2048 x 2560 took 27 us split three ways, 21 us on 64x64 tiles). The
+    // partials go through scratch memory.
+    const int nk = (int)ceil_div(a.K, kPK);
+    int ksplit = 1;
+    if (T == 128 && g_prefill_split != 0) {
+        const int tiles = tiles_x * tiles_y;
+        ksplit = g_prefill_split > 0 ? g_prefill_split : std::min(4, ctx->cu_count / std::max(1, tiles));
+        ksplit = std::max(1, std::min(ksplit, g_prefill_split > 0 ? nk / 2 : nk / 32));
+    }
+    a.split_stages = (int)(ceil_div(ceil_div(nk, ksplit), 2) * 2);
+    a.ksplit = (int)ceil_div(nk, a.split_stages);
+    a.Ypart = nullptr;
+    if (a.ksplit > 1) {
+        void *part = nullptr;
+        if (int rc = scratch_get(ctx, 0, (size_t)a.ksplit * a.M * a.N * sizeof(float), &part)) return rc;
+        a.Ypart = static_cast<float *>(part);
+    }
+    const dim3 g2(grid, (unsigned)a.ksplit);
     if (full)
-        mmnb_prefill_kernel<SG, T, true><<<dim3(grid), dim3(256), prefill_lds(T), ctx->stream>>>(a);
+        mmnb_prefill_kernel<SG, T, true><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
     else
-        mmnb_prefill_kernel<SG, T, false><<<dim3(grid), dim3(256), prefill_lds(T), ctx->stream>>>(a);
+        mmnb_prefill_kernel<SG, T, false><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
     HIPC_LAUNCHED(ctx);
+    if (a.ksplit > 1) {
+        const long total = (long)a.M * a.N;
+        mmnb_prefill_reduce_kernel<<<dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream>>>(a.Ypart, a.Y, total, a.ksplit);
+        HIPC_LAUNCHED(ctx);
+    }
     return HIPC_OK;
 }
 
@@ -303,7 +365,12 @@ int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
         const char *e = getenv("HIPC_PREFILL_TILE");
         return e ? atoi(e) : 0;
     }();
-    int tile = ceil_div(a.M, 128) * ceil_div(a.N, 128) >= 256 ? 128 : 64;  // at least one 128-tile per CU
+    // 128x128 tiles when they give every CU a workgroup, directly or (long k) with k split over up
+    // to four workgroups per tile; else 64x64
+    const int64_t tiles128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
+    const int nk = (int)ceil_div(a.K, kPK);
+    const bool by_split = g_prefill_split != 0 && tiles128 * std::min<int64_t>(4, nk / 32) >= 192;
+    int tile = tiles128 >= 256 || by_split ? 128 : 64;
     if (forced == 64 || forced == 128) tile = forced;
     return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_wide(ctx, a, SG);
 }
