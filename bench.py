@@ -39,7 +39,7 @@ BS = 32
 # HBM bytes per lm_head GEMV launch as the memory counters see them (FETCH_SIZE + WRITE_SIZE, each
 # scaled by its reading for a 256 MiB copy; profiles/mmnb_gemv_lm_head_1152x262144.txt). A counter
 # run cannot happen inside this program, so the figure is carried over from that profile.
-LM_HEAD_TRAFFIC_BYTES = 200.5e6
+LM_HEAD_TRAFFIC_BYTES = 199.6e6
 IN_GRAPH = 16   # instances of a small operator per captured graph: amortises the graph launch
 
 
