@@ -322,14 +322,17 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     const int my_tiles = wk < span ? (span - wk + p.WK - 1) / p.WK : 0;
     // the load cursor runs D - 1 tiles ahead of the one being multiplied: same group, or the first
     // tile of this wavefront's next group, or (past the end) tiles of a group that does not exist,
-    // which load_stage clamps onto the last one and the caches absorb
+    // which become loads of one tile that the caches hold
     int l_tile = first_tile, l_ng = ng, l_ti = 0;
     auto load_ahead = [&](GemvStage<T, SG> &dst) {
         const bool group_done = l_ti + 1 >= my_tiles;
         l_tile = group_done ? first_tile : l_tile + p.WK;
         l_ng = group_done ? l_ng + gstride : l_ng;
         l_ti = group_done ? 0 : l_ti + 1;
-        load_stage(min(l_ng, groups - 1), l_tile, dst);
+        // past the end: every wavefront asks for the same tile (0, 0), which the caches hold, instead
+        // of fetching another tile of its own that nobody will use
+        const bool past = l_ng >= groups;
+        load_stage(past ? 0 : l_ng, past ? 0 : l_tile, dst);
     };
     auto load_first = [&]() {
         load_stage(first_ng, first_tile, st[0]);
