@@ -115,8 +115,11 @@ __device__ __forceinline__ int dot_ones(uint4 v) {
 template <int MODE, int EPI>
 __device__ __forceinline__ void gemm_emit(const GemmArgs &p, int img, int gi, int gj, int v, float &fmn, float &fmx) {
     const size_t at = MODE == MODE_MM ? (size_t)gi * p.J + gj : ((size_t)img * p.I + gi) * p.J + gj;
+    // the int32 / float outputs are written once and are several times the operands: non-temporal
+    // stores keep them from displacing the operand tiles other workgroups are about to read
+    // (1000 x 1024 x 4096: 16.5 -> 14.9 us, 8192^3: 605 -> 585 us)
     if (EPI == EPI_I32) {
-        static_cast<int32_t *>(p.Y)[at] = v;
+        __builtin_nontemporal_store(v, static_cast<int32_t *>(p.Y) + at);
     } else if (EPI == EPI_SCALE_BIAS) {
         float s = p.scale[(size_t)gj * p.scale_step];
         if (p.product) s = __fmul_rn(s, p.product[(size_t)gj * p.product_step]);
@@ -126,7 +129,7 @@ __device__ __forceinline__ void gemm_emit(const GemmArgs &p, int img, int gi, in
         asm volatile("" : "+v"(o));
         if (p.bias) o = __fadd_rn(o, p.bias[(size_t)gj * p.bias_step]);
         if (p.relu) o = o > 0.f ? o : 0.f;
-        static_cast<float *>(p.Y)[at] = o;
+        __builtin_nontemporal_store(o, static_cast<float *>(p.Y) + at);
         fmn = fminf(fmn, o);
         fmx = fmaxf(fmx, o);
     } else {
@@ -167,13 +170,13 @@ template <int EPI>
 __device__ __forceinline__ void gemm_emit_mm(const GemmArgs &p, const EmitColumn &e, int gi, int gj, int v, float &fmn, float &fmx) {
     const size_t at = (size_t)gi * p.J + gj;
     if (EPI == EPI_I32) {
-        static_cast<int32_t *>(p.Y)[at] = v;
+        __builtin_nontemporal_store(v, static_cast<int32_t *>(p.Y) + at);
     } else if (EPI == EPI_SCALE_BIAS) {
         float o = __fmul_rn((float)v, e.s);
         asm volatile("" : "+v"(o));  // two roundings, as in gemm_emit
         if (p.bias) o = __fadd_rn(o, e.b);
         if (p.relu) o = o > 0.f ? o : 0.f;
-        static_cast<float *>(p.Y)[at] = o;
+        __builtin_nontemporal_store(o, static_cast<float *>(p.Y) + at);
         fmn = fminf(fmn, o);
         fmx = fmaxf(fmx, o);
     } else {
