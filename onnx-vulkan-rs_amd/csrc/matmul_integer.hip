@@ -189,8 +189,8 @@ bool wants_big_tiles(const GemmArgs &g) {
     return ceil_div(g.I, kBigTile) * ceil_div(g.J, kBigTile) >= 192;
 }
 
-// Products of at most two 64x64 tiles per CU run on the kernel that keeps B out of LDS and splits
-// k over the wavefronts of a workgroup. HIPC_GEMM_SMALL=0/1 overrides (tuning, tests).
+// Products of a few 64x64 tiles per CU and a long enough k run on the kernel that keeps B out of LDS
+// and splits k over the wavefronts of a workgroup. HIPC_GEMM_SMALL=0/1 overrides (tuning, tests).
 bool wants_small_tiles(hipc_ctx *ctx, const GemmArgs &g) {
     static const int forced = [] {
         const char *e = getenv("HIPC_GEMM_SMALL");
@@ -198,7 +198,10 @@ bool wants_small_tiles(hipc_ctx *ctx, const GemmArgs &g) {
     }();
     if (!g.p_aligned) return false;
     if (forced >= 0) return forced != 0;
-    return ceil_div(g.I, 64) * ceil_div(g.J, 64) <= 2 * (int64_t)ctx->cu_count && g.K >= 4 * kBK;
+    // measured against the LDS-staged 64x64 tiles: ahead up to four tiles per CU from k = 1024 on (14.1
+    // against 15.3 us for 1000 x 1024 x 4096), up to two per CU from k = 512 on; behind with k = 256
+    const int64_t tiles64 = ceil_div(g.I, 64) * ceil_div(g.J, 64);
+    return (tiles64 <= 2 * (int64_t)ctx->cu_count && g.K >= 4 * kBK) || (tiles64 <= 4 * (int64_t)ctx->cu_count && g.K >= 8 * kBK);
 }
 template <int EPI, bool DYN>
 int launch_mm_small_dyn(hipc_ctx *ctx, GemmArgs g) {
