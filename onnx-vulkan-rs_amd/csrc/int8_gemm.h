@@ -793,9 +793,17 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
 
     // the weight sums of the rows this lane will finish (fragment (wave >> 1, wave & 1)): asked for
     // before the hand-over, so that the epilogue does not start with a memory round trip
-    int my_csum[16];
+    // (and, for the requantising epilogue, their ratios and int32 biases)
+    int my_csum[16], my_qb[16];
+    float my_ratio[16];
 #pragma unroll
-    for (int r = 0; r < 16; r++) my_csum[r] = p.const_sum[i0 + (wave >> 1) * 32 + (r >> 2) * 8 + kg * 4 + (r & 3)];  // I_pad rows exist
+    for (int r = 0; r < 16; r++) {
+        const int row = i0 + (wave >> 1) * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
+        my_csum[r] = p.const_sum[row];  // I_pad rows exist
+        const int c = min(row, p.I - 1);
+        my_ratio[r] = EPI == EPI_REQUANT ? p.ratio[(size_t)c * p.ratio_step] : 0.f;
+        my_qb[r] = EPI == EPI_REQUANT && p.qbias ? p.qbias[c] : 0;
+    }
     // sums of the activations over this wavefront's product steps, per position: the two k halves live in lanes l and l + 32
     if (DYN) {
 #pragma unroll
@@ -840,7 +848,16 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
                 if (gi >= p.I || gj >= p.J) continue;
                 v = v - zd * my_csum[r] + kzz;
                 if (DYN) v -= zc * qs;
-                gemm_emit<MODE_CONV, EPI>(p, img, gi, gj, v, fmn, fmx);
+                if (EPI == EPI_REQUANT) {
+                    int q = (int)rintf(__fmul_rn((float)(v + my_qb[r]), my_ratio[r])) + p.y_zp;
+                    const size_t at = ((size_t)img * p.I + gi) * p.J + gj;
+                    if (p.out_signed)
+                        static_cast<int8_t *>(p.Y)[at] = (int8_t)min(max(q, -128), 127);
+                    else
+                        static_cast<uint8_t *>(p.Y)[at] = (uint8_t)min(max(q, 0), 255);
+                } else {
+                    gemm_emit<MODE_CONV, EPI>(p, img, gi, gj, v, fmn, fmx);
+                }
             }
         }
     }
