@@ -173,6 +173,28 @@ def bench_int8_ffn(pkg, ctx):
     ctx.graph_destroy(g)
     dql_bytes = x.size * 4 + x.size + 5
     out["dynamic_quantize_linear_1000x1024"] = dict(us=ns / 1e3, gbs=dql_bytes / ns, frac_hbm=dql_bytes / ns / HBM_PEAK_GBS)
+    # the FFN's middle: DynamicQuantizeLinear of the exact GELU of the first product's [1000, 4096] output,
+    # fused (two passes over x, the GELU never stored) against GELU kernel + DynamicQuantizeLinear
+    h = ctx.upload(pkg.synth.normal_f32(T * 4096, 3))
+    hg, hq = ctx.alloc(T * 4096 * 4), ctx.alloc(T * 4096)
+    sq2 = float(np.float32(np.sqrt(2.0)))
+    lib = ctx.lib
+    fused = lambda: ctx._check(lib.hipc_dynamic_quantize_linear_gelu(ctx.handle, h.ptr, T * 4096, sq2, 1.0, 0.5, 0, hq.ptr, dP.ptr, dP.ptr + 4, None))  # noqa: E731
+    def unfused():
+        ctx._check(lib.hipc_decomposed_gelu(ctx.handle, h.ptr, T * 4096, sq2, 1.0, 0.5, 0, hg.ptr))
+        ops.dynamic_quantize_linear_device(ctx, hg, T * 4096, hq, dP, dP.at(4))
+    for name, fn in [("gelu_quantize_fused_1000x4096", fused), ("gelu_then_quantize_1000x4096", unfused)]:
+        fn()
+        ctx.flush()
+        ctx.capture_begin()
+        for _ in range(IN_GRAPH):
+            fn()
+        g = ctx.capture_end()
+        ns, _ = median_ns(ctx, g, IN_GRAPH, samples=20, reps=4)
+        ctx.graph_destroy(g)
+        out[name] = dict(us=ns / 1e3)
+    for b in (h, hg, hq):
+        b.free()
     dS = ctx.upload(np.array([0.01], np.float32))
     for (K, N) in [(1024, 4096), (4096, 1024)]:
         w = ops.Int8Weight(ctx, pkg.synth.int8_weight(K, N, 22 + K))

@@ -160,6 +160,26 @@ int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hi
 int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out,
                                  void *zp_out, void *range, int range_ready);
 
+/*
+ * DecomposedGelu: the exact GELU written out as Div -> Erf -> Add -> Mul -> Mul, which the
+ * reference fuses at load time (rewrite.rs:683-698, kernel shaders/elementwise.rs:71-118):
+ *   e = erf(x / divisor) + offset;  y = (x * e) * factor,  or  x * (e * factor) with factor_first
+ * erf is the reference's polynomial (Abramowitz-Stegun 7.1.26); every step rounds on its own.
+ * X, Y: n f32 on the device.
+ */
+int hipc_decomposed_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor, float offset, float factor,
+                         int factor_first, void *Y);
+
+/*
+ * DecomposedGeluQuantize: DynamicQuantizeLinear of DecomposedGelu(x) without ever storing the
+ * GELU (rewrite.rs:699-735; shaders/dynamic_quantize.rs:224-247; interp.rs:1976-2030): both passes
+ * evaluate the GELU again from X. Byte for byte what hipc_decomposed_gelu followed by
+ * hipc_dynamic_quantize_linear gives (the reference's own test, tests/decomposed_gelu.rs).
+ * `range` as in hipc_dynamic_quantize_linear (NULL: the context's own).
+ */
+int hipc_dynamic_quantize_linear_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor, float offset, float factor,
+                                      int factor_first, void *Y, void *scale_out, void *zp_out, void *range);
+
 /* ------------------------------------------------------------ MatMulInteger */
 
 /* `packed_b` + `flipped_const` (interp.rs:2673-2768; shaders/matmul_integer.rs:135-158):

@@ -14,13 +14,45 @@
 
 namespace hipc {
 
+// What the quantizer reads: x itself, or DecomposedGelu(x), the exact GELU written out as
+// Div -> Erf -> Add -> Mul -> Mul and fused by the reference (rewrite.rs:683-735). Every step rounds
+// on its own, as the five kernels it replaces do (shaders/elementwise.rs:71-118): this file is
+// compiled with floating-point contraction off, so the fused quantizer and the plain GELU kernel
+// below evaluate bit for bit the same function.
+struct GeluParams {
+    int on;             // 0: the identity
+    float divisor, offset, factor;
+    int factor_first;   // x * ((erf + offset) * factor) instead of (x * (erf + offset)) * factor
+};
+
+__device__ __forceinline__ float erf_approx(float x) {  // shaders/elementwise.rs:71-80 (Abramowitz-Stegun 7.1.26)
+    const float s = x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f);
+    const float a = fabsf(x);
+    const float t = 1.f / (1.f + 0.3275911f * a);
+    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+    return s * (1.f - poly * expf(-a * a));
+}
+
+__device__ __forceinline__ float gelu_load(float v, const GeluParams &g) {
+    if (!g.on) return v;
+    const float e = erf_approx(v / g.divisor) + g.offset;
+    return g.factor_first ? v * (e * g.factor) : (v * e) * g.factor;
+}
+
+__global__ void __launch_bounds__(256)
+decomposed_gelu_kernel(const float *__restrict__ x, long n, GeluParams g, float *__restrict__ y) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = gelu_load(x[i], g);
+}
+
 __global__ void dql_clear_range_kernel(uint32_t *range) {
     if (threadIdx.x < 2) range[threadIdx.x] = 0u;
 }
 
 __global__ void __launch_bounds__(256)
-dql_range_kernel(const float *__restrict__ x, long n, uint32_t *__restrict__ range, int vec_ok, int per_block) {
+dql_range_kernel(const float *__restrict__ x, long n, uint32_t *__restrict__ range, int vec_ok, int per_block, GeluParams g) {
     float mn = 0.f, mx = 0.f;
+    auto L = [&](float4 v) { return g.on ? make_float4(gelu_load(v.x, g), gelu_load(v.y, g), gelu_load(v.z, g), gelu_load(v.w, g)) : v; };
     const long tid = (long)blockIdx.x * 256 + threadIdx.x;
     const long nthreads = (long)gridDim.x * 256;
     if (vec_ok) {
@@ -28,25 +60,27 @@ dql_range_kernel(const float *__restrict__ x, long n, uint32_t *__restrict__ ran
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
         long i = tid;
         for (; i + 3 * nthreads < n4; i += 4 * nthreads) {  // four independent loads in flight
-            const float4 a = x4[i], b = x4[i + nthreads], c = x4[i + 2 * nthreads], d = x4[i + 3 * nthreads];
+            const float4 a = L(x4[i]), b = L(x4[i + nthreads]), c = L(x4[i + 2 * nthreads]), d = L(x4[i + 3 * nthreads]);
             mn = fminf(mn, fminf(fminf(fminf(a.x, a.y), fminf(a.z, a.w)), fminf(fminf(b.x, b.y), fminf(b.z, b.w))));
             mn = fminf(mn, fminf(fminf(fminf(c.x, c.y), fminf(c.z, c.w)), fminf(fminf(d.x, d.y), fminf(d.z, d.w))));
             mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(a.x, a.y), fmaxf(a.z, a.w)), fmaxf(fmaxf(b.x, b.y), fmaxf(b.z, b.w))));
             mx = fmaxf(mx, fmaxf(fmaxf(fmaxf(c.x, c.y), fmaxf(c.z, c.w)), fmaxf(fmaxf(d.x, d.y), fmaxf(d.z, d.w))));
         }
         for (; i < n4; i += nthreads) {
-            const float4 v = x4[i];
+            const float4 v = L(x4[i]);
             mn = fminf(mn, fminf(fminf(v.x, v.y), fminf(v.z, v.w)));
             mx = fmaxf(mx, fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
         }
         for (long i = (n4 << 2) + tid; i < n; i += nthreads) {
-            mn = fminf(mn, x[i]);
-            mx = fmaxf(mx, x[i]);
+            const float v = gelu_load(x[i], g);
+            mn = fminf(mn, v);
+            mx = fmaxf(mx, v);
         }
     } else {
         for (long i = tid; i < n; i += nthreads) {
-            mn = fminf(mn, x[i]);
-            mx = fmaxf(mx, x[i]);
+            const float v = gelu_load(x[i], g);
+            mn = fminf(mn, v);
+            mx = fmaxf(mx, v);
         }
     }
 #pragma unroll
@@ -89,15 +123,16 @@ __device__ __forceinline__ uint32_t dql_one(float v, float scale, float zp) {
 // four values per thread, packed into one 32-bit store where the output allows it
 __global__ void __launch_bounds__(256)
 dql_quantize_kernel(const float *__restrict__ x, long n, const uint32_t *__restrict__ range, int nparts,
-                    uint8_t *__restrict__ y, float *__restrict__ scale_out, uint8_t *__restrict__ zp_out, int vec_ok) {
+                    uint8_t *__restrict__ y, float *__restrict__ scale_out, uint8_t *__restrict__ zp_out, int vec_ok,
+                    GeluParams g) {
     float scale, zp;
     if (nparts > 0) {
-        // range holds nparts pairs (nparts <= 256): every workgroup joins them itself; the maximum of
+        // range holds nparts pairs: every workgroup joins them itself; the maximum of
         // non-negative floats is the maximum of their bit patterns
         __shared__ uint32_t joined[2];
         __shared__ uint32_t wave_max[4][2];
         uint32_t a = 0, b = 0;
-        if ((int)threadIdx.x < nparts) a = range[2 * threadIdx.x], b = range[2 * threadIdx.x + 1];
+        for (int i = threadIdx.x; i < nparts; i += 256) a = max(a, range[2 * i]), b = max(b, range[2 * i + 1]);
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) {
             a = max(a, (uint32_t)__shfl_xor((int)a, off, 64));
@@ -122,12 +157,13 @@ dql_quantize_kernel(const float *__restrict__ x, long n, const uint32_t *__restr
     const long base = i4 << 2;
     if (base >= n) return;
     if (vec_ok && base + 4 <= n) {
-        const float4 v = reinterpret_cast<const float4 *>(x)[i4];
+        float4 v = reinterpret_cast<const float4 *>(x)[i4];
+        if (g.on) v = make_float4(gelu_load(v.x, g), gelu_load(v.y, g), gelu_load(v.z, g), gelu_load(v.w, g));
         const uint32_t packed = dql_one(v.x, scale, zp) | dql_one(v.y, scale, zp) << 8 |
                                 dql_one(v.z, scale, zp) << 16 | dql_one(v.w, scale, zp) << 24;
         reinterpret_cast<uint32_t *>(y)[i4] = packed;
     } else {
-        for (long i = base; i < n && i < base + 4; i++) y[i] = (uint8_t)dql_one(x[i], scale, zp);
+        for (long i = base; i < n && i < base + 4; i++) y[i] = (uint8_t)dql_one(gelu_load(x[i], g), scale, zp);
     }
 }
 
@@ -142,10 +178,10 @@ __global__ void dql_empty_kernel(float *scale_out, uint8_t *zp_out) {
 
 using namespace hipc;
 
-extern "C" int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out,
-                                            void *zp_out, void *range, int range_ready) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
+namespace {
+
+int dql_launch(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out, void *zp_out, void *range, int range_ready,
+               const GeluParams &gelu) {
     HIPC_REQUIRE(ctx, n >= 0, "DynamicQuantizeLinear: negative length");
     HIPC_REQUIRE(ctx, scale_out && zp_out, "DynamicQuantizeLinear: null scale or zero-point output");
     HIPC_REQUIRE(ctx, aligned(scale_out, 4), "DynamicQuantizeLinear: scale output must be 4-byte aligned");
@@ -167,7 +203,7 @@ extern "C" int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_
         // second pass -- no clearing launch and no atomics
         slot = reinterpret_cast<uint32_t *>(static_cast<char *>(ctx->params) + kParamParts);
         nparts = (int)std::min<long>(std::max<long>(ceil_div(n, 256 * 16), 1), kParamPartsMax);
-        dql_range_kernel<<<(unsigned)nparts, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 1);
+        dql_range_kernel<<<(unsigned)nparts, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 1, gelu);
         HIPC_LAUNCHED(ctx);
     } else if (!range_ready) {
         dql_clear_range_kernel<<<1, 64, 0, ctx->stream>>>(slot);
@@ -175,14 +211,58 @@ extern "C" int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_
         // enough workgroups to pull from every HBM channel, few enough that the atomics are noise
         const long want = ceil_div(n, 256 * 16);
         const unsigned grid = (unsigned)std::min<long>(std::max<long>(want, 1), 8L * ctx->cu_count);
-        dql_range_kernel<<<grid, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 0);
+        dql_range_kernel<<<grid, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 0, gelu);
         HIPC_LAUNCHED(ctx);
     }
     const long quads = ceil_div(n, 4);
     HIPC_REQUIRE(ctx, ceil_div(quads, 256) < (int64_t(1) << 31), "DynamicQuantizeLinear: tensor too large");
     dql_quantize_kernel<<<(unsigned)ceil_div(quads, 256), 256, 0, ctx->stream>>>(
         x, (long)n, slot, nparts, static_cast<uint8_t *>(Y), static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out),
-        vec_ok);
+        vec_ok, gelu);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }
+
+int gelu_params(hipc_ctx *ctx, float divisor, float offset, float factor, int factor_first, GeluParams *out) {
+    HIPC_REQUIRE(ctx, divisor == divisor && offset == offset && factor == factor && divisor != 0.f, "DecomposedGelu: bad constants");
+    *out = GeluParams{1, divisor, offset, factor, factor_first != 0};
+    return HIPC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out, void *zp_out,
+                                 void *range, int range_ready) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    return dql_launch(ctx, X, n, Y, scale_out, zp_out, range, range_ready, GeluParams{0, 1.f, 0.f, 1.f, 0});
+}
+
+int hipc_dynamic_quantize_linear_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor, float offset, float factor,
+                                      int factor_first, void *Y, void *scale_out, void *zp_out, void *range) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    GeluParams gp;
+    if (int rc = gelu_params(ctx, divisor, offset, factor, factor_first, &gp)) return rc;
+    return dql_launch(ctx, X, n, Y, scale_out, zp_out, range, 0, gp);
+}
+
+int hipc_decomposed_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor, float offset, float factor,
+                         int factor_first, void *Y) {
+    if (!ctx) return HIPC_ERR_INVALID;
+    Guard g(ctx);
+    HIPC_REQUIRE(ctx, n >= 0, "DecomposedGelu: negative length");
+    GeluParams gp;
+    if (int rc = gelu_params(ctx, divisor, offset, factor, factor_first, &gp)) return rc;
+    if (n == 0) return HIPC_OK;
+    HIPC_REQUIRE(ctx, X && Y && aligned(X, 4) && aligned(Y, 4), "DecomposedGelu: null or unaligned tensor");
+    HIPC_REQUIRE(ctx, ceil_div(n, 256) < (int64_t(1) << 31), "DecomposedGelu: tensor too large");
+    decomposed_gelu_kernel<<<(unsigned)ceil_div(n, 256), 256, 0, ctx->stream>>>(static_cast<const float *>(X), (long)n, gp,
+                                                                                static_cast<float *>(Y));
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
+
+}  // extern "C"

@@ -179,8 +179,8 @@ int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void
 
 // offsets inside ctx->params
 constexpr size_t kParamRange = 0;   // 8 B  {bits(-min), bits(max)}
-constexpr size_t kParamParts = 256; // 2 KiB: per-workgroup {bits(-min), bits(max)} pairs of DynamicQuantizeLinear
-constexpr int kParamPartsMax = 256;
+constexpr size_t kParamParts = 256; // 16 KiB: per-workgroup {bits(-min), bits(max)} pairs of DynamicQuantizeLinear
+constexpr int kParamPartsMax = 2048;
 constexpr size_t kParamBytes = 256 + 8 * kParamPartsMax;
 
 }  // namespace hipc

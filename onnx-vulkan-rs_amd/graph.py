@@ -21,7 +21,7 @@ from . import ops
 from .runtime import Context, ConvGeom
 
 HOT_OPS = ("MatMulNBits", "DynamicQuantizeLinear", "MatMulInteger", "MatMulIntegerScaleBias", "QLinearMatMul",
-           "QLinearConv", "ConvInteger")
+           "QLinearConv", "ConvInteger", "DecomposedGelu", "DecomposedGeluQuantize")
 
 
 class Unsupported(Exception):
@@ -143,6 +143,16 @@ def execute(ctx: Context, nodes: List[NodeIr], env: Dict[str, np.ndarray]) -> No
         elif node.op == "DynamicQuantizeLinear":
             y, s, z = ops.dynamic_quantize_linear(ctx, inp(0))
             env[node.outputs[0]], env[node.outputs[1]], env[node.outputs[2]] = y, np.float32(s), np.uint8(z)
+        elif node.op in ("DecomposedGelu", "DecomposedGeluQuantize"):
+            # the rewrite's nodes (rewrite.rs:660-735): inputs x and the graph's three scalar constants
+            # (what it divides by, adds, multiplies by), attribute factor_first
+            c = [float(np.asarray(env[name], np.float32).reshape(-1)[0]) for name in node.inputs[1:4]]
+            k = dict(divisor=c[0], offset=c[1], factor=c[2], factor_first=bool(node.attrs.get("factor_first", 0)))
+            if node.op == "DecomposedGelu":
+                env[node.outputs[0]] = ops.decomposed_gelu(ctx, inp(0), **k)
+            else:
+                y, s, z = ops.dynamic_quantize_linear_gelu(ctx, inp(0), **k)
+                env[node.outputs[0]], env[node.outputs[1]], env[node.outputs[2]] = y, np.float32(s), np.uint8(z)
         elif node.op == "MatMulInteger":
             a, b = inp(0), inp(1)
             if a.ndim < 2 or b.ndim != 2:

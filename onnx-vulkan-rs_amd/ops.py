@@ -104,6 +104,35 @@ def dynamic_quantize_linear(ctx: Context, x):
     return y, scale, zp
 
 
+SQRT2_F32 = float(np.float32(np.sqrt(2.0)))
+
+
+def decomposed_gelu(ctx: Context, x, divisor=SQRT2_F32, offset=1.0, factor=0.5, factor_first=False):
+    """The exact GELU as Div, Erf, Add, Mul, Mul in one kernel (``DecomposedGelu``)."""
+    x = np.ascontiguousarray(x, np.float32)
+    dX, dY = ctx.upload(x), ctx.alloc(max(x.nbytes, 4))
+    ctx._check(ctx.lib.hipc_decomposed_gelu(ctx.handle, dX.ptr, x.size, divisor, offset, factor, int(factor_first), dY.ptr))
+    y = ctx.download(dY, np.float32, x.shape)
+    dX.free(), dY.free()
+    return y
+
+
+def dynamic_quantize_linear_gelu(ctx: Context, x, divisor=SQRT2_F32, offset=1.0, factor=0.5, factor_first=False):
+    """DynamicQuantizeLinear(DecomposedGelu(x)) in two passes over x (``DecomposedGeluQuantize``)."""
+    x = np.ascontiguousarray(x, np.float32)
+    dX = ctx.upload(x)
+    dY = ctx.alloc(max(x.size, 4))
+    dP = ctx.alloc(8)
+    ctx._check(ctx.lib.hipc_dynamic_quantize_linear_gelu(ctx.handle, dX.ptr if x.size else None, x.size, divisor, offset, factor,
+                                                         int(factor_first), dY.ptr if x.size else None, dP.ptr, dP.ptr + 4, None))
+    y = ctx.download(dY, np.uint8, x.shape)
+    scale = ctx.download(dP, np.float32, (1,))[0]
+    zp = int(ctx.download(dP, np.uint8, (1,), offset=4)[0])
+    for b in (dX, dY, dP):
+        b.free()
+    return y, scale, zp
+
+
 # ------------------------------------------------------------------ MatMulInteger
 
 class Int8Weight:

@@ -93,6 +93,29 @@ def dynamic_quantize_linear(x):
     return y, np.float32(scale.value), int(zp.value)
 
 
+def erf_approx(x):
+    """The reference's erf (shaders/elementwise.rs:71-80: Abramowitz-Stegun 7.1.26), every step in float32."""
+    f = np.float32
+    x = np.asarray(x, f)
+    a = np.abs(x)
+    with np.errstate(over="ignore", invalid="ignore"):   # a * a overflows to inf for huge |x|: exp(-inf) = 0, erf = +-1
+        t = (f(1.0) / (f(1.0) + f(0.3275911) * a)).astype(f)
+        poly = t * (f(0.254829592) + t * (f(-0.284496736) + t * (f(1.421413741) + t * (f(-1.453152027) + t * f(1.061405429)))))
+        return (np.sign(x).astype(f) * (f(1.0) - poly.astype(f) * np.exp(-a * a).astype(f))).astype(f)
+
+
+def decomposed_gelu(x, divisor=np.float32(np.sqrt(2.0)), offset=1.0, factor=0.5, factor_first=False):
+    """Div -> Erf -> Add -> Mul -> Mul, each rounding to float32 (shaders/elementwise.rs:82-118):
+    (x * (erf(x / divisor) + offset)) * factor, or x * ((erf + offset) * factor) with factor_first."""
+    f = np.float32
+    x = np.asarray(x, f)
+    e = (erf_approx((x / f(divisor)).astype(f)) + f(offset)).astype(f)
+    with np.errstate(over="ignore", invalid="ignore"):
+        if factor_first:
+            return (x * (e * f(factor)).astype(f)).astype(f)
+        return ((x * e).astype(f) * f(factor)).astype(f)
+
+
 def _signed(a):
     return 1 if a.dtype == np.int8 else 0
 

@@ -305,6 +305,27 @@ def test_conv_geometry_known_answers(oracle):
     assert oracle.same_pads(10, 1, 1, 1) == (0, 0)
 
 
+# ------------------------------------------------------------- DecomposedGelu
+
+def test_decomposed_gelu_is_the_exact_gelu_to_the_polynomial_s_error(oracle):
+    """erf_approx is Abramowitz-Stegun 7.1.26 (|error| <= 1.5e-7); with divisor sqrt(2), offset 1 and
+    factor 0.5 the five steps are x * Phi(x). Against math.erf in float64, both product orders; and
+    the two orders differ from each other only by rounding."""
+    import math
+    x = np.linspace(-6.0, 6.0, 4001).astype(np.float32)
+    erf64 = np.array([math.erf(float(v)) for v in x])
+    assert np.max(np.abs(oracle.erf_approx(x).astype(np.float64) - erf64)) < 6e-7   # 1.5e-7 of the formula + float32 steps
+    assert oracle.erf_approx(np.float32(0.0)) == 0.0 and oracle.erf_approx(np.float32(-7.0)) == -1.0
+    want = x.astype(np.float64) * 0.5 * (1.0 + np.array([math.erf(float(v) / math.sqrt(2.0)) for v in x]))
+    for ff in (False, True):
+        got = oracle.decomposed_gelu(x, factor_first=ff).astype(np.float64)
+        assert np.max(np.abs(got - want)) < 3e-6, ff
+    a, b = oracle.decomposed_gelu(x), oracle.decomposed_gelu(x, factor_first=True)
+    assert np.max(np.abs(a - b)) <= 5e-7
+    # other constants: offset and factor enter as written (a plain erf: divisor 1, offset 0, factor 1 gives x * erf(x))
+    assert np.allclose(oracle.decomposed_gelu(x, 1.0, 0.0, 1.0), x * oracle.erf_approx(x), rtol=0, atol=0)
+
+
 # ------------------------------------------------------------- decoder glue
 
 def test_decoder_glue_against_float64_closed_forms(oracle):
