@@ -438,29 +438,37 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
         const bool more = t0 + kAttnPass < t_end;
         // 3a. scores. The row of `pos` as loaded is not the step's key: it counts as zero here and
         //     the thread that owns it takes the key from LDS below.
+        //     A thread's two positions (kp and kp + 32) share every q value it reads from LDS.
+        float dot[KP][G];
+#pragma unroll
+        for (int ps = 0; ps < KP; ps++)
+#pragma unroll
+            for (int g = 0; g < G; g++) dot[ps][g] = 0.f;
+#pragma unroll
+        for (int u = 0; u < NK; u++) {
+            float kf[KP][8];
+#pragma unroll
+            for (int ps = 0; ps < KP; ps++) {
+                const bool stale = min(t0 + kp + 32 * ps, t_end - 1) == pos;
+                const uint4 raw = stale ? make_uint4(0, 0, 0, 0) : kreg[ps][u];
+                const __half2 *h2 = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+                for (int e = 0; e < 4; e++) kf[ps][2 * e] = __low2float(h2[e]), kf[ps][2 * e + 1] = __high2float(h2[e]);
+            }
+            const int c0 = u * 64 + seg * 8;
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float4 qa = *reinterpret_cast<const float4 *>(qs + g * HD + c0);
+                const float4 qb = *reinterpret_cast<const float4 *>(qs + g * HD + c0 + 4);
+#pragma unroll
+                for (int ps = 0; ps < KP; ps++)
+                    dot[ps][g] += (qa.x * kf[ps][0] + qa.y * kf[ps][1]) + (qa.z * kf[ps][2] + qa.w * kf[ps][3]) +
+                                  (qb.x * kf[ps][4] + qb.y * kf[ps][5]) + (qb.z * kf[ps][6] + qb.w * kf[ps][7]);
+            }
+        }
 #pragma unroll
         for (int ps = 0; ps < KP; ps++) {
             const int tp = kp + 32 * ps;
-            const bool stale = min(t0 + tp, t_end - 1) == pos;
-            float dot[G];
-#pragma unroll
-            for (int g = 0; g < G; g++) dot[g] = 0.f;
-#pragma unroll
-            for (int u = 0; u < NK; u++) {
-                const uint4 raw = stale ? make_uint4(0, 0, 0, 0) : kreg[ps][u];
-                const __half2 *h2 = reinterpret_cast<const __half2 *>(&raw);
-                float kf[8];
-#pragma unroll
-                for (int e = 0; e < 4; e++) kf[2 * e] = __low2float(h2[e]), kf[2 * e + 1] = __high2float(h2[e]);
-                const int c0 = u * 64 + seg * 8;
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-                    const float4 qa = *reinterpret_cast<const float4 *>(qs + g * HD + c0);
-                    const float4 qb = *reinterpret_cast<const float4 *>(qs + g * HD + c0 + 4);
-                    dot[g] += (qa.x * kf[0] + qa.y * kf[1]) + (qa.z * kf[2] + qa.w * kf[3]) +
-                              (qb.x * kf[4] + qb.y * kf[5]) + (qb.z * kf[6] + qb.w * kf[7]);
-                }
-            }
             if (t0 + tp == pos) {
 #pragma unroll 1
                 for (int u = 0; u < NK; u++) {
@@ -470,14 +478,14 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
                     for (int g = 0; g < G; g++) {
                         const float4 qa = *reinterpret_cast<const float4 *>(qs + g * HD + c0);
                         const float4 qb = *reinterpret_cast<const float4 *>(qs + g * HD + c0 + 4);
-                        dot[g] += (qa.x * ka.x + qa.y * ka.y) + (qa.z * ka.z + qa.w * ka.w) +
-                                  (qb.x * kb.x + qb.y * kb.y) + (qb.z * kb.z + qb.w * kb.w);
+                        dot[ps][g] += (qa.x * ka.x + qa.y * ka.y) + (qa.z * ka.z + qa.w * ka.w) +
+                                      (qb.x * kb.x + qb.y * kb.y) + (qb.z * kb.z + qb.w * kb.w);
                     }
                 }
             }
 #pragma unroll
             for (int g = 0; g < G; g++) {
-                float v = dot[g];
+                float v = dot[ps][g];
                 v += __shfl_xor(v, 1, 64);
                 v += __shfl_xor(v, 2, 64);
                 v += __shfl_xor(v, 4, 64);
