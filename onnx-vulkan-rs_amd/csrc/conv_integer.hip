@@ -225,24 +225,8 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
     HIPC_REQUIRE(ctx, X && Y, "Conv: null tensor");
 
     if (W->Wp) {
-        // NHWC copy of the activation, shifted to the signed domain
-        void *xt = nullptr;
-        const size_t x_bytes = (size_t)(g->n * g->c_in * g->h * g->w);
-        rc = scratch_get(ctx, 1, x_bytes + 16, &xt);
-        if (rc != HIPC_OK) return rc;
-        const int HW = (int)(g->h * g->w);
-        if (g->c_in % 4 == 0 && HW % 4 == 0 && aligned(X, 4))
-            nchw_to_nhwc4_kernel<<<dim3((unsigned)ceil_div(HW, 64), (unsigned)ceil_div(g->c_in, 64), (unsigned)g->n), 256, 0,
-                                   ctx->stream>>>(static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
-                                                  x_dtype == HIPC_U8 ? 0x80808080u : 0u);
-        else
-            nchw_to_nhwc_kernel<<<dim3((unsigned)ceil_div(HW, 32), (unsigned)ceil_div(g->c_in, 32), (unsigned)g->n), 256, 0,
-                                  ctx->stream>>>(static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
-                                                 x_dtype == HIPC_U8 ? 0x80 : 0);
-        HIPC_LAUNCHED(ctx);
         GemmArgs ga{};
         ga.P = W->Wp;
-        ga.Q = static_cast<const uint8_t *>(xt);
         ga.const_sum = W->rowsum;
         ga.dyn_zp = static_cast<const uint8_t *>(x_zp), ga.const_zp = static_cast<const uint8_t *>(w_zp);
         ga.dyn_shift = x_dtype == HIPC_U8 ? 128 : 0, ga.const_shift = W->w_dtype == HIPC_U8 ? 128 : 0;
@@ -264,9 +248,51 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
         }();
         const int64_t tiles64 = ceil_div(ga.I, 64) * ceil_div(ga.J, 64) * g->n;
         const bool small = forced >= 0 ? forced != 0 : (tiles64 <= 2 * (int64_t)ctx->cu_count && ga.K_pad >= 4 * kBK);
+        // the row sums of the activations only matter when the weight's zero point, in the signed domain, is not zero
+        const bool zero_known = ga.const_shift == 0 && (host_zp ? w_zp_value == 0 : w_zp == nullptr);
+
+        // A convolution along W alone whose per-tile input slab fits LDS reads the NCHW activation
+        // directly: no transposed copy at all (HIPC_CONV_ROW=0 takes the general route: tuning, tests).
+        static const bool row_off = [] {
+            const char *e = getenv("HIPC_CONV_ROW");
+            return e && atoi(e) == 0;
+        }();
+        const int64_t slab_pos = (3 + 63 * g->stride_w + (g->kw - 1) * g->dil_w + 1 + 3) / 4 * 4;
+        const size_t slab_bytes = (size_t)(slab_pos * g->c_in);
+        if (small && !row_off && g->h == 1 && g->kh == 1 && ho == 1 && g->pad_top == 0 && g->w % 4 == 0 && aligned(X, 4) &&
+            slab_bytes <= 64 * 1024) {
+            ga.Q = static_cast<const uint8_t *>(X);
+            ga.slab_pos = (int)slab_pos;
+            const size_t lds = std::max(kSmallLds, slab_bytes);
+            const dim3 grid(gemm_grid(ga, 64), 1, (unsigned)g->n);
+            if (ep.requant) {
+                if (zero_known) int8_conv_row_kernel<EPI_REQUANT, false><<<grid, 256, lds, ctx->stream>>>(ga);
+                else int8_conv_row_kernel<EPI_REQUANT, true><<<grid, 256, lds, ctx->stream>>>(ga);
+            } else {
+                if (zero_known) int8_conv_row_kernel<EPI_I32, false><<<grid, 256, lds, ctx->stream>>>(ga);
+                else int8_conv_row_kernel<EPI_I32, true><<<grid, 256, lds, ctx->stream>>>(ga);
+            }
+            HIPC_LAUNCHED(ctx);
+            return HIPC_OK;
+        }
+
+        // NHWC copy of the activation, shifted to the signed domain
+        void *xt = nullptr;
+        const size_t x_bytes = (size_t)(g->n * g->c_in * g->h * g->w);
+        rc = scratch_get(ctx, 1, x_bytes + 16, &xt);
+        if (rc != HIPC_OK) return rc;
+        const int HW = (int)(g->h * g->w);
+        if (g->c_in % 4 == 0 && HW % 4 == 0 && aligned(X, 4))
+            nchw_to_nhwc4_kernel<<<dim3((unsigned)ceil_div(HW, 64), (unsigned)ceil_div(g->c_in, 64), (unsigned)g->n), 256, 0,
+                                   ctx->stream>>>(static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
+                                                  x_dtype == HIPC_U8 ? 0x80808080u : 0u);
+        else
+            nchw_to_nhwc_kernel<<<dim3((unsigned)ceil_div(HW, 32), (unsigned)ceil_div(g->c_in, 32), (unsigned)g->n), 256, 0,
+                                  ctx->stream>>>(static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
+                                                 x_dtype == HIPC_U8 ? 0x80 : 0);
+        HIPC_LAUNCHED(ctx);
+        ga.Q = static_cast<const uint8_t *>(xt);
         if (small) {
-            // the row sums of the activations only matter when the weight's zero point, in the signed domain, is not zero
-            const bool zero_known = ga.const_shift == 0 && (host_zp ? w_zp_value == 0 : w_zp == nullptr);
             const dim3 grid(gemm_grid(ga, 64), 1, (unsigned)g->n);
             if (ep.requant) {
                 if (zero_known) int8_conv_small_kernel<EPI_REQUANT, false><<<grid, 256, kSmallLds, ctx->stream>>>(ga);

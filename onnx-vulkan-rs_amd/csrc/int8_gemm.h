@@ -56,6 +56,7 @@ struct GemmArgs {
 
     // conv geometry (MODE_CONV); Q is [n][H][W][C]
     int C, H, W, Ho, Wo, kh, kw, sh, sw, dh, dw, pt, pl;
+    int slab_pos;  // int8_conv_row_kernel: input positions held per tile
 
     // epilogue
     void *Y;
@@ -669,128 +670,17 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
     if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
 }
 
-// The same arrangement for a convolution with few 64x64 tiles (MODE_CONV): the gathered activation
-// chunks (the Q operand: 64 output positions x 128 bytes of (kh, kw, c) per stage) go through LDS,
-// the fragments of the prepacked, fragment-major weight (the P operand) come straight from memory,
-// and the four wavefronts split the product steps of a stage and add up at the end.
+// What the k-split convolution kernels below end with: the four wavefronts hold partial products
+// of all four 32x32 fragments of the 64x64 tile; wavefront w finishes fragment (w >> 1, w & 1),
+// receiving the other three wavefronts' parts through LDS (lds_acc: [owner][source 0..2][16][64],
+// lds_sum: [4 wavefronts][64 positions] activation sums). Every wavefront must be past its last
+// read of whatever else lived in that LDS before this is called.
 template <int EPI, bool DYN>
-__global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) {
-    constexpr int T = 64;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    uint8_t *lds_q = lds_raw;                                              // [2][T * kPitch]
-    int *lds_acc = reinterpret_cast<int *>(lds_raw);                       // after the loop: [owner][source 0..2][16][64]
-    int *lds_sum = lds_acc + 4 * 3 * 16 * 64;                              // [4 wavefronts][64 positions]
+__device__ __forceinline__ void conv_small_finish(const GemmArgs &p, i32x16 (&acc)[2][2], int (&dsum)[2], int *lds_acc, int *lds_sum,
+                                                  int i0, int j0, int img, int zd, int zc) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r32 = lane & 31, kg = lane >> 5;
-    const int img = blockIdx.z;
     auto handed = [&](int owner, int slot, int r) -> int & { return lds_acc[((owner * 3 + slot) * 16 + r) * 64 + lane]; };
-
-    const int tiles_x = (p.J + T - 1) / T, tiles_y = (p.I + T - 1) / T;
-    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
-    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
-    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
-    const int i0 = ty * T, j0 = tx * T;
-    const int nk = p.K_pad / kBK;
-
-    const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
-    const int zc = (p.host_zp ? p.const_zp_value : zp_byte(p.const_zp, p.const_signed)) - p.const_shift;
-    const uint32_t pad_word = (uint32_t)(zd & 0xff) * 0x01010101u;
-
-    // Q: chunk c = tid + 256 u of a 64-position slab: position c / 8, 16-byte k chunk c % 8
-    int kc_[2], base_h[2], base_w[2];
-    bool pos_ok[2];
-    uint32_t l_off[2];
-    const uint8_t *q_img = p.Q + (size_t)img * p.H * p.W * p.C;
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        const int c = tid + 256 * u, row = c >> 3;
-        kc_[u] = c & 7;
-        const int gj = j0 + row;
-        pos_ok[u] = gj < p.J;
-        const int oh = gj / p.Wo, ow = gj - oh * p.Wo;
-        base_h[u] = oh * p.sh - p.pt;
-        base_w[u] = ow * p.sw - p.pl;
-        l_off[u] = row * kPitch + kc_[u] * 16;
-    }
-    // P: fragments i0 / 32 and i0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
-    const uint8_t *p_frag[2];
-#pragma unroll
-    for (int f = 0; f < 2; f++) p_frag[f] = p.P + qfrag_offset(i0 + f * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
-
-    uint4 rq[kSmallSets][2], rp[kSmallSets][2];
-    // beyond the problem: zeros; padding taps: the zero point (which contributes nothing)
-    auto load_q = [&](int set, int stage) {
-        const int k0 = min(stage, nk - 1) * kBK;
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const int gk = k0 + kc_[u] * 16;
-            const int gkc = min(gk, p.K - 16);
-            const int tap = gkc / p.C, c0 = gkc - tap * p.C;
-            const int r = tap / p.kw, s = tap - r * p.kw;
-            const int ih = base_h[u] + r * p.dh, iw = base_w[u] + s * p.dw;
-            const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-            const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
-            const uint4 v = *reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + c0);
-            const bool live = pos_ok[u] && gk < p.K;
-            const uint32_t alt = live ? pad_word : 0u;
-            const bool take = live && inside;
-            rq[set][u] = make_uint4(take ? v.x : alt, take ? v.y : alt, take ? v.z : alt, take ? v.w : alt);
-        }
-    };
-    auto load_p = [&](int set, int stage) {
-#pragma unroll
-        for (int f = 0; f < 2; f++) rp[set][f] = *reinterpret_cast<const uint4 *>(p_frag[f] + (size_t)min(stage, nk - 1) * kBK * 32);
-    };
-    // a stage past the end is stored as zeros: its products add nothing whatever the weight holds
-    auto store_q = [&](int set, int buf, bool live) {
-        const uint32_t keep = live ? 0xffffffffu : 0u;
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-            *reinterpret_cast<uint4 *>(lds_q + buf * T * kPitch + l_off[u]) =
-                make_uint4(rq[set][u].x & keep, rq[set][u].y & keep, rq[set][u].z & keep, rq[set][u].w & keep);
-    };
-
-    i32x16 acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
-    int dsum[2] = {0, 0};
-    const uint32_t frag_q = r32 * kPitch + wave * 32 + kg * 16;
-    auto compute = [&](int buf, int set) {
-        i32x4 b[2];
-#pragma unroll
-        for (int f = 0; f < 2; f++) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(lds_q + buf * T * kPitch + frag_q + f * 32 * kPitch);
-            b[f] = __builtin_bit_cast(i32x4, v);
-            if (DYN) dsum[f] += dot_ones(v);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, rp[set][i]), b[j], acc[i][j], 0, 0, 0);
-    };
-
-#pragma unroll
-    for (int d = 0; d < kSmallSets; d++) load_q(d, d), load_p(d, d);
-    store_q(0, 0, true);
-    load_q(0, kSmallSets);
-    __syncthreads();
-    for (int s = 0; s < nk; s += kSmallSets) {
-#pragma unroll
-        for (int d = 0; d < kSmallSets; d++) {
-            compute(d & 1, d);
-            load_p(d, s + d + kSmallSets);
-            store_q((d + 1) % kSmallSets, (d + 1) & 1, s + d + 1 < nk);
-            load_q((d + 1) % kSmallSets, s + d + 1 + kSmallSets);
-            __syncthreads();
-        }
-    }
-
     // the weight sums of the rows this lane will finish (fragment (wave >> 1, wave & 1)): asked for
     // before the hand-over, so that the epilogue does not start with a memory round trip
     // (and, for the requantising epilogue, their ratios and int32 biases)
@@ -861,6 +751,293 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
             }
         }
     }
+}
+
+// The same arrangement for a convolution with few 64x64 tiles (MODE_CONV): the gathered activation
+// chunks (the Q operand: 64 output positions x 128 bytes of (kh, kw, c) per stage) go through LDS,
+// the fragments of the prepacked, fragment-major weight (the P operand) come straight from memory,
+// and the four wavefronts split the product steps of a stage and add up at the end.
+template <int EPI, bool DYN>
+__global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) {
+    constexpr int T = 64;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint8_t *lds_q = lds_raw;                                              // [2][T * kPitch]
+    int *lds_acc = reinterpret_cast<int *>(lds_raw);                       // after the loop: [owner][source 0..2][16][64]
+    int *lds_sum = lds_acc + 4 * 3 * 16 * 64;                              // [4 wavefronts][64 positions]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r32 = lane & 31, kg = lane >> 5;
+    const int img = blockIdx.z;
+
+    const int tiles_x = (p.J + T - 1) / T, tiles_y = (p.I + T - 1) / T;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
+    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
+    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
+    const int i0 = ty * T, j0 = tx * T;
+    const int nk = p.K_pad / kBK;
+
+    const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
+    const int zc = (p.host_zp ? p.const_zp_value : zp_byte(p.const_zp, p.const_signed)) - p.const_shift;
+    const uint32_t pad_word = (uint32_t)(zd & 0xff) * 0x01010101u;
+
+    // Q: chunk c = tid + 256 u of a 64-position slab: position c / 8, 16-byte k chunk c % 8
+    int kc_[2], base_h[2], base_w[2];
+    bool pos_ok[2];
+    uint32_t l_off[2];
+    const uint8_t *q_img = p.Q + (size_t)img * p.H * p.W * p.C;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int c = tid + 256 * u, row = c >> 3;
+        kc_[u] = c & 7;
+        const int gj = j0 + row;
+        pos_ok[u] = gj < p.J;
+        const int oh = gj / p.Wo, ow = gj - oh * p.Wo;
+        base_h[u] = oh * p.sh - p.pt;
+        base_w[u] = ow * p.sw - p.pl;
+        l_off[u] = row * kPitch + kc_[u] * 16;
+    }
+    // P: fragments i0 / 32 and i0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
+    const uint8_t *p_frag[2];
+#pragma unroll
+    for (int f = 0; f < 2; f++) p_frag[f] = p.P + qfrag_offset(i0 + f * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
+
+    uint4 rq[kSmallSets][2], rp[kSmallSets][2];
+    // Where a chunk's 16 bytes sit in the filter window: (row, column, first channel) of the stage
+    // about to be loaded. load_q is called for stages 0, 1, 2, ... in turn, so the triple moves on
+    // by one stage (kBK bytes of k) per call with adds and compares only; the divisions are made
+    // once, here, and the step's own quotients are the same for every thread.
+    const int adv_tap = kBK / p.C, adv_c = kBK - adv_tap * p.C;
+    const int adv_r = adv_tap / p.kw, adv_s = adv_tap - adv_r * p.kw;
+    int q_k[2], q_r[2], q_s[2], q_c[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        q_k[u] = kc_[u] * 16;
+        const int tap = q_k[u] / p.C;
+        q_c[u] = q_k[u] - tap * p.C;
+        q_r[u] = tap / p.kw;
+        q_s[u] = tap - q_r[u] * p.kw;
+    }
+    // beyond the problem: zeros; padding taps: the zero point (which contributes nothing).
+    // Past K the triple points outside the window; the clamps keep the address inside the image.
+    auto load_q = [&](int set) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int ih = base_h[u] + q_r[u] * p.dh, iw = base_w[u] + q_s[u] * p.dw;
+            const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+            const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
+            const uint4 v = *reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + q_c[u]);
+            const bool live = pos_ok[u] && q_k[u] < p.K;
+            const uint32_t alt = live ? pad_word : 0u;
+            const bool take = live && inside;
+            rq[set][u] = make_uint4(take ? v.x : alt, take ? v.y : alt, take ? v.z : alt, take ? v.w : alt);
+            q_k[u] += kBK;
+            q_c[u] += adv_c;
+            const int wrap = q_c[u] >= p.C ? 1 : 0;
+            q_c[u] -= wrap ? p.C : 0;
+            q_s[u] += adv_s + wrap;
+            const int down = q_s[u] >= p.kw ? 1 : 0;
+            q_s[u] -= down ? p.kw : 0;
+            q_r[u] = min(q_r[u] + adv_r + down, 1 << 20);
+        }
+    };
+    auto load_p = [&](int set, int stage) {
+#pragma unroll
+        for (int f = 0; f < 2; f++) rp[set][f] = *reinterpret_cast<const uint4 *>(p_frag[f] + (size_t)min(stage, nk - 1) * kBK * 32);
+    };
+    // a stage past the end is stored as zeros: its products add nothing whatever the weight holds
+    auto store_q = [&](int set, int buf, bool live) {
+        const uint32_t keep = live ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            *reinterpret_cast<uint4 *>(lds_q + buf * T * kPitch + l_off[u]) =
+                make_uint4(rq[set][u].x & keep, rq[set][u].y & keep, rq[set][u].z & keep, rq[set][u].w & keep);
+    };
+
+    i32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    int dsum[2] = {0, 0};
+    const uint32_t frag_q = r32 * kPitch + wave * 32 + kg * 16;
+    auto compute = [&](int buf, int set) {
+        i32x4 b[2];
+#pragma unroll
+        for (int f = 0; f < 2; f++) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(lds_q + buf * T * kPitch + frag_q + f * 32 * kPitch);
+            b[f] = __builtin_bit_cast(i32x4, v);
+            if (DYN) dsum[f] += dot_ones(v);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, rp[set][i]), b[j], acc[i][j], 0, 0, 0);
+    };
+
+#pragma unroll
+    for (int d = 0; d < kSmallSets; d++) load_q(d), load_p(d, d);
+    store_q(0, 0, true);
+    load_q(0);
+    __syncthreads();
+    for (int s = 0; s < nk; s += kSmallSets) {
+#pragma unroll
+        for (int d = 0; d < kSmallSets; d++) {
+            compute(d & 1, d);
+            load_p(d, s + d + kSmallSets);
+            store_q((d + 1) % kSmallSets, (d + 1) & 1, s + d + 1 < nk);
+            load_q((d + 1) % kSmallSets);
+            __syncthreads();
+        }
+    }
+
+    conv_small_finish<EPI, DYN>(p, acc, dsum, lds_acc, lds_sum, i0, j0, img, zd, zc);
+}
+
+// A convolution along one axis (H = 1, a 1 x kw window) with few 64x64 tiles, straight from the
+// NCHW activation. The 64 output positions of a tile see 63 sw + (kw - 1) dw + 1 input positions
+// of every channel: that slab is read once, as 32-bit words along the positions, transposed 4 x 4
+// in registers and kept in LDS for the whole product as [16-channel chunk][position][16 bytes].
+// A lane's operand chunk of product step k = tap * C + c is then one 16-byte LDS read at position
+// (output position) * sw + tap * dw, consecutive lanes reading consecutive 16 bytes; nothing is
+// gathered from memory and the k loop has no barrier. The weight fragments come straight from
+// memory and the four wavefronts split the product steps, as in the kernel above.
+// p.Q is the NCHW activation as the caller gave it (uint8 is shifted to signed on the way in),
+// p.slab_pos the positions a slab holds (a multiple of 4). Needs W % 4 == 0 and 4-byte aligned images.
+constexpr int kRowBatch = 8;  // 16-quad blocks of the slab a wavefront has in flight
+template <int EPI, bool DYN>
+__global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
+    constexpr int T = 64;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint8_t *slab = lds_raw;                                               // [C / 16][slab_pos][16]
+    int *lds_acc = reinterpret_cast<int *>(lds_raw);                       // after the loop: [owner][source 0..2][16][64]
+    int *lds_sum = lds_acc + 4 * 3 * 16 * 64;                              // [4 wavefronts][64 positions]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r32 = lane & 31, kg = lane >> 5;
+    const int img = blockIdx.z;
+
+    const int tiles_x = (p.J + T - 1) / T, tiles_y = (p.I + T - 1) / T;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
+    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
+    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
+    const int i0 = ty * T, j0 = tx * T;
+    const int nk = p.K_pad / kBK;
+
+    const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
+    const int zc = (p.host_zp ? p.const_zp_value : zp_byte(p.const_zp, p.const_signed)) - p.const_shift;
+    const uint32_t pad_word = (uint32_t)(zd & 0xff) * 0x01010101u;
+    const uint32_t flip4 = p.dyn_shift ? 0x80808080u : 0u;
+
+    // P: fragments i0 / 32 and i0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
+    const uint8_t *p_frag[2];
+#pragma unroll
+    for (int f = 0; f < 2; f++) p_frag[f] = p.P + qfrag_offset(i0 + f * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
+    uint4 rp[kSmallSets][2];
+    auto load_p = [&](int set, int stage) {
+#pragma unroll
+        for (int f = 0; f < 2; f++) rp[set][f] = *reinterpret_cast<const uint4 *>(p_frag[f] + (size_t)min(stage, nk - 1) * kBK * 32);
+    };
+#pragma unroll
+    for (int d = 0; d < kSmallSets; d++) load_p(d, d);
+
+    // The slab starts at the 4-aligned input position at or below the tile's first one. A block is
+    // 16 position quads x one 16-channel chunk: lane (quad l >> 2, channel quad l & 3) reads four
+    // positions of four channels and writes four words, each the four channels of one position.
+    // Words outside the row hold the zero point (W % 4 == 0: a word is inside or outside as a whole).
+    const int SP = p.slab_pos, npq = SP >> 2, n_pq16 = (npq + 15) >> 4;
+    const int in0 = j0 * p.sw - p.pl;
+    const int base = in0 & ~3, lead = in0 - base;
+    const int n_blocks = (p.C >> 4) * n_pq16;
+    const uint8_t *x_img = p.Q + (size_t)img * p.C * p.W;
+    for (int b0 = wave; b0 < n_blocks; b0 += 4 * kRowBatch) {
+        uint32_t in[kRowBatch][4];
+#pragma unroll
+        for (int u = 0; u < kRowBatch; u++) {
+            const int b = min(b0 + 4 * u, n_blocks - 1);   // a repeated block rewrites the same words
+            const int chunk = b / n_pq16, pq = (b - chunk * n_pq16) * 16 + (lane >> 2);
+            const int gpos = base + 4 * pq;
+            const bool inside = pq < npq && gpos >= 0 && gpos < p.W;
+            const uint8_t *src = x_img + (size_t)(chunk * 16 + (lane & 3) * 4) * p.W + (inside ? gpos : 0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(src + (size_t)i * p.W);
+                in[u][i] = inside ? v ^ flip4 : pad_word;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kRowBatch; u++) {
+            const int b = min(b0 + 4 * u, n_blocks - 1);
+            const int chunk = b / n_pq16, pq = (b - chunk * n_pq16) * 16 + (lane >> 2);
+            if (pq >= npq) continue;
+            const uint32_t lo01 = __builtin_amdgcn_perm(in[u][1], in[u][0], 0x05010400u);  // a0 b0 a1 b1
+            const uint32_t hi01 = __builtin_amdgcn_perm(in[u][1], in[u][0], 0x07030602u);  // a2 b2 a3 b3
+            const uint32_t lo23 = __builtin_amdgcn_perm(in[u][3], in[u][2], 0x05010400u);  // c0 d0 c1 d1
+            const uint32_t hi23 = __builtin_amdgcn_perm(in[u][3], in[u][2], 0x07030602u);  // c2 d2 c3 d3
+            uint32_t *dst = reinterpret_cast<uint32_t *>(slab + ((size_t)chunk * SP + 4 * pq) * 16 + (lane & 3) * 4);
+            dst[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);   // a0 b0 c0 d0: position 4 pq
+            dst[4] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+            dst[8] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+            dst[12] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+        }
+    }
+
+    // This lane's 16 bytes of product step n (k = 128 n + 32 wave + 16 kg) are channels q_c.. of tap
+    // q_s; both move on by 128 bytes of k per step with adds and compares (the quotients of the
+    // step are the same for every thread). Past K the weight is zero and the position is clamped
+    // into the slab, so the product adds nothing; the activation sums skip those steps.
+    const int adv_tap = kBK / p.C, adv_c = kBK - adv_tap * p.C;
+    int q_k = wave * 32 + kg * 16;
+    int q_s = q_k / p.C, q_c = q_k - q_s * p.C;
+    const int pos0 = lead + r32 * p.sw;
+
+    i32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    int dsum[2] = {0, 0};
+    auto compute = [&](int set) {
+        i32x4 b[2];
+        const uint8_t *chunk = slab + (size_t)(q_c >> 4) * SP * 16;
+#pragma unroll
+        for (int f = 0; f < 2; f++) {
+            const int pos = min(pos0 + f * 32 * p.sw + q_s * p.dw, SP - 1);
+            const uint4 v = *reinterpret_cast<const uint4 *>(chunk + pos * 16);
+            b[f] = __builtin_bit_cast(i32x4, v);
+            if (DYN) dsum[f] += q_k < p.K ? dot_ones(v) : 0;
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, rp[set][i]), b[j], acc[i][j], 0, 0, 0);
+        q_k += kBK;
+        q_c += adv_c;
+        const int wrap = q_c >= p.C ? 1 : 0;
+        q_c -= wrap ? p.C : 0;
+        q_s = min(q_s + adv_tap + wrap, 1 << 20);
+    };
+
+    __syncthreads();
+    // whole rounds without a branch, so that the weight loads stay counted exactly; then the rest
+    int s = 0;
+    for (; s + kSmallSets <= nk; s += kSmallSets) {
+#pragma unroll
+        for (int d = 0; d < kSmallSets; d++) {
+            compute(d);
+            load_p(d, s + d + kSmallSets);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < kSmallSets - 1; d++)
+        if (s + d < nk) compute(d);
+    __syncthreads();   // the hand-over reuses the slab's LDS
+    conv_small_finish<EPI, DYN>(p, acc, dsum, lds_acc, lds_sum, i0, j0, img, zd, zc);
 }
 
 // ---- the large-problem variant (MODE_MM, aligned A) --------------------------------------

@@ -144,6 +144,34 @@ def test_geometries_and_signs(ctx, pkg, oracle, cfg, signs):
     assert np.array_equal(got, oracle.qlinear_conv(X, 0.03, x_zp, W, np.float32(0.004), w_zp, 0.7, 99, None, og))
 
 
+ROWS = [  # 1-D convolutions whose input slab stays in LDS: (c_in, c_out, t, kw, dilation, stride, pads l/r, batch)
+    (112, 70, 200, 5, 2, 2, (3, 6), 2),     # an odd number of 16-channel chunks, strided, lopsided pads, ragged tiles
+    (32, 64, 260, 17, 1, 3, (0, 5), 1),     # four taps per product step; no left pad
+    (208, 96, 128, 3, 7, 1, (7, 7), 3),     # a tap straddles product steps (208 = 128 + 80)
+    (512, 64, 64, 7, 20, 1, (60, 60), 1),   # the slab would not fit: the general route
+]
+
+
+@pytest.mark.parametrize("signs", [(np.uint8, np.int8), (np.int8, np.uint8)], ids=["u8xi8", "i8xu8"])
+@pytest.mark.parametrize("c_in,c_out,t,kw,dil,stride,pads,n", ROWS, ids=lambda v: str(v).replace(" ", ""))
+def test_row_convolutions_straight_from_nchw(ctx, pkg, oracle, c_in, c_out, t, kw, dil, stride, pads, n, signs):
+    """One filter axis, k >= 512: the kernel that keeps a tile's input positions in LDS and reads the
+    NCHW activation itself -- against the dense definition (tests/conv_integer_im2col.rs:58-89)
+    and the oracle's requantisation."""
+    X, W, w_scale, bias, kwargs = _qconv_case(pkg, c_in, c_out, t, kw, dil, seed=90 + c_in, n=n, stride=stride)
+    kwargs["pads"] = (0, pads[0], 0, pads[1])
+    kwargs["strides"] = (1, stride)
+    X, W = X.view(signs[0]), W.view(signs[1])
+    geom, og = pkg.ConvGeom.make(X.shape, W.shape, **kwargs), oracle.conv_geom(X.shape, W.shape, **kwargs)
+    x_zp = 100 if signs[0] == np.uint8 else -20
+    w_zp = 0 if signs[1] == np.int8 else 131
+    acc = pkg.ops.conv_integer(ctx, X, W, x_zp, w_zp, geom)
+    want = rc.conv_integer_dense(X, W, x_zp, w_zp, kwargs["strides"], kwargs["dilations"], kwargs["pads"], 1)
+    assert acc.shape == want.shape and np.array_equal(acc, want)
+    got = pkg.ops.qlinear_conv(ctx, X, 0.03, x_zp, W, np.float32(0.004), w_zp, 2.5, -5, bias, geom, y_signed=True)
+    assert np.array_equal(got, oracle.qlinear_conv(X, 0.03, x_zp, W, np.float32(0.004), w_zp, 2.5, -5, bias, og, True))
+
+
 def test_one_dimensional_node_with_auto_pad(ctx, pkg, oracle):
     X, W, w_scale, bias, _ = _qconv_case(pkg, 32, 32, 300, 7, 3, seed=80)
     node = pkg.graph.NodeIr("QLinearConv", ["x", "x_scale", "x_zp", "w", "w_scale", "w_zp", "y_scale", "y_zp", "B"],
