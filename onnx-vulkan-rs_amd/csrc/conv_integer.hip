@@ -252,14 +252,16 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
         const bool zero_known = ga.const_shift == 0 && (host_zp ? w_zp_value == 0 : w_zp == nullptr);
 
         // A convolution along W alone whose per-tile input slab fits LDS reads the NCHW activation
-        // directly: no transposed copy at all (HIPC_CONV_ROW=0 takes the general route: tuning, tests).
+        // directly: no transposed copy at all, whatever the number of tiles (on 8 x 512 x 4096 inputs,
+        // k = 7, it still finishes before the tiled route: 120 against 147 us).
+        // HIPC_CONV_ROW=0 takes the general route (tuning, tests).
         static const bool row_off = [] {
             const char *e = getenv("HIPC_CONV_ROW");
             return e && atoi(e) == 0;
         }();
         const int64_t slab_pos = (3 + 63 * g->stride_w + (g->kw - 1) * g->dil_w + 1 + 3) / 4 * 4;
         const size_t slab_bytes = (size_t)(slab_pos * g->c_in);
-        if (small && !row_off && g->h == 1 && g->kh == 1 && ho == 1 && g->pad_top == 0 && g->w % 4 == 0 && aligned(X, 4) &&
+        if (!row_off && g->h == 1 && g->kh == 1 && ho == 1 && g->pad_top == 0 && g->w % 4 == 0 && aligned(X, 4) &&
             slab_bytes <= 64 * 1024) {
             ga.Q = static_cast<const uint8_t *>(X);
             ga.slab_pos = (int)slab_pos;

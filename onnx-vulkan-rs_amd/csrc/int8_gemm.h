@@ -670,30 +670,40 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
     if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
 }
 
-// What the k-split convolution kernels below end with: the four wavefronts hold partial products
-// of all four 32x32 fragments of the 64x64 tile; wavefront w finishes fragment (w >> 1, w & 1),
-// receiving the other three wavefronts' parts through LDS (lds_acc: [owner][source 0..2][16][64],
-// lds_sum: [4 wavefronts][64 positions] activation sums). Every wavefront must be past its last
-// read of whatever else lived in that LDS before this is called.
+// What the k-split convolution kernels below end with. The four wavefronts hold partial products
+// of all four 32x32 fragments of the 64x64 tile, acc[j][i] = positions j*32.. x channels i*32..,
+// with the positions along the rows of the matrix-core result: register r of lane l is position
+// (r >> 2) * 8 + (l >> 5) * 4 + (r & 3), channel l & 31. Wavefront w finishes fragment
+// (j = w & 1, i = w >> 1), receiving the other three wavefronts' parts through LDS (lds_acc:
+// [owner][source 0..2][16][64], lds_sum: [4 wavefronts][64 positions] activation sums). A lane
+// then owns one output channel -- one weight sum, ratio and bias -- and runs of four consecutive
+// positions of it, which leave as one 32-bit (bytes) or 128-bit (int32) store. The code after the
+// hand-over is the same for all four wavefronts: it is run once per workgroup, so its size counts.
+// Every wavefront must be past its last read of whatever else lived in that LDS before this is called.
+struct ConvChannel {
+    int csum = 0, qb = 0;
+    float ratio = 0.f;
+};
+template <int EPI>
+__device__ __forceinline__ ConvChannel conv_small_channel(const GemmArgs &p, int i0) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ch = i0 + (wave >> 1) * 32 + (lane & 31);
+    ConvChannel c;
+    c.csum = p.const_sum[ch];  // I_pad rows exist
+    const int cc = min(ch, p.I - 1);
+    if (EPI == EPI_REQUANT) {
+        c.ratio = p.ratio[(size_t)cc * p.ratio_step];
+        if (p.qbias) c.qb = p.qbias[cc];
+    }
+    return c;
+}
+
 template <int EPI, bool DYN>
-__device__ __forceinline__ void conv_small_finish(const GemmArgs &p, i32x16 (&acc)[2][2], int (&dsum)[2], int *lds_acc, int *lds_sum,
-                                                  int i0, int j0, int img, int zd, int zc) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__device__ __forceinline__ void conv_small_finish(const GemmArgs &p, i32x16 (&acc)[2][2], int (&dsum)[2], const ConvChannel &chan,
+                                                  int *lds_acc, int *lds_sum, int i0, int j0, int img, int zd, int zc) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r32 = lane & 31, kg = lane >> 5;
     auto handed = [&](int owner, int slot, int r) -> int & { return lds_acc[((owner * 3 + slot) * 16 + r) * 64 + lane]; };
-    // the weight sums of the rows this lane will finish (fragment (wave >> 1, wave & 1)): asked for
-    // before the hand-over, so that the epilogue does not start with a memory round trip
-    // (and, for the requantising epilogue, their ratios and int32 biases)
-    int my_csum[16], my_qb[16];
-    float my_ratio[16];
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int row = i0 + (wave >> 1) * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
-        my_csum[r] = p.const_sum[row];  // I_pad rows exist
-        const int c = min(row, p.I - 1);
-        my_ratio[r] = EPI == EPI_REQUANT ? p.ratio[(size_t)c * p.ratio_step] : 0.f;
-        my_qb[r] = EPI == EPI_REQUANT && p.qbias ? p.qbias[c] : 0;
-    }
     // sums of the activations over this wavefront's product steps, per position: the two k halves live in lanes l and l + 32
     if (DYN) {
 #pragma unroll
@@ -704,50 +714,76 @@ __device__ __forceinline__ void conv_small_finish(const GemmArgs &p, i32x16 (&ac
         }
     }
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int j = 0; j < 2; j++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
+        for (int i = 0; i < 2; i++) {
             const int owner = i * 2 + j;
             if (owner == wave) continue;
             const int slot = wave < owner ? wave : wave - 1;
 #pragma unroll
-            for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[i][j][r];
+            for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[j][i][r];
         }
     __syncthreads();
 
+    // This wavefront's own part of its fragment, picked with masks of all ones or all zeros whose
+    // values the compiler is not told: a choice it can read as an index would send the
+    // accumulators through memory.
+    int is1 = wave == 1 ? -1 : 0, is2 = wave == 2 ? -1 : 0, is3 = wave == 3 ? -1 : 0;
+    asm("" : "+v"(is1), "+v"(is2), "+v"(is3));
+    i32x16 mine;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        int m = acc[0][0][r];
+        m = (acc[1][0][r] & is1) | (m & ~is1);
+        m = (acc[0][1][r] & is2) | (m & ~is2);
+        m = (acc[1][1][r] & is3) | (m & ~is3);
+        mine[r] = m;
+    }
+    const int jf = wave & 1, ifr = wave >> 1;
+    const int ch = i0 + ifr * 32 + r32;
     const int kzz = p.K * zd * zc;
-    float fmn = 0.f, fmx = 0.f;
+    int out[16];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (int r = 0; r < 16; r++) {
+        int v = mine[r];
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            if (i * 2 + j != wave) continue;
-            const int gj = j0 + j * 32 + r32;
+        for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
+        v = v - zd * chan.csum + kzz;
+        if (DYN) {
+            const int at = jf * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
             int qs = 0;
-            if (DYN) {
 #pragma unroll
-                for (int w = 0; w < 4; w++) qs += lds_sum[w * 64 + j * 32 + r32];
+            for (int w = 0; w < 4; w++) qs += lds_sum[w * 64 + at];
+            v -= zc * qs;
+        }
+        if (EPI == EPI_REQUANT) {
+            const int q = (int)rintf(__fmul_rn((float)(v + chan.qb), chan.ratio)) + p.y_zp;
+            v = p.out_signed ? min(max(q, -128), 127) & 0xff : min(max(q, 0), 255);
+        }
+        out[r] = v;
+    }
+    if (ch >= p.I) return;
+    const size_t row = ((size_t)img * p.I + ch) * p.J;
+    const bool wide = (p.J & 3) == 0 && (reinterpret_cast<uintptr_t>(p.Y) & (EPI == EPI_REQUANT ? 3 : 15)) == 0;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const int pos = j0 + jf * 32 + g * 8 + kg * 4;   // four consecutive positions: out[4 g ..]
+        if (wide && pos + 3 < p.J) {
+            if (EPI == EPI_REQUANT) {
+                const uint32_t word = (uint32_t)out[4 * g] | (uint32_t)out[4 * g + 1] << 8 | (uint32_t)out[4 * g + 2] << 16 |
+                                      (uint32_t)out[4 * g + 3] << 24;
+                *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(p.Y) + row + pos) = word;
+            } else {
+                // written once and several times the operands: kept from displacing them in the caches
+                i32x4 quad = {out[4 * g], out[4 * g + 1], out[4 * g + 2], out[4 * g + 3]};
+                __builtin_nontemporal_store(quad, reinterpret_cast<i32x4 *>(static_cast<int32_t *>(p.Y) + row + pos));
             }
+        } else {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);  // row inside the 32x32 fragment
-                const int gi = i0 + i * 32 + rf;
-                int v = acc[i][j][r];
-#pragma unroll
-                for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
-                if (gi >= p.I || gj >= p.J) continue;
-                v = v - zd * my_csum[r] + kzz;
-                if (DYN) v -= zc * qs;
-                if (EPI == EPI_REQUANT) {
-                    int q = (int)rintf(__fmul_rn((float)(v + my_qb[r]), my_ratio[r])) + p.y_zp;
-                    const size_t at = ((size_t)img * p.I + gi) * p.J + gj;
-                    if (p.out_signed)
-                        static_cast<int8_t *>(p.Y)[at] = (int8_t)min(max(q, -128), 127);
-                    else
-                        static_cast<uint8_t *>(p.Y)[at] = (uint8_t)min(max(q, 0), 255);
-                } else {
-                    gemm_emit<MODE_CONV, EPI>(p, img, gi, gj, v, fmn, fmx);
-                }
+            for (int e = 0; e < 4; e++) {
+                if (pos + e >= p.J) continue;
+                if (EPI == EPI_REQUANT) static_cast<uint8_t *>(p.Y)[row + pos + e] = (uint8_t)out[4 * g + e];
+                else static_cast<int32_t *>(p.Y)[row + pos + e] = out[4 * g + e];
             }
         }
     }
@@ -874,7 +910,7 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, rp[set][i]), b[j], acc[i][j], 0, 0, 0);
+                acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], __builtin_bit_cast(i32x4, rp[set][i]), acc[j][i], 0, 0, 0);
     };
 
 #pragma unroll
@@ -893,7 +929,9 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
         }
     }
 
-    conv_small_finish<EPI, DYN>(p, acc, dsum, lds_acc, lds_sum, i0, j0, img, zd, zc);
+    // asked for before the hand-over, so that the epilogue does not start with a memory round trip
+    const ConvChannel chan = conv_small_channel<EPI>(p, i0);
+    conv_small_finish<EPI, DYN>(p, acc, dsum, chan, lds_acc, lds_sum, i0, j0, img, zd, zc);
 }
 
 // A convolution along one axis (H = 1, a 1 x kw window) with few 64x64 tiles, straight from the
@@ -942,6 +980,8 @@ __global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
     };
 #pragma unroll
     for (int d = 0; d < kSmallSets; d++) load_p(d, d);
+    // the epilogue's per-channel constants travel with the first loads
+    const ConvChannel chan = conv_small_channel<EPI>(p, i0);
 
     // The slab starts at the 4-aligned input position at or below the tile's first one. A block is
     // 16 position quads x one 16-channel chunk: lane (quad l >> 2, channel quad l & 3) reads four
@@ -950,33 +990,40 @@ __global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
     const int SP = p.slab_pos, npq = SP >> 2, n_pq16 = (npq + 15) >> 4;
     const int in0 = j0 * p.sw - p.pl;
     const int base = in0 & ~3, lead = in0 - base;
-    const int n_blocks = (p.C >> 4) * n_pq16;
+    const int n_chunks = p.C >> 4;
     const uint8_t *x_img = p.Q + (size_t)img * p.C * p.W;
-    for (int b0 = wave; b0 < n_blocks; b0 += 4 * kRowBatch) {
+    // block b = wave + 4 u is (chunk b / n_pq16, quad block b % n_pq16): both are the same for the
+    // whole wavefront and move on by four blocks with adds and compares
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int step_chunk = 4 / n_pq16, step_pb = 4 - step_chunk * n_pq16;
+    int chunk = wave_u / n_pq16, pb = wave_u - chunk * n_pq16;
+    while (chunk < n_chunks) {
         uint32_t in[kRowBatch][4];
+        int at[kRowBatch];   // byte offset of the block's first word in the slab, or -1: nothing to store
 #pragma unroll
         for (int u = 0; u < kRowBatch; u++) {
-            const int b = min(b0 + 4 * u, n_blocks - 1);   // a repeated block rewrites the same words
-            const int chunk = b / n_pq16, pq = (b - chunk * n_pq16) * 16 + (lane >> 2);
+            const int pq = pb * 16 + (lane >> 2);
             const int gpos = base + 4 * pq;
-            const bool inside = pq < npq && gpos >= 0 && gpos < p.W;
-            const uint8_t *src = x_img + (size_t)(chunk * 16 + (lane & 3) * 4) * p.W + (inside ? gpos : 0);
+            const bool live = chunk < n_chunks && pq < npq;
+            const bool inside = live && gpos >= 0 && gpos < p.W;
+            const uint8_t *src = x_img + (size_t)(min(chunk, n_chunks - 1) * 16 + (lane & 3) * 4) * p.W + (inside ? gpos : 0);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const uint32_t v = *reinterpret_cast<const uint32_t *>(src + (size_t)i * p.W);
                 in[u][i] = inside ? v ^ flip4 : pad_word;
             }
+            at[u] = live ? (chunk * SP + 4 * pq) * 16 + (lane & 3) * 4 : -1;
+            pb += step_pb, chunk += step_chunk;
+            if (pb >= n_pq16) pb -= n_pq16, chunk++;
         }
 #pragma unroll
         for (int u = 0; u < kRowBatch; u++) {
-            const int b = min(b0 + 4 * u, n_blocks - 1);
-            const int chunk = b / n_pq16, pq = (b - chunk * n_pq16) * 16 + (lane >> 2);
-            if (pq >= npq) continue;
+            if (at[u] < 0) continue;
             const uint32_t lo01 = __builtin_amdgcn_perm(in[u][1], in[u][0], 0x05010400u);  // a0 b0 a1 b1
             const uint32_t hi01 = __builtin_amdgcn_perm(in[u][1], in[u][0], 0x07030602u);  // a2 b2 a3 b3
             const uint32_t lo23 = __builtin_amdgcn_perm(in[u][3], in[u][2], 0x05010400u);  // c0 d0 c1 d1
             const uint32_t hi23 = __builtin_amdgcn_perm(in[u][3], in[u][2], 0x07030602u);  // c2 d2 c3 d3
-            uint32_t *dst = reinterpret_cast<uint32_t *>(slab + ((size_t)chunk * SP + 4 * pq) * 16 + (lane & 3) * 4);
+            uint32_t *dst = reinterpret_cast<uint32_t *>(slab + at[u]);
             dst[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);   // a0 b0 c0 d0: position 4 pq
             dst[4] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
             dst[8] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
@@ -1015,7 +1062,7 @@ __global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, rp[set][i]), b[j], acc[i][j], 0, 0, 0);
+                acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], __builtin_bit_cast(i32x4, rp[set][i]), acc[j][i], 0, 0, 0);
         q_k += kBK;
         q_c += adv_c;
         const int wrap = q_c >= p.C ? 1 : 0;
@@ -1037,7 +1084,7 @@ __global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
     for (int d = 0; d < kSmallSets - 1; d++)
         if (s + d < nk) compute(d);
     __syncthreads();   // the hand-over reuses the slab's LDS
-    conv_small_finish<EPI, DYN>(p, acc, dsum, lds_acc, lds_sum, i0, j0, img, zd, zc);
+    conv_small_finish<EPI, DYN>(p, acc, dsum, chan, lds_acc, lds_sum, i0, j0, img, zd, zc);
 }
 
 // ---- the large-problem variant (MODE_MM, aligned A) --------------------------------------
