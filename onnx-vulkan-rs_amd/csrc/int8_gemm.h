@@ -671,14 +671,15 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
 }
 
 // What the k-split convolution kernels below end with. The four wavefronts hold partial products
-// of all four 32x32 fragments of the 64x64 tile, acc[j][i] = positions j*32.. x channels i*32..,
-// with the positions along the rows of the matrix-core result: register r of lane l is position
-// (r >> 2) * 8 + (l >> 5) * 4 + (r & 3), channel l & 31. Wavefront w finishes fragment
-// (j = w & 1, i = w >> 1), receiving the other three wavefronts' parts through LDS (lds_acc:
-// [owner][source 0..2][16][64], lds_sum: [4 wavefronts][64 positions] activation sums). A lane
-// then owns one output channel -- one weight sum, ratio and bias -- and runs of four consecutive
-// positions of it, which leave as one 32-bit (bytes) or 128-bit (int32) store. The code after the
-// hand-over is the same for all four wavefronts: it is run once per workgroup, so its size counts.
+// of all four 32x32 fragments of the 64x64 tile, positions x channels, with the positions along
+// the rows of the matrix-core result: register r of lane l is position (r >> 2) * 8 + (l >> 5) * 4
+// + (r & 3), channel l & 31. Wavefront w finishes fragment (positions jf = w & 1, channels
+// ifr = w >> 1), and every wavefront numbers its accumulators from that one: acc[dj][di] is
+// fragment (jf ^ dj, ifr ^ di), so its own part is acc[0][0] and needs no choosing. The other three
+// wavefronts' parts arrive through LDS (lds_acc: [owner][source 0..2][16][64], lds_sum:
+// [4 wavefronts][64 positions] activation sums, dsum[f] being those of positions fragment jf ^ f).
+// A lane then owns one output channel -- one weight sum, ratio and bias -- and runs of four
+// consecutive positions of it, which leave as one 32-bit (bytes) or 128-bit (int32) store.
 // Every wavefront must be past its last read of whatever else lived in that LDS before this is called.
 struct ConvChannel {
     int csum = 0, qb = 0;
@@ -704,62 +705,50 @@ __device__ __forceinline__ void conv_small_finish(const GemmArgs &p, i32x16 (&ac
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r32 = lane & 31, kg = lane >> 5;
     auto handed = [&](int owner, int slot, int r) -> int & { return lds_acc[((owner * 3 + slot) * 16 + r) * 64 + lane]; };
+    const int jf = wave & 1, ifr = wave >> 1;
     // sums of the activations over this wavefront's product steps, per position: the two k halves live in lanes l and l + 32
     if (DYN) {
 #pragma unroll
         for (int f = 0; f < 2; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
         if (kg == 0) {
 #pragma unroll
-            for (int f = 0; f < 2; f++) lds_sum[wave * 64 + f * 32 + r32] = dsum[f];
+            for (int f = 0; f < 2; f++) lds_sum[wave * 64 + (f ^ jf) * 32 + r32] = dsum[f];
         }
     }
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int dj = 0; dj < 2; dj++)
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int owner = i * 2 + j;
-            if (owner == wave) continue;
+        for (int di = 0; di < 2; di++) {
+            if (dj == 0 && di == 0) continue;
+            const int owner = ((ifr ^ di) << 1) | (jf ^ dj);
             const int slot = wave < owner ? wave : wave - 1;
 #pragma unroll
-            for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[j][i][r];
+            for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[dj][di][r];
         }
     __syncthreads();
 
-    // This wavefront's own part of its fragment, picked with masks of all ones or all zeros whose
-    // values the compiler is not told: a choice it can read as an index would send the
-    // accumulators through memory.
-    int is1 = wave == 1 ? -1 : 0, is2 = wave == 2 ? -1 : 0, is3 = wave == 3 ? -1 : 0;
-    asm("" : "+v"(is1), "+v"(is2), "+v"(is3));
-    i32x16 mine;
+    // all of the LDS reads first, so that their latency is paid once and not per output
+    int part[3][16], qs[16];
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        int m = acc[0][0][r];
-        m = (acc[1][0][r] & is1) | (m & ~is1);
-        m = (acc[0][1][r] & is2) | (m & ~is2);
-        m = (acc[1][1][r] & is3) | (m & ~is3);
-        mine[r] = m;
+    for (int slot = 0; slot < 3; slot++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) part[slot][r] = handed(wave, slot, r);
+    if (DYN) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int at = jf * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
+            qs[r] = lds_sum[at] + lds_sum[64 + at] + lds_sum[128 + at] + lds_sum[192 + at];
+        }
     }
-    const int jf = wave & 1, ifr = wave >> 1;
     const int ch = i0 + ifr * 32 + r32;
-    const int kzz = p.K * zd * zc;
+    const int fixed = p.K * zd * zc - zd * chan.csum + (EPI == EPI_REQUANT ? chan.qb : 0);
+    const int lo = p.out_signed ? -128 : 0, hi = p.out_signed ? 127 : 255;
     int out[16];
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-        int v = mine[r];
-#pragma unroll
-        for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
-        v = v - zd * chan.csum + kzz;
-        if (DYN) {
-            const int at = jf * 32 + (r >> 2) * 8 + kg * 4 + (r & 3);
-            int qs = 0;
-#pragma unroll
-            for (int w = 0; w < 4; w++) qs += lds_sum[w * 64 + at];
-            v -= zc * qs;
-        }
-        if (EPI == EPI_REQUANT) {
-            const int q = (int)rintf(__fmul_rn((float)(v + chan.qb), chan.ratio)) + p.y_zp;
-            v = p.out_signed ? min(max(q, -128), 127) & 0xff : min(max(q, 0), 255);
-        }
+        int v = acc[0][0][r] + part[0][r] + part[1][r] + part[2][r] + fixed;
+        if (DYN) v -= zc * qs[r];
+        if (EPI == EPI_REQUANT) v = min(max((int)rintf(__fmul_rn((float)v, chan.ratio)) + p.y_zp, lo), hi) & 0xff;
         out[r] = v;
     }
     if (ch >= p.I) return;
@@ -832,10 +821,12 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
         base_w[u] = ow * p.sw - p.pl;
         l_off[u] = row * kPitch + kc_[u] * 16;
     }
-    // P: fragments i0 / 32 and i0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
+    // P: fragments i0 / 32 and i0 / 32 + 1 of this wavefront's product step, the one this wavefront
+    // will finish first (see conv_small_finish); a step is 1 KB on, a stage 4 KB
     const uint8_t *p_frag[2];
 #pragma unroll
-    for (int f = 0; f < 2; f++) p_frag[f] = p.P + qfrag_offset(i0 + f * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
+    for (int f = 0; f < 2; f++)
+        p_frag[f] = p.P + qfrag_offset(i0 + (f ^ (wave >> 1)) * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
 
     uint4 rq[kSmallSets][2], rp[kSmallSets][2];
     // Where a chunk's 16 bytes sit in the filter window: (row, column, first channel) of the stage
@@ -902,7 +893,7 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
         i32x4 b[2];
 #pragma unroll
         for (int f = 0; f < 2; f++) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(lds_q + buf * T * kPitch + frag_q + f * 32 * kPitch);
+            const uint4 v = *reinterpret_cast<const uint4 *>(lds_q + buf * T * kPitch + frag_q + (f ^ (wave & 1)) * 32 * kPitch);
             b[f] = __builtin_bit_cast(i32x4, v);
             if (DYN) dsum[f] += dot_ones(v);
         }
@@ -972,7 +963,8 @@ __global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
     // P: fragments i0 / 32 and i0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
     const uint8_t *p_frag[2];
 #pragma unroll
-    for (int f = 0; f < 2; f++) p_frag[f] = p.P + qfrag_offset(i0 + f * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
+    for (int f = 0; f < 2; f++)
+        p_frag[f] = p.P + qfrag_offset(i0 + (f ^ (wave >> 1)) * 32, wave * 32, p.K_pad) + lane * 16;  // I_pad is a multiple of 128
     uint4 rp[kSmallSets][2];
     auto load_p = [&](int set, int stage) {
 #pragma unroll
@@ -1031,14 +1023,23 @@ __global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
         }
     }
 
-    // This lane's 16 bytes of product step n (k = 128 n + 32 wave + 16 kg) are channels q_c.. of tap
-    // q_s; both move on by 128 bytes of k per step with adds and compares (the quotients of the
-    // step are the same for every thread). Past K the weight is zero and the position is clamped
-    // into the slab, so the product adds nothing; the activation sums skip those steps.
+    // This lane's 16 bytes of product step n (k = 128 n + 32 wave + 16 kg) are channels q_c.. of some
+    // tap: in the slab, `off` bytes from its start for the lane's position in fragment 0. Both move
+    // on by 128 bytes of k per step with adds and compares (the quotients of the step are the same
+    // for every thread): (adv_c / 16) chunks and adv_tap taps on, and one tap on less a whole row
+    // of chunks when the channel wraps. Past K the weight is zero and the address is clamped into
+    // the slab, so the product adds nothing; the activation sums skip those steps.
     const int adv_tap = kBK / p.C, adv_c = kBK - adv_tap * p.C;
+    const int SP16 = SP * 16;
+    const int step_off = (adv_c >> 4) * SP16 + adv_tap * p.dw * 16, wrap_off = p.dw * 16 - (p.C >> 4) * SP16;
+    const int last_off = (p.C >> 4) * SP16 - 16;
     int q_k = wave * 32 + kg * 16;
-    int q_s = q_k / p.C, q_c = q_k - q_s * p.C;
-    const int pos0 = lead + r32 * p.sw;
+    const int tap0 = q_k / p.C;
+    int q_c = q_k - tap0 * p.C;
+    int off = (q_c >> 4) * SP16 + (lead + r32 * p.sw + tap0 * p.dw) * 16;
+    int frag_off[2];   // the wavefront's own positions fragment first (see conv_small_finish)
+#pragma unroll
+    for (int f = 0; f < 2; f++) frag_off[f] = (f ^ (wave & 1)) * 32 * p.sw * 16;
 
     i32x16 acc[2][2];
 #pragma unroll
@@ -1048,41 +1049,47 @@ __global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
     int dsum[2] = {0, 0};
-    auto compute = [&](int set) {
-        i32x4 b[2];
-        const uint8_t *chunk = slab + (size_t)(q_c >> 4) * SP * 16;
+    // the operand of the next step is read from LDS before this step's products are issued
+    uint4 bq[2][2];
+    auto read_q = [&](int par) {
 #pragma unroll
-        for (int f = 0; f < 2; f++) {
-            const int pos = min(pos0 + f * 32 * p.sw + q_s * p.dw, SP - 1);
-            const uint4 v = *reinterpret_cast<const uint4 *>(chunk + pos * 16);
-            b[f] = __builtin_bit_cast(i32x4, v);
-            if (DYN) dsum[f] += q_k < p.K ? dot_ones(v) : 0;
-        }
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-                acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], __builtin_bit_cast(i32x4, rp[set][i]), acc[j][i], 0, 0, 0);
-        q_k += kBK;
+        for (int f = 0; f < 2; f++) bq[par][f] = *reinterpret_cast<const uint4 *>(slab + min(off + frag_off[f], last_off));
+        off += step_off;
         q_c += adv_c;
-        const int wrap = q_c >= p.C ? 1 : 0;
+        const bool wrap = q_c >= p.C;
         q_c -= wrap ? p.C : 0;
-        q_s = min(q_s + adv_tap + wrap, 1 << 20);
+        off += wrap ? wrap_off : 0;
+    };
+    auto compute = [&](int set, int par) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if (DYN) dsum[j] += q_k < p.K ? dot_ones(bq[par][j]) : 0;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, bq[par][j]), __builtin_bit_cast(i32x4, rp[set][i]),
+                                                                  acc[j][i], 0, 0, 0);
+        }
+        q_k += kBK;
     };
 
     __syncthreads();
+    read_q(0);
     // whole rounds without a branch, so that the weight loads stay counted exactly; then the rest
     int s = 0;
     for (; s + kSmallSets <= nk; s += kSmallSets) {
 #pragma unroll
         for (int d = 0; d < kSmallSets; d++) {
-            compute(d);
+            read_q((d + 1) & 1);
+            compute(d, d & 1);
             load_p(d, s + d + kSmallSets);
         }
     }
 #pragma unroll
     for (int d = 0; d < kSmallSets - 1; d++)
-        if (s + d < nk) compute(d);
+        if (s + d < nk) {
+            read_q((d + 1) & 1);
+            compute(d, d & 1);
+        }
     __syncthreads();   // the hand-over reuses the slab's LDS
     conv_small_finish<EPI, DYN>(p, acc, dsum, chan, lds_acc, lds_sum, i0, j0, img, zd, zc);
 }
