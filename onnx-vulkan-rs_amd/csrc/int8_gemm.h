@@ -495,7 +495,7 @@ constexpr int kSmallSets = 4;  // register sets of A chunks and of B fragments: 
 constexpr size_t kSmallLds = 4 * 3 * 16 * 64 * sizeof(int) + 4 * 64 * sizeof(int);
 
 template <int EPI, bool DYN>
-__global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) {
+__global__ void __launch_bounds__(256, 3) int8_gemm_small_kernel(const GemmArgs p) {  // three workgroups per CU (LDS allows no more): 168 registers
     constexpr int T = 64;                       // edge of the workgroup's tile
     constexpr int kCh = T / 32;                 // 16-byte chunks of an A slab per thread
     constexpr int kSteps = 1;                   // product steps of a stage per wavefront
@@ -527,12 +527,15 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
         p_off[u] = (uint32_t)min(i0 + row, p.I - 1) * (uint32_t)p.K + kc * 16;  // rows past I: clamped, never stored
         l_off[u] = row * kPitch + kc * 16;
     }
-    // B: fragments j0 / 32 and j0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB
+    // B: fragments j0 / 32 and j0 / 32 + 1 of this wavefront's product step; a step is 1 KB on, a stage 4 KB.
+    // Wavefront w will finish fragment (rows w >> 1, columns w & 1) and numbers its operands and
+    // accumulators from that one: acc[di][dj] is fragment ((w >> 1) ^ di, (w & 1) ^ dj), so its own
+    // part is acc[0][0] whatever w is and the epilogue is one piece of code.
     const int j_last = (p.J + kBN - 1) / kBN * kBN - 1;  // B is packed in whole 128-column tiles
     uint32_t q_off[2];
 #pragma unroll
     for (int f = 0; f < 2; f++)
-        q_off[f] = qfrag_offset(min(j0 + f * 32, j_last - 31), wave * 32, p.K_pad) + lane * 16;
+        q_off[f] = qfrag_offset(min(j0 + (f ^ (wave & 1)) * 32, j_last - 31), wave * 32, p.K_pad) + lane * 16;
     const __amdgpu_buffer_rsrc_t rsrc_p = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t *>(p.P), 0, (int)((uint32_t)p.I * (uint32_t)p.K), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
@@ -579,7 +582,7 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
         for (int step = 0; step < kSteps; step++)
 #pragma unroll
             for (int f = 0; f < 2; f++)
-                av[step][f] = *reinterpret_cast<const uint4 *>(lds_a + buf * T * kPitch + frag_a + f * 32 * kPitch + step * 32);
+                av[step][f] = *reinterpret_cast<const uint4 *>(lds_a + buf * T * kPitch + frag_a + (f ^ (wave >> 1)) * 32 * kPitch + step * 32);
 #pragma unroll
         for (int step = 0; step < kSteps; step++) {
             if (DYN) {
@@ -616,55 +619,56 @@ __global__ void __launch_bounds__(256) int8_gemm_small_kernel(const GemmArgs p) 
     }
 
     // row sums of A over this wavefront's product steps: the two k halves of a row live in lanes l and l + 32
+    const int ifr = wave >> 1, jf = wave & 1;
     if (DYN) {
 #pragma unroll
         for (int f = 0; f < 2; f++) dsum[f] += __shfl_xor(dsum[f], 32, 64);
         if (kg == 0) {
 #pragma unroll
-            for (int f = 0; f < 2; f++) lds_sum[wave * 64 + f * 32 + r32] = dsum[f];
+            for (int f = 0; f < 2; f++) lds_sum[wave * 64 + (f ^ ifr) * 32 + r32] = dsum[f];
         }
     }
-    // wavefront w finishes fragment (w >> 1, w & 1); the other three it hands over (the A buffers
-    // are free: the loop ended with a barrier)
-    {
+    // the other three fragments are handed over (the A buffers are free: the loop ended with a barrier)
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+    for (int di = 0; di < 2; di++)
 #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const int owner = i * 2 + j;
-                if (owner == wave) continue;
-                const int slot = wave < owner ? wave : wave - 1;  // 0..2 among the three sources
+        for (int dj = 0; dj < 2; dj++) {
+            if (di == 0 && dj == 0) continue;
+            const int owner = ((ifr ^ di) << 1) | (jf ^ dj);
+            const int slot = wave < owner ? wave : wave - 1;  // 0..2 among the three sources
 #pragma unroll
-                for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[i][j][r];
-            }
-    }
+            for (int r = 0; r < 16; r++) handed(owner, slot, r) = acc[di][dj][r];
+        }
     __syncthreads();
 
-    const int kzz = p.K * zd * zc;
+    // The handed-over parts are read four output rows ahead of their use: the LDS latency is paid
+    // once, not per output, and the stores still leave spread out (other workgroups of the CU are
+    // in their product loops meanwhile).
+    const int fixed = p.K * zd * zc - zd * my_csum;
+    const int gj = j0 + jf * 32 + r32;
     float fmn = 0.f, fmx = 0.f;
+    int part[2][4], rs[2][4];
+    auto read_group = [&](int g, int par) {
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            if (i * 2 + j != wave) continue;
-            const int gj = j0 + j * 32 + r32;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);  // row inside the 32x32 fragment
-                const int gi = i0 + i * 32 + rf;
-                int v = acc[i][j][r];
-#pragma unroll
-                for (int slot = 0; slot < 3; slot++) v += handed(wave, slot, r);
-                if (gi >= p.I || gj >= p.J) continue;
-                v = v - zd * my_csum + kzz;
-                if (DYN) {
-                    int rs = 0;
-#pragma unroll
-                    for (int w = 0; w < 4; w++) rs += lds_sum[w * 64 + i * 32 + rf];
-                    v -= zc * rs;
-                }
-                gemm_emit_mm<EPI>(p, my_emit, gi, gj, v, fmn, fmx);
+        for (int e = 0; e < 4; e++) {
+            const int r = 4 * g + e;
+            part[par][e] = handed(wave, 0, r) + handed(wave, 1, r) + handed(wave, 2, r);
+            if (DYN) {
+                const int at = ifr * 32 + g * 8 + kg * 4 + e;
+                rs[par][e] = lds_sum[at] + lds_sum[64 + at] + lds_sum[128 + at] + lds_sum[192 + at];
             }
+        }
+    };
+    read_group(0, 0);
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        if (g + 1 < 4) read_group(g + 1, (g + 1) & 1);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int gi = i0 + ifr * 32 + g * 8 + kg * 4 + e;
+            int v = acc[0][0][4 * g + e] + part[g & 1][e] + fixed;
+            if (DYN) v -= zc * rs[g & 1][e];
+            if (gi < p.I && gj < p.J) gemm_emit_mm<EPI>(p, my_emit, gi, gj, v, fmn, fmx);
         }
     }
     if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
@@ -937,7 +941,7 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
 // p.slab_pos the positions a slab holds (a multiple of 4). Needs W % 4 == 0 and 4-byte aligned images.
 constexpr int kRowBatch = 8;  // 16-quad blocks of the slab a wavefront has in flight
 template <int EPI, bool DYN>
-__global__ void __launch_bounds__(256) int8_conv_row_kernel(const GemmArgs p) {
+__global__ void __launch_bounds__(256, 3) int8_conv_row_kernel(const GemmArgs p) {
     constexpr int T = 64;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     uint8_t *slab = lds_raw;                                               // [C / 16][slab_pos][16]
