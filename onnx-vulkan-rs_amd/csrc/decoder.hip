@@ -18,6 +18,7 @@
 #include <hip/hip_fp16.h>
 
 #include <cstdlib>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -303,7 +304,7 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
 
 // ---- the context chunks of one decode step's attention in one launch (head_dim 64 / 128 / 256) ----
 // Workgroup (split, kvh) owns attn_chunk(span) consecutive visible positions of kv head kvh, walks them
-// kAttnPass at a time and serves all G query heads of the group. It
+// kAttnPass at a time (kAttnShortPass when that is the whole chunk) and serves all G query heads of the group. It
 //   1. asks for the fused qkv vector's pieces it needs and for the K and V rows of its first pass
 //      (16-byte pieces, every load of a pass independent of every other),
 //   2. prepares the step's own q, k, v: per-head RMS norm and half-split rotary embedding for q
@@ -323,12 +324,10 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
                        int max_seq, float scale, int window, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
                        float *__restrict__ part_ml, float *__restrict__ part_o) {
     constexpr int GH = G * HD, NK = HD / 64, HALF = HD / 2;
-    constexpr int KP = kAttnPass / 32;         // passes of 32 positions over the keys (8 threads per position)
     constexpr int VT = HD / 8;                 // threads per value row (8 channels each)
     constexpr int VPP = 256 / VT;              // value rows in flight per pass of the workgroup
-    constexpr int VI = kAttnPass / VPP;        // value rows per thread
     constexpr int ROWS = (G + 1 + 3) / 4;      // q heads and the k head, dealt to four wavefronts
-    static_assert(kAttnPass == 64, "one lane per position of a pass");
+    static_assert(kAttnPass == 64 && kAttnShortPass == 32, "at most one lane per position of a pass");
     __shared__ __attribute__((aligned(16))) float qs[GH];      // query heads, normed and rotated
     __shared__ __attribute__((aligned(16))) float kn[HD];      // the step's key, as the cache will hold it
     __shared__ __attribute__((aligned(16))) float vn[HD];      // the step's value
@@ -366,6 +365,14 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
     //    K: thread (kp, seg) reads the 16-byte piece `seg` of every 128-byte run of rows kp and
     //    kp + 32 (a row is read in whole cache lines); V: thread (pg, cb) reads 8 channels of rows
     //    pg, pg + VPP, ...  Rows past the end repeat the last one (their weights are zero).
+    // Everything from here on is written once for a pass of P positions and instantiated for the
+    // two pass lengths; a launch runs one of them (chunks of 32 positions are walked 32 at a time:
+    // half the score and value work per workgroup, on twice as many CUs).
+    auto walk = [&](auto pass_length) {
+    constexpr int P = decltype(pass_length)::value;
+    constexpr int KP = P / 32;                 // passes of 32 positions over the keys (8 threads per position)
+    constexpr int VI = P / VPP;                // value rows per thread
+    static_assert(VI >= 1, "a pass holds at least one value row per thread");
     const int kp = tid >> 3, seg = tid & 7;
     const int pg = tid / VT, cb = tid % VT;
     const __half *k_head = k_cache + (size_t)kvh * max_seq * HD + seg * 8;
@@ -433,9 +440,9 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 #pragma unroll
         for (int e = 0; e < 8; e++) o[g][e] = 0.f;
 
-    for (int t0 = t_begin; t0 < t_end; t0 += kAttnPass) {
-        const int cnt = min(kAttnPass, t_end - t0);
-        const bool more = t0 + kAttnPass < t_end;
+    for (int t0 = t_begin; t0 < t_end; t0 += P) {
+        const int cnt = min(P, t_end - t0);
+        const bool more = t0 + P < t_end;
         // 3a. scores. The row of `pos` as loaded is not the step's key: it counts as zero here and
         //     the thread that owns it takes the key from LDS below.
         //     A thread's two positions (kp and kp + 32) share every q value it reads from LDS.
@@ -489,14 +496,14 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
                 v += __shfl_xor(v, 1, 64);
                 v += __shfl_xor(v, 2, 64);
                 v += __shfl_xor(v, 4, 64);
-                if (seg == 0) sc[g * kAttnPass + tp] = v * scale;
+                if (seg == 0) sc[g * P + tp] = v * scale;
             }
         }
-        if (more) load_k(t0 + kAttnPass);
+        if (more) load_k(t0 + P);
         __syncthreads();
         // 3b. one wavefront per head: the pass's max and sum join the running pair
         for (int g = wave; g < G; g += 4) {
-            const float x = lane < cnt ? sc[g * kAttnPass + lane] : -3.0e38f;
+            const float x = lane < cnt ? sc[g * P + lane] : -3.0e38f;
             const float m_old = mrun[g], l_old = lrun[g];
             float m = x;
 #pragma unroll
@@ -507,7 +514,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
             const float f = __expf(m_old - m);
-            sc[g * kAttnPass + lane] = pv;
+            if (lane < P) sc[g * P + lane] = pv;
             if (lane == 0) mrun[g] = m, lrun[g] = l_old * f + l, fac[g] = f;
         }
         __syncthreads();
@@ -531,23 +538,23 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
                 for (int e = 0; e < 4; e++) vf[2 * e] = __low2float(h2[e]), vf[2 * e + 1] = __high2float(h2[e]);
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    const float w = sc[g * kAttnPass + tp];  // zero past the end of the pass
+                    const float w = sc[g * P + tp];  // zero past the end of the pass
 #pragma unroll
                     for (int e = 0; e < 8; e++) o[g][e] += w * vf[e];
                 }
             }
             const int own = pos - t0;  // the step's own position, if this pass holds it
-            if (own >= 0 && own < kAttnPass && (own % VPP) == pg) {
+            if (own >= 0 && own < P && (own % VPP) == pg) {
                 const float4 va = *reinterpret_cast<const float4 *>(vn + cb * 8), vb = *reinterpret_cast<const float4 *>(vn + cb * 8 + 4);
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    const float w = sc[g * kAttnPass + own];
+                    const float w = sc[g * P + own];
                     o[g][0] += w * va.x, o[g][1] += w * va.y, o[g][2] += w * va.z, o[g][3] += w * va.w;
                     o[g][4] += w * vb.x, o[g][5] += w * vb.y, o[g][6] += w * vb.z, o[g][7] += w * vb.w;
                 }
             }
         }
-        if (more) load_v(t0 + kAttnPass);
+        if (more) load_v(t0 + P);
         // the next pass rewrites sc only after the barrier that follows its scores' LDS reads of qs;
         // its writes to sc must not overtake this pass's reads of sc
         __syncthreads();
@@ -572,7 +579,11 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
         po[idx] = (ored[idx] + ored[GH + idx]) + (ored[2 * GH + idx] + ored[3 * GH + idx]);
     float *ml = part_ml + ((size_t)kvh * kAttnSplits + split) * G * 2;
     if (tid < G) ml[tid * 2] = mrun[tid], ml[tid * 2 + 1] = lrun[tid];
+    };
+    if (chunk == kAttnShortPass) walk(std::integral_constant<int, kAttnShortPass>{});
+    else walk(std::integral_constant<int, kAttnPass>{});
 }
+
 
 // h[i] = gelu_tanh(gu[i]) * gu[ffn + i]
 __global__ void __launch_bounds__(256) dec_gelu_mul_kernel(const float *__restrict__ gu, int ffn, float *__restrict__ h) {

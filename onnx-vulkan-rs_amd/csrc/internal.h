@@ -155,11 +155,15 @@ struct GemvPrologue {
 };
 // Decode attention splits the visible context of a kv head (`span` positions: all of them, or the
 // last `window`) over kAttnSplits workgroups. Each takes `attn_chunk(span)` consecutive positions,
-// a multiple of kAttnPass, so that all splits together cover the span; the first
-// attn_live_chunks(span) splits hold at least one position and only those write a partial.
+// so that all splits together cover the span: kAttnShortPass positions while that is enough
+// (span <= 2048: up to 64 workgroups of 32 positions rather than 32 of 64), else a multiple of
+// kAttnPass. The first attn_live_chunks(span) splits hold at least one position and only those
+// write a partial.
 constexpr int kAttnPass = 64;
+constexpr int kAttnShortPass = 32;
 constexpr int kAttnSplits = 64;
 __host__ __device__ inline int attn_chunk(int total) {
+    if (total <= kAttnShortPass * kAttnSplits) return kAttnShortPass;
     return kAttnPass * ((total + kAttnPass * kAttnSplits - 1) / (kAttnPass * kAttnSplits));
 }
 __host__ __device__ inline int attn_live_chunks(int total) {
