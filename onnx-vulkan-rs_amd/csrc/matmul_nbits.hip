@@ -263,7 +263,9 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     float *asum = reinterpret_cast<float *>(As + (size_t)nch * (4 * NT) * M);
     float *red = asum + ((nch * M + 3) & ~3);  // [WN][WK][T][NR][64]
 
-    const int lane = tid & 63, wave = tid >> 6;
+    // the wavefront's number is told to the compiler as the scalar it is: the tile cursors derived
+    // from it then live in scalar registers and cost the vector unit nothing
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wk = wave % p.WK, wn = wave / p.WK;
     const int i16 = lane & 15, g4 = lane >> 4;
     const int groups = (p.n_tiles + T - 1) / T;
