@@ -939,7 +939,7 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
 // memory and the four wavefronts split the product steps, as in the kernel above.
 // p.Q is the NCHW activation as the caller gave it (uint8 is shifted to signed on the way in),
 // p.slab_pos the positions a slab holds (a multiple of 4). Needs W % 4 == 0 and 4-byte aligned images.
-constexpr int kRowBatch = 8;  // 16-quad blocks of the slab a wavefront has in flight
+constexpr int kRowBatch = 4;  // steps of the slab loader whose loads are in flight together
 template <int EPI, bool DYN>
 __global__ void __launch_bounds__(256, 3) int8_conv_row_kernel(const GemmArgs p) {
     constexpr int T = 64;
@@ -979,38 +979,42 @@ __global__ void __launch_bounds__(256, 3) int8_conv_row_kernel(const GemmArgs p)
     // the epilogue's per-channel constants travel with the first loads
     const ConvChannel chan = conv_small_channel<EPI>(p, i0);
 
-    // The slab starts at the 4-aligned input position at or below the tile's first one. A block is
-    // 16 position quads x one 16-channel chunk: lane (quad l >> 2, channel quad l & 3) reads four
-    // positions of four channels and writes four words, each the four channels of one position.
-    // Words outside the row hold the zero point (W % 4 == 0: a word is inside or outside as a whole).
-    const int SP = p.slab_pos, npq = SP >> 2, n_pq16 = (npq + 15) >> 4;
+    // The slab starts at the 4-aligned input position at or below the tile's first one. Its
+    // (16-channel chunk, position quad) pairs are numbered chunk * npq + quad and dealt 16 to a
+    // wavefront instruction, 64 to a step of the workgroup: lane l takes pair 16 wave + (l >> 2) +
+    // 64 step and, of it, channel quad l & 3 -- it reads four positions of four channels and writes
+    // four words, each the four channels of one position. A lane's pair moves on by 64 per step:
+    // 64 / npq chunks and 64 % npq quads, with adds and compares. Words outside the row hold the
+    // zero point (W % 4 == 0: a word is inside or outside as a whole).
+    const int SP = p.slab_pos, npq = SP >> 2;
     const int in0 = j0 * p.sw - p.pl;
     const int base = in0 & ~3, lead = in0 - base;
-    const int n_chunks = p.C >> 4;
+    const int n_chunks = p.C >> 4, n_pairs = n_chunks * npq;
     const uint8_t *x_img = p.Q + (size_t)img * p.C * p.W;
-    // block b = wave + 4 u is (chunk b / n_pq16, quad block b % n_pq16): both are the same for the
-    // whole wavefront and move on by four blocks with adds and compares
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const int step_chunk = 4 / n_pq16, step_pb = 4 - step_chunk * n_pq16;
-    int chunk = wave_u / n_pq16, pb = wave_u - chunk * n_pq16;
-    while (chunk < n_chunks) {
+    const int cq4 = (lane & 3) * 4;
+    const int adv_chunk = 64 / npq, adv_pq = 64 - adv_chunk * npq;
+    int pair = wave * 16 + (lane >> 2);
+    int chunk = pair / npq, pq = pair - chunk * npq;
+    for (int first = 0; first < n_pairs; first += 64 * kRowBatch) {   // the same count for every lane
         uint32_t in[kRowBatch][4];
-        int at[kRowBatch];   // byte offset of the block's first word in the slab, or -1: nothing to store
+        int at[kRowBatch];   // byte offset of the pair's first word in the slab, or -1: nothing to store
 #pragma unroll
         for (int u = 0; u < kRowBatch; u++) {
-            const int pq = pb * 16 + (lane >> 2);
+            at[u] = -1;
+            if (first + 64 * u >= n_pairs) continue;   // a step with no pair at all asks for nothing
             const int gpos = base + 4 * pq;
-            const bool live = chunk < n_chunks && pq < npq;
+            const bool live = pair < n_pairs;
             const bool inside = live && gpos >= 0 && gpos < p.W;
-            const uint8_t *src = x_img + (size_t)(min(chunk, n_chunks - 1) * 16 + (lane & 3) * 4) * p.W + (inside ? gpos : 0);
+            const uint8_t *src = x_img + (size_t)(min(chunk, n_chunks - 1) * 16 + cq4) * p.W + (inside ? gpos : 0);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const uint32_t v = *reinterpret_cast<const uint32_t *>(src + (size_t)i * p.W);
                 in[u][i] = inside ? v ^ flip4 : pad_word;
             }
-            at[u] = live ? (chunk * SP + 4 * pq) * 16 + (lane & 3) * 4 : -1;
-            pb += step_pb, chunk += step_chunk;
-            if (pb >= n_pq16) pb -= n_pq16, chunk++;
+            at[u] = live ? (chunk * SP + 4 * pq) * 16 + cq4 : -1;
+            pair += 64;
+            pq += adv_pq, chunk += adv_chunk;
+            if (pq >= npq) pq -= npq, chunk++;
         }
 #pragma unroll
         for (int u = 0; u < kRowBatch; u++) {
