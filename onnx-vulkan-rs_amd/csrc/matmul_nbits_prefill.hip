@@ -177,10 +177,7 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
 #pragma unroll
             for (int j = 0; j < kF; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    total[i][j][r] = fmaf(raw[i][j][r], s[j], total[i][j][r]);
-                    raw[i][j][r] = 0.f;
-                }
+                for (int r = 0; r < 16; r++) total[i][j][r] = fmaf(raw[i][j][r], s[j], total[i][j][r]);
     };
 
     // One stage = four k steps of 16. `half` is the stage's parity inside its 128-k weight tile;
@@ -197,7 +194,12 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
             else if (half == 1) s1[j] = scale_of(j, cg, 0);
         }
     };
+    // the first product of a quantisation block starts from zero instead of from a cleared register
+    f32x16 zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.f;
     auto compute = [&](int buf, int half) {
+        auto opens_block = [&](int step) { return SG == 4 ? (step & 1) == 0 : SG == 2 ? step == 0 : step == 0 && half == 0; };
         const uint8_t *ba = lds_a + buf * T * kPPitch + (wm * kWT + r32) * kPPitch + kg * 16;
         const uint8_t *bw = lds_w + buf * T * kPPitch + (wn * kWT + r32) * kPPitch + kg * 16;
 #pragma unroll
@@ -211,7 +213,7 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
             for (int i = 0; i < kF; i++)
 #pragma unroll
                 for (int j = 0; j < kF; j++)
-                    raw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], raw[i][j], 0, 0, 0);
+                    raw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], opens_block(step) ? zero : raw[i][j], 0, 0, 0);
             if (SG == 4 && step == 1) fold(s0);
             if (step == 3 && (SG != 1 || half == 1)) fold(s1);
         }
