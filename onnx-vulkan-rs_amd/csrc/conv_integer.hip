@@ -13,6 +13,10 @@
 // match. Padding taps read the zero point, so they contribute nothing and the
 // zero-point algebra of the plain matmul applies unchanged
 // (shaders/conv_integer.rs:112-119, 350-371).
+// A window along one axis (H = 1, 1 x kw: the vocoder shapes) skips even that
+// copy: each workgroup reads the input positions its 64 outputs see straight
+// from NCHW, transposes them in registers and keeps them in LDS for the whole
+// product (int8_conv_row_kernel).
 // Grouped convolutions and channel counts that are not multiples of 16 take a
 // direct kernel, one output per thread, as the reference does for grouped ones.
 #include <algorithm>
