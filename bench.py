@@ -457,7 +457,7 @@ def main():
         "metric": "int4 MatMulNBits HBM GB/s (% peak); int8 GEMM TOPS (% MFMA); tok/s",
         "value": head["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int4 weights x f32 activations (bf16x3 MFMA, f32 accumulate)", "data": "synthetic",
+        "dtype": "int4 weights x f32 activations (each activation as two bf16 terms on the MFMA, f32 accumulate)", "data": "synthetic",
         "config": {"workload": "int4 MatMulNBits decode GEMVs of one gemma3-1b-shaped token: 26 layers x "
                                "(q|k|v fused, o, gate|up fused, down) + lm_head 1152->262144, block 32 + zero points, "
                                "M=1, every weight distinct and HBM-resident, graph replay",
