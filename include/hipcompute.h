@@ -16,7 +16,14 @@
  *     crates/vk-compute/src/pipeline.rs:12-21) in the ONNX layout of the operator;
  *   - operator calls only ENQUEUE on the context's stream, in call order; the
  *     host blocks only in `hipc_flush` and `hipc_download`
- *     (crates/vk-compute/src/stream.rs:8-28, 370-383, 702);
+ *     (crates/vk-compute/src/stream.rs:8-28, 370-383, 702). `hipc_upload` copies the
+ *     bytes into a pinned staging ring and records the transfer; it waits (for the
+ *     ring's oldest slot, not for the stream) only while more than the ring's 16 MiB
+ *     are in flight;
+ *   - memory the library itself retires while recorded graphs exist (a scratch block
+ *     that had to grow, requantisation ratios that changed, a replaced decoder weight)
+ *     stays allocated until the context's last graph is destroyed, so replaying an
+ *     older graph never touches freed memory and keeps the scales it was recorded with;
  *   - zero points of the integer operators are read ON THE DEVICE, never read
  *     back (crates/onnx-vulkan-core/src/shaders/matmul_integer.rs:55-56);
  *   - a context may be used from any thread; calls are serialised inside
@@ -64,15 +71,28 @@ const char *hipc_last_error(hipc_ctx *ctx);
 const char *hipc_version(void);
 /* the `hipStream_t` operators are enqueued on */
 void *hipc_stream(hipc_ctx *ctx);
+/* Route and launch-shape overrides, for experiments and for tests that must reach every kernel
+ * (the reference keeps the same kind of switch in its tactic keys, crates/onnx-vulkan-core/src/tuning.rs).
+ * `name` is one of HIPC_GEMV_T, HIPC_GEMV_WAVES, HIPC_GEMV_PER_CU, HIPC_GEMM_TILE, HIPC_GEMM_BIG,
+ * HIPC_GEMM_SMALL, HIPC_GEMM_SPLITK, HIPC_CONV_ROW, HIPC_PREFILL_TILE, HIPC_PREFILL_SPLIT,
+ * HIPC_DEC_FUSED_GLUE, HIPC_DEC_FUSED_ATTN, HIPC_DEC_PERSISTENT; a context starts from the environment
+ * variables of the same names; value < 0 returns the choice to the library. */
+int hipc_set_option(hipc_ctx *ctx, const char *name, int value);
 
 /* ------------------------------------------------------------------ buffers */
 
-/* `create_storage_buffer` (crates/vk-compute/src/buffer.rs:239). 256-byte aligned. */
+/* `create_storage_buffer` + `take_scratch_buffer` (crates/vk-compute/src/buffer.rs:239, 303-341).
+ * 256-byte aligned. Requests are served by size class (a power of two up to 1 MiB, whole MiB above)
+ * from the blocks earlier frees left behind; only a class with no free block allocates. */
 int hipc_alloc(hipc_ctx *ctx, size_t bytes, void **dptr);
-/* `defer_destroy` (crates/vk-compute/src/stream.rs:691): the memory stays valid for
- * everything already enqueued and is released at the next flush. */
+/* `defer_destroy` + `recycle_*` (crates/vk-compute/src/stream.rs:691, buffer.rs:303-341): the memory
+ * stays valid for everything already enqueued; at the next flush it returns to its size class's
+ * free list (up to 1 GiB waiting in all), or to the device. */
 int hipc_free_deferred(hipc_ctx *ctx, void *dptr);
-/* `stream_upload_at` (stream.rs:310-321): `host` may be reused when the call returns. */
+/* pool counters (the reference's alloc / pool-hit counters, crates/vk-compute/src/stats.rs:302-312);
+ * any pointer may be NULL */
+int hipc_pool_stats(hipc_ctx *ctx, size_t *hits, size_t *misses, size_t *bytes_waiting);
+/* `stream_upload_at` (stream.rs:310-321): records only; `host` may be reused when the call returns. */
 int hipc_upload(hipc_ctx *ctx, void *dst, size_t dst_offset, const void *host, size_t bytes);
 /* `stream_download` (stream.rs:773-918): flushes, then copies to `host`. */
 int hipc_download(hipc_ctx *ctx, void *host, const void *src, size_t src_offset, size_t bytes);
@@ -86,10 +106,12 @@ int hipc_flush(hipc_ctx *ctx);
 
 /* ------------------------------------------------------- capture and replay */
 
-/* `begin_capture` / `end_capture` / `replay` (crates/vk-compute/src/stream.rs:537-572):
- * everything enqueued between begin and end is recorded instead of run, and
- * `hipc_graph_launch` re-issues it. Buffers named while recording must stay alive
- * and keep their addresses (the reference's preconditions, crates/onnx-vulkan-core/src/plan.rs:21-29). */
+/* `begin_capture` / `end_capture` / `replay` (crates/vk-compute/src/capture.rs:29-126,
+ * crates/vk-compute/src/stream.rs:537-572): everything enqueued between begin and end is recorded
+ * instead of run, and `hipc_graph_launch` re-issues it. Buffers and weight handles the CALLER named
+ * while recording must stay alive and keep their addresses until the graph is destroyed (the
+ * reference's preconditions, crates/onnx-vulkan-core/src/plan.rs:21-29); the library's own
+ * temporaries are kept alive for it (see the conventions above). */
 int hipc_capture_begin(hipc_ctx *ctx);
 int hipc_capture_end(hipc_ctx *ctx, hipc_graph **out);
 int hipc_graph_launch(hipc_ctx *ctx, hipc_graph *graph);
@@ -303,6 +325,11 @@ int hipc_qlinear_conv(hipc_ctx *ctx, const void *X, int x_dtype, float x_scale, 
  * followed by logits = rmsnorm(x, w_final) W_lm_head and token = argmax(logits).
  * The current token and position live in device memory and are advanced by the step itself,
  * so a captured graph of one step replays without patching.
+ * Limits kept on the device: the cache holds `max_seq` positions, so at most `max_seq` steps can
+ * follow a reset to position 0. A step enqueued (or replayed) with the cache full writes nothing,
+ * leaves token and position as they are and raises a sticky flag that `hipc_decoder_read` reports
+ * as HIPC_ERR_INVALID until the next `hipc_decoder_reset`. The chosen token is always inside
+ * [0, vocab): if no logit compares (all NaN) it is 0, ArgMax's answer for such a row.
  */
 typedef struct hipc_decoder hipc_decoder;
 typedef struct {
@@ -352,7 +379,8 @@ int hipc_decoder_kv_cache(hipc_ctx *ctx, hipc_decoder *dec, int layer, void **k_
 /* enqueue one decode step (capturable) */
 int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *dec);
 /* flush, then read the state: next token, next position, the last step's logits [vocab] (or NULL),
- * and the tokens chosen at positions 0..n_history-1 (or NULL) */
+ * and the tokens chosen at positions 0..n_history-1 (or NULL). Returns HIPC_ERR_INVALID (outputs
+ * still filled) when a step was enqueued with the cache full. */
 int hipc_decoder_read(hipc_ctx *ctx, hipc_decoder *dec, int32_t *token, int32_t *pos, float *logits,
                       int32_t *history, int32_t n_history);
 

@@ -245,11 +245,8 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
         ga.out_signed = ep.out_signed;
         HIPC_REQUIRE(ctx, g->n <= 65535, "Conv: batch %ld too large", (long)g->n);
         // few 64x64 tiles and a long k: the wavefronts of a workgroup split k and the weight stays out of LDS
-        // (HIPC_GEMM_SMALL=0/1 overrides: tuning, tests)
-        static const int forced = [] {
-            const char *e = getenv("HIPC_GEMM_SMALL");
-            return e ? atoi(e) : -1;
-        }();
+        // (the gemm_small option, 0 / 1, overrides: tuning, tests)
+        const int forced = ctx->tune.gemm_small;
         const int64_t tiles64 = ceil_div(ga.I, 64) * ceil_div(ga.J, 64) * g->n;
         const bool small = forced >= 0 ? forced != 0 : (tiles64 <= 2 * (int64_t)ctx->cu_count && ga.K_pad >= 4 * kBK);
         // the row sums of the activations only matter when the weight's zero point, in the signed domain, is not zero
@@ -258,11 +255,8 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
         // A convolution along W alone whose per-tile input slab fits LDS reads the NCHW activation
         // directly: no transposed copy at all, whatever the number of tiles (on 8 x 512 x 4096 inputs,
         // k = 7, it still finishes before the tiled route: 120 against 147 us).
-        // HIPC_CONV_ROW=0 takes the general route (tuning, tests).
-        static const bool row_off = [] {
-            const char *e = getenv("HIPC_CONV_ROW");
-            return e && atoi(e) == 0;
-        }();
+        // The conv_row option set to 0 takes the general route (tuning, tests).
+        const bool row_off = ctx->tune.conv_row == 0;
         const int64_t slab_pos = (3 + 63 * g->stride_w + (g->kw - 1) * g->dil_w + 1 + 3) / 4 * 4;
         const size_t slab_bytes = (size_t)(slab_pos * g->c_in);
         if (!row_off && g->h == 1 && g->kh == 1 && ho == 1 && g->pad_top == 0 && g->w % 4 == 0 && aligned(X, 4) &&
@@ -355,92 +349,94 @@ void hipc_same_pads(int64_t in, int64_t kernel, int64_t stride, int64_t dilation
 }
 
 int hipc_prepack_conv_w(hipc_ctx *ctx, const void *W, int w_dtype, const hipc_conv_geom *g, hipc_conv_weight **out) {
-    if (!ctx || !out) return HIPC_ERR_INVALID;
-    Guard gd(ctx);
-    *out = nullptr;
-    HIPC_REFUSE(ctx, ctx->capturing, "Conv prepack while a capture is open");
-    HIPC_REFUSE(ctx, !is_byte_dtype(w_dtype), "Conv: W must be uint8 or int8, got %d", w_dtype);
-    HIPC_REQUIRE(ctx, W && g, "Conv prepack: null argument");
-    HIPC_REQUIRE(ctx, g->c_in > 0 && g->c_out > 0 && g->kh > 0 && g->kw > 0 && g->group > 0 && g->c_in % g->group == 0 &&
-                          g->c_out % g->group == 0 && g->c_in * g->kh * g->kw < (int64_t(1) << 30),
-                 "Conv prepack: bad weight shape");
-    hipc_conv_weight *w = new hipc_conv_weight();
-    w->geom = *g;
-    w->w_dtype = w_dtype;
-    const size_t raw_bytes = (size_t)(g->c_out * (g->c_in / g->group) * g->kh * g->kw);
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->raw), raw_bytes);
-    if (e == hipSuccess)
-        e = hipMemcpyAsync(w->raw, W, raw_bytes, hipMemcpyDeviceToDevice, ctx->stream);
-    const bool mfma = g->group == 1 && g->c_in % 16 == 0;
-    if (e == hipSuccess && mfma) {
-        w->O_pad = (int)(ceil_div(g->c_out, kBM) * kBM);
-        w->K_pad = (int)(ceil_div(g->c_in * g->kh * g->kw, kBK) * kBK);
-        e = hipMalloc(reinterpret_cast<void **>(&w->Wp), (size_t)w->O_pad * w->K_pad);
-        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&w->rowsum), (size_t)w->O_pad * 4);
-        if (e == hipSuccess) {
-            pack_conv_w_kernel<<<dim3((unsigned)w->O_pad), 256, 0, ctx->stream>>>(
-                static_cast<const uint8_t *>(W), w->Wp, w->rowsum, (int)g->c_out, (int)g->c_in, (int)g->kh, (int)g->kw,
-                w->O_pad, w->K_pad, w_dtype == HIPC_I8, w_dtype == HIPC_U8 ? 128 : 0);
-            e = hipGetLastError();
+    if (!out) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        *out = nullptr;
+        HIPC_REFUSE(ctx, ctx->capturing, "Conv prepack while a capture is open");
+        HIPC_REFUSE(ctx, !is_byte_dtype(w_dtype), "Conv: W must be uint8 or int8, got %d", w_dtype);
+        HIPC_REQUIRE(ctx, W && g, "Conv prepack: null argument");
+        HIPC_REQUIRE(ctx, g->c_in > 0 && g->c_out > 0 && g->kh > 0 && g->kw > 0 && g->group > 0 && g->c_in % g->group == 0 &&
+                              g->c_out % g->group == 0 && g->c_in * g->kh * g->kw < (int64_t(1) << 30),
+                     "Conv prepack: bad weight shape");
+        hipc_conv_weight *w = new hipc_conv_weight();
+        w->geom = *g;
+        w->w_dtype = w_dtype;
+        const size_t raw_bytes = (size_t)(g->c_out * (g->c_in / g->group) * g->kh * g->kw);
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->raw), raw_bytes);
+        if (e == hipSuccess)
+            e = hipMemcpyAsync(w->raw, W, raw_bytes, hipMemcpyDeviceToDevice, ctx->stream);
+        const bool mfma = g->group == 1 && g->c_in % 16 == 0;
+        if (e == hipSuccess && mfma) {
+            w->O_pad = (int)(ceil_div(g->c_out, kBM) * kBM);
+            w->K_pad = (int)(ceil_div(g->c_in * g->kh * g->kw, kBK) * kBK);
+            e = hipMalloc(reinterpret_cast<void **>(&w->Wp), (size_t)w->O_pad * w->K_pad);
+            if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&w->rowsum), (size_t)w->O_pad * 4);
+            if (e == hipSuccess) {
+                pack_conv_w_kernel<<<dim3((unsigned)w->O_pad), 256, 0, ctx->stream>>>(
+                    static_cast<const uint8_t *>(W), w->Wp, w->rowsum, (int)g->c_out, (int)g->c_in, (int)g->kh, (int)g->kw,
+                    w->O_pad, w->K_pad, w_dtype == HIPC_I8, w_dtype == HIPC_U8 ? 128 : 0);
+                e = hipGetLastError();
+            }
         }
-    }
-    if (e != hipSuccess) {
-        if (w->raw) (void)hipFree(w->raw);
-        if (w->Wp) (void)hipFree(w->Wp);
-        if (w->rowsum) (void)hipFree(w->rowsum);
-        delete w;
-        return fail(ctx, HIPC_ERR_BACKEND, "Conv prepack: %s", hipGetErrorString(e));
-    }
-    *out = w;
-    return HIPC_OK;
+        if (e != hipSuccess) {
+            if (w->raw) (void)hipFree(w->raw);
+            if (w->Wp) (void)hipFree(w->Wp);
+            if (w->rowsum) (void)hipFree(w->rowsum);
+            delete w;
+            return fail(ctx, HIPC_ERR_BACKEND, "Conv prepack: %s", hipGetErrorString(e));
+        }
+        *out = w;
+        return HIPC_OK;
+    });
 }
 
 void hipc_conv_weight_destroy(hipc_ctx *ctx, hipc_conv_weight *w) {
-    if (!ctx || !w) return;
-    Guard g(ctx);
-    if (w->raw) ctx->deferred.push_back(w->raw);
-    if (w->Wp) ctx->deferred.push_back(w->Wp);
-    if (w->rowsum) ctx->deferred.push_back(w->rowsum);
-    ratio_release(ctx, w->ratios);
-    delete w;
+    if (!w) return;
+    entry_void(ctx, [&] {
+        if (w->raw) ctx->deferred.push_back(w->raw);
+        if (w->Wp) ctx->deferred.push_back(w->Wp);
+        if (w->rowsum) ctx->deferred.push_back(w->rowsum);
+        ratio_release(ctx, w->ratios);
+        delete w;
+    });
 }
 
 int hipc_conv_integer(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *W, const void *x_zp,
                       const void *w_zp, const hipc_conv_geom *g, void *Y) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard gd(ctx);
-    return run_conv(ctx, X, x_dtype, W, x_zp, w_zp, 0, 0, 0, g, Y, ConvEpilogue{});
+    return entry(ctx, [&]() -> int {
+        return run_conv(ctx, X, x_dtype, W, x_zp, w_zp, 0, 0, 0, g, Y, ConvEpilogue{});
+    });
 }
 
 int hipc_qlinear_conv(hipc_ctx *ctx, const void *X, int x_dtype, float x_scale, int32_t x_zp, const hipc_conv_weight *W,
                       const float *w_scale, int64_t n_w_scale, int32_t w_zp, float y_scale, int32_t y_zp, int y_dtype,
                       const void *bias, const hipc_conv_geom *g, void *Y) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard gd(ctx);
-    HIPC_REQUIRE(ctx, g && w_scale, "QLinearConv: null geometry or scale");
-    HIPC_REFUSE(ctx, !is_byte_dtype(y_dtype), "QLinearConv: output must be uint8 or int8, got %d", y_dtype);
-    // the accepted envelope of `unsupported_quantization` (interp.rs:781-847)
-    HIPC_REQUIRE(ctx, n_w_scale == 1 || n_w_scale == g->c_out, "QLinearConv: %ld weight scales for %ld channels",
-                 (long)n_w_scale, (long)g->c_out);
-    HIPC_REFUSE(ctx, n_w_scale > 1 && w_zp != 0, "QLinearConv: w per-channel zero point is not zero (asymmetric weights)");
-    HIPC_REQUIRE(ctx, y_scale != 0.f, "QLinear: y_scale is zero");
-    HIPC_REQUIRE(ctx, W, "QLinearConv: null weight");
-    // ratio[c] = x_scale * w_scale[c] / y_scale (interp.rs:4693); a per-tensor scale is
-    // broadcast to c_out so the bias stays per channel (interp.rs:4815-4823)
-    std::vector<float> ratio((size_t)g->c_out);
-    for (int64_t c = 0; c < g->c_out; c++) {
-        volatile float t = x_scale * w_scale[n_w_scale == 1 ? 0 : c];
-        ratio[(size_t)c] = t / y_scale;
-    }
-    const float *dratio = nullptr;
-    int rc = ratio_resident(ctx, W->ratios, ratio, &dratio);
-    if (rc != HIPC_OK) return rc;
-    ConvEpilogue ep;
-    ep.requant = 1;
-    ep.ratio = dratio, ep.ratio_step = 1;
-    ep.qbias = static_cast<const int32_t *>(bias);
-    ep.y_zp = y_zp, ep.out_signed = y_dtype == HIPC_I8;
-    return run_conv(ctx, X, x_dtype, W, nullptr, nullptr, 1, x_zp, w_zp, g, Y, ep);
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, g && w_scale, "QLinearConv: null geometry or scale");
+        HIPC_REFUSE(ctx, !is_byte_dtype(y_dtype), "QLinearConv: output must be uint8 or int8, got %d", y_dtype);
+        // the accepted envelope of `unsupported_quantization` (interp.rs:781-847)
+        HIPC_REQUIRE(ctx, n_w_scale == 1 || n_w_scale == g->c_out, "QLinearConv: %ld weight scales for %ld channels",
+                     (long)n_w_scale, (long)g->c_out);
+        HIPC_REFUSE(ctx, n_w_scale > 1 && w_zp != 0, "QLinearConv: w per-channel zero point is not zero (asymmetric weights)");
+        HIPC_REQUIRE(ctx, y_scale != 0.f, "QLinear: y_scale is zero");
+        HIPC_REQUIRE(ctx, W, "QLinearConv: null weight");
+        // ratio[c] = x_scale * w_scale[c] / y_scale (interp.rs:4693); a per-tensor scale is
+        // broadcast to c_out so the bias stays per channel (interp.rs:4815-4823)
+        std::vector<float> ratio((size_t)g->c_out);
+        for (int64_t c = 0; c < g->c_out; c++) {
+            volatile float t = x_scale * w_scale[n_w_scale == 1 ? 0 : c];
+            ratio[(size_t)c] = t / y_scale;
+        }
+        const float *dratio = nullptr;
+        int rc = ratio_resident(ctx, W->ratios, ratio, &dratio);
+        if (rc != HIPC_OK) return rc;
+        ConvEpilogue ep;
+        ep.requant = 1;
+        ep.ratio = dratio, ep.ratio_step = 1;
+        ep.qbias = static_cast<const int32_t *>(bias);
+        ep.y_zp = y_zp, ep.out_signed = y_dtype == HIPC_I8;
+        return run_conv(ctx, X, x_dtype, W, nullptr, nullptr, 1, x_zp, w_zp, g, Y, ep);
+    });
 }
 
 }  // extern "C"

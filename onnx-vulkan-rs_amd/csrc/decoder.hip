@@ -28,9 +28,10 @@ namespace hipc {
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-struct DecState {   // device-resident loop state
-    int32_t token;  // the token the next step consumes
-    int32_t pos;    // its position = number of tokens already in the cache
+struct DecState {      // device-resident loop state
+    int32_t token;     // the token the next step consumes
+    int32_t pos;       // its position = number of tokens already in the cache
+    int32_t overflow;  // sticky: a step was asked for with the cache full (pos == max_seq); that step did nothing
 };
 
 __device__ __forceinline__ float block_sum(float v, float *red) {
@@ -120,6 +121,7 @@ dec_qkv_kernel(const DecState *st, const float *__restrict__ qkv, const float *_
     __shared__ float buf[512];
     const int head = blockIdx.x;
     const int pos = st->pos;
+    if (pos >= max_seq) return;  // the cache is full: the step is a no-op (dec_argmax_final_kernel reports it)
     const float *src = qkv + (size_t)head * hd;
     const bool is_q = head < n_q, is_k = !is_q && head < n_q + n_kv;
     if (!is_q && !is_k) {  // a value head: straight into the cache
@@ -163,6 +165,7 @@ dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const _
     __shared__ float sc[kMaxGroup][kAttnChunk];
     const int split = blockIdx.x, kvh = blockIdx.y, nsplit = gridDim.x;
     const int G = n_q / n_kv;
+    if (st->pos >= max_seq) return;  // the cache is full: the step is a no-op
     const int total = st->pos + 1;  // the step's own key is already in the cache
     const int t0 = split * kAttnChunk;
     const int tid = threadIdx.x;
@@ -337,6 +340,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int pos = st->pos, total = pos + 1;
+    if (pos >= max_seq) return;  // the cache is full: the step is a no-op
     const int t_first = attn_first(total, window);  // a local layer sees the last `window` positions only
     const int chunk = attn_chunk(total - t_first);
     const int t_begin = t_first + split * chunk;
@@ -621,9 +625,12 @@ dec_argmax_partial_kernel(const float *__restrict__ logits, int n, float *__rest
     }
 }
 
+// The state only ever holds a token inside the vocabulary and a position inside the cache: a
+// candidate outside [0, vocab) (every logit NaN: no comparison succeeds) becomes token 0, and a step
+// taken with the cache full (pos == max_seq) changes nothing and raises the sticky overflow flag.
 __global__ void __launch_bounds__(64)
 dec_argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int nparts, DecState *st,
-                        int32_t *__restrict__ history, int max_hist) {
+                        int32_t *__restrict__ history, int max_hist, int vocab) {
     float best = -3.4e38f;
     int bi = 0x7fffffff;
     for (int i = threadIdx.x; i < nparts; i += 64) {
@@ -637,14 +644,19 @@ dec_argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi
     }
     if (threadIdx.x == 0) {
         const int pos = st->pos;
-        if (pos < max_hist) history[pos] = bi;
-        st->token = bi;
-        st->pos = pos + 1;
+        if (pos >= max_hist) {
+            st->overflow = 1;
+        } else {
+            if (bi < 0 || bi >= vocab) bi = 0;
+            history[pos] = bi;
+            st->token = bi;
+            st->pos = pos + 1;
+        }
     }
 }
 
 __global__ void dec_set_state_kernel(DecState *st, int token, int pos) {
-    if (threadIdx.x == 0) st->token = token, st->pos = pos;
+    if (threadIdx.x == 0) st->token = token, st->pos = pos, st->overflow = 0;
 }
 
 }  // namespace hipc
@@ -735,282 +747,293 @@ bool complete(const hipc_decoder *d) {
 extern "C" {
 
 int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_decoder **out) {
-    if (!ctx || !cfg || !out) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    *out = nullptr;
-    HIPC_REFUSE(ctx, ctx->capturing, "decoder create while a capture is open");
-    const hipc_decoder_config &c = *cfg;
-    HIPC_REQUIRE(ctx, c.n_layers > 0 && c.hidden > 0 && c.ffn > 0 && c.n_q_heads > 0 && c.n_kv_heads > 0 && c.head_dim > 0 &&
-                          c.vocab > 0 && c.max_seq > 0, "decoder: non-positive dimension");
-    HIPC_REQUIRE(ctx, c.n_q_heads % c.n_kv_heads == 0 && c.n_q_heads / c.n_kv_heads <= kMaxGroup,
-                 "decoder: %d query heads over %d kv heads (at most %d per group)", c.n_q_heads, c.n_kv_heads, kMaxGroup);
-    HIPC_REQUIRE(ctx, c.head_dim % 64 == 0 && c.head_dim <= 512, "decoder: head_dim %d must be a multiple of 64, at most 512", c.head_dim);
-    HIPC_REQUIRE(ctx, is_pow2(c.block_size) && c.block_size >= 32, "decoder: block_size %d", c.block_size);
-    HIPC_REQUIRE(ctx, c.hidden <= 256 * kNormPer, "decoder: hidden %d exceeds %d", c.hidden, 256 * kNormPer);
-    HIPC_REQUIRE(ctx, c.max_seq <= 8192 * kAttnChunk, "decoder: max_seq %d exceeds %d", c.max_seq, 8192 * kAttnChunk);
-    hipc_decoder *d = new hipc_decoder();
-    d->cfg = c;
-    d->layers.resize(c.n_layers);
-    d->nsplit = (int)ceil_div(c.max_seq, kAttnChunk);
-    const size_t kv = (size_t)c.n_kv_heads * c.max_seq * c.head_dim;
-    const int G = c.n_q_heads / c.n_kv_heads;
-    int rc = HIPC_OK;
-    auto A = [&](auto **p, size_t n) { if (rc == HIPC_OK) rc = dev_alloc(ctx, d, p, n); };
-    for (DecLayer &l : d->layers) {
-        A(&l.k_cache, kv);
-        A(&l.v_cache, kv);
-    }
-    A(&d->state, 1), A(&d->history, (size_t)c.max_seq);
-    A(&d->x, c.hidden), A(&d->xn, c.hidden), A(&d->qkv, (size_t)(c.n_q_heads + 2 * c.n_kv_heads) * c.head_dim);
-    A(&d->q, (size_t)c.n_q_heads * c.head_dim), A(&d->attn, (size_t)c.n_q_heads * c.head_dim), A(&d->y, c.hidden);
-    A(&d->gu, (size_t)2 * c.ffn), A(&d->h, c.ffn), A(&d->logits, c.vocab);
-    const size_t parts = (size_t)c.n_kv_heads * std::max(d->nsplit, kAttnSplits) * G;
-    A(&d->part_ml, parts * 2), A(&d->part_o, parts * c.head_dim);
-    A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
-    A(&d->rope, (size_t)2 * c.head_dim), A(&d->x2, c.hidden);
-    {
-        const char *e = getenv("HIPC_DEC_FUSED_GLUE");  // 0: keep the separate norm / GELU kernels (tests of that path)
-        d->fused_glue = c.hidden % 8 == 0 && c.ffn % 8 == 0 && !(e && atoi(e) == 0);
-    }
-    {
-        const char *e = getenv("HIPC_DEC_FUSED_ATTN");  // 0: keep the three-kernel attention (tests of that path)
-        d->one_launch_attn = (c.head_dim == 64 || c.head_dim == 128 || c.head_dim == 256) && (G == 1 || G == 2 || G == 4 || G == 8) &&
-                             !(e && atoi(e) == 0);
-    }
-    if (rc == HIPC_OK) {
-        for (DecLayer &l : d->layers) {  // an unwritten cache row must not hold NaN bit patterns
-            if (hipMemsetAsync(l.k_cache, 0, kv * 2, ctx->stream) != hipSuccess || hipMemsetAsync(l.v_cache, 0, kv * 2, ctx->stream) != hipSuccess)
-                rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the KV cache");
+    if (!cfg || !out) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        *out = nullptr;
+        HIPC_REFUSE(ctx, ctx->capturing, "decoder create while a capture is open");
+        const hipc_decoder_config &c = *cfg;
+        HIPC_REQUIRE(ctx, c.n_layers > 0 && c.hidden > 0 && c.ffn > 0 && c.n_q_heads > 0 && c.n_kv_heads > 0 && c.head_dim > 0 &&
+                              c.vocab > 0 && c.max_seq > 0, "decoder: non-positive dimension");
+        HIPC_REQUIRE(ctx, c.n_q_heads % c.n_kv_heads == 0 && c.n_q_heads / c.n_kv_heads <= kMaxGroup,
+                     "decoder: %d query heads over %d kv heads (at most %d per group)", c.n_q_heads, c.n_kv_heads, kMaxGroup);
+        HIPC_REQUIRE(ctx, c.head_dim % 64 == 0 && c.head_dim <= 512, "decoder: head_dim %d must be a multiple of 64, at most 512", c.head_dim);
+        HIPC_REQUIRE(ctx, is_pow2(c.block_size) && c.block_size >= 32, "decoder: block_size %d", c.block_size);
+        HIPC_REQUIRE(ctx, c.hidden <= 256 * kNormPer, "decoder: hidden %d exceeds %d", c.hidden, 256 * kNormPer);
+        HIPC_REQUIRE(ctx, c.max_seq <= 8192 * kAttnChunk, "decoder: max_seq %d exceeds %d", c.max_seq, 8192 * kAttnChunk);
+        hipc_decoder *d = new hipc_decoder();
+        d->cfg = c;
+        d->layers.resize(c.n_layers);
+        d->nsplit = (int)ceil_div(c.max_seq, kAttnChunk);
+        const size_t kv = (size_t)c.n_kv_heads * c.max_seq * c.head_dim;
+        const int G = c.n_q_heads / c.n_kv_heads;
+        int rc = HIPC_OK;
+        auto A = [&](auto **p, size_t n) { if (rc == HIPC_OK) rc = dev_alloc(ctx, d, p, n); };
+        for (DecLayer &l : d->layers) {
+            A(&l.k_cache, kv);
+            A(&l.v_cache, kv);
         }
-        dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, 0, 0);
-    }
-    if (rc != HIPC_OK) {
-        for (void *p : d->owned) (void)hipFree(p);
-        delete d;
-        return rc;
-    }
-    *out = d;
-    return HIPC_OK;
+        A(&d->state, 1), A(&d->history, (size_t)c.max_seq);
+        A(&d->x, c.hidden), A(&d->xn, c.hidden), A(&d->qkv, (size_t)(c.n_q_heads + 2 * c.n_kv_heads) * c.head_dim);
+        A(&d->q, (size_t)c.n_q_heads * c.head_dim), A(&d->attn, (size_t)c.n_q_heads * c.head_dim), A(&d->y, c.hidden);
+        A(&d->gu, (size_t)2 * c.ffn), A(&d->h, c.ffn), A(&d->logits, c.vocab);
+        const size_t parts = (size_t)c.n_kv_heads * std::max(d->nsplit, kAttnSplits) * G;
+        A(&d->part_ml, parts * 2), A(&d->part_o, parts * c.head_dim);
+        A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
+        A(&d->rope, (size_t)2 * c.head_dim), A(&d->x2, c.hidden);
+        // options read when the decoder is created: dec_fused_glue = 0 keeps the separate norm / GELU
+        // kernels, dec_fused_attn = 0 the three-kernel attention (tests of those paths)
+        d->fused_glue = c.hidden % 8 == 0 && c.ffn % 8 == 0 && ctx->tune.dec_fused_glue != 0;
+        d->one_launch_attn = (c.head_dim == 64 || c.head_dim == 128 || c.head_dim == 256) && (G == 1 || G == 2 || G == 4 || G == 8) &&
+                             ctx->tune.dec_fused_attn != 0;
+        if (rc == HIPC_OK) {
+            for (DecLayer &l : d->layers) {  // an unwritten cache row must not hold NaN bit patterns
+                if (hipMemsetAsync(l.k_cache, 0, kv * 2, ctx->stream) != hipSuccess || hipMemsetAsync(l.v_cache, 0, kv * 2, ctx->stream) != hipSuccess)
+                    rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the KV cache");
+            }
+            dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, 0, 0);
+        }
+        if (rc != HIPC_OK) {
+            for (void *p : d->owned) (void)hipFree(p);
+            delete d;
+            return rc;
+        }
+        *out = d;
+        return HIPC_OK;
+    });
 }
 
 void hipc_decoder_destroy(hipc_ctx *ctx, hipc_decoder *d) {
-    if (!ctx || !d) return;
-    Guard g(ctx);
-    for (DecLayer &l : d->layers) {
-        nbits_release(ctx, l.qkv), nbits_release(ctx, l.o), nbits_release(ctx, l.gate_up), nbits_release(ctx, l.down);
-    }
-    nbits_release(ctx, d->lm_head);
-    for (void *p : d->owned) ctx->deferred.push_back(p);
-    delete d;
+    if (!d) return;
+    entry_void(ctx, [&] {
+        for (DecLayer &l : d->layers) {
+            nbits_release(ctx, l.qkv), nbits_release(ctx, l.o), nbits_release(ctx, l.gate_up), nbits_release(ctx, l.down);
+        }
+        nbits_release(ctx, d->lm_head);
+        for (void *p : d->owned) ctx->deferred.push_back(p);
+        delete d;
+    });
 }
 
 int hipc_decoder_set_linear(hipc_ctx *ctx, hipc_decoder *d, int layer, int which, const void *B, size_t b_len,
                             const void *scales, size_t scales_len, const void *zp, size_t zp_len) {
-    if (!ctx || !d) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    const hipc_decoder_config &c = d->cfg;
-    const int64_t qd = (int64_t)c.n_q_heads * c.head_dim, kvd = (int64_t)c.n_kv_heads * c.head_dim;
-    int64_t K = 0, N = 0;
-    hipc_nbits_weight **slot = nullptr;
-    if (which == HIPC_DEC_LM_HEAD) {
-        K = c.hidden, N = c.vocab, slot = &d->lm_head;
-    } else {
-        HIPC_REQUIRE(ctx, layer >= 0 && layer < c.n_layers, "decoder: layer %d out of range", layer);
-        DecLayer &l = d->layers[layer];
-        switch (which) {
-            case HIPC_DEC_QKV: K = c.hidden, N = qd + 2 * kvd, slot = &l.qkv; break;
-            case HIPC_DEC_O: K = qd, N = c.hidden, slot = &l.o; break;
-            case HIPC_DEC_GATE_UP: K = c.hidden, N = 2 * (int64_t)c.ffn, slot = &l.gate_up; break;
-            case HIPC_DEC_DOWN: K = c.ffn, N = c.hidden, slot = &l.down; break;
-            default: return fail(ctx, HIPC_ERR_INVALID, "decoder: unknown linear %d", which);
+    if (!d) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        const hipc_decoder_config &c = d->cfg;
+        const int64_t qd = (int64_t)c.n_q_heads * c.head_dim, kvd = (int64_t)c.n_kv_heads * c.head_dim;
+        int64_t K = 0, N = 0;
+        hipc_nbits_weight **slot = nullptr;
+        if (which == HIPC_DEC_LM_HEAD) {
+            K = c.hidden, N = c.vocab, slot = &d->lm_head;
+        } else {
+            HIPC_REQUIRE(ctx, layer >= 0 && layer < c.n_layers, "decoder: layer %d out of range", layer);
+            DecLayer &l = d->layers[layer];
+            switch (which) {
+                case HIPC_DEC_QKV: K = c.hidden, N = qd + 2 * kvd, slot = &l.qkv; break;
+                case HIPC_DEC_O: K = qd, N = c.hidden, slot = &l.o; break;
+                case HIPC_DEC_GATE_UP: K = c.hidden, N = 2 * (int64_t)c.ffn, slot = &l.gate_up; break;
+                case HIPC_DEC_DOWN: K = c.ffn, N = c.hidden, slot = &l.down; break;
+                default: return fail(ctx, HIPC_ERR_INVALID, "decoder: unknown linear %d", which);
+            }
         }
-    }
-    if (*slot) nbits_release(ctx, *slot), *slot = nullptr;
-    return nbits_prepack(ctx, B, b_len, scales, HIPC_F32, scales_len, zp, zp_len, K, N, c.block_size, slot);
+        if (*slot) {  // a recorded step may still name the old weight: it is retired, not freed
+            retire(ctx, (*slot)->Wq), retire(ctx, (*slot)->Sc), retire(ctx, (*slot)->Zb);
+            delete *slot;
+            *slot = nullptr;
+        }
+        return nbits_prepack(ctx, B, b_len, scales, HIPC_F32, scales_len, zp, zp_len, K, N, c.block_size, slot);
+    });
 }
 
 int hipc_decoder_set_norm(hipc_ctx *ctx, hipc_decoder *d, int layer, int which, const void *w) {
-    if (!ctx || !d || !w) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    const hipc_decoder_config &c = d->cfg;
-    float **slot = nullptr;
-    size_t n = c.hidden;
-    if (which == HIPC_DEC_NORM_FINAL) {
-        slot = &d->final_norm;
-    } else {
-        HIPC_REQUIRE(ctx, layer >= 0 && layer < c.n_layers, "decoder: layer %d out of range", layer);
-        HIPC_REQUIRE(ctx, which >= 0 && which < 6, "decoder: unknown norm %d", which);
-        slot = &d->layers[layer].norm[which];
-        if (which == HIPC_DEC_NORM_Q || which == HIPC_DEC_NORM_K) n = c.head_dim;
-    }
-    if (!*slot) {
-        int rc = dev_alloc(ctx, d, slot, n);
-        if (rc != HIPC_OK) return rc;
-    }
-    HIPC_TRY(ctx, hipMemcpyAsync(*slot, w, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
-    return HIPC_OK;
+    if (!d || !w) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        const hipc_decoder_config &c = d->cfg;
+        float **slot = nullptr;
+        size_t n = c.hidden;
+        if (which == HIPC_DEC_NORM_FINAL) {
+            slot = &d->final_norm;
+        } else {
+            HIPC_REQUIRE(ctx, layer >= 0 && layer < c.n_layers, "decoder: layer %d out of range", layer);
+            HIPC_REQUIRE(ctx, which >= 0 && which < 6, "decoder: unknown norm %d", which);
+            slot = &d->layers[layer].norm[which];
+            if (which == HIPC_DEC_NORM_Q || which == HIPC_DEC_NORM_K) n = c.head_dim;
+        }
+        if (!*slot) {
+            int rc = dev_alloc(ctx, d, slot, n);
+            if (rc != HIPC_OK) return rc;
+        }
+        HIPC_TRY(ctx, hipMemcpyAsync(*slot, w, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        return HIPC_OK;
+    });
 }
 
 int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *d, const void *B, size_t b_len, const void *scales,
                                size_t scales_len, const void *zp, size_t zp_len) {
-    if (!ctx || !d || !B || !scales) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    const hipc_decoder_config &c = d->cfg;
-    const size_t nb = (size_t)ceil_div(c.hidden, c.block_size);
-    const size_t qb = (size_t)c.vocab * nb * c.block_size / 2, sb = (size_t)c.vocab * nb, zb = (size_t)c.vocab * ((nb + 1) / 2);
-    HIPC_REQUIRE(ctx, b_len >= qb && scales_len >= sb && (!zp || zp_len >= zb), "decoder: embedding table is short");
-    if (!d->emb_q) {
-        int rc = dev_alloc(ctx, d, &d->emb_q, qb);
-        if (rc == HIPC_OK) rc = dev_alloc(ctx, d, &d->emb_scales, sb);
-        if (rc == HIPC_OK && zp) rc = dev_alloc(ctx, d, &d->emb_zp, zb);
-        if (rc != HIPC_OK) return rc;
-    }
-    HIPC_TRY(ctx, hipMemcpyAsync(d->emb_q, B, qb, hipMemcpyDeviceToDevice, ctx->stream));
-    HIPC_TRY(ctx, hipMemcpyAsync(d->emb_scales, scales, sb * 4, hipMemcpyDeviceToDevice, ctx->stream));
-    if (zp) HIPC_TRY(ctx, hipMemcpyAsync(d->emb_zp, zp, zb, hipMemcpyDeviceToDevice, ctx->stream));
-    return HIPC_OK;
+    if (!d || !B || !scales) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        const hipc_decoder_config &c = d->cfg;
+        const size_t nb = (size_t)ceil_div(c.hidden, c.block_size);
+        const size_t qb = (size_t)c.vocab * nb * c.block_size / 2, sb = (size_t)c.vocab * nb, zb = (size_t)c.vocab * ((nb + 1) / 2);
+        HIPC_REQUIRE(ctx, b_len >= qb && scales_len >= sb && (!zp || zp_len >= zb), "decoder: embedding table is short");
+        if (!d->emb_q) {
+            int rc = dev_alloc(ctx, d, &d->emb_q, qb);
+            if (rc == HIPC_OK) rc = dev_alloc(ctx, d, &d->emb_scales, sb);
+            if (rc == HIPC_OK && zp) rc = dev_alloc(ctx, d, &d->emb_zp, zb);
+            if (rc != HIPC_OK) return rc;
+        }
+        HIPC_TRY(ctx, hipMemcpyAsync(d->emb_q, B, qb, hipMemcpyDeviceToDevice, ctx->stream));
+        HIPC_TRY(ctx, hipMemcpyAsync(d->emb_scales, scales, sb * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        if (zp) HIPC_TRY(ctx, hipMemcpyAsync(d->emb_zp, zp, zb, hipMemcpyDeviceToDevice, ctx->stream));
+        return HIPC_OK;
+    });
 }
 
 int hipc_decoder_set_layer_attention(hipc_ctx *ctx, hipc_decoder *d, int layer, int32_t window, float rope_theta) {
-    if (!ctx || !d) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REFUSE(ctx, ctx->capturing, "decoder: layer attention changed while a capture is open");
-    HIPC_REQUIRE(ctx, layer >= 0 && layer < d->cfg.n_layers, "decoder: layer %d out of range", layer);
-    HIPC_REQUIRE(ctx, !(rope_theta < 0.f) && rope_theta == rope_theta, "decoder: bad rotary base");
-    DecLayer &l = d->layers[layer];
-    int table = 0;
-    if (rope_theta > 0.f && rope_theta != d->cfg.rope_theta) {
-        HIPC_REQUIRE(ctx, d->theta2 == 0.f || d->theta2 == rope_theta,
-                     "decoder: a third rotary base (%g beside %g and %g)", rope_theta, d->cfg.rope_theta, d->theta2);
-        d->theta2 = rope_theta;
-        table = 1;
-    }
-    l.window = window > 0 ? window : 0;
-    l.rope_table = table;
-    return HIPC_OK;
+    if (!d) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        HIPC_REFUSE(ctx, ctx->capturing, "decoder: layer attention changed while a capture is open");
+        HIPC_REQUIRE(ctx, layer >= 0 && layer < d->cfg.n_layers, "decoder: layer %d out of range", layer);
+        HIPC_REQUIRE(ctx, !(rope_theta < 0.f) && rope_theta == rope_theta, "decoder: bad rotary base");
+        DecLayer &l = d->layers[layer];
+        int table = 0;
+        if (rope_theta > 0.f && rope_theta != d->cfg.rope_theta) {
+            HIPC_REQUIRE(ctx, d->theta2 == 0.f || d->theta2 == rope_theta,
+                         "decoder: a third rotary base (%g beside %g and %g)", rope_theta, d->cfg.rope_theta, d->theta2);
+            d->theta2 = rope_theta;
+            table = 1;
+        }
+        l.window = window > 0 ? window : 0;
+        l.rope_table = table;
+        return HIPC_OK;
+    });
 }
 
 int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *d, int32_t token, int32_t pos) {
-    if (!ctx || !d) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, token >= 0 && token < d->cfg.vocab && pos >= 0 && pos < d->cfg.max_seq, "decoder: bad token %d or position %d", token, pos);
-    dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, token, pos);
-    HIPC_LAUNCHED(ctx);
-    return HIPC_OK;
+    if (!d) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, token >= 0 && token < d->cfg.vocab && pos >= 0 && pos < d->cfg.max_seq, "decoder: bad token %d or position %d", token, pos);
+        dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, token, pos);
+        HIPC_LAUNCHED(ctx);
+        return HIPC_OK;
+    });
 }
 
 int hipc_decoder_kv_cache(hipc_ctx *ctx, hipc_decoder *d, int layer, void **k_cache, void **v_cache) {
-    if (!ctx || !d || !k_cache || !v_cache) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, layer >= 0 && layer < d->cfg.n_layers, "decoder: layer %d out of range", layer);
-    *k_cache = d->layers[layer].k_cache, *v_cache = d->layers[layer].v_cache;
-    return HIPC_OK;
+    if (!d || !k_cache || !v_cache) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, layer >= 0 && layer < d->cfg.n_layers, "decoder: layer %d out of range", layer);
+        *k_cache = d->layers[layer].k_cache, *v_cache = d->layers[layer].v_cache;
+        return HIPC_OK;
+    });
 }
 
 int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
-    if (!ctx || !d) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, complete(d), "decoder: not every weight has been set");
-    const hipc_decoder_config &c = d->cfg;
-    hipStream_t s = ctx->stream;
-    const int nb = (int)ceil_div(c.hidden, c.block_size);
-    const int heads = c.n_q_heads + 2 * c.n_kv_heads;
-    const float scale = c.attn_scale > 0.f ? c.attn_scale : 1.f / sqrtf((float)c.head_dim);
-    const int terms = 2;
-    int rc;
-    dec_embed_kernel<<<1, 256, 0, s>>>(d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
-                                       d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn, c.head_dim, c.rope_theta,
-                                       d->theta2, d->rope);
-    HIPC_LAUNCHED(ctx);
-    // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
-    // branch into the stream reads one and (its first workgroup) writes the other.
-    float *xc = d->x, *xo = d->x2;
-    for (int li = 0; li < c.n_layers; li++) {
-        DecLayer &l = d->layers[li];
-        if (d->fused_glue && li > 0) {
-            GemvPrologue pro;
-            pro.mode = 2, pro.x = xc, pro.y = d->y, pro.w_post = d->layers[li - 1].norm[HIPC_DEC_NORM_POST_FFN];
-            pro.w_in = l.norm[HIPC_DEC_NORM_INPUT], pro.x_out = xo, pro.eps = c.rms_eps;
-            if ((rc = nbits_gemv(ctx, xc, HIPC_F32, l.qkv, d->qkv, 1, terms, &pro)) != HIPC_OK) return rc;
-            std::swap(xc, xo);
-        } else {
-            if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.qkv, d->qkv, 1, terms)) != HIPC_OK) return rc;
-        }
-        if (d->one_launch_attn) {
-            if ((rc = launch_attn_chunks(ctx, d, l, scale)) != HIPC_OK) return rc;
-            if (d->fused_glue) {  // the output projection joins the chunks' partials in its prologue
-                GemvPrologue merge;
-                merge.mode = 3, merge.part_o = d->part_o, merge.part_ml = d->part_ml, merge.pos = &d->state->pos;
-                merge.group = c.n_q_heads / c.n_kv_heads, merge.head_dim = c.head_dim, merge.window = l.window;
-                if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms, &merge)) != HIPC_OK) return rc;
+    if (!d) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, complete(d), "decoder: not every weight has been set");
+        const hipc_decoder_config &c = d->cfg;
+        hipStream_t s = ctx->stream;
+        const int nb = (int)ceil_div(c.hidden, c.block_size);
+        const int heads = c.n_q_heads + 2 * c.n_kv_heads;
+        const float scale = c.attn_scale > 0.f ? c.attn_scale : 1.f / sqrtf((float)c.head_dim);
+        const int terms = 2;
+        int rc;
+        dec_embed_kernel<<<1, 256, 0, s>>>(d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
+                                           d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn, c.head_dim, c.rope_theta,
+                                           d->theta2, d->rope);
+        HIPC_LAUNCHED(ctx);
+        // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
+        // branch into the stream reads one and (its first workgroup) writes the other.
+        float *xc = d->x, *xo = d->x2;
+        for (int li = 0; li < c.n_layers; li++) {
+            DecLayer &l = d->layers[li];
+            if (d->fused_glue && li > 0) {
+                GemvPrologue pro;
+                pro.mode = 2, pro.x = xc, pro.y = d->y, pro.w_post = d->layers[li - 1].norm[HIPC_DEC_NORM_POST_FFN];
+                pro.w_in = l.norm[HIPC_DEC_NORM_INPUT], pro.x_out = xo, pro.eps = c.rms_eps;
+                if ((rc = nbits_gemv(ctx, xc, HIPC_F32, l.qkv, d->qkv, 1, terms, &pro)) != HIPC_OK) return rc;
+                std::swap(xc, xo);
             } else {
-                dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)kAttnSplits * sizeof(float), s>>>(
-                    d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads, c.head_dim, kAttnSplits, 1, l.window, d->attn);
+                if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.qkv, d->qkv, 1, terms)) != HIPC_OK) return rc;
+            }
+            if (d->one_launch_attn) {
+                if ((rc = launch_attn_chunks(ctx, d, l, scale)) != HIPC_OK) return rc;
+                if (d->fused_glue) {  // the output projection joins the chunks' partials in its prologue
+                    GemvPrologue merge;
+                    merge.mode = 3, merge.part_o = d->part_o, merge.part_ml = d->part_ml, merge.pos = &d->state->pos;
+                    merge.group = c.n_q_heads / c.n_kv_heads, merge.head_dim = c.head_dim, merge.window = l.window;
+                    if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms, &merge)) != HIPC_OK) return rc;
+                } else {
+                    dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)kAttnSplits * sizeof(float), s>>>(
+                        d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads, c.head_dim, kAttnSplits, 1, l.window, d->attn);
+                    HIPC_LAUNCHED(ctx);
+                    if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
+                }
+            } else {
+                dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
+                                                     c.n_kv_heads, c.head_dim, c.rms_eps, l.rope_table ? d->theta2 : c.rope_theta, c.max_seq, d->q,
+                                                     l.k_cache, l.v_cache);
+                HIPC_LAUNCHED(ctx);
+                dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
+                                                                                     c.head_dim, c.max_seq, scale, l.window, d->part_ml, d->part_o);
+                HIPC_LAUNCHED(ctx);
+                dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
+                                                                                                 c.head_dim, d->nsplit, 0, l.window, d->attn);
                 HIPC_LAUNCHED(ctx);
                 if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
             }
-        } else {
-            dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
-                                                 c.n_kv_heads, c.head_dim, c.rms_eps, l.rope_table ? d->theta2 : c.rope_theta, c.max_seq, d->q,
-                                                 l.k_cache, l.v_cache);
-            HIPC_LAUNCHED(ctx);
-            dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
-                                                                                 c.head_dim, c.max_seq, scale, l.window, d->part_ml, d->part_o);
-            HIPC_LAUNCHED(ctx);
-            dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
-                                                                                             c.head_dim, d->nsplit, 0, l.window, d->attn);
-            HIPC_LAUNCHED(ctx);
-            if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
+            if (d->fused_glue) {
+                GemvPrologue pro;
+                pro.mode = 2, pro.x = xc, pro.y = d->y, pro.w_post = l.norm[HIPC_DEC_NORM_POST_ATTN];
+                pro.w_in = l.norm[HIPC_DEC_NORM_PRE_FFN], pro.x_out = xo, pro.eps = c.rms_eps;
+                if ((rc = nbits_gemv(ctx, xc, HIPC_F32, l.gate_up, d->gu, 1, terms, &pro)) != HIPC_OK) return rc;
+                std::swap(xc, xo);
+                GemvPrologue gelu;
+                gelu.mode = 1;
+                if ((rc = nbits_gemv(ctx, d->gu, HIPC_F32, l.down, d->y, 1, terms, &gelu)) != HIPC_OK) return rc;
+            } else {
+                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->xn);
+                HIPC_LAUNCHED(ctx);
+                if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.gate_up, d->gu, 1, terms)) != HIPC_OK) return rc;
+                dec_gelu_mul_kernel<<<(unsigned)ceil_div(c.ffn, 256), 256, 0, s>>>(d->gu, c.ffn, d->h);
+                HIPC_LAUNCHED(ctx);
+                if ((rc = nbits_gemv(ctx, d->h, HIPC_F32, l.down, d->y, 1, terms)) != HIPC_OK) return rc;
+                const float *next = li + 1 < c.n_layers ? d->layers[li + 1].norm[HIPC_DEC_NORM_INPUT] : d->final_norm;
+                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->xn);
+                HIPC_LAUNCHED(ctx);
+            }
         }
         if (d->fused_glue) {
-            GemvPrologue pro;
-            pro.mode = 2, pro.x = xc, pro.y = d->y, pro.w_post = l.norm[HIPC_DEC_NORM_POST_ATTN];
-            pro.w_in = l.norm[HIPC_DEC_NORM_PRE_FFN], pro.x_out = xo, pro.eps = c.rms_eps;
-            if ((rc = nbits_gemv(ctx, xc, HIPC_F32, l.gate_up, d->gu, 1, terms, &pro)) != HIPC_OK) return rc;
-            std::swap(xc, xo);
-            GemvPrologue gelu;
-            gelu.mode = 1;
-            if ((rc = nbits_gemv(ctx, d->gu, HIPC_F32, l.down, d->y, 1, terms, &gelu)) != HIPC_OK) return rc;
-        } else {
-            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->xn);
-            HIPC_LAUNCHED(ctx);
-            if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.gate_up, d->gu, 1, terms)) != HIPC_OK) return rc;
-            dec_gelu_mul_kernel<<<(unsigned)ceil_div(c.ffn, 256), 256, 0, s>>>(d->gu, c.ffn, d->h);
-            HIPC_LAUNCHED(ctx);
-            if ((rc = nbits_gemv(ctx, d->h, HIPC_F32, l.down, d->y, 1, terms)) != HIPC_OK) return rc;
-            const float *next = li + 1 < c.n_layers ? d->layers[li + 1].norm[HIPC_DEC_NORM_INPUT] : d->final_norm;
-            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->xn);
+            // the unembedding streams ~200 MB: its workgroups start on the weights at once and the
+            // final norm stays a launch of its own
+            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], d->final_norm, c.hidden,
+                                                       c.rms_eps, xc, d->xn);
             HIPC_LAUNCHED(ctx);
         }
-    }
-    if (d->fused_glue) {
-        // the unembedding streams ~200 MB: its workgroups start on the weights at once and the
-        // final norm stays a launch of its own
-        dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], d->final_norm, c.hidden,
-                                                   c.rms_eps, xc, d->xn);
+        if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;
+        dec_argmax_partial_kernel<<<kArgmaxParts, 256, 0, s>>>(d->logits, c.vocab, d->am_v, d->am_i);
         HIPC_LAUNCHED(ctx);
-    }
-    if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;
-    dec_argmax_partial_kernel<<<kArgmaxParts, 256, 0, s>>>(d->logits, c.vocab, d->am_v, d->am_i);
-    HIPC_LAUNCHED(ctx);
-    dec_argmax_final_kernel<<<1, 64, 0, s>>>(d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq);
-    HIPC_LAUNCHED(ctx);
-    return HIPC_OK;
+        dec_argmax_final_kernel<<<1, 64, 0, s>>>(d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq, c.vocab);
+        HIPC_LAUNCHED(ctx);
+        return HIPC_OK;
+    });
 }
 
 int hipc_decoder_read(hipc_ctx *ctx, hipc_decoder *d, int32_t *token, int32_t *pos, float *logits, int32_t *history, int32_t n_history) {
-    if (!ctx || !d) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REFUSE(ctx, ctx->capturing, "decoder read while a capture is open");
-    HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));
-    DecState st{};
-    HIPC_TRY(ctx, hipMemcpy(&st, d->state, sizeof st, hipMemcpyDeviceToHost));
-    if (token) *token = st.token;
-    if (pos) *pos = st.pos;
-    if (logits) HIPC_TRY(ctx, hipMemcpy(logits, d->logits, (size_t)d->cfg.vocab * 4, hipMemcpyDeviceToHost));
-    if (history && n_history > 0)
-        HIPC_TRY(ctx, hipMemcpy(history, d->history, (size_t)std::min<int32_t>(n_history, d->cfg.max_seq) * 4, hipMemcpyDeviceToHost));
-    return HIPC_OK;
+    if (!d) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        HIPC_REFUSE(ctx, ctx->capturing, "decoder read while a capture is open");
+        HIPC_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        DecState st{};
+        HIPC_TRY(ctx, hipMemcpy(&st, d->state, sizeof st, hipMemcpyDeviceToHost));
+        if (token) *token = st.token;
+        if (pos) *pos = st.pos;
+        if (logits) HIPC_TRY(ctx, hipMemcpy(logits, d->logits, (size_t)d->cfg.vocab * 4, hipMemcpyDeviceToHost));
+        if (history && n_history > 0)
+            HIPC_TRY(ctx, hipMemcpy(history, d->history, (size_t)std::min<int32_t>(n_history, d->cfg.max_seq) * 4, hipMemcpyDeviceToHost));
+        HIPC_REQUIRE(ctx, !st.overflow, "decoder: a step was enqueued with the cache full (%d positions); it did nothing", d->cfg.max_seq);
+        return HIPC_OK;
+    });
 }
 
 }  // extern "C"

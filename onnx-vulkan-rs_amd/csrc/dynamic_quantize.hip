@@ -235,34 +235,34 @@ extern "C" {
 
 int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out, void *zp_out,
                                  void *range, int range_ready) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    return dql_launch(ctx, X, n, Y, scale_out, zp_out, range, range_ready, GeluParams{0, 1.f, 0.f, 1.f, 0});
+    return entry(ctx, [&]() -> int {
+        return dql_launch(ctx, X, n, Y, scale_out, zp_out, range, range_ready, GeluParams{0, 1.f, 0.f, 1.f, 0});
+    });
 }
 
 int hipc_dynamic_quantize_linear_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor, float offset, float factor,
                                       int factor_first, void *Y, void *scale_out, void *zp_out, void *range) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    GeluParams gp;
-    if (int rc = gelu_params(ctx, divisor, offset, factor, factor_first, &gp)) return rc;
-    return dql_launch(ctx, X, n, Y, scale_out, zp_out, range, 0, gp);
+    return entry(ctx, [&]() -> int {
+        GeluParams gp;
+        if (int rc = gelu_params(ctx, divisor, offset, factor, factor_first, &gp)) return rc;
+        return dql_launch(ctx, X, n, Y, scale_out, zp_out, range, 0, gp);
+    });
 }
 
 int hipc_decomposed_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor, float offset, float factor,
                          int factor_first, void *Y) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, n >= 0, "DecomposedGelu: negative length");
-    GeluParams gp;
-    if (int rc = gelu_params(ctx, divisor, offset, factor, factor_first, &gp)) return rc;
-    if (n == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, X && Y && aligned(X, 4) && aligned(Y, 4), "DecomposedGelu: null or unaligned tensor");
-    HIPC_REQUIRE(ctx, ceil_div(n, 256) < (int64_t(1) << 31), "DecomposedGelu: tensor too large");
-    decomposed_gelu_kernel<<<(unsigned)ceil_div(n, 256), 256, 0, ctx->stream>>>(static_cast<const float *>(X), (long)n, gp,
-                                                                                static_cast<float *>(Y));
-    HIPC_LAUNCHED(ctx);
-    return HIPC_OK;
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, n >= 0, "DecomposedGelu: negative length");
+        GeluParams gp;
+        if (int rc = gelu_params(ctx, divisor, offset, factor, factor_first, &gp)) return rc;
+        if (n == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, X && Y && aligned(X, 4) && aligned(Y, 4), "DecomposedGelu: null or unaligned tensor");
+        HIPC_REQUIRE(ctx, ceil_div(n, 256) < (int64_t(1) << 31), "DecomposedGelu: tensor too large");
+        decomposed_gelu_kernel<<<(unsigned)ceil_div(n, 256), 256, 0, ctx->stream>>>(static_cast<const float *>(X), (long)n, gp,
+                                                                                    static_cast<float *>(Y));
+        HIPC_LAUNCHED(ctx);
+        return HIPC_OK;
+    });
 }
 
 }  // extern "C"

@@ -448,12 +448,9 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
 
 // ---- host side: tile choice and launch of the kernel above ---------------------------------
 // 64x64 tiles until 128x128 ones would give every CU at least two workgroups;
-// HIPC_GEMM_TILE=64/128 overrides (tuning, tests).
-inline int gemm_tile(const GemmArgs &g, unsigned batch) {
-    static const int forced = [] {
-        const char *e = getenv("HIPC_GEMM_TILE");
-        return e ? atoi(e) : 0;
-    }();
+// the gemm_tile option (64 / 128) overrides (tuning, tests).
+inline int gemm_tile(hipc_ctx *ctx, const GemmArgs &g, unsigned batch) {
+    const int forced = ctx->tune.gemm_tile;
     if (forced == 64 || forced == 128) return forced;
     const int64_t tiles = ceil_div(g.I, kBM) * ceil_div(g.J, kBN) * (int64_t)batch;
     return tiles >= 512 ? 128 : 64;
@@ -471,7 +468,7 @@ int gemm_launch_tile(hipc_ctx *ctx, GemmArgs g, unsigned batch) {
 
 template <int MODE, int EPI, bool ALIGNED>
 int gemm_launch(hipc_ctx *ctx, const GemmArgs &g, unsigned batch) {
-    return gemm_tile(g, batch) == 64 ? gemm_launch_tile<MODE, EPI, ALIGNED, 64>(ctx, g, batch)
+    return gemm_tile(ctx, g, batch) == 64 ? gemm_launch_tile<MODE, EPI, ALIGNED, 64>(ctx, g, batch)
                                      : gemm_launch_tile<MODE, EPI, ALIGNED, 128>(ctx, g, batch);
 }
 

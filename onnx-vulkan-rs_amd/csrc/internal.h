@@ -7,8 +7,12 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <exception>
+#include <map>
 #include <mutex>
+#include <new>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/hipcompute.h"
@@ -25,6 +29,37 @@ struct Scratch {
     size_t bytes = 0;
 };
 
+// Route and launch-shape overrides (experiments, and tests that must reach every kernel that
+// ships). -1 leaves the choice to the library. A context starts from the environment variables of
+// the same names (HIPC_GEMV_T ...) and hipc_set_option changes one afterwards.
+struct Tuning {
+    int gemv_t = -1;          // HIPC_GEMV_T         16-column tiles per GEMV wavefront: 1, 2 or 4
+    int gemv_waves = -1;      // HIPC_GEMV_WAVES     wavefronts the GEMV aims for when it splits k inside a workgroup
+    int gemv_per_cu = -1;     // HIPC_GEMV_PER_CU    resident GEMV wavefronts per CU of the persistent grid
+    int gemm_tile = -1;       // HIPC_GEMM_TILE      LDS-staged int8 tiles: 64 or 128
+    int gemm_big = -1;        // HIPC_GEMM_BIG       256x256 int8 tiles: 0 never, 1 whenever A allows
+    int gemm_small = -1;      // HIPC_GEMM_SMALL     the k-split 64x64 kernels: 0 never, 1 whenever A allows
+    int gemm_splitk = -1;     // HIPC_GEMM_SPLITK    the k-split-over-workgroups 128x128 kernel: 0 never, n >= 1 forces n ways
+    int conv_row = -1;        // HIPC_CONV_ROW       0: convolutions along one axis take the general route
+    int prefill_tile = -1;    // HIPC_PREFILL_TILE   64 or 128
+    int prefill_split = -1;   // HIPC_PREFILL_SPLIT  0 never splits k, n forces n ways
+    int dec_fused_glue = -1;  // HIPC_DEC_FUSED_GLUE 0 keeps the separate norm / GELU kernels (read when a decoder is created)
+    int dec_fused_attn = -1;  // HIPC_DEC_FUSED_ATTN 0 keeps the three-kernel attention (read when a decoder is created)
+    int dec_persistent = -1;  // HIPC_DEC_PERSISTENT 0: one launch per operator; 1: the whole step in one persistent launch
+};
+
+// Pinned staging ring of hipc_upload: the bytes are copied into a slot and travel from there, so the
+// call returns without waiting for the stream. A slot is reused once the copies that read it are done.
+constexpr int kStageSlots = 4;
+constexpr size_t kStageSlotBytes = size_t(4) << 20;
+struct StageRing {
+    char *base = nullptr;               // kStageSlots * kStageSlotBytes of pinned host memory (allocated on first use)
+    hipEvent_t done[kStageSlots] = {};  // recorded when the ring leaves a slot
+    bool pending[kStageSlots] = {};
+    int slot = 0;
+    size_t used = 0;                    // bytes of the current slot handed out
+};
+
 }  // namespace hipc
 
 struct hipc_ctx {
@@ -35,9 +70,22 @@ struct hipc_ctx {
     std::mutex mu;
     std::string err;
     std::vector<void *> deferred;        // released at the next flush
+    // Blocks the library itself retired (a scratch slot that grew, requantisation ratios that changed, a
+    // replaced decoder weight) while recorded graphs exist: a graph may hold their addresses, so they stay
+    // allocated until the last graph of the context is destroyed.
+    std::vector<void *> retained;
+    int live_graphs = 0;
     hipc::Scratch scratch[hipc::kScratchSlots];
     void *params = nullptr;              // small device block: range slot, scalars, range partials
     int cu_count = 256;
+    hipc::Tuning tune;
+    hipc::StageRing stage;
+    // hipc_alloc's blocks by size class (the reference's pooled scratch buffers,
+    // crates/vk-compute/src/buffer.rs:303-341): a freed block waits in `pool` for the next request of its class
+    std::unordered_map<void *, size_t> alloc_class;      // live hipc_alloc blocks -> class bytes
+    std::map<size_t, std::vector<void *>> pool;          // class bytes -> free blocks
+    size_t pool_bytes = 0;                               // bytes waiting in `pool`
+    size_t pool_hits = 0, pool_misses = 0;
 };
 
 struct hipc_graph {
@@ -75,6 +123,45 @@ struct Guard {
     std::unique_lock<std::mutex> lock;
     explicit Guard(hipc_ctx *ctx) : lock(ctx->mu) { (void)hipSetDevice(ctx->device); }
 };
+
+// The body of an entry point: takes the context's lock, makes its device current and keeps C++
+// exceptions (a failed host allocation, a length error) from crossing the C ABI -- they become
+// HIPC_ERR_BACKEND with a message, under the same lock.
+template <typename F>
+int entry(hipc_ctx *ctx, F &&body) noexcept {
+    if (!ctx) return HIPC_ERR_INVALID;
+    try {
+        Guard g(ctx);
+        try {
+            return body();
+        } catch (const std::bad_alloc &) {
+            return fail(ctx, HIPC_ERR_BACKEND, "out of host memory");
+        } catch (const std::exception &e) {
+            return fail(ctx, HIPC_ERR_BACKEND, "internal error: %s", e.what());
+        } catch (...) {
+            return fail(ctx, HIPC_ERR_BACKEND, "internal error");
+        }
+    } catch (...) {
+        return HIPC_ERR_BACKEND;
+    }
+}
+template <typename F>
+void entry_void(hipc_ctx *ctx, F &&body) noexcept {
+    if (!ctx) return;
+    try {
+        Guard g(ctx);
+        body();
+    } catch (...) {
+    }
+}
+
+// A block of the library's own that later work no longer uses: freed at the next flush, or, while
+// recorded graphs exist (they may hold its address), when the last of them is destroyed.
+inline void retire(hipc_ctx *ctx, void *p) {
+    if (!p) return;
+    if (ctx->live_graphs > 0) ctx->retained.push_back(p);
+    else ctx->deferred.push_back(p);
+}
 
 #define HIPC_TRY(ctx, expr)                                                                      \
     do {                                                                                         \
@@ -125,6 +212,8 @@ int allow_dynamic_lds(hipc_ctx *ctx, K kernel, size_t bytes, bool (&done)[kMaxDe
 // Returns ctx->scratch[slot] grown to at least `bytes`. Growth allocates, so it is
 // refused while a capture is open.
 int scratch_get(hipc_ctx *ctx, int slot, size_t bytes, void **out);
+// host bytes -> device through the context's pinned staging ring; records only (see StageRing)
+int stage_upload(hipc_ctx *ctx, void *dst, const void *host, size_t bytes);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }

@@ -178,24 +178,18 @@ int launch_mm_big(hipc_ctx *ctx, const GemmArgs &g) {
     return zero_known ? launch_mm_big_dyn<EPI, false>(ctx, g) : launch_mm_big_dyn<EPI, true>(ctx, g);
 }
 
-// 256x256 tiles once they fill most of the chip's 256 CUs; HIPC_GEMM_BIG=0/1 overrides (tuning, tests)
-bool wants_big_tiles(const GemmArgs &g) {
-    static const int forced = [] {
-        const char *e = getenv("HIPC_GEMM_BIG");
-        return e ? atoi(e) : -1;
-    }();
+// 256x256 tiles once they fill most of the chip's 256 CUs; the gemm_big option (0 / 1) overrides (tuning, tests)
+bool wants_big_tiles(hipc_ctx *ctx, const GemmArgs &g) {
+    const int forced = ctx->tune.gemm_big;
     if (!g.p_aligned) return false;
     if (forced >= 0) return forced != 0;
     return ceil_div(g.I, kBigTile) * ceil_div(g.J, kBigTile) >= 192;
 }
 
 // Products of a few 64x64 tiles per CU and a long enough k run on the kernel that keeps B out of LDS
-// and splits k over the wavefronts of a workgroup. HIPC_GEMM_SMALL=0/1 overrides (tuning, tests).
+// and splits k over the wavefronts of a workgroup. The gemm_small option (0 / 1) overrides (tuning, tests).
 bool wants_small_tiles(hipc_ctx *ctx, const GemmArgs &g) {
-    static const int forced = [] {
-        const char *e = getenv("HIPC_GEMM_SMALL");
-        return e ? atoi(e) : -1;
-    }();
+    const int forced = ctx->tune.gemm_small;
     if (!g.p_aligned) return false;
     if (forced >= 0) return forced != 0;
     // measured against the LDS-staged 64x64 tiles: ahead up to four tiles per CU from k = 1024 on (14.1
@@ -218,7 +212,7 @@ int launch_mm_small(hipc_ctx *ctx, const GemmArgs &g) {
 template <int EPI>
 int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
     if (g.I == 0 || g.J == 0) return HIPC_OK;
-    if (wants_big_tiles(g)) return launch_mm_big<EPI>(ctx, g);
+    if (wants_big_tiles(ctx, g)) return launch_mm_big<EPI>(ctx, g);
     if (wants_small_tiles(ctx, g)) return launch_mm_small<EPI>(ctx, g);
     return g.p_aligned ? gemm_launch<MODE_MM, EPI, true>(ctx, g, 1) : gemm_launch<MODE_MM, EPI, false>(ctx, g, 1);
 }
@@ -228,193 +222,196 @@ int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
 extern "C" {
 
 int hipc_probe_int8_mfma(hipc_ctx *ctx, int random_operands, int waves_per_simd, int iterations, double *tops) {
-    if (!ctx || !tops) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, (waves_per_simd == 1 || waves_per_simd == 2) && iterations > 0 && iterations <= (1 << 20),
-                 "hipc_probe_int8_mfma: waves_per_simd must be 1 or 2, iterations in 1..2^20");
-    HIPC_REFUSE(ctx, ctx->capturing, "hipc_probe_int8_mfma while a capture is open");
-    hipEvent_t t0, t1;
-    HIPC_TRY(ctx, hipEventCreate(&t0));
-    HIPC_TRY(ctx, hipEventCreate(&t1));
-    int *sink = reinterpret_cast<int *>(static_cast<char *>(ctx->params) + 128);
-    const unsigned grid = (unsigned)(ctx->cu_count * waves_per_simd);  // 4 wavefronts per workgroup, one per SIMD
-    int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(64, 1u, random_operands, sink);  // warm the clocks and the code
-    hipError_t e = hipEventRecord(t0, ctx->stream);
-    int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(iterations, 7u, random_operands, sink);
-    if (e == hipSuccess) e = hipGetLastError();
-    if (e == hipSuccess) e = hipEventRecord(t1, ctx->stream);
-    if (e == hipSuccess) e = hipEventSynchronize(t1);
-    float ms = 0.f;
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    if (e != hipSuccess) return fail(ctx, HIPC_ERR_BACKEND, "hipc_probe_int8_mfma: %s", hipGetErrorString(e));
-    const double ops = 2.0 * 32 * 32 * 32 * 8.0 * iterations * 4.0 * grid;
-    *tops = ops / (ms * 1e-3) / 1e12;
-    return HIPC_OK;
+    if (!tops) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, (waves_per_simd == 1 || waves_per_simd == 2) && iterations > 0 && iterations <= (1 << 20),
+                     "hipc_probe_int8_mfma: waves_per_simd must be 1 or 2, iterations in 1..2^20");
+        HIPC_REFUSE(ctx, ctx->capturing, "hipc_probe_int8_mfma while a capture is open");
+        hipEvent_t t0, t1;
+        HIPC_TRY(ctx, hipEventCreate(&t0));
+        HIPC_TRY(ctx, hipEventCreate(&t1));
+        int *sink = reinterpret_cast<int *>(static_cast<char *>(ctx->params) + 128);
+        const unsigned grid = (unsigned)(ctx->cu_count * waves_per_simd);  // 4 wavefronts per workgroup, one per SIMD
+        int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(64, 1u, random_operands, sink);  // warm the clocks and the code
+        hipError_t e = hipEventRecord(t0, ctx->stream);
+        int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(iterations, 7u, random_operands, sink);
+        if (e == hipSuccess) e = hipGetLastError();
+        if (e == hipSuccess) e = hipEventRecord(t1, ctx->stream);
+        if (e == hipSuccess) e = hipEventSynchronize(t1);
+        float ms = 0.f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+        (void)hipEventDestroy(t0);
+        (void)hipEventDestroy(t1);
+        if (e != hipSuccess) return fail(ctx, HIPC_ERR_BACKEND, "hipc_probe_int8_mfma: %s", hipGetErrorString(e));
+        const double ops = 2.0 * 32 * 32 * 32 * 8.0 * iterations * 4.0 * grid;
+        *tops = ops / (ms * 1e-3) / 1e12;
+        return HIPC_OK;
+    });
 }
 
 int hipc_prepack_int8_b(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, int64_t N, hipc_int8_weight **out) {
-    if (!ctx || !out) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    *out = nullptr;
-    HIPC_REFUSE(ctx, ctx->capturing, "MatMulInteger prepack while a capture is open");
-    HIPC_REFUSE(ctx, !is_byte_dtype(b_dtype), "MatMulInteger: B must be uint8 or int8, got %d", b_dtype);
-    HIPC_REQUIRE(ctx, B && K > 0 && N > 0 && K < (int64_t(1) << 30) && N < (int64_t(1) << 30),
-                 "MatMulInteger prepack: bad shape K=%ld N=%ld", (long)K, (long)N);
-    hipc_int8_weight *w = new hipc_int8_weight();
-    w->K = K, w->N = N, w->b_dtype = b_dtype;
-    w->K_pad = (int)(ceil_div(K, kBK) * kBK);
-    w->N_pad = (int)(ceil_div(N, kBN) * kBN);
-    if ((int64_t)w->K_pad * w->N_pad >= (int64_t(1) << 32)) {
-        delete w;
-        return fail(ctx, HIPC_ERR_UNSUPPORTED, "MatMulInteger prepack: a %ld x %ld weight exceeds the 4 GiB the kernel addresses", (long)K, (long)N);
-    }
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->Bp), (size_t)w->K_pad * w->N_pad);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&w->colsum), (size_t)w->N_pad * 4);
-    if (e != hipSuccess) {
-        if (w->Bp) (void)hipFree(w->Bp);
-        delete w;
-        return fail(ctx, HIPC_ERR_BACKEND, "MatMulInteger prepack: %s", hipGetErrorString(e));
-    }
-    int rc = pack_into(ctx, B, b_dtype, K, N, w->K_pad, w->N_pad, w->Bp, w->colsum);
-    if (rc != HIPC_OK) {
-        (void)hipFree(w->Bp);
-        (void)hipFree(w->colsum);
-        delete w;
-        return rc;
-    }
-    *out = w;
-    return HIPC_OK;
+    if (!out) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        *out = nullptr;
+        HIPC_REFUSE(ctx, ctx->capturing, "MatMulInteger prepack while a capture is open");
+        HIPC_REFUSE(ctx, !is_byte_dtype(b_dtype), "MatMulInteger: B must be uint8 or int8, got %d", b_dtype);
+        HIPC_REQUIRE(ctx, B && K > 0 && N > 0 && K < (int64_t(1) << 30) && N < (int64_t(1) << 30),
+                     "MatMulInteger prepack: bad shape K=%ld N=%ld", (long)K, (long)N);
+        hipc_int8_weight *w = new hipc_int8_weight();
+        w->K = K, w->N = N, w->b_dtype = b_dtype;
+        w->K_pad = (int)(ceil_div(K, kBK) * kBK);
+        w->N_pad = (int)(ceil_div(N, kBN) * kBN);
+        if ((int64_t)w->K_pad * w->N_pad >= (int64_t(1) << 32)) {
+            delete w;
+            return fail(ctx, HIPC_ERR_UNSUPPORTED, "MatMulInteger prepack: a %ld x %ld weight exceeds the 4 GiB the kernel addresses", (long)K, (long)N);
+        }
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->Bp), (size_t)w->K_pad * w->N_pad);
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&w->colsum), (size_t)w->N_pad * 4);
+        if (e != hipSuccess) {
+            if (w->Bp) (void)hipFree(w->Bp);
+            delete w;
+            return fail(ctx, HIPC_ERR_BACKEND, "MatMulInteger prepack: %s", hipGetErrorString(e));
+        }
+        int rc = pack_into(ctx, B, b_dtype, K, N, w->K_pad, w->N_pad, w->Bp, w->colsum);
+        if (rc != HIPC_OK) {
+            (void)hipFree(w->Bp);
+            (void)hipFree(w->colsum);
+            delete w;
+            return rc;
+        }
+        *out = w;
+        return HIPC_OK;
+    });
 }
 
 void hipc_int8_weight_destroy(hipc_ctx *ctx, hipc_int8_weight *w) {
-    if (!ctx || !w) return;
-    Guard g(ctx);
-    if (w->Bp) ctx->deferred.push_back(w->Bp);
-    if (w->colsum) ctx->deferred.push_back(w->colsum);
-    ratio_release(ctx, w->ratios);
-    delete w;
+    if (!w) return;
+    entry_void(ctx, [&] {
+        if (w->Bp) ctx->deferred.push_back(w->Bp);
+        if (w->colsum) ctx->deferred.push_back(w->colsum);
+        ratio_release(ctx, w->ratios);
+        delete w;
+    });
 }
 
 int hipc_matmul_integer(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_int8_weight *B, const void *a_zp,
                         const void *b_zp, void *Y, int64_t M) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, B, "MatMulInteger: null weight");
-    GemmArgs ga;
-    int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
-    if (rc != HIPC_OK) return rc;
-    if (M == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, A && Y, "MatMulInteger: null operand");
-    ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
-    ga.const_zp = static_cast<const uint8_t *>(b_zp);
-    ga.Y = Y;
-    return launch_mm<EPI_I32>(ctx, ga);
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, B, "MatMulInteger: null weight");
+        GemmArgs ga;
+        int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
+        if (rc != HIPC_OK) return rc;
+        if (M == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, A && Y, "MatMulInteger: null operand");
+        ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
+        ga.const_zp = static_cast<const uint8_t *>(b_zp);
+        ga.Y = Y;
+        return launch_mm<EPI_I32>(ctx, ga);
+    });
 }
 
 int hipc_matmul_integer_raw(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, int b_dtype, const void *a_zp,
                             const void *b_zp, void *Y, int64_t M, int64_t K, int64_t N) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REFUSE(ctx, !is_byte_dtype(b_dtype), "MatMulInteger: B must be uint8 or int8, got %d", b_dtype);
-    HIPC_REQUIRE(ctx, K > 0 && N >= 0 && K < (int64_t(1) << 30) && N < (int64_t(1) << 30),
-                 "MatMulInteger: bad shape K=%ld N=%ld", (long)K, (long)N);
-    if (M == 0 || N == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, A && B && Y, "MatMulInteger: null operand");
-    const int K_pad = (int)(ceil_div(K, kBK) * kBK), N_pad = (int)(ceil_div(N, kBN) * kBN);
-    HIPC_REFUSE(ctx, (int64_t)K_pad * N_pad >= (int64_t(1) << 32), "MatMulInteger: a %ld x %ld weight exceeds the 4 GiB the kernel addresses", (long)K, (long)N);
-    void *scratch = nullptr;
-    const size_t bp_bytes = (size_t)K_pad * N_pad;
-    int rc = scratch_get(ctx, 1, bp_bytes + (size_t)N_pad * 4, &scratch);
-    if (rc != HIPC_OK) return rc;
-    uint8_t *Bp = static_cast<uint8_t *>(scratch);
-    int32_t *colsum = reinterpret_cast<int32_t *>(Bp + bp_bytes);
-    rc = pack_into(ctx, B, b_dtype, K, N, K_pad, N_pad, Bp, colsum);
-    if (rc != HIPC_OK) return rc;
-    GemmArgs ga;
-    rc = fill_common(ctx, MmOperands{A, a_dtype, Bp, colsum, b_dtype, M, K, N, K_pad}, ga);
-    if (rc != HIPC_OK) return rc;
-    ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
-    ga.const_zp = static_cast<const uint8_t *>(b_zp);
-    ga.Y = Y;
-    return launch_mm<EPI_I32>(ctx, ga);
+    return entry(ctx, [&]() -> int {
+        HIPC_REFUSE(ctx, !is_byte_dtype(b_dtype), "MatMulInteger: B must be uint8 or int8, got %d", b_dtype);
+        HIPC_REQUIRE(ctx, K > 0 && N >= 0 && K < (int64_t(1) << 30) && N < (int64_t(1) << 30),
+                     "MatMulInteger: bad shape K=%ld N=%ld", (long)K, (long)N);
+        if (M == 0 || N == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, A && B && Y, "MatMulInteger: null operand");
+        const int K_pad = (int)(ceil_div(K, kBK) * kBK), N_pad = (int)(ceil_div(N, kBN) * kBN);
+        HIPC_REFUSE(ctx, (int64_t)K_pad * N_pad >= (int64_t(1) << 32), "MatMulInteger: a %ld x %ld weight exceeds the 4 GiB the kernel addresses", (long)K, (long)N);
+        void *scratch = nullptr;
+        const size_t bp_bytes = (size_t)K_pad * N_pad;
+        int rc = scratch_get(ctx, 1, bp_bytes + (size_t)N_pad * 4, &scratch);
+        if (rc != HIPC_OK) return rc;
+        uint8_t *Bp = static_cast<uint8_t *>(scratch);
+        int32_t *colsum = reinterpret_cast<int32_t *>(Bp + bp_bytes);
+        rc = pack_into(ctx, B, b_dtype, K, N, K_pad, N_pad, Bp, colsum);
+        if (rc != HIPC_OK) return rc;
+        GemmArgs ga;
+        rc = fill_common(ctx, MmOperands{A, a_dtype, Bp, colsum, b_dtype, M, K, N, K_pad}, ga);
+        if (rc != HIPC_OK) return rc;
+        ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
+        ga.const_zp = static_cast<const uint8_t *>(b_zp);
+        ga.Y = Y;
+        return launch_mm<EPI_I32>(ctx, ga);
+    });
 }
 
 int hipc_matmul_integer_scale_bias(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_int8_weight *B,
                                    const void *a_zp, const void *b_zp, const void *scale, int scale_step,
                                    const void *product, int product_step, const void *bias, int bias_step, int relu,
                                    void *range, void *Y, int64_t M) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, B, "MatMulIntegerScaleBias: null weight");
-    HIPC_REQUIRE(ctx, scale, "MatMulIntegerScaleBias: null scale");
-    HIPC_REQUIRE(ctx, (scale_step | 1) == 1 && (product_step | 1) == 1 && (bias_step | 1) == 1,
-                 "MatMulIntegerScaleBias: broadcast steps must be 0 (scalar) or 1 (per column)");
-    GemmArgs ga;
-    int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
-    if (rc != HIPC_OK) return rc;
-    if (M == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, A && Y, "MatMulIntegerScaleBias: null operand");
-    ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
-    ga.const_zp = static_cast<const uint8_t *>(b_zp);
-    ga.Y = Y;
-    ga.scale = static_cast<const float *>(scale), ga.scale_step = scale_step;
-    ga.product = static_cast<const float *>(product), ga.product_step = product_step;
-    ga.bias = static_cast<const float *>(bias), ga.bias_step = bias_step;
-    ga.relu = relu;
-    ga.range = static_cast<uint32_t *>(range);
-    return launch_mm<EPI_SCALE_BIAS>(ctx, ga);
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, B, "MatMulIntegerScaleBias: null weight");
+        HIPC_REQUIRE(ctx, scale, "MatMulIntegerScaleBias: null scale");
+        HIPC_REQUIRE(ctx, (scale_step | 1) == 1 && (product_step | 1) == 1 && (bias_step | 1) == 1,
+                     "MatMulIntegerScaleBias: broadcast steps must be 0 (scalar) or 1 (per column)");
+        GemmArgs ga;
+        int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
+        if (rc != HIPC_OK) return rc;
+        if (M == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, A && Y, "MatMulIntegerScaleBias: null operand");
+        ga.dyn_zp = static_cast<const uint8_t *>(a_zp);
+        ga.const_zp = static_cast<const uint8_t *>(b_zp);
+        ga.Y = Y;
+        ga.scale = static_cast<const float *>(scale), ga.scale_step = scale_step;
+        ga.product = static_cast<const float *>(product), ga.product_step = product_step;
+        ga.bias = static_cast<const float *>(bias), ga.bias_step = bias_step;
+        ga.relu = relu;
+        ga.range = static_cast<uint32_t *>(range);
+        return launch_mm<EPI_SCALE_BIAS>(ctx, ga);
+    });
 }
 
 int hipc_requantize(hipc_ctx *ctx, const void *acc, const void *bias, const void *ratio, int64_t n, int64_t inner,
                     int64_t axis_len, int32_t y_zp, int out_dtype, void *out) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REFUSE(ctx, !is_byte_dtype(out_dtype), "Requantize: output must be uint8 or int8, got %d", out_dtype);
-    HIPC_REQUIRE(ctx, n >= 0, "Requantize: negative length");
-    HIPC_REQUIRE(ctx, axis_len > 0, "Requantize: empty scale");  // interp.rs:4732
-    if (n == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, acc && ratio && out, "Requantize: null operand");
-    const long words = ceil_div(n, 4);
-    requantize_kernel<<<dim3((unsigned)ceil_div(words, 256)), 256, 0, ctx->stream>>>(
-        static_cast<const int32_t *>(acc), static_cast<const int32_t *>(bias), static_cast<const float *>(ratio), (long)n,
-        (long)std::max<int64_t>(inner, 1), (long)axis_len, y_zp, out_dtype == HIPC_I8, static_cast<uint8_t *>(out));
-    HIPC_LAUNCHED(ctx);
-    return HIPC_OK;
+    return entry(ctx, [&]() -> int {
+        HIPC_REFUSE(ctx, !is_byte_dtype(out_dtype), "Requantize: output must be uint8 or int8, got %d", out_dtype);
+        HIPC_REQUIRE(ctx, n >= 0, "Requantize: negative length");
+        HIPC_REQUIRE(ctx, axis_len > 0, "Requantize: empty scale");  // interp.rs:4732
+        if (n == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, acc && ratio && out, "Requantize: null operand");
+        const long words = ceil_div(n, 4);
+        requantize_kernel<<<dim3((unsigned)ceil_div(words, 256)), 256, 0, ctx->stream>>>(
+            static_cast<const int32_t *>(acc), static_cast<const int32_t *>(bias), static_cast<const float *>(ratio), (long)n,
+            (long)std::max<int64_t>(inner, 1), (long)axis_len, y_zp, out_dtype == HIPC_I8, static_cast<uint8_t *>(out));
+        HIPC_LAUNCHED(ctx);
+        return HIPC_OK;
+    });
 }
 
 int hipc_qlinear_matmul(hipc_ctx *ctx, const void *A, int a_dtype, float a_scale, int32_t a_zp,
                         const hipc_int8_weight *B, const float *b_scale, int64_t n_b_scale, int32_t b_zp, float y_scale,
                         int32_t y_zp, int y_dtype, void *Y, int64_t M) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, B && b_scale, "QLinearMatMul: null weight or scale");
-    HIPC_REFUSE(ctx, !is_byte_dtype(y_dtype), "QLinearMatMul: output must be uint8 or int8, got %d", y_dtype);
-    // the accepted envelope of `unsupported_quantization` (interp.rs:781-847, :4862-4866)
-    HIPC_REQUIRE(ctx, n_b_scale == 1 || n_b_scale == B->N, "QLinearMatMul: %ld scales for %ld columns", (long)n_b_scale,
-                 (long)B->N);
-    HIPC_REFUSE(ctx, n_b_scale > 1 && b_zp != 0, "QLinearMatMul: b per-channel zero point is not zero (asymmetric weights)");
-    HIPC_REQUIRE(ctx, y_scale != 0.f, "QLinear: y_scale is zero");
-    GemmArgs ga;
-    int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
-    if (rc != HIPC_OK) return rc;
-    if (M == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, A && Y, "QLinearMatMul: null operand");
-    // ratio[c] = a_scale * b_scale[c] / y_scale, f32, left to right (interp.rs:4693)
-    std::vector<float> ratio((size_t)n_b_scale);
-    for (int64_t c = 0; c < n_b_scale; c++) {
-        volatile float t = a_scale * b_scale[c];
-        ratio[(size_t)c] = t / y_scale;
-    }
-    const float *dratio = nullptr;
-    rc = ratio_resident(ctx, B->ratios, ratio, &dratio);
-    if (rc != HIPC_OK) return rc;
-    ga.host_zp = 1, ga.dyn_zp_value = a_zp, ga.const_zp_value = b_zp;
-    ga.Y = Y;
-    ga.ratio = dratio, ga.ratio_step = n_b_scale > 1 ? 1 : 0;
-    ga.y_zp = y_zp, ga.out_signed = y_dtype == HIPC_I8;
-    return launch_mm<EPI_REQUANT>(ctx, ga);
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, B && b_scale, "QLinearMatMul: null weight or scale");
+        HIPC_REFUSE(ctx, !is_byte_dtype(y_dtype), "QLinearMatMul: output must be uint8 or int8, got %d", y_dtype);
+        // the accepted envelope of `unsupported_quantization` (interp.rs:781-847, :4862-4866)
+        HIPC_REQUIRE(ctx, n_b_scale == 1 || n_b_scale == B->N, "QLinearMatMul: %ld scales for %ld columns", (long)n_b_scale,
+                     (long)B->N);
+        HIPC_REFUSE(ctx, n_b_scale > 1 && b_zp != 0, "QLinearMatMul: b per-channel zero point is not zero (asymmetric weights)");
+        HIPC_REQUIRE(ctx, y_scale != 0.f, "QLinear: y_scale is zero");
+        GemmArgs ga;
+        int rc = fill_common(ctx, MmOperands{A, a_dtype, B->Bp, B->colsum, B->b_dtype, M, B->K, B->N, B->K_pad}, ga);
+        if (rc != HIPC_OK) return rc;
+        if (M == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, A && Y, "QLinearMatMul: null operand");
+        // ratio[c] = a_scale * b_scale[c] / y_scale, f32, left to right (interp.rs:4693)
+        std::vector<float> ratio((size_t)n_b_scale);
+        for (int64_t c = 0; c < n_b_scale; c++) {
+            volatile float t = a_scale * b_scale[c];
+            ratio[(size_t)c] = t / y_scale;
+        }
+        const float *dratio = nullptr;
+        rc = ratio_resident(ctx, B->ratios, ratio, &dratio);
+        if (rc != HIPC_OK) return rc;
+        ga.host_zp = 1, ga.dyn_zp_value = a_zp, ga.const_zp_value = b_zp;
+        ga.Y = Y;
+        ga.ratio = dratio, ga.ratio_step = n_b_scale > 1 ? 1 : 0;
+        ga.y_zp = y_zp, ga.out_signed = y_dtype == HIPC_I8;
+        return launch_mm<EPI_REQUANT>(ctx, ga);
+    });
 }
 
 }  // extern "C"

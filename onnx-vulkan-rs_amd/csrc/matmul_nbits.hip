@@ -14,9 +14,10 @@
 //            load per lane; nibbles become bf16 integers 128+q with four
 //            and-or operations per word and go straight into
 //            v_mfma_f32_16x16x32_bf16 as the B operand. The f32 activations are
-//            split once per workgroup into three bf16 terms (hi + mid + lo,
-//            24 significant bits) that are the A operands of three chained MFMAs,
-//            so products are exact and the sum is f32. The +128 bias and the
+//            split once per workgroup into bf16 terms that are the A operands of
+//            chained MFMAs, so products are exact and the sum is f32: two terms
+//            by default (hi + lo, 16 significant bits), three (hi + mid + lo, all
+//            24 bits) with accuracy_level 1. The +128 bias and the
 //            zero point leave in the per-block epilogue:
 //                acc += scale * (dot - (128 + zp) * sum_k a_k).
 //            HBM-bound: 16 B of nibbles + 4 B scale + 1 B zero point per 32 weights.
@@ -738,18 +739,9 @@ using namespace hipc;
 
 namespace {
 
-// Launch-shape overrides for experiments: HIPC_GEMV_T (16-column tiles per wavefront: 1, 2 or
-// 4), HIPC_GEMV_WAVES (wavefronts to aim for when k is split inside a workgroup) and
-// HIPC_GEMV_PER_CU (resident wavefronts per CU of the persistent grid).
-struct GemvTune {
-    int T = 0, waves = 0, per_cu = 0;
-    GemvTune() {
-        if (const char *e = getenv("HIPC_GEMV_T")) T = atoi(e);
-        if (const char *e = getenv("HIPC_GEMV_WAVES")) waves = atoi(e);
-        if (const char *e = getenv("HIPC_GEMV_PER_CU")) per_cu = atoi(e);
-    }
-};
-const GemvTune g_tune;
+// Launch-shape overrides (the context's Tuning): gemv_t (16-column tiles per wavefront: 1, 2 or 4),
+// gemv_waves (wavefronts to aim for when k is split inside a workgroup) and gemv_per_cu (resident
+// wavefronts per CU of the persistent grid).
 
 int log2i(int64_t v) {
     int s = 0;
@@ -857,11 +849,11 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
 
     // columns per wavefront: wide outputs amortise the activation operands over more tiles
     int T = n_tiles >= 2048 ? 2 : 1;
-    if (g_tune.T == 1 || g_tune.T == 2 || g_tune.T == 4) T = g_tune.T;
+    if (ctx->tune.gemv_t == 1 || ctx->tune.gemv_t == 2 || ctx->tune.gemv_t == 4) T = ctx->tune.gemv_t;
     if (NR == 4 && T == 4) T = 2;  // four tiles x four accumulator registers do not fit the register file
     const int groups = (int)ceil_div(n_tiles, T);
     // k partition inside a workgroup: enough wavefronts to cover the chip a few times over
-    const int want_waves = g_tune.waves > 0 ? g_tune.waves : 8 * ctx->cu_count;
+    const int want_waves = ctx->tune.gemv_waves > 0 ? ctx->tune.gemv_waves : 8 * ctx->cu_count;
     const int kparts = (int)std::min<int64_t>(n_cg, std::max<int64_t>(1, ceil_div(want_waves, groups)));
     // the activation slice of a workgroup must fit the LDS budget: NT*64 + 4 bytes per row per 32-k
     // chunk; only then is k also split across workgroups (partials + a reduce launch)
@@ -888,7 +880,7 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
     }
     // persistent over the column groups once there are more workgroups than the chip holds at the
     // occupancy aimed for (16 wavefronts per CU unless overridden)
-    const int waves_per_cu = g_tune.per_cu > 0 ? g_tune.per_cu : 16;
+    const int waves_per_cu = ctx->tune.gemv_per_cu > 0 ? ctx->tune.gemv_per_cu : 16;
     const int resident = std::max(1, ctx->cu_count * std::max(1, waves_per_cu / (WK * WN)) / ksplit);
     const dim3 grid((unsigned)std::min<int64_t>(ceil_div(groups, WN), resident), (unsigned)ksplit);
     const dim3 block(64 * WK * WN);
@@ -941,29 +933,30 @@ extern "C" {
 int hipc_matmul_nbits(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, size_t b_len, const void *scales,
                       int scale_dtype, size_t scales_len, const void *zp, size_t zp_len, void *Y, int64_t M, int64_t K,
                       int64_t N, int64_t block_size, int accuracy_level) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
-    HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 3,
-                "MatMulNBits: accuracy_level %d asks for quantised activations", accuracy_level);
-    int rc = check_nbits_shape(ctx, M, K, N, block_size, b_len, scales_len, zp, zp_len, scale_dtype);
-    if (rc != HIPC_OK) return rc;
-    if (M == 0 || N == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, A && B && scales && Y, "MatMulNBits: null operand");
-    HIPC_REQUIRE(ctx, aligned(B, 4), "MatMulNBits: packed weight must be 4-byte aligned");
-    const bool af16 = a_dtype == HIPC_F16, sf16 = scale_dtype == HIPC_F16;
-    if (af16 && sf16) return launch_direct<__half, __half>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
-    if (af16) return launch_direct<__half, float>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
-    if (sf16) return launch_direct<float, __half>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
-    return launch_direct<float, float>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
+    return entry(ctx, [&]() -> int {
+        HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
+        HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 3,
+                    "MatMulNBits: accuracy_level %d asks for quantised activations", accuracy_level);
+        int rc = check_nbits_shape(ctx, M, K, N, block_size, b_len, scales_len, zp, zp_len, scale_dtype);
+        if (rc != HIPC_OK) return rc;
+        if (M == 0 || N == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, A && B && scales && Y, "MatMulNBits: null operand");
+        HIPC_REQUIRE(ctx, aligned(B, 4), "MatMulNBits: packed weight must be 4-byte aligned");
+        const bool af16 = a_dtype == HIPC_F16, sf16 = scale_dtype == HIPC_F16;
+        if (af16 && sf16) return launch_direct<__half, __half>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
+        if (af16) return launch_direct<__half, float>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
+        if (sf16) return launch_direct<float, __half>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
+        return launch_direct<float, float>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
+    });
 }
 
 int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype,
                               size_t scales_len, const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size,
                               hipc_nbits_weight **out) {
-    if (!ctx || !out) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    return hipc::nbits_prepack(ctx, B, b_len, scales, scale_dtype, scales_len, zp, zp_len, K, N, block_size, out);
+    if (!out) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        return hipc::nbits_prepack(ctx, B, b_len, scales, scale_dtype, scales_len, zp, zp_len, K, N, block_size, out);
+    });
 }
 
 }  // extern "C"
@@ -1049,37 +1042,38 @@ int64_t hipc::nbits_depth(const hipc_nbits_weight *w) { return w->K; }
 extern "C" {
 
 void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w) {
-    if (!ctx || !w) return;
-    Guard g(ctx);
-    hipc::nbits_release(ctx, w);
+    if (!w) return;
+    entry_void(ctx, [&] {
+        hipc::nbits_release(ctx, w);
+    });
 }
 
 size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w) { return w ? w->bytes : 0; }
 
 int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int64_t M,
                              int accuracy_level) {
-    if (!ctx) return HIPC_ERR_INVALID;
-    Guard g(ctx);
-    HIPC_REQUIRE(ctx, w, "MatMulNBits: null weight");
-    HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
-    HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 3,
-                "MatMulNBits: accuracy_level %d asks for quantised activations", accuracy_level);
-    HIPC_REQUIRE(ctx, M >= 0 && M < (int64_t(1) << 30), "MatMulNBits: bad M=%ld", (long)M);
-    if (M == 0) return HIPC_OK;
-    HIPC_REQUIRE(ctx, A && Y, "MatMulNBits: null operand");
-    const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
-    // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
-    // terms). Unset, or 2 / 3 (f16 / bf16 are enough): 2 terms. f16 activations are exact in 2.
-    const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
-    // many rows of f16: the tiled kernel reads the weight once per row tile instead of once per 16 rows
-    if (a_dtype == HIPC_F16 && nbits_prefill_takes(A, w, M)) return nbits_prefill(ctx, A, w, Y, M);
-    for (int64_t m0 = 0; m0 < M; m0 += 16) {
-        const int rows = (int)std::min<int64_t>(16, M - m0);
-        int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,
-                             static_cast<char *>(Y) + (size_t)m0 * w->N * esz, rows, NT);
-        if (rc != HIPC_OK) return rc;
-    }
-    return HIPC_OK;
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, w, "MatMulNBits: null weight");
+        HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
+        HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 3,
+                    "MatMulNBits: accuracy_level %d asks for quantised activations", accuracy_level);
+        HIPC_REQUIRE(ctx, M >= 0 && M < (int64_t(1) << 30), "MatMulNBits: bad M=%ld", (long)M);
+        if (M == 0) return HIPC_OK;
+        HIPC_REQUIRE(ctx, A && Y, "MatMulNBits: null operand");
+        const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
+        // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
+        // terms). Unset, or 2 / 3 (f16 / bf16 are enough): 2 terms. f16 activations are exact in 2.
+        const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
+        // many rows of f16: the tiled kernel reads the weight once per row tile instead of once per 16 rows
+        if (a_dtype == HIPC_F16 && nbits_prefill_takes(A, w, M)) return nbits_prefill(ctx, A, w, Y, M);
+        for (int64_t m0 = 0; m0 < M; m0 += 16) {
+            const int rows = (int)std::min<int64_t>(16, M - m0);
+            int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,
+                                 static_cast<char *>(Y) + (size_t)m0 * w->N * esz, rows, NT);
+            if (rc != HIPC_OK) return rc;
+        }
+        return HIPC_OK;
+    });
 }
 
 }  // extern "C"

@@ -284,11 +284,7 @@ mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ 
 
 namespace {
 
-// HIPC_PREFILL_SPLIT: 0 never splits k, n > 0 forces n ways (tuning, tests); unset: chosen by shape
-const int g_prefill_split = [] {
-    const char *e = getenv("HIPC_PREFILL_SPLIT");
-    return e ? atoi(e) : -1;
-}();
+// the prefill_split option: 0 never splits k, n > 0 forces n ways (tuning, tests); unset: chosen by shape
 
 template <int SG, int T>
 int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
@@ -311,6 +307,7 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
     // partials go through scratch memory.
     const int nk = (int)ceil_div(a.K, kPK);
     int ksplit = 1;
+    const int g_prefill_split = ctx->tune.prefill_split;
     if (T == 128 && g_prefill_split != 0) {
         const int tiles = tiles_x * tiles_y;
         ksplit = g_prefill_split > 0 ? g_prefill_split : std::min(4, ctx->cu_count / std::max(1, tiles));
@@ -363,10 +360,7 @@ namespace {
 
 template <int SG>
 int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
-    static const int forced = [] {
-        const char *e = getenv("HIPC_PREFILL_TILE");
-        return e ? atoi(e) : 0;
-    }();
+    const int forced = ctx->tune.prefill_tile, g_prefill_split = ctx->tune.prefill_split;
     // 128x128 tiles when they give every CU a workgroup, directly or (long k) with k split over up
     // to four workgroups per tile; else 64x64
     const int64_t tiles128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);

@@ -5,6 +5,7 @@ enqueue-only calls, one explicit ``flush``.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import os
 
@@ -62,6 +63,8 @@ SIGNATURES = {
     "hipc_last_error": (C.c_char_p, [_vp]),
     "hipc_version": (C.c_char_p, []),
     "hipc_stream": (_vp, [_vp]),
+    "hipc_set_option": (_int, [_vp, C.c_char_p, _int]),
+    "hipc_pool_stats": (_int, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "hipc_alloc": (_int, [_vp, _sz, C.POINTER(_vp)]),
     "hipc_free_deferred": (_int, [_vp, _vp]),
     "hipc_upload": (_int, [_vp, _vp, _sz, _vp, _sz]),
@@ -186,6 +189,27 @@ class Context:
     @property
     def stream(self) -> int:
         return self.lib.hipc_stream(self.handle)
+
+    def set_option(self, name: str, value: int):
+        """A route / launch-shape override (``hipc_set_option``); a negative value restores the default."""
+        self._check(self.lib.hipc_set_option(self.handle, name.encode(), int(value)))
+
+    @contextlib.contextmanager
+    def options(self, **values):
+        """``with ctx.options(HIPC_GEMM_TILE=128): ...`` -- overrides for the duration of the block."""
+        for k, v in values.items():
+            self.set_option(k, v)
+        try:
+            yield self
+        finally:
+            for k in values:
+                self.set_option(k, -1)
+
+    def pool_stats(self):
+        """(hits, misses, bytes waiting) of the allocation pool."""
+        h, m, b = _sz(), _sz(), _sz()
+        self._check(self.lib.hipc_pool_stats(self.handle, C.byref(h), C.byref(m), C.byref(b)))
+        return h.value, m.value, b.value
 
     # ---- buffers
     def alloc(self, nbytes: int) -> Buffer:

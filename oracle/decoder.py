@@ -123,3 +123,22 @@ class Decoder:
             xn = rmsnorm(x, nxt, c["rms_eps"])
         logits = self._lin(xn, 0, LM_HEAD)
         return logits, int(np.argmax(logits))
+
+
+def advance_state(token, pos, logits, max_seq):
+    """The loop state after one step: (token, pos, overflow).
+
+    ArgMax keeps the smallest index among equal maxima (shaders/reduction.rs:76-191); a row in which
+    no comparison succeeds (every logit NaN) yields index 0. A step asked for with the cache full
+    (pos == max_seq: row `pos` does not exist) changes nothing and reports overflow; the caller must
+    not have run the step's writes in that case.
+    """
+    if pos >= max_seq:
+        return token, pos, True
+    best, bi = -np.inf, None
+    for i, v in enumerate(np.asarray(logits, np.float32)):
+        if v > best:
+            best, bi = v, i
+    if bi is None:
+        bi = 0
+    return int(bi), pos + 1, False

@@ -47,18 +47,31 @@ DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / 
     (128, 4, 2, 130),    # three live chunks only
     (192, 2, 1, 100),    # no instance for this head_dim: the three-kernel path
 ]
-PATHS = [{}, {"HIPC_DEC_FUSED_GLUE": "0"}, {"HIPC_DEC_FUSED_ATTN": "0"}]
+PATHS = [{}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
+
+
+@pytest.fixture
+def route(ctx):
+    """Sets route options on the shared context for one test and restores the defaults afterwards."""
+    touched = []
+
+    def apply(options):
+        for k, v in options.items():
+            ctx.set_option(k, v)
+            touched.append(k)
+    yield apply
+    for k in touched:
+        ctx.set_option(k, -1)
 
 
 @pytest.mark.parametrize("env", PATHS, ids=["default", "separate-glue", "three-kernel-attention"])
 @pytest.mark.parametrize("hd,nq,nkv,p0", DEEP)
-def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, monkeypatch, hd, nq, nkv, p0, env):
+def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, route, hd, nq, nkv, p0, env):
     """Steps taken deep into a context whose cache rows hold random f16 values on both sides: the
     chunked attention (several passes per workgroup, the join in the output projection's prologue
     or in the merge kernel) against the oracle's softmax over the whole context."""
     from oracle import decoder as od
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)   # read when the decoder is created
+    route(env)                     # read when the decoder is created
     cfg = dict(SMALL, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd)
     steps, max_seq = 3, p0 + 8
     w = pkg.decoder.build_weights(cfg, seed=11)
@@ -97,13 +110,12 @@ WINDOWS = [  # (head_dim, query heads, kv heads, first position, window of layer
 
 @pytest.mark.parametrize("env", PATHS, ids=["default", "separate-glue", "three-kernel-attention"])
 @pytest.mark.parametrize("hd,nq,nkv,p0,w0,w1", WINDOWS)
-def test_sliding_windows_and_a_second_rotary_base(ctx, pkg, oracle, monkeypatch, hd, nq, nkv, p0, w0, w1, env):
+def test_sliding_windows_and_a_second_rotary_base(ctx, pkg, oracle, route, hd, nq, nkv, p0, w0, w1, env):
     """Local layers: the last `window` positions only, the step's own included (the reference's
     bound, shaders/attention.rs:202-214), rotating with their own base; against the oracle over a
     filled cache, across the step at which the window starts to cut."""
     from oracle import decoder as od
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    route(env)
     cfg = dict(SMALL, n_q_heads=nq, n_kv_heads=nkv, head_dim=hd, rope_theta=1.0e6)
     steps, max_seq = 5, p0 + 8
     w = pkg.decoder.build_weights(cfg, seed=12)
@@ -183,3 +195,86 @@ def test_refuses_incomplete_models_and_bad_shapes(ctx, pkg):
     dec.destroy()
     with pytest.raises(pkg.HipComputeError):
         pkg.decoder.Decoder(ctx, dict(SMALL, head_dim=48), 16)
+
+
+def test_the_cache_limit_is_kept_on_the_device(ctx, pkg, oracle):
+    """max_seq steps fit after a reset to 0; one more (eager or replayed) writes nothing, leaves token
+    and position alone and is reported by the next read -- the rule of oracle.decoder.advance_state."""
+    from oracle.decoder import advance_state
+    max_seq = 6
+    w = pkg.decoder.build_weights(SMALL, seed=5)
+    dec = pkg.decoder.Decoder(ctx, SMALL, max_seq)
+    dec.load(w)
+    dec.reset(3, 0)
+    tok, pos, over = 3, 0, False
+    for _ in range(max_seq):
+        dec.step()
+        got_tok, got_pos, logits, _ = dec.read(want_logits=True)
+        tok, pos, over = advance_state(tok, pos, logits, max_seq)
+        assert (got_tok, got_pos) == (tok, pos) and not over
+    assert pos == max_seq
+    k_before = ctx.download(dec.kv_cache(0)[0], np.float16, (SMALL["n_kv_heads"] * max_seq * SMALL["head_dim"],))
+    dec.step()                                           # one step too many
+    with pytest.raises(pkg.HipComputeError) as e:
+        dec.read()
+    assert e.value.code == 1 and "cache full" in e.value.message
+    tok2, pos2 = ctypes_state(ctx, dec)
+    assert (tok2, pos2) == advance_state(tok, pos, None, max_seq)[:2] == (tok, max_seq)
+    assert np.array_equal(ctx.download(dec.kv_cache(0)[0], np.float16, k_before.shape), k_before)
+    dec.reset(3, 0)                                      # a reset clears the flag
+    dec.step()
+    assert dec.read()[1] == 1
+    dec.destroy()
+
+
+def ctypes_state(ctx, dec):
+    """token and position as hipc_decoder_read fills them, whatever status it returns"""
+    import ctypes as C
+    tok, pos = C.c_int32(), C.c_int32()
+    ctx.lib.hipc_decoder_read(ctx.handle, dec.handle, C.byref(tok), C.byref(pos), None, None, 0)
+    return tok.value, pos.value
+
+
+def test_gemma3_1b_shape_at_context_2040(ctx, pkg, oracle):
+    """The decoder configuration at its real size -- 26 layers, hidden 1152, ffn 6912, 4 query heads on
+    1 kv head of 256, vocabulary 262144, 22 local layers (window 512, base 10000) and 4 global ones
+    (base 1e6) -- three steps from position 2040 over a cache filled with random f16 rows on both
+    sides, logits against the oracle at 2e-3 + 2e-3 |ref|. These are the code paths the tokens-per-
+    second figure runs: the one-item-per-thread norm prologue, the gated-GELU prologue of a
+    k-split down projection, the attention join of 64 chunks."""
+    from oracle import decoder as od
+    D = pkg.decoder
+    cfg = dict(D.GEMMA3_1B)
+    p0, steps = 2040, 3
+    max_seq = p0 + steps + 5
+    w = D.build_weights(cfg, seed=9)
+    dec = D.Decoder(ctx, cfg, max_seq)
+    dec.load(w)
+    ref = od.Decoder(w, max_seq)
+    for li in range(cfg["n_layers"]):
+        if (li + 1) % 6 != 0:
+            dec.set_layer_attention(li, 512, 10000.0), ref.set_layer_attention(li, 512, 10000.0)
+        else:
+            dec.set_layer_attention(li, 0, 1.0e6), ref.set_layer_attention(li, 0, 1.0e6)
+    rng = np.random.default_rng(2040)
+    for li in range(cfg["n_layers"]):
+        kptr, vptr = dec.kv_cache(li)
+        for ptr, dst in ((kptr, ref.k), (vptr, ref.v)):
+            rows = (rng.standard_normal((1, max_seq, 256)) * 0.5).astype(np.float16)
+            dst[li] = rows
+            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, rows.ctypes.data, rows.nbytes))
+    token = 1234
+    dec.reset(token, p0)
+    for pos in range(p0, p0 + steps):
+        dec.step()
+        got_tok, got_pos, logits, _ = dec.read(want_logits=True)
+        want_logits, want_tok = ref.step(token, pos)
+        assert got_pos == pos + 1
+        err = np.abs(logits - want_logits)
+        assert np.all(err <= 2e-3 + 2e-3 * np.abs(want_logits)), (pos, float(err.max()))
+        top2 = np.sort(want_logits)[-2:]
+        if top2[1] - top2[0] > 1e-2:
+            assert got_tok == want_tok, pos
+        token = got_tok
+    dec.destroy()
+    ctx.flush()

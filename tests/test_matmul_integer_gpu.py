@@ -224,3 +224,52 @@ def test_requantize_alone(ctx, pkg, oracle):
         assert np.array_equal(got, oracle.requantize(acc, bias, ratio, 11, zp, signed))
     got = pkg.ops.requantize(ctx, acc.reshape(-1)[:229], None, ratio[:1], 1, 7, False)   # ragged tail, scalar ratio
     assert np.array_equal(got, oracle.requantize(acc.reshape(-1)[:229], None, ratio[:1], 1, 7, False))
+
+
+SIGNS = [(np.uint8, np.int8), (np.uint8, np.uint8), (np.int8, np.int8), (np.int8, np.uint8)]
+
+
+def _mm_three_epilogues(ctx, pkg, oracle, m, k, n, a_dt, b_dt, seed):
+    """int32, rescaled float and requantised byte outputs of one product against the oracle."""
+    a = rc.pseudo_plus1(m * k, seed).view(a_dt).reshape(m, k)
+    b = rc.pseudo_plus1(k * n, seed + 1).view(b_dt).reshape(k, n)
+    za = -9 if a_dt == np.int8 else 200
+    zb = 17 if b_dt == np.int8 else 3
+    want = oracle.matmul_integer(a, b, za, zb)
+    weight = pkg.ops.Int8Weight(ctx, b)
+    assert np.array_equal(pkg.ops.matmul_integer(ctx, a, b, za, zb, weight=weight), want)
+    scale = np.float32(0.003)
+    bias = pkg.synth.uniform_f32(n, seed + 2, -0.5, 0.5)
+    got = pkg.ops.matmul_integer_scale_bias(ctx, a, b, za, zb, scale, bias, relu=True, weight=weight)
+    assert np.array_equal(got.view(np.uint32), oracle.rescale(want, scale, bias, relu=True).view(np.uint32))
+    ys = float(0.02 * 0.01 * 74 * 73 * np.sqrt(k) / 100.0)
+    got = pkg.ops.qlinear_matmul(ctx, a, 0.02, za, b, np.float32(0.01), zb, ys, 7, True, weight=weight)
+    assert np.array_equal(got, oracle.qlinear_matmul(a, 0.02, za, b, np.float32(0.01), zb, ys, 7, True))
+    weight.destroy()
+
+
+@pytest.mark.parametrize("a_dt,b_dt", SIGNS)
+@pytest.mark.parametrize("shape", [(2048, 384, 4096), (2017, 200, 4001), (3000, 256, 3000)], ids=lambda s: "M%d_K%d_N%d" % s)
+def test_many_tiles_take_the_128x128_kernel(ctx, pkg, oracle, shape, a_dt, b_dt):
+    """512 or more 128x128 tiles but fewer than 192 of 256x256 (or an A the large-tile kernel does not
+    take): the LDS-staged 128x128 kernel, in its aligned form (k a multiple of 128), its unaligned
+    form (k = 200, ragged rows and columns) and with an even stage count; every sign combination,
+    both zero points non-zero, all three epilogues."""
+    m, k, n = shape
+    _mm_three_epilogues(ctx, pkg, oracle, m, k, n, a_dt, b_dt, seed=61)
+
+
+ROUTES = [  # (options, M, K, N): every alternative route of the integer product once, forced in process
+    ({"HIPC_GEMM_TILE": 128, "HIPC_GEMM_BIG": 0, "HIPC_GEMM_SMALL": 0}, 300, 640, 260),
+    ({"HIPC_GEMM_TILE": 64, "HIPC_GEMM_BIG": 0, "HIPC_GEMM_SMALL": 0}, 1000, 1024, 520),
+    ({"HIPC_GEMM_BIG": 1}, 700, 384, 520),
+    ({"HIPC_GEMM_SMALL": 1, "HIPC_GEMM_BIG": 0}, 2100, 256, 1030),
+    ({"HIPC_GEMM_SMALL": 0, "HIPC_GEMM_BIG": 0}, 1000, 1024, 1024),
+]
+
+
+@pytest.mark.parametrize("options,m,k,n", ROUTES, ids=lambda v: str(v).replace(" ", "") if isinstance(v, dict) else str(v))
+def test_every_route_of_the_integer_product_can_be_forced(ctx, pkg, oracle, options, m, k, n):
+    with ctx.options(**options):
+        _mm_three_epilogues(ctx, pkg, oracle, m, k, n, np.uint8, np.int8, seed=71)
+        _mm_three_epilogues(ctx, pkg, oracle, m, k, n, np.int8, np.uint8, seed=73)

@@ -173,3 +173,39 @@ def test_refusals_and_short_buffers(ctx, pkg):
     assert e.value.code == 1
     y = pkg.ops.matmul_nbits(ctx, np.zeros((0, k), np.float32), B, scales, zp, k, n, bs)   # no rows: a no-op
     assert y.shape == (0, n)
+
+
+def _unpack(B, zp, k, n, bs):
+    nb = -(-k // bs)
+    flat = B.reshape(n, -1)
+    nib = np.empty((n, nb * bs), np.uint8)
+    nib[:, 0::2], nib[:, 1::2] = flat & 15, flat >> 4
+    z = np.empty((n, 2 * zp.shape[1]), np.uint8)
+    z[:, 0::2], z[:, 1::2] = zp & 15, zp >> 4
+    return nib[:, :k], z[:, :nb]
+
+
+@pytest.mark.parametrize("shape", [(1, 1152, 6912), (1, 6912, 1152), (8, 1152, 512)], ids=lambda s: "M%d_K%d_N%d" % s)
+def test_accuracy_levels(ctx, pkg, oracle, shape):
+    """accuracy_level 0 (unset), 2 and 3 let an f32 activation enter the matrix cores as two bf16 terms;
+    1 pins f32 and sends all 24 bits (three terms). Every level meets the operator's tolerance
+    against the oracle; level 1 is held to a tighter bound against the float64 product -- 2e-5 of
+    the row's largest output, what the f32 accumulation of the +128-biased block dots leaves --
+    and must not be worse than the default."""
+    m, k, n = shape
+    bs = 32
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=300 + n)
+    a = pkg.synth.normal_f32(m * k, 301).reshape(m, k)
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    nib, z = _unpack(B, zp, k, n, bs)
+    f64 = rc.matmul_nbits_f64(a, nib, z, scales.reshape(n, -1), bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    err = {}
+    for level in (0, 1, 2, 3):
+        got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, accuracy_level=level, weight=w)
+        assert close(got, want, RTOL32), (level, worst(got, want))
+        err[level] = float(np.max(np.abs(got - f64)))
+    w.destroy()
+    assert err[1] <= 2e-5 * float(np.max(np.abs(f64))), err
+    assert err[1] <= err[0] * 1.05 + 1e-7, err
+    assert err[2] == err[0] and err[3] == err[0], err     # the same kernel instance as the default

@@ -382,3 +382,123 @@ def test_gather_block_quantized_is_a_row_of_the_dequantised_table(oracle, pkg):
         blk = np.arange(100) // 32
         want = (nib[row].astype(np.float32) - zp[row][blk]) * scale[row][blk]
         assert np.array_equal(od.gather_block_quantized(table, row, 100, 32), want)
+
+
+# ---------------------------------------------------------------- the decode step as a whole
+
+def _dense_f64(lin, K, bs):
+    """(B, scales, zp) in the MatMulNBits layout -> float64 [N, K], written out from the format's
+    definition (low nibble first, zero-point nibble b & 1 of byte b / 2) without the oracle."""
+    B, scales, zp = lin
+    N, nb = B.shape[0], B.shape[1]
+    q = np.empty((N, nb * bs), np.float64)
+    flat = B.reshape(N, -1)
+    q[:, 0::2], q[:, 1::2] = flat & 15, flat >> 4
+    z = np.empty((N, 2 * zp.shape[1]), np.float64)
+    z[:, 0::2], z[:, 1::2] = zp & 15, zp >> 4
+    w = (q.reshape(N, nb, bs) - z[:, :nb, None]) * scales.reshape(N, nb, 1).astype(np.float64)
+    return w.reshape(N, nb * bs)[:, :K]
+
+
+def _step_f64(w, caches, token, pos, windows, thetas):
+    """One decode step in float64 from the layer formula of the C header (rmsnorm -> qkv -> per-head
+    norm + rotary -> f16 cache -> attention -> o -> post-norm residual -> pre-norm -> gated GELU ->
+    down -> post-norm residual; final norm -> lm_head). No call into oracle.decoder."""
+    from oracle import decoder as od
+    c = w.cfg
+    hd, nq, nkv, H, F, bs = c["head_dim"], c["n_q_heads"], c["n_kv_heads"], c["hidden"], c["ffn"], c["block_size"]
+
+    def rms(x, g):
+        return x / np.sqrt(np.mean(x * x) + c["rms_eps"]) * g.astype(np.float64)
+
+    def rope(x, theta):
+        half = hd // 2
+        ang = pos * theta ** (-2.0 * np.arange(half) / hd)
+        cs, sn = np.cos(ang), np.sin(ang)
+        return np.concatenate([x[:half] * cs - x[half:] * sn, x[half:] * cs + x[:half] * sn])
+
+    scale = c["attn_scale"] if c["attn_scale"] > 0 else 1.0 / np.sqrt(hd)
+    x = _dense_f64(w.embedding, H, bs)[token] * c["embed_scale"]
+    for li in range(c["n_layers"]):
+        n = lambda which: w.norms[(li, which)]
+        qkv = _dense_f64(w.linears[(li, od.QKV)], H, bs) @ rms(x, n(od.NORM_INPUT))
+        q = qkv[: nq * hd].reshape(nq, hd)
+        k = qkv[nq * hd: (nq + nkv) * hd].reshape(nkv, hd)
+        v = qkv[(nq + nkv) * hd:].reshape(nkv, hd)
+        K, V = caches[li]
+        for h in range(nkv):
+            K[h, pos] = rope(rms(k[h], n(od.NORM_K)), thetas[li]).astype(np.float16)
+            V[h, pos] = v[h].astype(np.float16)
+        first = max(0, pos + 1 - windows[li]) if windows[li] > 0 else 0
+        a = np.empty((nq, hd))
+        for h in range(nq):
+            qh = rope(rms(q[h], n(od.NORM_Q)), thetas[li])
+            kv = h // (nq // nkv)
+            s = K[kv, first: pos + 1].astype(np.float64) @ qh * scale
+            p = np.exp(s - s.max())
+            a[h] = (p / p.sum()) @ V[kv, first: pos + 1].astype(np.float64)
+        x = x + rms(_dense_f64(w.linears[(li, od.O)], nq * hd, bs) @ a.reshape(-1), n(od.NORM_POST_ATTN))
+        gu = _dense_f64(w.linears[(li, od.GATE_UP)], H, bs) @ rms(x, n(od.NORM_PRE_FFN))
+        g, u = gu[:F], gu[F:]
+        hcur = 0.5 * g * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (g + 0.044715 * g ** 3))) * u
+        x = x + rms(_dense_f64(w.linears[(li, od.DOWN)], F, bs) @ hcur, n(od.NORM_POST_FFN))
+    return _dense_f64(w.linears[(0, od.LM_HEAD)], H, bs) @ rms(x, w.norms[(0, od.NORM_FINAL)])
+
+
+_TINY = dict(n_layers=2, hidden=64, ffn=96, n_q_heads=4, n_kv_heads=2, head_dim=32, vocab=80, block_size=32,
+             rms_eps=1e-6, rope_theta=10000.0, attn_scale=0.0, embed_scale=8.0)
+
+
+def test_decoder_step_composition_against_a_float64_route(oracle, pkg):
+    """The wiring of Decoder.step (where the four norms sit, the order of the residual adds, the
+    embedding scale, the gate | up split, the window bound, the per-layer rotary base) against a
+    float64 evaluation with dense matrices, over several positions so that the cache and the
+    window are exercised. A misplaced norm or a swapped gate / up moves the logits by O(1)."""
+    from oracle import decoder as od
+    w = pkg.decoder.build_weights(_TINY, seed=21)
+    max_seq = 12
+    ref = od.Decoder(w, max_seq)
+    ref.set_layer_attention(1, 3, 500.0)
+    windows, thetas = [0, 3], [_TINY["rope_theta"], 500.0]
+    caches = [(np.zeros((2, max_seq, 32), np.float16), np.zeros((2, max_seq, 32), np.float16)) for _ in range(2)]
+    token = 7
+    for pos in range(8):
+        got, nxt = ref.step(token, pos)
+        want = _step_f64(w, caches, token, pos, windows, thetas)
+        assert got.dtype == np.float32 and got.shape == (80,)
+        assert np.all(np.abs(got - want) <= 1e-3 + 1e-3 * np.abs(want)), (pos, float(np.abs(got - want).max()))
+        assert np.ptp(want) > 0.5, "the case must not be degenerate"
+        assert nxt == int(np.argmax(got))
+        token = nxt
+
+
+def test_decoder_step_with_silent_branches_is_the_unembedded_embedding(oracle, pkg):
+    """With the output and down projections at zero (all scales 0) both residual branches add
+    rmsnorm(0) = 0, so the logits are lm_head(rmsnorm(embed_scale * embedding row, w_final)):
+    a closed form that involves none of the per-layer code."""
+    from oracle import decoder as od
+    w = pkg.decoder.build_weights(_TINY, seed=22)
+    for li in range(2):
+        for which in (od.O, od.DOWN):
+            B, scales, zp = w.linears[(li, which)]
+            w.linears[(li, which)] = (B, np.zeros_like(scales), zp)
+    ref = od.Decoder(w, 4)
+    for token in (0, 5, 79):
+        got, _ = ref.step(token, 1)
+        x = _dense_f64(w.embedding, 64, 32)[token] * _TINY["embed_scale"]
+        xn = x / np.sqrt(np.mean(x * x) + 1e-6) * w.norms[(0, od.NORM_FINAL)]
+        want = _dense_f64(w.linears[(0, od.LM_HEAD)], 64, 32) @ xn
+        assert np.all(np.abs(got - want) <= 1e-4 + 1e-4 * np.abs(want)), token
+
+
+def test_decoder_state_rule(oracle):
+    """advance_state: smallest index among equal maxima, index 0 when nothing compares, and a step
+    at a full cache changes nothing and is reported."""
+    from oracle.decoder import advance_state
+    logits = np.array([0.5, 3.0, -1.0, 3.0, 2.0], np.float32)
+    assert advance_state(9, 4, logits, 8) == (1, 5, False)
+    assert advance_state(9, 7, logits, 8) == (1, 8, False)          # the last row of the cache is usable
+    assert advance_state(9, 8, logits, 8) == (9, 8, True)           # full: nothing moves
+    assert advance_state(9, 2, np.full(5, np.nan, np.float32), 8) == (0, 3, False)
+    assert advance_state(9, 2, np.array([np.nan, -np.inf, 1.0], np.float32), 8) == (2, 3, False)
+    assert advance_state(9, 2, np.full(4, -np.inf, np.float32), 8)[0] == 0

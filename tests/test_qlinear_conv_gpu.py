@@ -112,8 +112,8 @@ def test_replays_from_a_graph_once_its_ratios_are_resident(ctx, pkg, oracle):
 
 
 def test_wide_decoder_variant(ctx, pkg, oracle):
-    """512 -> 512 channels, kernel 7, stride 1; T shortened to keep the oracle in seconds."""
-    X, W, w_scale, bias, kw = _qconv_case(pkg, 512, 512, 1024, 7, 1, seed=60)
+    """512 -> 512 channels, kernel 7, stride 1, T = 4096: the size the benchmark times."""
+    X, W, w_scale, bias, kw = _qconv_case(pkg, 512, 512, 4096, 7, 1, seed=60)
     geom, og = pkg.ConvGeom.make(X.shape, W.shape, **kw), oracle.conv_geom(X.shape, W.shape, **kw)
     ys = _y_scale(0.02, w_scale, 512 * 7)
     got = pkg.ops.qlinear_conv(ctx, X, 0.02, 128, W, w_scale, 0, ys, 128, bias, geom)
@@ -198,3 +198,75 @@ def test_refusals(ctx, pkg):
     bad = pkg.ConvGeom.make((1, 16, 1, 2), W.shape)     # the window does not fit
     with pytest.raises(ValueError):
         pkg.ops.conv_integer(ctx, X[..., :2], W, 0, 0, bad)
+
+
+@pytest.mark.parametrize("signs", [(np.uint8, np.int8), (np.int8, np.uint8)], ids=["u8xi8", "i8xu8"])
+def test_many_tiles_in_two_dimensions_take_the_128x128_kernel(ctx, pkg, oracle, signs):
+    """A 3x3 convolution over a 192 x 200 image: 2 x 300 tiles of 128x128, the LDS-staged
+    128x128 kernel in its gathering form (NHWC copy, padding taps read the zero point)."""
+    X, W, w_scale, bias, kw = _qconv_case(pkg, 32, 200, 200, 3, 1, seed=140, h=192, kh=3)
+    X, W = X.view(signs[0]), W.view(signs[1])
+    geom, og = pkg.ConvGeom.make(X.shape, W.shape, **kw), oracle.conv_geom(X.shape, W.shape, **kw)
+    x_zp = 100 if signs[0] == np.uint8 else -20
+    w_zp = 0 if signs[1] == np.int8 else 131
+    acc = pkg.ops.conv_integer(ctx, X, W, x_zp, w_zp, geom)
+    assert np.array_equal(acc, oracle.conv_integer(X, W, x_zp, w_zp, og))
+    got = pkg.ops.qlinear_conv(ctx, X, 0.03, x_zp, W, np.float32(0.004), w_zp, 0.7, -5, bias, geom, y_signed=True)
+    assert np.array_equal(got, oracle.qlinear_conv(X, 0.03, x_zp, W, np.float32(0.004), w_zp, 0.7, -5, bias, og, True))
+
+
+CONV_ROUTES = [  # every alternative route of a convolution along one axis, forced in process
+    {"HIPC_CONV_ROW": 0},                                               # NHWC copy + the k-split gathering kernel
+    {"HIPC_CONV_ROW": 0, "HIPC_GEMM_SMALL": 0, "HIPC_GEMM_TILE": 64},   # ... + LDS-staged 64x64 tiles
+    {"HIPC_CONV_ROW": 0, "HIPC_GEMM_SMALL": 0, "HIPC_GEMM_TILE": 128},  # ... + LDS-staged 128x128 tiles
+]
+
+
+@pytest.mark.parametrize("options", CONV_ROUTES, ids=lambda o: ",".join("%s=%d" % kv for kv in o.items()))
+def test_every_route_of_a_row_convolution_can_be_forced(ctx, pkg, oracle, options):
+    X, W, w_scale, bias, kw = _qconv_case(pkg, 96, 80, 700, 7, 3, seed=150, n=2)
+    geom, og = pkg.ConvGeom.make(X.shape, W.shape, **kw), oracle.conv_geom(X.shape, W.shape, **kw)
+    ys = _y_scale(0.02, w_scale, 96 * 7)
+    want_acc = oracle.conv_integer(X, W, 128, 0, og)
+    want = oracle.qlinear_conv(X, 0.02, 128, W, w_scale, 0, ys, 128, bias, og)
+    with ctx.options(**options):
+        assert np.array_equal(pkg.ops.conv_integer(ctx, X, W, 128, 0, geom), want_acc)
+        assert np.array_equal(pkg.ops.qlinear_conv(ctx, X, 0.02, 128, W, w_scale, 0, ys, 128, bias, geom), want)
+
+
+def test_a_recorded_graph_survives_scratch_growth_and_new_scales(ctx, pkg, oracle):
+    """A captured QLinearConv on the route that transposes into scratch, then a larger one run
+    eagerly (the scratch block must grow) with other scales on the same weight (new ratios), a flush,
+    and the replay: the graph still owns the block and the ratios it was recorded with."""
+    with ctx.options(HIPC_CONV_ROW=0):
+        X, W, w_scale, bias, kw = _qconv_case(pkg, 64, 64, 512, 7, 3, seed=160)
+        geom, og = pkg.ConvGeom.make(X.shape, W.shape, **kw), oracle.conv_geom(X.shape, W.shape, **kw)
+        ys = _y_scale(0.02, w_scale, 64 * 7)
+        weight = pkg.ops.ConvWeight(ctx, W, geom)
+        dX, dY, dB = ctx.upload(X), ctx.alloc(X.size), ctx.upload(bias.astype(np.int32))
+        run = lambda s: pkg.ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, 128, weight, w_scale, 0, s, 128, pkg.U8, dB, geom, dY)
+        run(ys)
+        ctx.flush()
+        ctx.capture_begin()
+        run(ys)
+        graph = ctx.capture_end()
+        # eager work that retires both blocks the graph names
+        Xb, Wb, wsb, bb, kwb = _qconv_case(pkg, 64, 64, 70000, 7, 3, seed=161, n=4)   # 18 MB to transpose: the scratch grows
+        gb, ogb = pkg.ConvGeom.make(Xb.shape, Wb.shape, **kwb), oracle.conv_geom(Xb.shape, Wb.shape, **kwb)
+        big = pkg.ops.qlinear_conv(ctx, Xb, 0.02, 128, Wb, wsb, 0, ys, 128, bb, gb)
+        assert np.array_equal(big[:, :, :, :300], oracle.qlinear_conv(Xb[:, :, :, :320], 0.02, 128, Wb, wsb, 0, ys, 128, bb,
+                                                                    oracle.conv_geom(Xb[:, :, :, :320].shape, Wb.shape, **kwb))[:, :, :, :300])
+        run(3 * ys)                        # new ratios on the recorded weight
+        ctx.flush()
+        filler = [ctx.alloc(1 << 20) for _ in range(8)]   # whatever was freed is handed out again
+        for b in filler:
+            ctx.fill(b, 0, 1 << 20, 0xFFFFFFFF)
+        ctx.flush()
+        ctx.graph_launch(graph)
+        got = ctx.download(dY, np.uint8, X.shape)
+        assert np.array_equal(got, oracle.qlinear_conv(X, 0.02, 128, W, w_scale, 0, ys, 128, bias, og))
+        ctx.graph_destroy(graph)
+        weight.destroy()
+        for b in [dX, dY, dB] + filler:
+            b.free()
+        ctx.flush()

@@ -90,3 +90,60 @@ def test_a_second_context_on_a_caller_stream(ctx, pkg, oracle):
         wy, ws, wz = oracle.dynamic_quantize_linear(x)
         assert np.array_equal(y, wy) and z == wz
     assert hip.hipStreamDestroy(stream) == 0
+
+
+def test_freed_blocks_are_handed_out_again_by_size_class(ctx):
+    """hipc_alloc serves a request from the blocks earlier frees of its size class left behind
+    (crates/vk-compute/src/buffer.rs:303-341): after a flush the same address comes back and no
+    device allocation happens."""
+    ctx.flush()
+    a = ctx.alloc(3000)                    # class 4096
+    first = a.ptr
+    a.free()
+    b = ctx.alloc(3500)                    # before the flush the block is still in use: another one
+    assert b.ptr != first
+    ctx.flush()
+    hits0, misses0, _ = ctx.pool_stats()
+    c = ctx.alloc(4096)
+    assert c.ptr == first
+    hits1, misses1, waiting = ctx.pool_stats()
+    assert (hits1, misses1) == (hits0 + 1, misses0)
+    big = ctx.alloc((5 << 20) + 1)         # whole MiB above 1 MiB: class 6 MiB
+    p = big.ptr
+    big.free()
+    ctx.flush()
+    again = ctx.alloc(6 << 20)
+    assert again.ptr == p
+    for x in (b, c, again):
+        x.free()
+    ctx.flush()
+
+
+def test_uploads_only_record(ctx):
+    """hipc_upload stages the bytes and returns: the source may be overwritten at once, uploads
+    larger than the staging ring arrive whole, and order with other stream work is call order."""
+    n = 50 << 20                            # three times the ring
+    src = np.arange(n // 4, dtype=np.uint32)
+    d = ctx.alloc(n)
+    ctx.fill(d, 0, n, 0)
+    ctx.upload(src, d)
+    src[:] = 0                              # the call has copied what it needs
+    ctx.fill(d, 4 * 1000, 4 * 10, 7)        # later stream work lands on top
+    out = ctx.download(d, np.uint32, (n // 4,))
+    want = np.arange(n // 4, dtype=np.uint32)
+    want[1000:1010] = 7
+    assert np.array_equal(out, want)
+    small = [ctx.upload(np.full(5, i, np.int32)) for i in range(300)]   # many small uploads share slots
+    for i in (0, 150, 299):
+        assert np.array_equal(ctx.download(small[i], np.int32, (5,)), np.full(5, i, np.int32))
+    for b in small + [d]:
+        b.free()
+    ctx.flush()
+
+
+def test_unknown_options_are_refused(ctx, pkg):
+    with pytest.raises(pkg.HipComputeError) as e:
+        ctx.set_option("HIPC_NO_SUCH_THING", 1)
+    assert e.value.code == 1
+    ctx.set_option("HIPC_GEMM_TILE", 128)
+    ctx.set_option("HIPC_GEMM_TILE", -1)
