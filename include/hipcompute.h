@@ -202,6 +202,21 @@ int hipc_decomposed_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor,
 int hipc_dynamic_quantize_linear_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor, float offset, float factor,
                                       int factor_first, void *Y, void *scale_out, void *zp_out, void *range);
 
+/*
+ * hipc_dynamic_quantize_linear (range == NULL) for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the
+ * reference. The call allocates nothing, on the device or through any library: the per-workgroup
+ * range pairs of the first pass live in a 16 KiB array that is part of the library's own device
+ * image (one copy per GPU, held until the process ends), whose address on the context's device was
+ * looked up when the context was created. Results are bit for bit those of
+ * hipc_dynamic_quantize_linear. n is limited to HIPC_DQL_STATIC_MAX_N elements (HIPC_ERR_INVALID
+ * beyond). Every call on one GPU shares that GPU's array, whatever the context: calls that may
+ * overlap on one GPU (two contexts, two streams) race; calls on one context are ordered by its stream.
+ */
+#define HIPC_DQL_STATIC_MAX_N ((int64_t)1 << 30)
+int hipc_dynamic_quantize_linear_static(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out,
+                                        void *zp_out);
+
 /* ------------------------------------------------------------ MatMulInteger */
 
 /* `packed_b` + `flipped_const` (interp.rs:2673-2768; shaders/matmul_integer.rs:135-158):

@@ -132,7 +132,8 @@ int create(int device, void *stream, bool adopt, hipc_ctx **out) {
     }
     for (const OptionName &o : kOptions) ctx->tune.*(o.field) = env_int(o.name);
     if (hipMalloc(&ctx->params, kParamBytes) != hipSuccess ||
-        hipMemsetAsync(ctx->params, 0, kParamBytes, ctx->stream) != hipSuccess) {
+        hipMemsetAsync(ctx->params, 0, kParamBytes, ctx->stream) != hipSuccess ||
+        dql_static_init(ctx) != HIPC_OK) {
         if (ctx->params) (void)hipFree(ctx->params);
         if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
         delete ctx;

@@ -14,6 +14,20 @@
 
 namespace hipc {
 
+// Range partials of hipc_dynamic_quantize_linear_static: {bits(-min), bits(max)} per workgroup of
+// the first pass, kParamPartsMax pairs = 16 KiB, part of the library's device image. In host code
+// this name is a stand-in, not a device address: dql_static_init asks the runtime where the array
+// lives on the context's device, and every launch gets that pointer.
+static __device__ __align__(256) __attribute__((used)) uint32_t scratch[2 * kParamPartsMax];
+
+int dql_static_init(hipc_ctx *ctx) {
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return HIPC_ERR_BACKEND;
+    ctx->dql_static = ptr;
+    return HIPC_OK;
+}
+
 // What the quantizer reads: x itself, or DecomposedGelu(x), the exact GELU written out as
 // Div -> Erf -> Add -> Mul -> Mul and fused by the reference (rewrite.rs:683-735). Every step rounds
 // on its own, as the five kernels it replaces do (shaders/elementwise.rs:71-118): this file is
@@ -180,8 +194,10 @@ using namespace hipc;
 
 namespace {
 
+// `parts`: where the per-workgroup range pairs of a call without a caller-owned slot go (the
+// context's own block, or this device's static array)
 int dql_launch(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out, void *zp_out, void *range, int range_ready,
-               const GeluParams &gelu) {
+               const GeluParams &gelu, uint32_t *parts = nullptr) {
     HIPC_REQUIRE(ctx, n >= 0, "DynamicQuantizeLinear: negative length");
     HIPC_REQUIRE(ctx, scale_out && zp_out, "DynamicQuantizeLinear: null scale or zero-point output");
     HIPC_REQUIRE(ctx, aligned(scale_out, 4), "DynamicQuantizeLinear: scale output must be 4-byte aligned");
@@ -201,7 +217,7 @@ int dql_launch(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out
     if (!range_ready && !range) {
         // no slot of the caller's to fill: per-workgroup pairs in the context's block, joined by the
         // second pass -- no clearing launch and no atomics
-        slot = reinterpret_cast<uint32_t *>(static_cast<char *>(ctx->params) + kParamParts);
+        slot = parts ? parts : reinterpret_cast<uint32_t *>(static_cast<char *>(ctx->params) + kParamParts);
         nparts = (int)std::min<long>(std::max<long>(ceil_div(n, 256 * 16), 1), kParamPartsMax);
         dql_range_kernel<<<(unsigned)nparts, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 1, gelu);
         HIPC_LAUNCHED(ctx);
@@ -237,6 +253,18 @@ int hipc_dynamic_quantize_linear(hipc_ctx *ctx, const void *X, int64_t n, void *
                                  void *range, int range_ready) {
     return entry(ctx, [&]() -> int {
         return dql_launch(ctx, X, n, Y, scale_out, zp_out, range, range_ready, GeluParams{0, 1.f, 0.f, 1.f, 0});
+    });
+}
+
+int hipc_dynamic_quantize_linear_static(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out, void *zp_out) {
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, n <= HIPC_DQL_STATIC_MAX_N, "DynamicQuantizeLinear (static): %ld elements exceed the limit of %ld", (long)n,
+                     (long)HIPC_DQL_STATIC_MAX_N);
+        HIPC_REQUIRE(ctx, ctx->dql_static, "DynamicQuantizeLinear (static): the static array was not found on this device");
+        // every pair the second pass reads is written by the first pass of this same call, so
+        // what an earlier (larger) call left in the array is never seen and nothing needs clearing
+        return dql_launch(ctx, X, n, Y, scale_out, zp_out, nullptr, 0, GeluParams{0, 1.f, 0.f, 1.f, 0},
+                          static_cast<uint32_t *>(ctx->dql_static));
     });
 }
 

@@ -77,6 +77,7 @@ struct hipc_ctx {
     int live_graphs = 0;
     hipc::Scratch scratch[hipc::kScratchSlots];
     void *params = nullptr;              // small device block: range slot, scalars, range partials
+    void *dql_static = nullptr;          // this device's address of the static range-partials array (see dynamic_quantize.hip)
     int cu_count = 256;
     hipc::Tuning tune;
     hipc::StageRing stage;
@@ -214,6 +215,9 @@ int allow_dynamic_lds(hipc_ctx *ctx, K kernel, size_t bytes, bool (&done)[kMaxDe
 int scratch_get(hipc_ctx *ctx, int slot, size_t bytes, void **out);
 // host bytes -> device through the context's pinned staging ring; records only (see StageRing)
 int stage_upload(hipc_ctx *ctx, void *dst, const void *host, size_t bytes);
+// looks up this device's address of the static range-partials array of the DynamicQuantizeLinear
+// variant that allocates nothing, and keeps it in ctx->dql_static (dynamic_quantize.hip)
+int dql_static_init(hipc_ctx *ctx);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }

@@ -104,6 +104,22 @@ def dynamic_quantize_linear(ctx: Context, x):
     return y, scale, zp
 
 
+def dynamic_quantize_linear_static(ctx: Context, x):
+    """The same through the entry point that allocates nothing (``hipc_dynamic_quantize_linear_static``)."""
+    x = np.ascontiguousarray(x, np.float32)
+    dX = ctx.upload(x)
+    dY = ctx.alloc(max(x.size, 4))
+    dP = ctx.alloc(8)
+    ctx._check(ctx.lib.hipc_dynamic_quantize_linear_static(ctx.handle, dX.ptr if x.size else None, x.size,
+                                                           dY.ptr if x.size else None, dP.ptr, dP.ptr + 4))
+    y = ctx.download(dY, np.uint8, x.shape)
+    scale = ctx.download(dP, np.float32, (1,))[0]
+    zp = int(ctx.download(dP, np.uint8, (1,), offset=4)[0])
+    for b in (dX, dY, dP):
+        b.free()
+    return y, scale, zp
+
+
 SQRT2_F32 = float(np.float32(np.sqrt(2.0)))
 
 

@@ -86,6 +86,7 @@ SIGNATURES = {
     "hipc_nbits_weight_bytes": (_sz, [_vp]),
     "hipc_matmul_nbits_packed": (_int, [_vp, _vp, _int, _vp, _vp, _i64, _int]),
     "hipc_dynamic_quantize_linear": (_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _int]),
+    "hipc_dynamic_quantize_linear_static": (_int, [_vp, _vp, _i64, _vp, _vp, _vp]),
     "hipc_decomposed_gelu": (_int, [_vp, _vp, _i64, _f, _f, _f, _int, _vp]),
     "hipc_dynamic_quantize_linear_gelu": (_int, [_vp, _vp, _i64, _f, _f, _f, _int, _vp, _vp, _vp, _vp]),
     "hipc_prepack_int8_b": (_int, [_vp, _vp, _int, _i64, _i64, C.POINTER(_vp)]),
