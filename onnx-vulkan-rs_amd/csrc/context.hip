@@ -109,7 +109,8 @@ const OptionName kOptions[] = {
     {"HIPC_PREFILL_SPLIT", &Tuning::prefill_split},
     {"HIPC_DEC_FUSED_GLUE", &Tuning::dec_fused_glue},
     {"HIPC_DEC_FUSED_ATTN", &Tuning::dec_fused_attn},
-    {"HIPC_DEC_PERSISTENT", &Tuning::dec_persistent},
+    {"HIPC_GEMV_LEAN", &Tuning::gemv_lean},
+    {"HIPC_DEC_LEAN", &Tuning::dec_lean},
 };
 
 int create(int device, void *stream, bool adopt, hipc_ctx **out) {

@@ -82,16 +82,18 @@ dec_embed_kernel(const DecState *st, const uint8_t *__restrict__ q, const float 
 // x += rmsnorm(y, w_post); xn = rmsnorm(x, w_next). One workgroup of 256; every operand is read once,
 // up front (hidden <= 256 * kNormPer), so the kernel costs one memory round trip and two reductions.
 constexpr int kNormPer = 8;
+// y may arrive as y_slices partial rows (the k slices of the product that made it), hidden apart.
 __global__ void __launch_bounds__(256)
-dec_norm_residual_kernel(const float *__restrict__ y, const float *__restrict__ w_post, const float *__restrict__ w_next,
-                         int hidden, float eps, float *__restrict__ x, float *__restrict__ xn) {
+dec_norm_residual_kernel(const float *__restrict__ y, int y_slices, const float *__restrict__ w_post, const float *__restrict__ w_next,
+                         int hidden, float eps, const float *__restrict__ x_in, float *__restrict__ x, float *__restrict__ xn) {
     __shared__ float red[4];
     float yv[kNormPer], xv[kNormPer], wp[kNormPer], wn[kNormPer];
 #pragma unroll
     for (int e = 0; e < kNormPer; e++) {
         const int c = threadIdx.x + e * 256;
         const bool ok = c < hidden;
-        yv[e] = ok ? y[c] : 0.f, xv[e] = ok ? x[c] : 0.f, wp[e] = ok ? w_post[c] : 0.f, wn[e] = ok ? w_next[c] : 0.f;
+        yv[e] = ok ? y[c] : 0.f, xv[e] = ok ? x_in[c] : 0.f, wp[e] = ok ? w_post[c] : 0.f, wn[e] = ok ? w_next[c] : 0.f;
+        for (int s = 1; s < y_slices; s++) yv[e] += ok ? y[(size_t)s * hidden + c] : 0.f;
     }
     float sq = 0.f;
 #pragma unroll
@@ -687,6 +689,13 @@ struct hipc_decoder {
     float theta2 = 0.f;         // the second rotary base (0: none in use)
     float *x2 = nullptr;        // second buffer of the residual stream
     bool fused_glue = false;    // norms, residual adds and the gated GELU run inside the GEMV prologues
+    // The default path: every per-layer product on the one-row kernel built for latency, the gated
+    // GELU in the gate|up product's epilogue (its weight prepacked with interleaved halves), the
+    // output and down projections cut into k slices whose partial rows the next kernel adds up.
+    bool lean = false;
+    int o_slices = 1, down_slices = 1;
+    float *yo = nullptr, *yd = nullptr;      // [o_slices][hidden], [down_slices][hidden] partial rows
+    uint4 *h_split = nullptr;                // the gated row in operand order (see LeanArgs)
     int nsplit = 0;
     bool one_launch_attn = false;  // head_dim and group size have an instance of dec_attn_chunks_kernel
     std::vector<void *> owned;
@@ -785,6 +794,33 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         d->fused_glue = c.hidden % 8 == 0 && c.ffn % 8 == 0 && ctx->tune.dec_fused_glue != 0;
         d->one_launch_attn = (c.head_dim == 64 || c.head_dim == 128 || c.head_dim == 256) && (G == 1 || G == 2 || G == 4 || G == 8) &&
                              ctx->tune.dec_fused_attn != 0;
+        // the lean path (the dec_lean option set to 0 keeps the streaming kernel and its prologues)
+        {
+            const int n_cg_h = (int)ceil_div(c.hidden, 128), n_cg_o = (int)ceil_div((int64_t)c.n_q_heads * c.head_dim, 128);
+            const int n_cg_f = (int)ceil_div(c.ffn, 128);
+            d->lean = d->fused_glue && d->one_launch_attn && ctx->tune.dec_lean != 0 && c.ffn % 16 == 0 && n_cg_h <= 32 &&
+                      c.hidden % 8 == 0;
+            // output projection: a k slice is one head (or one 128-k tile when heads are shorter), at most 8 slices
+            int o_tiles = std::max(1, c.head_dim / 128);
+            while (ceil_div(n_cg_o, o_tiles) > 8 && o_tiles < 4) o_tiles *= 2;
+            d->o_slices = (int)ceil_div(n_cg_o, o_tiles);
+            if (d->o_slices > 8 || o_tiles > 4) d->lean = false;
+            // down projection: 18 k tiles per slice (six wavefronts of three tiles), at most 8 slices
+            d->down_slices = (int)std::max<int64_t>(1, ceil_div(n_cg_f, 18));
+            if (d->down_slices > 8) d->lean = false;
+            if (d->lean) {
+                A(&d->yo, (size_t)d->o_slices * c.hidden), A(&d->yd, (size_t)d->down_slices * c.hidden);
+                const size_t chunks = (size_t)n_cg_f * 4;
+                A(&d->h_split, chunks * 2 * 4);
+                // the join in the output projection's prologue reads a chunk's partials before it knows whether
+                // the chunk is live (and weighs them with zero if not): they must be finite from the start
+                if (rc == HIPC_OK &&
+                    (hipMemsetAsync(d->h_split, 0, chunks * 2 * 4 * 16, ctx->stream) != hipSuccess ||
+                     hipMemsetAsync(d->part_o, 0, parts * c.head_dim * 4, ctx->stream) != hipSuccess ||
+                     hipMemsetAsync(d->part_ml, 0, parts * 2 * 4, ctx->stream) != hipSuccess))
+                    rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the gated row and the attention partials");
+            }
+        }
         if (rc == HIPC_OK) {
             for (DecLayer &l : d->layers) {  // an unwritten cache row must not hold NaN bit patterns
                 if (hipMemsetAsync(l.k_cache, 0, kv * 2, ctx->stream) != hipSuccess || hipMemsetAsync(l.v_cache, 0, kv * 2, ctx->stream) != hipSuccess)
@@ -840,7 +876,8 @@ int hipc_decoder_set_linear(hipc_ctx *ctx, hipc_decoder *d, int layer, int which
             delete *slot;
             *slot = nullptr;
         }
-        return nbits_prepack(ctx, B, b_len, scales, HIPC_F32, scales_len, zp, zp_len, K, N, c.block_size, slot);
+        const int half = (d->lean && which == HIPC_DEC_GATE_UP) ? c.ffn : 0;
+        return nbits_prepack(ctx, B, b_len, scales, HIPC_F32, scales_len, zp, zp_len, K, N, c.block_size, slot, half);
     });
 }
 
@@ -945,7 +982,53 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
         // branch into the stream reads one and (its first workgroup) writes the other.
         float *xc = d->x, *xo = d->x2;
-        for (int li = 0; li < c.n_layers; li++) {
+        for (int li = 0; li < c.n_layers && d->lean; li++) {
+            DecLayer &l = d->layers[li];
+            LeanPlan pl;
+            // qkv: row = rmsnorm(x', w_input), x' = x + rmsnorm(sum of the down projection's partial rows, w_post_ffn of the layer before)
+            {
+                LeanArgs a{};
+                a.x = xc, a.w_in = l.norm[HIPC_DEC_NORM_INPUT], a.x_out = xo, a.eps = c.rms_eps;
+                if (li > 0) a.yparts = d->yd, a.y_slices = d->down_slices, a.w_post = d->layers[li - 1].norm[HIPC_DEC_NORM_POST_FFN];
+                a.Y = d->qkv;
+                HIPC_REQUIRE(ctx, lean_plan(ctx, l.qkv, 1, 1, &pl), "decoder: no launch plan for the qkv projection");
+                if ((rc = lean_gemv(ctx, l.qkv, pl, a, 2, 0, terms)) != HIPC_OK) return rc;
+                std::swap(xc, xo);
+            }
+            if ((rc = launch_attn_chunks(ctx, d, l, scale)) != HIPC_OK) return rc;
+            // output projection: a k slice per head, joined from the attention partials; partial rows out
+            {
+                LeanArgs a{};
+                a.part_o = d->part_o, a.part_ml = d->part_ml, a.pos = &d->state->pos;
+                a.lg_group = __builtin_ctz((unsigned)(c.n_q_heads / c.n_kv_heads)), a.lg_hd = __builtin_ctz((unsigned)c.head_dim);   // powers of two where the one-launch attention runs
+                a.n_kv = c.n_kv_heads, a.window = l.window;
+                a.Y = d->yo;
+                const int per_slice = (int)ceil_div(l.o->n_cg, d->o_slices);
+                pl = LeanPlan{1, per_slice, 4, d->o_slices};   // four wavefronts, each all k tiles of the slice: no sum over wavefronts
+                if ((rc = lean_gemv(ctx, l.o, pl, a, 3, 0, terms)) != HIPC_OK) return rc;
+            }
+            // gate | up: row = rmsnorm(x'', w_pre_ffn), x'' = x' + rmsnorm(sum of the output projection's partial rows, w_post_attn);
+            // epilogue gelu_tanh(gate) * up in operand order
+            {
+                LeanArgs a{};
+                a.x = xc, a.w_in = l.norm[HIPC_DEC_NORM_PRE_FFN], a.x_out = xo, a.eps = c.rms_eps;
+                a.yparts = d->yo, a.y_slices = d->o_slices, a.w_post = l.norm[HIPC_DEC_NORM_POST_ATTN];
+                a.h_split = d->h_split;
+                HIPC_REQUIRE(ctx, lean_plan(ctx, l.gate_up, 1, 2, &pl), "decoder: no launch plan for the gate | up projection");
+                if ((rc = lean_gemv(ctx, l.gate_up, pl, a, 2, 1, terms)) != HIPC_OK) return rc;
+                std::swap(xc, xo);
+            }
+            // down: the gated row straight into the operand registers; partial rows out
+            {
+                LeanArgs a{};
+                a.a_split = d->h_split;
+                a.Y = d->yd;
+                HIPC_REQUIRE(ctx, lean_plan(ctx, l.down, d->down_slices, 1, &pl, 8),
+                             "decoder: no launch plan for the down projection");
+                if ((rc = lean_gemv(ctx, l.down, pl, a, 4, 0, terms)) != HIPC_OK) return rc;
+            }
+        }
+        for (int li = 0; li < c.n_layers && !d->lean; li++) {
             DecLayer &l = d->layers[li];
             if (d->fused_glue && li > 0) {
                 GemvPrologue pro;
@@ -992,22 +1075,23 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 gelu.mode = 1;
                 if ((rc = nbits_gemv(ctx, d->gu, HIPC_F32, l.down, d->y, 1, terms, &gelu)) != HIPC_OK) return rc;
             } else {
-                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->xn);
+                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, 1, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->x, d->xn);
                 HIPC_LAUNCHED(ctx);
                 if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.gate_up, d->gu, 1, terms)) != HIPC_OK) return rc;
                 dec_gelu_mul_kernel<<<(unsigned)ceil_div(c.ffn, 256), 256, 0, s>>>(d->gu, c.ffn, d->h);
                 HIPC_LAUNCHED(ctx);
                 if ((rc = nbits_gemv(ctx, d->h, HIPC_F32, l.down, d->y, 1, terms)) != HIPC_OK) return rc;
                 const float *next = li + 1 < c.n_layers ? d->layers[li + 1].norm[HIPC_DEC_NORM_INPUT] : d->final_norm;
-                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->xn);
+                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, 1, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->x, d->xn);
                 HIPC_LAUNCHED(ctx);
             }
         }
         if (d->fused_glue) {
             // the unembedding streams ~200 MB: its workgroups start on the weights at once and the
             // final norm stays a launch of its own
-            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], d->final_norm, c.hidden,
-                                                       c.rms_eps, xc, d->xn);
+            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->lean ? d->yd : d->y, d->lean ? d->down_slices : 1,
+                                                       d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], d->final_norm, c.hidden,
+                                                       c.rms_eps, xc, xc, d->xn);
             HIPC_LAUNCHED(ctx);
         }
         if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;

@@ -45,7 +45,8 @@ struct Tuning {
     int prefill_split = -1;   // HIPC_PREFILL_SPLIT  0 never splits k, n forces n ways
     int dec_fused_glue = -1;  // HIPC_DEC_FUSED_GLUE 0 keeps the separate norm / GELU kernels (read when a decoder is created)
     int dec_fused_attn = -1;  // HIPC_DEC_FUSED_ATTN 0 keeps the three-kernel attention (read when a decoder is created)
-    int dec_persistent = -1;  // HIPC_DEC_PERSISTENT 0: one launch per operator; 1: the whole step in one persistent launch
+    int gemv_lean = -1;       // HIPC_GEMV_LEAN      0: one-row products keep the streaming GEMV kernel
+    int dec_lean = -1;        // HIPC_DEC_LEAN       0: the decoder keeps the streaming GEMV and its prologues (read when a decoder is created)
 };
 
 // Pinned staging ring of hipc_upload: the bytes are copied into a slot and travel from there, so the
@@ -101,6 +102,7 @@ struct hipc_graph {
 struct hipc_nbits_weight {
     int64_t K = 0, N = 0, block_size = 0;
     int n_tiles = 0, n_cg = 0, SG = 0;
+    int interleave_half = 0;  // > 0: column tiles alternate between the two halves of N (see mmnb_prepack_kernel)
     uint4 *Wq = nullptr;
     float *Sc = nullptr;
     uint8_t *Zb = nullptr;
@@ -226,7 +228,8 @@ inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_
 
 // MatMulNBits pieces other operators of the library build on (the caller holds the lock)
 int nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype, size_t scales_len,
-                  const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size, hipc_nbits_weight **out);
+                  const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size, hipc_nbits_weight **out,
+                  int interleave_half = 0);
 void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
 // rows [0, M), M <= 16, of A against a prepacked weight; `terms` = bf16 terms per activation (2 or 3)
 // What the single activation row of a decode GEMV is computed from (mode 0 / null: A as given):
@@ -267,6 +270,44 @@ __host__ __device__ inline int attn_live_chunks(int total) {
 __host__ __device__ inline int attn_first(int total, int window) { return window > 0 && total > window ? total - window : 0; }
 int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
                const GemvPrologue *pro = nullptr);
+
+// ---- the latency-built kernel for one f32 row (gemv_lean.hip) -------------------------------------
+// A row "in operand order": per 32-k chunk c, NT terms x 4 k groups of 8 bf16 (16 bytes each), term
+// major -- split[(c * NT + term) * 4 + group] -- so that a lane's matrix-core A operand is one
+// 16-byte load. (The sums over a quantisation block's activations, which take the +128 bias of the
+// weights out again, are formed by the consumer on the matrix cores: a product against ones.)
+struct LeanArgs {
+    const uint4 *Wq;
+    const float *Sc;
+    const uint8_t *Zb;
+    int K, N, n_tiles, n_cg;
+    int WK, KT, WN, slices;      // wavefronts along k, k tiles per wavefront (<= 4), column tiles per workgroup, k slices (gridDim.y)
+    uint32_t nib_mask, magic;    // 0x000f000f and 0x43004300 (bf16 128.0 in both halves)
+    const float *A;              // PRO 0: the row
+    // PRO 2: row = rmsnorm(x', w_in), x' = x + rmsnorm(sum of y_slices rows of yparts, w_post) (x' = x when yparts is null);
+    //        workgroup (0, 0) also writes x' to x_out
+    const float *x, *yparts, *w_post, *w_in;
+    float *x_out;
+    int y_slices;
+    float eps;
+    // PRO 3: the attention output joined from the flash-decoding partials (see GemvPrologue mode 3)
+    const float *part_o, *part_ml;
+    const int *pos;
+    int lg_group, lg_hd, n_kv, window;   // log2 of the query heads per kv head and of head_dim (both powers of two), kv heads
+    // PRO 4: the row in operand order
+    const uint4 *a_split;
+    float *Y;                    // EPI 0: [slices][N] partial rows (the row itself when slices == 1)
+    // EPI 1: gelu_tanh(gate) * up of the interleaved (gate, up) tile pairs, in operand order
+    uint4 *h_split;
+};
+struct LeanPlan {
+    int WK, KT, WN, slices;
+};
+// false when the shape does not fit the kernel (k tiles per wavefront would exceed 4)
+bool lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int WN, LeanPlan *out, int max_waves = 16);
+// `a` carries the prologue / epilogue operands; weight and launch-shape fields are filled in here
+int lean_gemv(hipc_ctx *ctx, const hipc_nbits_weight *w, const LeanPlan &pl, LeanArgs a, int pro, int epi, int NT);
+
 int64_t nbits_cols(const hipc_nbits_weight *w);
 int64_t nbits_depth(const hipc_nbits_weight *w);
 // f16 activations, any M: tiled matrix-core kernel that dequantises the weight on its way to LDS.

@@ -112,14 +112,21 @@ template <typename ST>
 __global__ void __launch_bounds__(256)
 mmnb_prepack_kernel(const uint32_t *__restrict__ B, const ST *__restrict__ scales, const uint8_t *__restrict__ zp,
                     uint4 *__restrict__ Wq, float *__restrict__ Sc, uint8_t *__restrict__ Zb, int N, int n_blocks,
-                    int row_words, int zp_row, long n_tile_total, int n_cg, int cpb_shift, int SG) {
+                    int row_words, int zp_row, long n_tile_total, int n_cg, int cpb_shift, int SG, int half) {
     const long idx = (long)blockIdx.x * 256 + threadIdx.x;
     const long tile = idx >> 6;
     if (tile >= n_tile_total) return;
     const int lane = (int)(idx & 63);
     const int nt = (int)(tile / n_cg), cg = (int)(tile % n_cg);
     const int i16 = lane & 15, w = lane >> 4;
-    const int n = nt * 16 + i16;
+    // half > 0: the weight is two matrices side by side ([gate | up], `half` columns each) and the
+    // packed column tiles alternate between them: tile 2 b holds columns 16 b .. of the first, tile
+    // 2 b + 1 the same columns of the second, so that one workgroup holds both halves of an output
+    int n = nt * 16 + i16;
+    if (half > 0) {
+        const int c = (nt >> 1) * 16 + i16;
+        n = c < half ? c + (nt & 1) * half : N;
+    }
     uint32_t v[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -838,6 +845,18 @@ void launch_gemv_nt(const GemvArgs &a, int pro, int NT, int NR, int SG, dim3 gri
 // rows [0, M) with M <= 16 of one activation matrix against a prepacked weight
 int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int NT,
                 const GemvPrologue *pro = nullptr) {
+    HIPC_REQUIRE(ctx, w->interleave_half == 0, "MatMulNBits gemv: this weight was prepacked with interleaved halves for the decoder");
+    // one plain f32 row on a narrow output: the kernel built for latency (gemv_lean.hip); the
+    // gemv_lean option set to 0 keeps this kernel (tuning, tests)
+    if (M == 1 && a_dtype == HIPC_F32 && !(pro && pro->mode) && aligned(A, 16) && aligned(Y, 4) && w->n_tiles < 2048 &&
+        ctx->tune.gemv_lean != 0) {
+        LeanPlan pl;
+        if (lean_plan(ctx, w, 1, 1, &pl)) {
+            LeanArgs la{};
+            la.A = static_cast<const float *>(A), la.Y = static_cast<float *>(Y);
+            return lean_gemv(ctx, w, pl, la, 0, 0, NT);
+        }
+    }
     GemvArgs a{};
     a.A = A, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = Y, a.Ypart = nullptr;
     a.M = M, a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
@@ -964,8 +983,10 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
 // The same operations for callers inside the library that already hold the context's lock.
 int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype,
                         size_t scales_len, const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size,
-                        hipc_nbits_weight **out) {
+                        hipc_nbits_weight **out, int interleave_half) {
     *out = nullptr;
+    HIPC_REQUIRE(ctx, interleave_half == 0 || (interleave_half % 16 == 0 && 2 * (int64_t)interleave_half == N),
+                 "MatMulNBits prepack: interleaved halves of %d columns do not make up N=%ld in whole tiles", interleave_half, (long)N);
     HIPC_REFUSE(ctx, ctx->capturing, "MatMulNBits prepack while a capture is open");
     int rc = check_nbits_shape(ctx, 1, K, N, block_size, b_len, scales_len, zp, zp_len, scale_dtype);
     if (rc != HIPC_OK) return rc;
@@ -975,6 +996,7 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
                 (long)block_size);
     hipc_nbits_weight *w = new hipc_nbits_weight();
     w->K = K, w->N = N, w->block_size = block_size;
+    w->interleave_half = interleave_half;
     const int n_blocks = (int)ceil_div(K, block_size);
     const int n_chunks = (int)ceil_div(K, 32);
     w->n_tiles = (int)ceil_div(N, 16);
@@ -1008,11 +1030,11 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
     if (scale_dtype == HIPC_F16)
         mmnb_prepack_kernel<__half><<<grid, block, 0, ctx->stream>>>(
             static_cast<const uint32_t *>(B), static_cast<const __half *>(scales), static_cast<const uint8_t *>(zp),
-            w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG);
+            w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, interleave_half);
     else
         mmnb_prepack_kernel<float><<<grid, block, 0, ctx->stream>>>(
             static_cast<const uint32_t *>(B), static_cast<const float *>(scales), static_cast<const uint8_t *>(zp),
-            w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG);
+            w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, interleave_half);
     e = hipGetLastError();
     if (e != hipSuccess) {
         cleanup();

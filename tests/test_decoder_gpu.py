@@ -47,7 +47,7 @@ DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / 
     (128, 4, 2, 130),    # three live chunks only
     (192, 2, 1, 100),    # no instance for this head_dim: the three-kernel path
 ]
-PATHS = [{}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
+PATHS = [{}, {"HIPC_DEC_LEAN": 0}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
 
 
 @pytest.fixture
@@ -64,7 +64,7 @@ def route(ctx):
         ctx.set_option(k, -1)
 
 
-@pytest.mark.parametrize("env", PATHS, ids=["default", "separate-glue", "three-kernel-attention"])
+@pytest.mark.parametrize("env", PATHS, ids=["default", "streaming-gemv", "separate-glue", "three-kernel-attention"])
 @pytest.mark.parametrize("hd,nq,nkv,p0", DEEP)
 def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, route, hd, nq, nkv, p0, env):
     """Steps taken deep into a context whose cache rows hold random f16 values on both sides: the
@@ -108,7 +108,7 @@ WINDOWS = [  # (head_dim, query heads, kv heads, first position, window of layer
 ]
 
 
-@pytest.mark.parametrize("env", PATHS, ids=["default", "separate-glue", "three-kernel-attention"])
+@pytest.mark.parametrize("env", PATHS, ids=["default", "streaming-gemv", "separate-glue", "three-kernel-attention"])
 @pytest.mark.parametrize("hd,nq,nkv,p0,w0,w1", WINDOWS)
 def test_sliding_windows_and_a_second_rotary_base(ctx, pkg, oracle, route, hd, nq, nkv, p0, w0, w1, env):
     """Local layers: the last `window` positions only, the step's own included (the reference's

@@ -209,3 +209,22 @@ def test_accuracy_levels(ctx, pkg, oracle, shape):
     assert err[1] <= 2e-5 * float(np.max(np.abs(f64))), err
     assert err[1] <= err[0] * 1.05 + 1e-7, err
     assert err[2] == err[0] and err[3] == err[0], err     # the same kernel instance as the default
+
+
+@pytest.mark.parametrize("shape", [(1, 1152, 6912, 32, True), (1, 6912, 1152, 32, True), (1, 2048, 2560, 128, False),
+                                   (1, 300, 100, 64, True), (1, 1024, 48, 32, True)], ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_one_row_on_the_streaming_kernel(ctx, pkg, oracle, shape):
+    """One f32 row takes the kernel built for latency by default; with the HIPC_GEMV_LEAN option at 0 the
+    same product runs on the streaming kernel: both against the oracle, and against each other."""
+    m, k, n, bs, with_zp = shape
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=400 + n, with_zp=with_zp)
+    a = pkg.synth.normal_f32(m * k, 401).reshape(m, k)
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    lean = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    with ctx.options(HIPC_GEMV_LEAN=0):
+        streaming = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    assert close(lean, want, RTOL32), ("lean", worst(lean, want))
+    assert close(streaming, want, RTOL32), ("streaming", worst(streaming, want))
+    assert close(lean, streaming, RTOL32)
