@@ -281,11 +281,9 @@ def bench_decoder(pkg, ctx, steps, warmup, context=2048):
     dec = D.Decoder(ctx, cfg, max_seq)
     dec.load(w)
     rng = np.random.default_rng(1)
-    filler = (rng.standard_normal(context * cfg["head_dim"]) * 0.5).astype(np.float16)
+    filler = (rng.standard_normal((cfg["n_kv_heads"], context, cfg["head_dim"])) * 0.5).astype(np.float16)
     for li in range(cfg["n_layers"]):
-        k, v = dec.kv_cache(li)
-        for ptr in (k, v):
-            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, filler.ctypes.data, filler.nbytes))
+        dec.fill_cache(li, filler, filler)
     log(f"[bench] decoder: weights built and loaded in {time.time() - t0:.1f}s")
     def timed():
         dec.reset(1234, context - 1)

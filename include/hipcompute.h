@@ -389,7 +389,11 @@ int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *dec, const void *B, 
 int hipc_decoder_set_layer_attention(hipc_ctx *ctx, hipc_decoder *dec, int layer, int32_t window, float rope_theta);
 /* the token the next step consumes and its position (= tokens already in the cache) */
 int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *dec, int32_t token, int32_t pos);
-/* device pointers of one layer's resident f16 cache, [n_kv_heads, max_seq, head_dim] each */
+/* Device pointers of one layer's resident f16 cache. Keys: [n_kv_heads, max_seq, head_dim]. Values are
+ * kept transposed, [n_kv_heads, head_dim, v_stride] with v_stride = max_seq rounded up to a multiple of
+ * 64, so that the positions a channel is summed over are consecutive (a matrix-core operand is then
+ * one 16-byte load). A caller that fills the cache itself (a prefill) writes position t of channel c of
+ * kv head h at v_cache[(h * head_dim + c) * v_stride + t]. */
 int hipc_decoder_kv_cache(hipc_ctx *ctx, hipc_decoder *dec, int layer, void **k_cache, void **v_cache);
 /* enqueue one decode step (capturable) */
 int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *dec);

@@ -23,6 +23,7 @@
 #include <vector>
 
 #include "internal.h"
+#include "lanes.h"
 
 namespace hipc {
 
@@ -114,10 +115,10 @@ dec_norm_residual_kernel(const float *__restrict__ y, int y_slices, const float 
 }
 
 // One workgroup per head of the fused qkv vector: q heads and k heads get a per-head RMS norm and
-// the half-split rotary embedding at `pos`; k and v go to the f16 cache row `pos`; q stays f32.
+// the half-split rotary embedding at `pos`; k goes to the f16 cache row `pos`, v to column `pos` of the transposed value cache; q stays f32.
 __global__ void __launch_bounds__(256)
 dec_qkv_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
-               const float *__restrict__ k_norm, int n_q, int n_kv, int hd, float eps, float theta, int max_seq,
+               const float *__restrict__ k_norm, int n_q, int n_kv, int hd, float eps, float theta, int max_seq, int v_stride,
                float *__restrict__ q_out, __half *__restrict__ k_cache, __half *__restrict__ v_cache) {
     __shared__ float red[4];
     __shared__ float buf[512];
@@ -129,7 +130,7 @@ dec_qkv_kernel(const DecState *st, const float *__restrict__ qkv, const float *_
     if (!is_q && !is_k) {  // a value head: straight into the cache
         const int kvh = head - n_q - n_kv;
         for (int d = threadIdx.x; d < hd; d += 256)
-            v_cache[((size_t)kvh * max_seq + pos) * hd + d] = __float2half(src[d]);
+            v_cache[((size_t)kvh * hd + d) * v_stride + pos] = __float2half(src[d]);
         return;
     }
     const float *w = is_q ? q_norm : k_norm;
@@ -161,7 +162,7 @@ constexpr int kAttnChunk = 16;
 constexpr int kMaxGroup = 8;
 __global__ void __launch_bounds__(256)
 dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const __half *__restrict__ k_cache,
-                        const __half *__restrict__ v_cache, int n_q, int n_kv, int hd, int max_seq, float scale, int window,
+                        const __half *__restrict__ v_cache, int n_q, int n_kv, int hd, int max_seq, int v_stride, float scale, int window,
                         float *__restrict__ part_ml, float *__restrict__ part_o) {
     __shared__ float qs[kMaxGroup * 512];
     __shared__ float sc[kMaxGroup][kAttnChunk];
@@ -180,15 +181,20 @@ dec_attn_partial_kernel(const DecState *st, const float *__restrict__ q, const _
             for (int i = tid; i < G * hd; i += 256) part_o[((size_t)kvh * nsplit + split) * G * hd + i] = 0.f;
         return;
     }
-    // values first: thread d owns channel d (and d + 256) of every row of the chunk
+    // values first: thread d owns channel d (and d + 256): the chunk's 16 positions are 32 consecutive
+    // bytes of the transposed cache (positions past the end have weight zero below)
     float vreg[2][kAttnChunk];
+    static_assert(kAttnChunk == 16, "two 16-byte loads per channel");
 #pragma unroll
     for (int c = 0; c < 2; c++) {
-        const int d = tid + c * 256;
+        const int d = min(tid + c * 256, hd - 1);
+        const uint4 *src = reinterpret_cast<const uint4 *>(v_cache + ((size_t)kvh * hd + d) * v_stride + t0);
+        const uint4 va = src[0], vb = src[1];
+        const __half2 *ha = reinterpret_cast<const __half2 *>(&va), *hb = reinterpret_cast<const __half2 *>(&vb);
 #pragma unroll
-        for (int t = 0; t < kAttnChunk; t++) {
-            const int tt = min(t, cnt - 1);
-            vreg[c][t] = d < hd ? __half2float(v_cache[((size_t)kvh * max_seq + t0 + tt) * hd + d]) : 0.f;
+        for (int e = 0; e < 4; e++) {
+            vreg[c][2 * e] = __low2float(ha[e]), vreg[c][2 * e + 1] = __high2float(ha[e]);
+            vreg[c][8 + 2 * e] = __low2float(hb[e]), vreg[c][8 + 2 * e + 1] = __high2float(hb[e]);
         }
     }
     // keys: 16 threads per position, 16 channels (32 bytes) each per pass over the head
@@ -268,7 +274,7 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
     const int G = n_q / n_kv, kvh = head / G, g = head % G;
     // chunks holding at least one position: kAttnChunk each, or the context dealt evenly to kAttnSplits
     const int total = st->pos + 1;
-    const int live = even_chunks ? attn_live_chunks(total - attn_first(total, window)) : min(nsplit, (st->pos + kAttnChunk) / kAttnChunk);
+    const int live = even_chunks ? attn_live_chunks(attn_span(total, window)) : min(nsplit, (st->pos + kAttnChunk) / kAttnChunk);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float m = -3.0e38f;
     for (int s = tid; s < live; s += 256) m = fmaxf(m, part_ml[(((size_t)kvh * nsplit + s) * G + g) * 2]);
@@ -308,51 +314,59 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
 }
 
 // ---- the context chunks of one decode step's attention in one launch (head_dim 64 / 128 / 256) ----
-// Workgroup (split, kvh) owns attn_chunk(span) consecutive visible positions of kv head kvh, walks them
-// kAttnPass at a time (kAttnShortPass when that is the whole chunk) and serves all G query heads of the group. It
-//   1. asks for the fused qkv vector's pieces it needs and for the K and V rows of its first pass
-//      (16-byte pieces, every load of a pass independent of every other),
-//   2. prepares the step's own q, k, v: per-head RMS norm and half-split rotary embedding for q
-//      and k (every workgroup does this redundantly: 1.3 k values), k and v rounded to f16 as the
-//      cache holds them; the workgroup whose chunk holds position `pos` writes them into the cache,
-//      and every use of that position takes the LDS copy,
-//   3. per pass: scores, running max / sum (rescaling what it has), unnormalised output, and
-//   4. writes the chunk's (max, sum) pairs and unnormalised output: the flash-decoding partial.
-// The partials of the live chunks are joined by the consumer (the output projection's prologue,
-// or dec_attn_merge_kernel). HD and G are template parameters so that the body is straight-line
-// code: with them as run-time values it was several times as long, and a workgroup that runs its
-// code once pays for every instruction-cache line it touches.
+// Workgroup (split, kvh) owns attn_chunk(span) consecutive positions of kv head kvh and serves all G
+// query heads of the group; a wavefront owns 16 positions of every pass of 64 and never waits for
+// another wavefront between the first barrier (q ready) and the last (the join). Both products run
+// on the matrix cores:
+//   scores   S[row, t] = sum_d q[row, d] K[t, d]    16x16x32 f16: the B operand of position t is
+//            16 bytes of the row-major key cache as they lie; the A operand's rows 2 g and 2 g + 1
+//            are head g's query as two f16 terms (hi = f16(q), lo = f16(q - hi): 22 bits), so that a
+//            lane's result registers (rows 4 j .. 4 j + 3) add up to two heads' scores;
+//   outputs  O[row, d] = sum_t p[row, t] V[t, d]    32x32x16 f16: the B operand of channel d is 16
+//            bytes (8 positions) of the TRANSPOSED value cache [kv head][channel][position]; the A
+//            operand's rows are the heads' weights as two f16 terms, turned from the scores' layout
+//            (lane = position) into the operand's (lane = row) through the wavefront's own LDS rows.
+// The step's own position never comes from the cache: the workgroup that owns it (the last live one)
+// writes the cache rows and joins q.k_new / v_new as a fifth partial beside its wavefronts' four.
+// A workgroup writes (max, sum) per head and the unnormalised output: the flash-decoding partial
+// that the consumer joins over the live chunks (the output projection's prologue, or
+// dec_attn_merge_kernel). HD and G are template parameters so that the body is straight-line code.
+typedef _Float16 dh16x8 __attribute__((ext_vector_type(8)));
+typedef float df32x4 __attribute__((ext_vector_type(4)));
+typedef float df32x16 __attribute__((ext_vector_type(16)));
+
 template <int HD, int G>
 __global__ void __launch_bounds__(256)
 dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
                        const float *__restrict__ k_norm, int n_q, int n_kv, float eps, const float *__restrict__ rope,
-                       int max_seq, float scale, int window, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
+                       int max_seq, int v_stride, float scale, int window, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
                        float *__restrict__ part_ml, float *__restrict__ part_o) {
     constexpr int GH = G * HD, NK = HD / 64, HALF = HD / 2;
-    constexpr int VT = HD / 8;                 // threads per value row (8 channels each)
-    constexpr int VPP = 256 / VT;              // value rows in flight per pass of the workgroup
+    constexpr int KS = HD / 32;                // 32-channel steps of the score product
+    constexpr int NB = HD / 32;                // 32-channel blocks of the output product
+    constexpr int R = 2 * G;                   // operand rows in use: two terms per head
     constexpr int ROWS = (G + 1 + 3) / 4;      // q heads and the k head, dealt to four wavefronts
-    static_assert(kAttnPass == 64 && kAttnShortPass == 32, "at most one lane per position of a pass");
-    __shared__ __attribute__((aligned(16))) float qs[GH];      // query heads, normed and rotated
-    __shared__ __attribute__((aligned(16))) float kn[HD];      // the step's key, as the cache will hold it
-    __shared__ __attribute__((aligned(16))) float vn[HD];      // the step's value
-    __shared__ __attribute__((aligned(16))) float sc[G * kAttnPass];
-    __shared__ __attribute__((aligned(16))) float ored[4 * GH];
-    __shared__ float mrun[G], lrun[G], fac[G];
+    constexpr int QS = HD + 8;                 // halfs per operand row of q (16 bytes of padding: rows start in different banks)
+    constexpr int PS = 24;                     // halfs per operand row of p
+    constexpr int HL = (G + 1) / 2;            // rows of 16 lanes that hold scores (two heads each)
+    constexpr int JN = G == 8 ? 8 : 4;         // result registers of an output block that hold rows in use
+    constexpr float NEG = -3.0e38f;
+    static_assert(kAttnPass == 64, "four wavefronts of 16 positions");
+    __shared__ __attribute__((aligned(16))) __half qa[R * QS];       // query heads, normed, rotated, scaled: rows 2 g + term
+    __shared__ __attribute__((aligned(16))) __half pa[4][16 * PS];    // per wavefront: the pass's weights, rows as in qa
+    __shared__ __attribute__((aligned(16))) float ow[4][GH];          // per wavefront: unnormalised outputs
+    __shared__ __attribute__((aligned(16))) float kn[HD];             // the step's key, as the cache will hold it
+    __shared__ __attribute__((aligned(16))) float vn[HD];             // the step's value
+    __shared__ float mw[4][G], lw[4][G], sown[G];
 
     const int split = blockIdx.x, kvh = blockIdx.y;
-    const int pos = st->pos, total = pos + 1;
-    if (pos >= max_seq) return;  // the cache is full: the step is a no-op
-    const int t_first = attn_first(total, window);  // a local layer sees the last `window` positions only
-    const int chunk = attn_chunk(total - t_first);
-    const int t_begin = t_first + split * chunk;
-    if (t_begin >= total) return;  // no position of this chunk exists yet
-    const int t_end = min(total, t_begin + chunk);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int i16 = lane & 15, g4 = lane >> 4, n32 = lane & 31, h32 = lane >> 5;
 
-    // 1. the step's own rows first (they come out of L2 and are needed first): rows 0..G-1 are the
-    //    query heads, row G the key head; wavefront w prepares rows w, w + 4, ...; lane l holds
-    //    elements l + 64 i of a row
+    // 1. the step's own rows (they come out of L2 and are needed first): rows 0..G-1 are the query
+    //    heads, row G the key head; wavefront w prepares rows w, w + 4, ...; lane l holds elements
+    //    l + 64 i of a row
     float px[ROWS][NK], pw[ROWS][NK], pc[NK], psn[NK];
 #pragma unroll
     for (int i = 0; i < NK; i++) {
@@ -368,50 +382,55 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
         for (int i = 0; i < NK; i++) px[rr][i] = src[lane + 64 * i], pw[rr][i] = w[lane + 64 * i];
     }
     const float pv_own = qkv[(size_t)(n_q + n_kv + kvh) * HD + min(tid, HD - 1)];
-    //    K: thread (kp, seg) reads the 16-byte piece `seg` of every 128-byte run of rows kp and
-    //    kp + 32 (a row is read in whole cache lines); V: thread (pg, cb) reads 8 channels of rows
-    //    pg, pg + VPP, ...  Rows past the end repeat the last one (their weights are zero).
-    // Everything from here on is written once for a pass of P positions and instantiated for the
-    // two pass lengths; a launch runs one of them (chunks of 32 positions are walked 32 at a time:
-    // half the score and value work per workgroup, on twice as many CUs).
-    auto walk = [&](auto pass_length) {
-    constexpr int P = decltype(pass_length)::value;
-    constexpr int KP = P / 32;                 // passes of 32 positions over the keys (8 threads per position)
-    constexpr int VI = P / VPP;                // value rows per thread
-    static_assert(VI >= 1, "a pass holds at least one value row per thread");
-    const int kp = tid >> 3, seg = tid & 7;
-    const int pg = tid / VT, cb = tid % VT;
-    const __half *k_head = k_cache + (size_t)kvh * max_seq * HD + seg * 8;
-    const __half *v_head = v_cache + (size_t)kvh * max_seq * HD + cb * 8;
-    uint4 kreg[KP][NK], vreg[VI];
+
+    const int pos = st->pos, total = pos + 1;
+    if (pos >= max_seq) return;  // the cache is full: the step is a no-op
+    const int t_first = attn_first(total, window);  // a local layer sees the last `window` positions only
+    const int base = t_first & ~15;
+    const int chunk = attn_chunk(total - base);
+    const int t_begin = base + split * chunk;
+    if (t_begin >= total) return;  // no position of this chunk exists yet
+    const int t_end = min(total, t_begin + chunk);
+    const bool is_last = t_end == total;        // this workgroup owns the step's own position
+    const int hist_end = min(t_end, pos);       // positions below come from the cache
+
+    //    K: lane (position i16, quarter g4) reads its position's channels g4 HD/4 .. + HD/4, 16 bytes
+    //    per step (the query operand takes the same channel order); V: lane (channel n32, half h32)
+    //    reads positions 8 h32 .. + 8 of its wavefront's 16 for channel 32 b + n32. Rows past the end
+    //    of the cache are padding; positions that do not count are masked below.
+    const __amdgpu_buffer_rsrc_t r_k = __builtin_amdgcn_make_buffer_rsrc(k_cache, 0, (int)(((uint32_t)n_kv * (uint32_t)max_seq + kAttnPass) * HD * 2u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t r_v = __builtin_amdgcn_make_buffer_rsrc(v_cache, 0, (int)((uint32_t)n_kv * HD * (uint32_t)v_stride * 2u), 0x00020000);
+    const uint32_t v_k = (uint32_t)((wave * 16 + i16) * HD + g4 * (HD / 4)) * 2u;
+    const uint32_t v_v = ((uint32_t)n32 * (uint32_t)v_stride + (uint32_t)(wave * 16 + h32 * 8)) * 2u;
+    uint4 kreg[KS], vreg[NB];
     auto load_k = [&](int t0) {
+        const uint32_t s_k = ((uint32_t)kvh * (uint32_t)max_seq + (uint32_t)t0) * HD * 2u;
 #pragma unroll
-        for (int ps = 0; ps < KP; ps++) {
-            const __half *krow = k_head + (size_t)min(t0 + kp + 32 * ps, t_end - 1) * HD;
-#pragma unroll
-            for (int u = 0; u < NK; u++) kreg[ps][u] = *reinterpret_cast<const uint4 *>(krow + u * 64);
-        }
+        for (int u = 0; u < KS; u++) kreg[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r_k, (int)(v_k + u * 16u), (int)s_k, 0));
     };
     auto load_v = [&](int t0) {
 #pragma unroll
-        for (int i = 0; i < VI; i++)
-            vreg[i] = *reinterpret_cast<const uint4 *>(v_head + (size_t)min(t0 + pg + VPP * i, t_end - 1) * HD);
+        for (int b = 0; b < NB; b++) {
+            const uint32_t s_v = (((uint32_t)kvh * HD + b * 32u) * (uint32_t)v_stride + (uint32_t)t0) * 2u;
+            vreg[b] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r_v, (int)v_v, (int)s_v, 0));
+        }
     };
     load_k(t_begin);
     load_v(t_begin);
 
     // 2. per-head RMS norm and half-split rotary embedding (pairs d, d + HD/2), one wavefront per
     //    row and no workgroup barrier: with HD = 128 or 256 both members of a pair sit in one lane
-    //    (elements i and i + NK/2), with HD = 64 in lanes l and l + 32
+    //    (elements i and i + NK/2), with HD = 64 in lanes l and l + 32. Query rows are scaled and
+    //    kept (for the step's own score); only the workgroup that owns the position prepares k.
+    float rq[ROWS][NK];
 #pragma unroll
     for (int rr = 0; rr < ROWS; rr++) {
         const int row = wave + 4 * rr;
-        if (row <= G) {
+        if (row < G || (row == G && is_last)) {
             float sq = 0.f;
 #pragma unroll
             for (int i = 0; i < NK; i++) sq += px[rr][i] * px[rr][i];
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) sq += __shfl_xor(sq, off, 64);
+            sq = lean_wave_sum(sq);
             const float inv = rsqrtf(sq / (float)HD + eps);
             float x[NK], r[NK];
 #pragma unroll
@@ -427,167 +446,140 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
                     r[(i + HK) % NK] = x[(i + HK) % NK] * pc[i] + x[i] * psn[i];
                 }
             }
-            float *dst = row < G ? qs + row * HD : kn;
+            if (row < G) {
 #pragma unroll
-            for (int i = 0; i < NK; i++) dst[lane + 64 * i] = row < G ? r[i] : __half2float(__float2half(r[i]));
+                for (int i = 0; i < NK; i++) {
+                    const float v = r[i] * scale;
+                    const __half hi = __float2half(v);
+                    rq[rr][i] = v;
+                    qa[(2 * row) * QS + lane + 64 * i] = hi;
+                    qa[(2 * row + 1) * QS + lane + 64 * i] = __float2half(v - __half2float(hi));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NK; i++) kn[lane + 64 * i] = __half2float(__float2half(r[i]));
+            }
         }
     }
-    if (tid < HD) vn[tid] = __half2float(__float2half(pv_own));
-    if (tid < G) mrun[tid] = -3.0e38f, lrun[tid] = 0.f;
+    if (is_last && tid < HD) vn[tid] = __half2float(__float2half(pv_own));
     __syncthreads();
-    if (pos >= t_begin && tid < HD) {  // pos = total - 1 lies in the last live chunk
-        k_cache[((size_t)kvh * max_seq + pos) * HD + tid] = __float2half(kn[tid]);
-        v_cache[((size_t)kvh * max_seq + pos) * HD + tid] = __float2half(vn[tid]);
+    if (is_last) {
+        if (tid < HD) {
+            k_cache[((size_t)kvh * max_seq + pos) * HD + tid] = __float2half(kn[tid]);
+            v_cache[((size_t)kvh * HD + tid) * v_stride + pos] = __float2half(vn[tid]);
+        }
+#pragma unroll
+        for (int rr = 0; rr < ROWS; rr++) {
+            const int row = wave + 4 * rr;
+            if (row < G) {
+                float dot = 0.f;
+#pragma unroll
+                for (int i = 0; i < NK; i++) dot = fmaf(rq[rr][i], kn[lane + 64 * i], dot);
+                dot = lean_wave_sum(dot);
+                if (lane == 0) sown[row] = dot;
+            }
+        }
     }
 
-    float o[G][8];
+    // 3. the query operand: row i16 (rows past the last in use: zeros), channels in the key loads' order
+    dh16x8 aq[KS];
 #pragma unroll
-    for (int g = 0; g < G; g++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[g][e] = 0.f;
-
-    for (int t0 = t_begin; t0 < t_end; t0 += P) {
-        const int cnt = min(P, t_end - t0);
-        const bool more = t0 + P < t_end;
-        // 3a. scores. The row of `pos` as loaded is not the step's key: it counts as zero here and
-        //     the thread that owns it takes the key from LDS below.
-        //     A thread's two positions (kp and kp + 32) share every q value it reads from LDS.
-        float dot[KP][G];
-#pragma unroll
-        for (int ps = 0; ps < KP; ps++)
-#pragma unroll
-            for (int g = 0; g < G; g++) dot[ps][g] = 0.f;
-#pragma unroll
-        for (int u = 0; u < NK; u++) {
-            float kf[KP][8];
-#pragma unroll
-            for (int ps = 0; ps < KP; ps++) {
-                const bool stale = min(t0 + kp + 32 * ps, t_end - 1) == pos;
-                const uint4 raw = stale ? make_uint4(0, 0, 0, 0) : kreg[ps][u];
-                const __half2 *h2 = reinterpret_cast<const __half2 *>(&raw);
-#pragma unroll
-                for (int e = 0; e < 4; e++) kf[ps][2 * e] = __low2float(h2[e]), kf[ps][2 * e + 1] = __high2float(h2[e]);
-            }
-            const int c0 = u * 64 + seg * 8;
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                const float4 qa = *reinterpret_cast<const float4 *>(qs + g * HD + c0);
-                const float4 qb = *reinterpret_cast<const float4 *>(qs + g * HD + c0 + 4);
-#pragma unroll
-                for (int ps = 0; ps < KP; ps++)
-                    dot[ps][g] += (qa.x * kf[ps][0] + qa.y * kf[ps][1]) + (qa.z * kf[ps][2] + qa.w * kf[ps][3]) +
-                                  (qb.x * kf[ps][4] + qb.y * kf[ps][5]) + (qb.z * kf[ps][6] + qb.w * kf[ps][7]);
-            }
-        }
-#pragma unroll
-        for (int ps = 0; ps < KP; ps++) {
-            const int tp = kp + 32 * ps;
-            if (t0 + tp == pos) {
-#pragma unroll 1
-                for (int u = 0; u < NK; u++) {
-                    const int c0 = u * 64 + seg * 8;
-                    const float4 ka = *reinterpret_cast<const float4 *>(kn + c0), kb = *reinterpret_cast<const float4 *>(kn + c0 + 4);
-#pragma unroll
-                    for (int g = 0; g < G; g++) {
-                        const float4 qa = *reinterpret_cast<const float4 *>(qs + g * HD + c0);
-                        const float4 qb = *reinterpret_cast<const float4 *>(qs + g * HD + c0 + 4);
-                        dot[ps][g] += (qa.x * ka.x + qa.y * ka.y) + (qa.z * ka.z + qa.w * ka.w) +
-                                      (qb.x * kb.x + qb.y * kb.y) + (qb.z * kb.z + qb.w * kb.w);
-                    }
-                }
-            }
-#pragma unroll
-            for (int g = 0; g < G; g++) {
-                float v = dot[ps][g];
-                v += __shfl_xor(v, 1, 64);
-                v += __shfl_xor(v, 2, 64);
-                v += __shfl_xor(v, 4, 64);
-                if (seg == 0) sc[g * P + tp] = v * scale;
-            }
-        }
-        if (more) load_k(t0 + P);
-        __syncthreads();
-        // 3b. one wavefront per head: the pass's max and sum join the running pair
-        for (int g = wave; g < G; g += 4) {
-            const float x = lane < cnt ? sc[g * P + lane] : -3.0e38f;
-            const float m_old = mrun[g], l_old = lrun[g];
-            float m = x;
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-            m = fmaxf(m, m_old);
-            const float pv = lane < cnt ? __expf(x - m) : 0.f;
-            float l = pv;
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
-            const float f = __expf(m_old - m);
-            if (lane < P) sc[g * P + lane] = pv;
-            if (lane == 0) mrun[g] = m, lrun[g] = l_old * f + l, fac[g] = f;
-        }
-        __syncthreads();
-        // 3c. unnormalised output: 8 channels x G heads per thread over its rows
-        {
-            float fg[G];
-#pragma unroll
-            for (int g = 0; g < G; g++) fg[g] = fac[g];
-#pragma unroll
-            for (int g = 0; g < G; g++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) o[g][e] *= fg[g];
-#pragma unroll
-            for (int i = 0; i < VI; i++) {
-                const int tp = pg + VPP * i;
-                const bool stale = min(t0 + tp, t_end - 1) == pos;
-                const uint4 raw = stale ? make_uint4(0, 0, 0, 0) : vreg[i];
-                const __half2 *h2 = reinterpret_cast<const __half2 *>(&raw);
-                float vf[8];
-#pragma unroll
-                for (int e = 0; e < 4; e++) vf[2 * e] = __low2float(h2[e]), vf[2 * e + 1] = __high2float(h2[e]);
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-                    const float w = sc[g * P + tp];  // zero past the end of the pass
-#pragma unroll
-                    for (int e = 0; e < 8; e++) o[g][e] += w * vf[e];
-                }
-            }
-            const int own = pos - t0;  // the step's own position, if this pass holds it
-            if (own >= 0 && own < P && (own % VPP) == pg) {
-                const float4 va = *reinterpret_cast<const float4 *>(vn + cb * 8), vb = *reinterpret_cast<const float4 *>(vn + cb * 8 + 4);
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-                    const float w = sc[g * P + own];
-                    o[g][0] += w * va.x, o[g][1] += w * va.y, o[g][2] += w * va.z, o[g][3] += w * va.w;
-                    o[g][4] += w * vb.x, o[g][5] += w * vb.y, o[g][6] += w * vb.z, o[g][7] += w * vb.w;
-                }
-            }
-        }
-        if (more) load_v(t0 + P);
-        // the next pass rewrites sc only after the barrier that follows its scores' LDS reads of qs;
-        // its writes to sc must not overtake this pass's reads of sc
-        __syncthreads();
+    for (int u = 0; u < KS; u++) {
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (i16 < R) raw = *reinterpret_cast<const uint4 *>(qa + i16 * QS + g4 * (HD / 4) + u * 8);
+        aq[u] = __builtin_bit_cast(dh16x8, raw);
     }
-    // 4. lanes VT apart hold the same channels of neighbouring rows; then the four wavefronts
+
+    float m_run0 = NEG, m_run1 = NEG, l_run0 = 0.f, l_run1 = 0.f;   // heads 2 g4 and 2 g4 + 1, the same in every lane of a row of 16
+    df32x16 o[NB];
 #pragma unroll
-    for (int g = 0; g < G; g++) {
+    for (int b = 0; b < NB; b++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
+        for (int j = 0; j < 16; j++) o[b][j] = 0.f;
+
+    for (int t0 = t_begin; t0 < t_end; t0 += kAttnPass) {
+        const bool more = t0 + kAttnPass < t_end;
+        // 3a. scores of this wavefront's 16 positions, all heads
+        df32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int off = VT; off < 64; off <<= 1) o[g][e] += __shfl_xor(o[g][e], off, 64);
+        for (int u = 0; u < KS; u++) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[u], __builtin_bit_cast(dh16x8, kreg[u]), acc, 0, 0, 0);
+        if (more) load_k(t0 + kAttnPass);
+        const int t = t0 + wave * 16 + i16;
+        const bool valid = t >= t_first && t < hist_end;
+        const float s0 = valid ? acc[0] + acc[1] : NEG, s1 = valid ? acc[2] + acc[3] : NEG;
+        // 3b. the pass's max and sum join the running pair (a row of 16 lanes = the 16 positions)
+        const float m0 = fmaxf(m_run0, lean_row_max(s0)), m1 = fmaxf(m_run1, lean_row_max(s1));
+        const float f0 = __expf(m_run0 - m0), f1 = __expf(m_run1 - m1);
+        const float p0 = valid ? __expf(s0 - m0) : 0.f, p1 = valid ? __expf(s1 - m1) : 0.f;
+        l_run0 = fmaf(l_run0, f0, lean_row_sum(p0)), l_run1 = fmaf(l_run1, f1, lean_row_sum(p1));
+        m_run0 = m0, m_run1 = m1;
+        //     weights as two f16 terms into the wavefront's LDS rows 4 g4 .. 4 g4 + 3, column = position
+        if (g4 < HL) {
+            const __half h0 = __float2half(p0), h1 = __float2half(p1);
+            __half *dst = pa[wave] + (4 * g4) * PS + i16;
+            dst[0] = h0, dst[PS] = __float2half(p0 - __half2float(h0));
+            dst[2 * PS] = h1, dst[3 * PS] = __float2half(p1 - __half2float(h1));
         }
-        if (lane < VT) {
-            float4 *dst = reinterpret_cast<float4 *>(ored + (wave * G + g) * HD + cb * 8);
-            dst[0] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
-            dst[1] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
+        // the rows are this wavefront's own: its LDS operations complete in order, the compiler only must not reorder them
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        uint4 praw = make_uint4(0, 0, 0, 0);
+        if (n32 < R) praw = *reinterpret_cast<const uint4 *>(pa[wave] + n32 * PS + h32 * 8);
+        const dh16x8 ap = __builtin_bit_cast(dh16x8, praw);
+        // 3c. unnormalised outputs. Result register j of a lane holds row 8 (j / 4) + 4 h32 + j % 4,
+        //     i.e. head 4 (j / 4) + 2 h32 + (j % 4) / 2; what the earlier passes left is rescaled first.
+        if (t0 != t_begin) {
+            float fh[8];
+#pragma unroll
+            for (int g = 0; g < 8; g++) fh[g] = g < G ? lean_lane((g & 1) ? f1 : f0, 16 * (g >> 1)) : 1.f;
+#pragma unroll
+            for (int j = 0; j < JN; j++) {
+                const int ga = 4 * (j >> 2) + ((j & 3) >> 1);
+                const float fj = h32 ? fh[ga + 2] : fh[ga];
+#pragma unroll
+                for (int b = 0; b < NB; b++) o[b][j] *= fj;
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) o[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ap, __builtin_bit_cast(dh16x8, vreg[b]), o[b], 0, 0, 0);
+        if (more) load_v(t0 + kAttnPass);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the next pass rewrites the weight rows
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // 4. the wavefront's partial: (max, sum) per head and the outputs (the two terms' rows added)
+    if (i16 == 0 && g4 < HL) {
+        mw[wave][2 * g4] = m_run0, lw[wave][2 * g4] = l_run0;
+        if (2 * g4 + 1 < G) mw[wave][2 * g4 + 1] = m_run1, lw[wave][2 * g4 + 1] = l_run1;
+    }
+#pragma unroll
+    for (int jj = 0; jj < JN / 2; jj++) {
+        const int head = 4 * (jj >> 1) + 2 * h32 + (jj & 1);
+        if (head < G) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) ow[wave][head * HD + b * 32 + n32] = o[b][2 * jj] + o[b][2 * jj + 1];
         }
     }
     __syncthreads();
+    // 5. the four wavefronts' partials and, in the workgroup that owns it, the step's own position
     float *po = part_o + ((size_t)kvh * kAttnSplits + split) * GH;
-    for (int idx = tid; idx < GH; idx += 256)
-        po[idx] = (ored[idx] + ored[GH + idx]) + (ored[2 * GH + idx] + ored[3 * GH + idx]);
     float *ml = part_ml + ((size_t)kvh * kAttnSplits + split) * G * 2;
-    if (tid < G) ml[tid * 2] = mrun[tid], ml[tid * 2 + 1] = lrun[tid];
-    };
-    if (chunk == kAttnShortPass) walk(std::integral_constant<int, kAttnShortPass>{});
-    else walk(std::integral_constant<int, kAttnPass>{});
+    for (int idx = tid; idx < GH; idx += 256) {
+        const int g = idx / HD, ch = idx % HD;
+        const float ma = mw[0][g], mb = mw[1][g], mc = mw[2][g], md = mw[3][g];
+        const float so = is_last ? sown[g] : NEG;
+        const float M = fmaxf(fmaxf(fmaxf(ma, mb), fmaxf(mc, md)), so);
+        const float ea = __expf(ma - M), eb = __expf(mb - M), ec = __expf(mc - M), ed = __expf(md - M);
+        const float eo = is_last ? __expf(so - M) : 0.f;
+        float out = (ea * ow[0][idx] + eb * ow[1][idx]) + (ec * ow[2][idx] + ed * ow[3][idx]);
+        if (is_last) out = fmaf(eo, vn[ch], out);
+        po[idx] = out;
+        if (ch == 0) {
+            ml[g * 2] = M;
+            ml[g * 2 + 1] = (ea * lw[0][g] + eb * lw[1][g]) + (ec * lw[2][g] + ed * lw[3][g]) + eo;
+        }
+    }
 }
 
 
@@ -717,7 +709,8 @@ void attn_chunks_launch(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale
     const hipc_decoder_config &c = d->cfg;
     dec_attn_chunks_kernel<HD, G><<<dim3(kAttnSplits, c.n_kv_heads), 256, 0, ctx->stream>>>(
         d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.rms_eps,
-        d->rope + (size_t)l.rope_table * c.head_dim, c.max_seq, scale, l.window, l.k_cache, l.v_cache, d->part_ml, d->part_o);
+        d->rope + (size_t)l.rope_table * c.head_dim, c.max_seq, attn_v_stride(c.max_seq), scale, l.window, l.k_cache, l.v_cache,
+        d->part_ml, d->part_o);
 }
 
 template <int HD>
@@ -773,13 +766,16 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         d->cfg = c;
         d->layers.resize(c.n_layers);
         d->nsplit = (int)ceil_div(c.max_seq, kAttnChunk);
-        const size_t kv = (size_t)c.n_kv_heads * c.max_seq * c.head_dim;
+        // keys [kv head][position][channel] with a pass of padding rows behind the last head (the one-launch
+        // attention reads whole passes); values transposed, [kv head][channel][position], rows of v_stride
+        const size_t k_halfs = ((size_t)c.n_kv_heads * c.max_seq + kAttnPass) * c.head_dim;
+        const size_t v_halfs = (size_t)c.n_kv_heads * c.head_dim * attn_v_stride(c.max_seq);
         const int G = c.n_q_heads / c.n_kv_heads;
         int rc = HIPC_OK;
         auto A = [&](auto **p, size_t n) { if (rc == HIPC_OK) rc = dev_alloc(ctx, d, p, n); };
         for (DecLayer &l : d->layers) {
-            A(&l.k_cache, kv);
-            A(&l.v_cache, kv);
+            A(&l.k_cache, k_halfs);
+            A(&l.v_cache, v_halfs);
         }
         A(&d->state, 1), A(&d->history, (size_t)c.max_seq);
         A(&d->x, c.hidden), A(&d->xn, c.hidden), A(&d->qkv, (size_t)(c.n_q_heads + 2 * c.n_kv_heads) * c.head_dim);
@@ -793,6 +789,7 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         // kernels, dec_fused_attn = 0 the three-kernel attention (tests of those paths)
         d->fused_glue = c.hidden % 8 == 0 && c.ffn % 8 == 0 && ctx->tune.dec_fused_glue != 0;
         d->one_launch_attn = (c.head_dim == 64 || c.head_dim == 128 || c.head_dim == 256) && (G == 1 || G == 2 || G == 4 || G == 8) &&
+                             k_halfs * 2 < (1ull << 32) && v_halfs * 2 < (1ull << 32) &&   // 32-bit buffer offsets
                              ctx->tune.dec_fused_attn != 0;
         // the lean path (the dec_lean option set to 0 keeps the streaming kernel and its prologues)
         {
@@ -823,7 +820,8 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         }
         if (rc == HIPC_OK) {
             for (DecLayer &l : d->layers) {  // an unwritten cache row must not hold NaN bit patterns
-                if (hipMemsetAsync(l.k_cache, 0, kv * 2, ctx->stream) != hipSuccess || hipMemsetAsync(l.v_cache, 0, kv * 2, ctx->stream) != hipSuccess)
+                if (hipMemsetAsync(l.k_cache, 0, k_halfs * 2, ctx->stream) != hipSuccess ||
+                    hipMemsetAsync(l.v_cache, 0, v_halfs * 2, ctx->stream) != hipSuccess)
                     rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the KV cache");
             }
             dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, 0, 0);
@@ -1054,11 +1052,11 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 }
             } else {
                 dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
-                                                     c.n_kv_heads, c.head_dim, c.rms_eps, l.rope_table ? d->theta2 : c.rope_theta, c.max_seq, d->q,
-                                                     l.k_cache, l.v_cache);
+                                                     c.n_kv_heads, c.head_dim, c.rms_eps, l.rope_table ? d->theta2 : c.rope_theta, c.max_seq,
+                                                     attn_v_stride(c.max_seq), d->q, l.k_cache, l.v_cache);
                 HIPC_LAUNCHED(ctx);
                 dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
-                                                                                     c.head_dim, c.max_seq, scale, l.window, d->part_ml, d->part_o);
+                                                                                     c.head_dim, c.max_seq, attn_v_stride(c.max_seq), scale, l.window, d->part_ml, d->part_o);
                 HIPC_LAUNCHED(ctx);
                 dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
                                                                                                  c.head_dim, d->nsplit, 0, l.window, d->attn);

@@ -35,6 +35,7 @@
 #include <algorithm>
 
 #include "internal.h"
+#include "lanes.h"
 
 namespace hipc {
 
@@ -77,38 +78,6 @@ struct ScaleVecLean<1> {
 
 __device__ __forceinline__ float lean_gelu_tanh(float v) {
     return 0.5f * v * (1.f + tanhf(0.79788456080286536f * fmaf(0.044715f, v * v * v, v)));
-}
-
-// ---- cross-lane helpers on the vector unit (no LDS round trip)
-template <int CTRL>
-__device__ __forceinline__ float lean_dpp(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
-}
-// every lane ends with the sum (maximum) of its row of 16 lanes: neighbours, pairs, then rotations by 4 and 8
-__device__ __forceinline__ float lean_row_sum(float v) {
-    v += lean_dpp<0xB1>(v);    // quad_perm [1,0,3,2]
-    v += lean_dpp<0x4E>(v);    // quad_perm [2,3,0,1]
-    v += lean_dpp<0x124>(v);   // row_ror:4
-    v += lean_dpp<0x128>(v);   // row_ror:8
-    return v;
-}
-__device__ __forceinline__ float lean_row_max(float v) {
-    v = fmaxf(v, lean_dpp<0xB1>(v));
-    v = fmaxf(v, lean_dpp<0x4E>(v));
-    v = fmaxf(v, lean_dpp<0x124>(v));
-    v = fmaxf(v, lean_dpp<0x128>(v));
-    return v;
-}
-__device__ __forceinline__ float lean_lane(float v, int l) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
-}
-__device__ __forceinline__ float lean_wave_sum(float v) {
-    v = lean_row_sum(v);
-    return (lean_lane(v, 0) + lean_lane(v, 16)) + (lean_lane(v, 32) + lean_lane(v, 48));
-}
-__device__ __forceinline__ float lean_wave_max(float v) {
-    v = lean_row_max(v);
-    return fmaxf(fmaxf(lean_lane(v, 0), lean_lane(v, 16)), fmaxf(lean_lane(v, 32), lean_lane(v, 48)));
 }
 
 // ---- buffer loads: a uniform descriptor, a per-lane byte offset computed once and a SCALAR offset per
@@ -343,9 +312,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
             const uint2 ml_raw = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r_ml, (int)((uint32_t)lane * (uint32_t)G * 8u),
                                                                                               (int)(((uint32_t)kvh * kAttnSplits * G + g) * 8u), 0));
             const int total = *p.pos + 1;
-            const int span = total - attn_first(total, p.window);
-            const int live = span <= kAttnShortPass * kAttnSplits ? (span + kAttnShortPass - 1) >> 5 : attn_live_chunks(span);
-            static_assert(kAttnShortPass == 32, "the shift above");
+            const int live = attn_live_chunks(attn_span(total, p.window));
 #pragma unroll
             for (int q = 1; q < 4; q++) {
                 if (q * 16 < live) {   // wave-uniform: a quarter of the chunks at a time

@@ -249,25 +249,28 @@ struct GemvPrologue {
     const int *pos = nullptr;
     int group = 0, head_dim = 0, window = 0;
 };
-// Decode attention splits the visible context of a kv head (`span` positions: all of them, or the
-// last `window`) over kAttnSplits workgroups. Each takes `attn_chunk(span)` consecutive positions,
-// so that all splits together cover the span: kAttnShortPass positions while that is enough
-// (span <= 2048: up to 64 workgroups of 32 positions rather than 32 of 64), else a multiple of
-// kAttnPass. The first attn_live_chunks(span) splits hold at least one position and only those
-// write a partial.
+// Decode attention splits the visible context of a kv head over kAttnSplits workgroups. The split
+// starts at attn_base: the first visible position rounded down to 16 (a wavefront's 16 positions are
+// then 32-byte aligned in the transposed value cache; positions before the first visible one are
+// masked). Each workgroup takes attn_chunk(span) consecutive positions of the span from there to the
+// end, kAttnPass at a time: one pass while span <= kAttnPass * kAttnSplits = 4096 positions. The first
+// attn_live_chunks(span) splits hold at least one position and only those write a partial.
 constexpr int kAttnPass = 64;
-constexpr int kAttnShortPass = 32;
 constexpr int kAttnSplits = 64;
-__host__ __device__ inline int attn_chunk(int total) {
-    if (total <= kAttnShortPass * kAttnSplits) return kAttnShortPass;
-    return kAttnPass * ((total + kAttnPass * kAttnSplits - 1) / (kAttnPass * kAttnSplits));
-}
-__host__ __device__ inline int attn_live_chunks(int total) {
-    const int c = attn_chunk(total);
-    return (total + c - 1) / c;
-}
 // first visible position of a step that sees `total` positions through a window (<= 0: no window)
 __host__ __device__ inline int attn_first(int total, int window) { return window > 0 && total > window ? total - window : 0; }
+__host__ __device__ inline int attn_base(int total, int window) { return attn_first(total, window) & ~15; }
+__host__ __device__ inline int attn_span(int total, int window) { return total - attn_base(total, window); }
+__host__ __device__ inline int attn_chunk(int span) {
+    return kAttnPass * ((span + kAttnPass * kAttnSplits - 1) / (kAttnPass * kAttnSplits));
+}
+__host__ __device__ inline int attn_live_chunks(int span) {
+    if (span <= kAttnPass * kAttnSplits) return (span + kAttnPass - 1) / kAttnPass;   // no run-time division on the common path
+    const int c = attn_chunk(span);
+    return (span + c - 1) / c;
+}
+// the transposed value cache's row length: max_seq rounded up to a pass
+__host__ __device__ inline int attn_v_stride(int max_seq) { return (max_seq + kAttnPass - 1) / kAttnPass * kAttnPass; }
 int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
                const GemvPrologue *pro = nullptr);
 

@@ -418,7 +418,7 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     float *minv = nullptr;
     if (PRO == 3) {
         const int total = *p.npos + 1;
-        const int live = attn_live_chunks(total - attn_first(total, p.nwindow));
+        const int live = attn_live_chunks(attn_span(total, p.nwindow));
         const int G = p.ngroup, hd = p.nhd, GH = G * hd, n_q = p.K / hd;
         float *wgt = reinterpret_cast<float *>(reinterpret_cast<char *>(smem) + p.pro_off);  // [n_q][kAttnSplits]
         minv = wgt + n_q * kAttnSplits;                                                     // [n_q]

@@ -109,6 +109,23 @@ class Decoder:
         self.ctx._check(self.ctx.lib.hipc_decoder_kv_cache(self.ctx.handle, self.handle, layer, C.byref(k), C.byref(v)))
         return k.value, v.value
 
+    def fill_cache(self, layer: int, k_rows: np.ndarray, v_rows: np.ndarray):
+        """Write the first positions of a layer's cache from ``[n_kv_heads, n, head_dim]`` f16 rows
+        (what a prefill would leave): keys as they are, values transposed into the library's
+        ``[n_kv_heads, head_dim, v_stride]`` layout."""
+        nkv, hd = self.cfg["n_kv_heads"], self.cfg["head_dim"]
+        n = k_rows.shape[1]
+        assert k_rows.shape == (nkv, n, hd) and v_rows.shape == (nkv, n, hd) and n <= self.max_seq
+        kptr, vptr = self.kv_cache(layer)
+        stride = (self.max_seq + 63) // 64 * 64
+        up = self.ctx.lib.hipc_upload
+        for h in range(nkv):
+            rows = np.ascontiguousarray(k_rows[h], np.float16)
+            self.ctx._check(up(self.ctx.handle, kptr, h * self.max_seq * hd * 2, rows.ctypes.data, rows.nbytes))
+        vt = np.zeros((nkv, hd, stride), np.float16)
+        vt[:, :, :n] = np.transpose(v_rows, (0, 2, 1))
+        self.ctx._check(up(self.ctx.handle, vptr, 0, vt.ctypes.data, vt.nbytes))
+
     def step(self):
         self.ctx._check(self.ctx.lib.hipc_decoder_step(self.ctx.handle, self.handle))
 

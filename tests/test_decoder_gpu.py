@@ -80,11 +80,9 @@ def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, route, hd, nq, nkv
     ref = od.Decoder(w, max_seq)
     rng = np.random.default_rng(hd + p0)
     for li in range(cfg["n_layers"]):
-        kptr, vptr = dec.kv_cache(li)
-        for ptr, dst in ((kptr, ref.k), (vptr, ref.v)):
-            rows = (rng.standard_normal((nkv, max_seq, hd)) * 0.7).astype(np.float16)
-            dst[li] = rows
-            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, rows.ctypes.data, rows.nbytes))
+        k_rows, v_rows = ((rng.standard_normal((nkv, max_seq, hd)) * 0.7).astype(np.float16) for _ in range(2))
+        ref.k[li], ref.v[li] = k_rows, v_rows
+        dec.fill_cache(li, k_rows, v_rows)
     token = 23
     dec.reset(token, p0)
     for pos in range(p0, p0 + steps):
@@ -96,6 +94,9 @@ def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, route, hd, nq, nkv
         assert np.all(err <= 2e-3 + 2e-3 * np.abs(want_logits)), (pos, float(err.max()))
         k_row = ctx.download(dec.kv_cache(1)[0], np.float16, (hd,), offset=((nkv - 1) * max_seq + pos) * hd * 2)
         assert np.allclose(k_row.astype(np.float32), ref.k[1, nkv - 1, pos].astype(np.float32), atol=2e-3, rtol=2e-3), pos
+        stride = (max_seq + 63) // 64 * 64       # values are kept transposed: [kv head, channel, position]
+        v_t = ctx.download(dec.kv_cache(1)[1], np.float16, (nkv, hd, stride))
+        assert np.allclose(v_t[nkv - 1, :, pos].astype(np.float32), ref.v[1, nkv - 1, pos].astype(np.float32), atol=2e-3, rtol=2e-3), pos
         token = got_tok
     dec.destroy()
 
@@ -128,11 +129,9 @@ def test_sliding_windows_and_a_second_rotary_base(ctx, pkg, oracle, route, hd, n
         ref.set_layer_attention(li, win, theta)
     rng = np.random.default_rng(hd + p0)
     for li in range(cfg["n_layers"]):
-        kptr, vptr = dec.kv_cache(li)
-        for ptr, dst in ((kptr, ref.k), (vptr, ref.v)):
-            rows = (rng.standard_normal((nkv, max_seq, hd)) * 0.7).astype(np.float16)
-            dst[li] = rows
-            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, rows.ctypes.data, rows.nbytes))
+        k_rows, v_rows = ((rng.standard_normal((nkv, max_seq, hd)) * 0.7).astype(np.float16) for _ in range(2))
+        ref.k[li], ref.v[li] = k_rows, v_rows
+        dec.fill_cache(li, k_rows, v_rows)
     token = 31
     dec.reset(token, p0)
     for pos in range(p0, p0 + steps):
@@ -258,11 +257,9 @@ def test_gemma3_1b_shape_at_context_2040(ctx, pkg, oracle):
             dec.set_layer_attention(li, 0, 1.0e6), ref.set_layer_attention(li, 0, 1.0e6)
     rng = np.random.default_rng(2040)
     for li in range(cfg["n_layers"]):
-        kptr, vptr = dec.kv_cache(li)
-        for ptr, dst in ((kptr, ref.k), (vptr, ref.v)):
-            rows = (rng.standard_normal((1, max_seq, 256)) * 0.5).astype(np.float16)
-            dst[li] = rows
-            ctx._check(ctx.lib.hipc_upload(ctx.handle, ptr, 0, rows.ctypes.data, rows.nbytes))
+        k_rows, v_rows = ((rng.standard_normal((1, max_seq, 256)) * 0.5).astype(np.float16) for _ in range(2))
+        ref.k[li], ref.v[li] = k_rows, v_rows
+        dec.fill_cache(li, k_rows, v_rows)
     token = 1234
     dec.reset(token, p0)
     for pos in range(p0, p0 + steps):
