@@ -314,26 +314,33 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
 }
 
 // ---- the context chunks of one decode step's attention in one launch (head_dim 64 / 128 / 256) ----
-// Workgroup (split, kvh) owns attn_chunk(span) consecutive positions of kv head kvh and serves all G
-// query heads of the group; a wavefront owns 16 positions of every pass of 64 and never waits for
-// another wavefront between the first barrier (q ready) and the last (the join). Both products run
-// on the matrix cores:
-//   scores   S[row, t] = sum_d q[row, d] K[t, d]    16x16x32 f16: the B operand of position t is
-//            16 bytes of the row-major key cache as they lie; the A operand's rows 2 g and 2 g + 1
-//            are head g's query as two f16 terms (hi = f16(q), lo = f16(q - hi): 22 bits), so that a
-//            lane's result registers (rows 4 j .. 4 j + 3) add up to two heads' scores;
-//   outputs  O[row, d] = sum_t p[row, t] V[t, d]    32x32x16 f16: the B operand of channel d is 16
-//            bytes (8 positions) of the TRANSPOSED value cache [kv head][channel][position]; the A
-//            operand's rows are the heads' weights as two f16 terms, turned from the scores' layout
-//            (lane = position) into the operand's (lane = row) through the wavefront's own LDS rows.
-// The step's own position never comes from the cache: the workgroup that owns it (the last live one)
-// writes the cache rows and joins q.k_new / v_new as a fifth partial beside its wavefronts' four.
-// A workgroup writes (max, sum) per head and the unnormalised output: the flash-decoding partial
-// that the consumer joins over the live chunks (the output projection's prologue, or
-// dec_attn_merge_kernel). HD and G are template parameters so that the body is straight-line code.
+// Workgroup (split, kvh) owns attn_chunk(span) consecutive positions of kv head kvh, walks them
+// kAttnPass = 32 at a time and serves all G query heads of the group. What bounds the kernel is the
+// rate at which one CU takes K and V in (64 bytes a clock), so a chunk is as short as the join of the
+// partials allows: 32 positions while the span is at most 2048. Both products run on the matrix
+// cores, 16x16x32 f16:
+//   scores   S[row, t] = sum_d q[row, d] K[t, d]: wavefront (pb, dh) multiplies positions 16 pb .. + 16
+//            by half dh of the channels; the B operand of position t is 16 bytes of the row-major key
+//            cache as they lie; the A operand's rows 2 g and 2 g + 1 are head g's query as two f16
+//            terms (hi = f16(q), lo = f16(q - hi): 22 bits), so that a lane's result registers (rows
+//            4 j .. 4 j + 3) add up to two heads' scores. The halves meet in LDS (one barrier);
+//   softmax  every wavefront forms the pass's weights for all 32 positions (the same arithmetic in
+//            each: nothing to exchange, and all hold the same running max and sum);
+//   outputs  O[row, c] = sum_t p[row, t] V[t, c]: wavefront w multiplies all 32 positions by its
+//            quarter of the channels; the B operand of channel c is 16 bytes (8 positions) of the
+//            TRANSPOSED value cache [kv head][channel][position]; the A operand's rows are the heads'
+//            weights as two f16 terms, turned from the scores' layout (lane = position) into the
+//            operand's (lane = row) through the wavefront's own LDS rows.
+// A wavefront's outputs are complete for its channels, so there is nothing to join at the end. The
+// step's own position never comes from the cache: the workgroup that owns it (the last live one)
+// writes the cache rows and adds q.k_new / v_new to its running triple. A workgroup writes (max, sum)
+// per head and the unnormalised output: the flash-decoding partial that the consumer joins over the
+// live chunks (the output projection's prologue, or dec_attn_merge_kernel).
+// Nothing branches on the position before the end: a workgroup without positions runs on with empty
+// descriptors and skips the stores. (An early exit would let the compiler sink the first loads
+// below the wait for the position.) HD and G are template parameters: straight-line code.
 typedef _Float16 dh16x8 __attribute__((ext_vector_type(8)));
 typedef float df32x4 __attribute__((ext_vector_type(4)));
-typedef float df32x16 __attribute__((ext_vector_type(16)));
 
 template <int HD, int G>
 __global__ void __launch_bounds__(256)
@@ -342,27 +349,28 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
                        int max_seq, int v_stride, float scale, int window, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
                        float *__restrict__ part_ml, float *__restrict__ part_o) {
     constexpr int GH = G * HD, NK = HD / 64, HALF = HD / 2;
-    constexpr int KS = HD / 32;                // 32-channel steps of the score product
-    constexpr int NB = HD / 32;                // 32-channel blocks of the output product
+    constexpr int KS = HD / 64;                // 32-channel steps of a wavefront's half of the score product
+    constexpr int NB = HD / 64;                // 16-channel blocks of a wavefront's quarter of the output product
     constexpr int R = 2 * G;                   // operand rows in use: two terms per head
     constexpr int ROWS = (G + 1 + 3) / 4;      // q heads and the k head, dealt to four wavefronts
     constexpr int QS = HD + 8;                 // halfs per operand row of q (16 bytes of padding: rows start in different banks)
-    constexpr int PS = 24;                     // halfs per operand row of p
+    constexpr int PS = kAttnPass + 8;          // halfs per operand row of p
     constexpr int HL = (G + 1) / 2;            // rows of 16 lanes that hold scores (two heads each)
-    constexpr int JN = G == 8 ? 8 : 4;         // result registers of an output block that hold rows in use
     constexpr float NEG = -3.0e38f;
-    static_assert(kAttnPass == 64, "four wavefronts of 16 positions");
+    static_assert(kAttnPass == 32, "two blocks of 16 positions; the output product's k");
     __shared__ __attribute__((aligned(16))) __half qa[R * QS];       // query heads, normed, rotated, scaled: rows 2 g + term
+    __shared__ __attribute__((aligned(16))) float4 sp[4][64];          // per wavefront: its half of the scores, as the lanes hold them
     __shared__ __attribute__((aligned(16))) __half pa[4][16 * PS];    // per wavefront: the pass's weights, rows as in qa
-    __shared__ __attribute__((aligned(16))) float ow[4][GH];          // per wavefront: unnormalised outputs
     __shared__ __attribute__((aligned(16))) float kn[HD];             // the step's key, as the cache will hold it
     __shared__ __attribute__((aligned(16))) float vn[HD];             // the step's value
-    __shared__ float mw[4][G], lw[4][G], sown[G];
+    __shared__ float sown[2 * HL];                                      // the step's own scores
 
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int i16 = lane & 15, g4 = lane >> 4, n32 = lane & 31, h32 = lane >> 5;
+    const int pb = wave & 1, dh = wave >> 1;
+    const int i16 = lane & 15, g4 = lane >> 4;
+    const int pos = st->pos;
 
     // 1. the step's own rows (they come out of L2 and are needed first): rows 0..G-1 are the query
     //    heads, row G the key head; wavefront w prepares rows w, w + 4, ...; lane l holds elements
@@ -383,25 +391,26 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
     }
     const float pv_own = qkv[(size_t)(n_q + n_kv + kvh) * HD + min(tid, HD - 1)];
 
-    const int pos = st->pos, total = pos + 1;
-    if (pos >= max_seq) return;  // the cache is full: the step is a no-op
+    const int total = pos + 1;
     const int t_first = attn_first(total, window);  // a local layer sees the last `window` positions only
     const int base = t_first & ~15;
     const int chunk = attn_chunk(total - base);
     const int t_begin = base + split * chunk;
-    if (t_begin >= total) return;  // no position of this chunk exists yet
+    const bool dead = pos >= max_seq || t_begin >= total;   // the cache is full (the step is a no-op), or no position of this chunk exists yet
     const int t_end = min(total, t_begin + chunk);
-    const bool is_last = t_end == total;        // this workgroup owns the step's own position
-    const int hist_end = min(t_end, pos);       // positions below come from the cache
+    const bool is_last = !dead && t_end == total;           // this workgroup owns the step's own position
+    const int hist_end = min(t_end, pos);                   // positions below come from the cache
 
-    //    K: lane (position i16, quarter g4) reads its position's channels g4 HD/4 .. + HD/4, 16 bytes
-    //    per step (the query operand takes the same channel order); V: lane (channel n32, half h32)
-    //    reads positions 8 h32 .. + 8 of its wavefront's 16 for channel 32 b + n32. Rows past the end
-    //    of the cache are padding; positions that do not count are masked below.
-    const __amdgpu_buffer_rsrc_t r_k = __builtin_amdgcn_make_buffer_rsrc(k_cache, 0, (int)(((uint32_t)n_kv * (uint32_t)max_seq + kAttnPass) * HD * 2u), 0x00020000);
-    const __amdgpu_buffer_rsrc_t r_v = __builtin_amdgcn_make_buffer_rsrc(v_cache, 0, (int)((uint32_t)n_kv * HD * (uint32_t)v_stride * 2u), 0x00020000);
-    const uint32_t v_k = (uint32_t)((wave * 16 + i16) * HD + g4 * (HD / 4)) * 2u;
-    const uint32_t v_v = ((uint32_t)n32 * (uint32_t)v_stride + (uint32_t)(wave * 16 + h32 * 8)) * 2u;
+    //    K: lane (position i16 of block pb, quarter g4) reads HD/8 channels of half dh, 16 bytes per
+    //    step (the query operand takes the same channel order); V: lane (channel i16 of a block,
+    //    quarter g4) reads positions 8 g4 .. + 8 of the pass. Rows past the end of the cache are
+    //    padding; positions that do not count are masked below.
+    const __amdgpu_buffer_rsrc_t r_k = __builtin_amdgcn_make_buffer_rsrc(
+        k_cache, 0, dead ? 0 : (int)(((uint32_t)n_kv * (uint32_t)max_seq + 64u) * HD * 2u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t r_v = __builtin_amdgcn_make_buffer_rsrc(
+        v_cache, 0, dead ? 0 : (int)((uint32_t)n_kv * HD * (uint32_t)v_stride * 2u), 0x00020000);
+    const uint32_t v_k = (uint32_t)((pb * 16 + i16) * HD + dh * HALF + g4 * (HD / 8)) * 2u;
+    const uint32_t v_v = ((uint32_t)(wave * (HD / 4) + i16) * (uint32_t)v_stride + (uint32_t)(g4 * 8)) * 2u;
     uint4 kreg[KS], vreg[NB];
     auto load_k = [&](int t0) {
         const uint32_t s_k = ((uint32_t)kvh * (uint32_t)max_seq + (uint32_t)t0) * HD * 2u;
@@ -411,7 +420,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
     auto load_v = [&](int t0) {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            const uint32_t s_v = (((uint32_t)kvh * HD + b * 32u) * (uint32_t)v_stride + (uint32_t)t0) * 2u;
+            const uint32_t s_v = (((uint32_t)kvh * HD + b * 16u) * (uint32_t)v_stride + (uint32_t)t0) * 2u;
             vreg[b] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r_v, (int)v_v, (int)s_v, 0));
         }
     };
@@ -486,98 +495,94 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 #pragma unroll
     for (int u = 0; u < KS; u++) {
         uint4 raw = make_uint4(0, 0, 0, 0);
-        if (i16 < R) raw = *reinterpret_cast<const uint4 *>(qa + i16 * QS + g4 * (HD / 4) + u * 8);
+        if (i16 < R) raw = *reinterpret_cast<const uint4 *>(qa + i16 * QS + dh * HALF + g4 * (HD / 8) + u * 8);
         aq[u] = __builtin_bit_cast(dh16x8, raw);
     }
 
-    float m_run0 = NEG, m_run1 = NEG, l_run0 = 0.f, l_run1 = 0.f;   // heads 2 g4 and 2 g4 + 1, the same in every lane of a row of 16
-    df32x16 o[NB];
+    float m_run0 = NEG, m_run1 = NEG, l_run0 = 0.f, l_run1 = 0.f;   // heads 2 g4 and 2 g4 + 1; the same in every lane of a row of 16 and in every wavefront
+    df32x4 o[NB];
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) o[b][j] = 0.f;
+    for (int b = 0; b < NB; b++) o[b] = df32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int t0 = t_begin; t0 < t_end; t0 += kAttnPass) {
+    for (int t0 = t_begin; t0 < t_end; t0 += kAttnPass) {   // (a workgroup without positions: not once)
         const bool more = t0 + kAttnPass < t_end;
-        // 3a. scores of this wavefront's 16 positions, all heads
+        // 3a. this wavefront's half of the scores of its 16 positions, all heads
         df32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int u = 0; u < KS; u++) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[u], __builtin_bit_cast(dh16x8, kreg[u]), acc, 0, 0, 0);
+        sp[wave][lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
         if (more) load_k(t0 + kAttnPass);
-        const int t = t0 + wave * 16 + i16;
-        const bool valid = t >= t_first && t < hist_end;
-        const float s0 = valid ? acc[0] + acc[1] : NEG, s1 = valid ? acc[2] + acc[3] : NEG;
-        // 3b. the pass's max and sum join the running pair (a row of 16 lanes = the 16 positions)
-        const float m0 = fmaxf(m_run0, lean_row_max(s0)), m1 = fmaxf(m_run1, lean_row_max(s1));
+        __syncthreads();
+        // 3b. all 32 positions' scores (block b: wavefronts b and b + 2), the pass's max and sum
+        float s0[2], s1[2], p0[2], p1[2];
+        bool valid[2];
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const float4 lo = sp[b][lane], hi = sp[b + 2][lane];
+            const int t = t0 + b * 16 + i16;
+            valid[b] = t >= t_first && t < hist_end;
+            s0[b] = valid[b] ? (lo.x + hi.x) + (lo.y + hi.y) : NEG;
+            s1[b] = valid[b] ? (lo.z + hi.z) + (lo.w + hi.w) : NEG;
+        }
+        const float m0 = fmaxf(m_run0, lean_row_max(fmaxf(s0[0], s0[1]))), m1 = fmaxf(m_run1, lean_row_max(fmaxf(s1[0], s1[1])));
         const float f0 = __expf(m_run0 - m0), f1 = __expf(m_run1 - m1);
-        const float p0 = valid ? __expf(s0 - m0) : 0.f, p1 = valid ? __expf(s1 - m1) : 0.f;
-        l_run0 = fmaf(l_run0, f0, lean_row_sum(p0)), l_run1 = fmaf(l_run1, f1, lean_row_sum(p1));
+#pragma unroll
+        for (int b = 0; b < 2; b++) p0[b] = valid[b] ? __expf(s0[b] - m0) : 0.f, p1[b] = valid[b] ? __expf(s1[b] - m1) : 0.f;
+        l_run0 = fmaf(l_run0, f0, lean_row_sum(p0[0] + p0[1])), l_run1 = fmaf(l_run1, f1, lean_row_sum(p1[0] + p1[1]));
         m_run0 = m0, m_run1 = m1;
         //     weights as two f16 terms into the wavefront's LDS rows 4 g4 .. 4 g4 + 3, column = position
         if (g4 < HL) {
-            const __half h0 = __float2half(p0), h1 = __float2half(p1);
-            __half *dst = pa[wave] + (4 * g4) * PS + i16;
-            dst[0] = h0, dst[PS] = __float2half(p0 - __half2float(h0));
-            dst[2 * PS] = h1, dst[3 * PS] = __float2half(p1 - __half2float(h1));
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                const __half h0 = __float2half(p0[b]), h1 = __float2half(p1[b]);
+                __half *dst = pa[wave] + (4 * g4) * PS + b * 16 + i16;
+                dst[0] = h0, dst[PS] = __float2half(p0[b] - __half2float(h0));
+                dst[2 * PS] = h1, dst[3 * PS] = __float2half(p1[b] - __half2float(h1));
+            }
         }
         // the rows are this wavefront's own: its LDS operations complete in order, the compiler only must not reorder them
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         uint4 praw = make_uint4(0, 0, 0, 0);
-        if (n32 < R) praw = *reinterpret_cast<const uint4 *>(pa[wave] + n32 * PS + h32 * 8);
+        if (i16 < R) praw = *reinterpret_cast<const uint4 *>(pa[wave] + i16 * PS + g4 * 8);
         const dh16x8 ap = __builtin_bit_cast(dh16x8, praw);
-        // 3c. unnormalised outputs. Result register j of a lane holds row 8 (j / 4) + 4 h32 + j % 4,
-        //     i.e. head 4 (j / 4) + 2 h32 + (j % 4) / 2; what the earlier passes left is rescaled first.
-        if (t0 != t_begin) {
-            float fh[8];
+        // 3c. unnormalised outputs of this wavefront's channels: a lane's result registers are rows
+        //     4 g4 .. + 3, the heads whose factors it holds
 #pragma unroll
-            for (int g = 0; g < 8; g++) fh[g] = g < G ? lean_lane((g & 1) ? f1 : f0, 16 * (g >> 1)) : 1.f;
-#pragma unroll
-            for (int j = 0; j < JN; j++) {
-                const int ga = 4 * (j >> 2) + ((j & 3) >> 1);
-                const float fj = h32 ? fh[ga + 2] : fh[ga];
-#pragma unroll
-                for (int b = 0; b < NB; b++) o[b][j] *= fj;
-            }
+        for (int b = 0; b < NB; b++) {
+            o[b][0] *= f0, o[b][1] *= f0, o[b][2] *= f1, o[b][3] *= f1;
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ap, __builtin_bit_cast(dh16x8, vreg[b]), o[b], 0, 0, 0);
         }
-#pragma unroll
-        for (int b = 0; b < NB; b++) o[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ap, __builtin_bit_cast(dh16x8, vreg[b]), o[b], 0, 0, 0);
-        if (more) load_v(t0 + kAttnPass);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the next pass rewrites the weight rows
-        __builtin_amdgcn_wave_barrier();
+        if (more) {
+            load_v(t0 + kAttnPass);
+            __syncthreads();   // the next pass's scores must not overtake this pass's reads of sp
+        }
     }
 
-    // 4. the wavefront's partial: (max, sum) per head and the outputs (the two terms' rows added)
-    if (i16 == 0 && g4 < HL) {
-        mw[wave][2 * g4] = m_run0, lw[wave][2 * g4] = l_run0;
-        if (2 * g4 + 1 < G) mw[wave][2 * g4 + 1] = m_run1, lw[wave][2 * g4 + 1] = l_run1;
+    // 4. the step's own position joins in the workgroup that owns it; then the partial goes out
+    float e0 = 1.f, e1 = 1.f, eo0 = 0.f, eo1 = 0.f;
+    if (is_last) {
+        const float so0 = sown[min(2 * g4, 2 * HL - 1)], so1 = sown[min(2 * g4 + 1, 2 * HL - 1)];
+        const float M0 = fmaxf(m_run0, so0), M1 = fmaxf(m_run1, so1);
+        e0 = __expf(m_run0 - M0), e1 = __expf(m_run1 - M1), eo0 = __expf(so0 - M0), eo1 = __expf(so1 - M1);
+        m_run0 = M0, m_run1 = M1;
+        l_run0 = fmaf(l_run0, e0, eo0), l_run1 = fmaf(l_run1, e1, eo1);
     }
-#pragma unroll
-    for (int jj = 0; jj < JN / 2; jj++) {
-        const int head = 4 * (jj >> 1) + 2 * h32 + (jj & 1);
-        if (head < G) {
-#pragma unroll
-            for (int b = 0; b < NB; b++) ow[wave][head * HD + b * 32 + n32] = o[b][2 * jj] + o[b][2 * jj + 1];
-        }
-    }
-    __syncthreads();
-    // 5. the four wavefronts' partials and, in the workgroup that owns it, the step's own position
+    if (dead) return;
     float *po = part_o + ((size_t)kvh * kAttnSplits + split) * GH;
     float *ml = part_ml + ((size_t)kvh * kAttnSplits + split) * G * 2;
-    for (int idx = tid; idx < GH; idx += 256) {
-        const int g = idx / HD, ch = idx % HD;
-        const float ma = mw[0][g], mb = mw[1][g], mc = mw[2][g], md = mw[3][g];
-        const float so = is_last ? sown[g] : NEG;
-        const float M = fmaxf(fmaxf(fmaxf(ma, mb), fmaxf(mc, md)), so);
-        const float ea = __expf(ma - M), eb = __expf(mb - M), ec = __expf(mc - M), ed = __expf(md - M);
-        const float eo = is_last ? __expf(so - M) : 0.f;
-        float out = (ea * ow[0][idx] + eb * ow[1][idx]) + (ec * ow[2][idx] + ed * ow[3][idx]);
-        if (is_last) out = fmaf(eo, vn[ch], out);
-        po[idx] = out;
-        if (ch == 0) {
-            ml[g * 2] = M;
-            ml[g * 2 + 1] = (ea * lw[0][g] + eb * lw[1][g]) + (ec * lw[2][g] + ed * lw[3][g]) + eo;
+    if (g4 < HL) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const int ch = wave * (HD / 4) + b * 16 + i16;
+            const float own = is_last ? vn[ch] : 0.f;
+            po[(2 * g4) * HD + ch] = fmaf(o[b][0] + o[b][1], e0, eo0 * own);
+            if (2 * g4 + 1 < G) po[(2 * g4 + 1) * HD + ch] = fmaf(o[b][2] + o[b][3], e1, eo1 * own);
+        }
+        if (wave == 0 && i16 == 0) {
+            ml[4 * g4] = m_run0, ml[4 * g4 + 1] = l_run0;
+            if (2 * g4 + 1 < G) ml[4 * g4 + 2] = m_run1, ml[4 * g4 + 3] = l_run1;
         }
     }
 }
@@ -768,7 +773,7 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         d->nsplit = (int)ceil_div(c.max_seq, kAttnChunk);
         // keys [kv head][position][channel] with a pass of padding rows behind the last head (the one-launch
         // attention reads whole passes); values transposed, [kv head][channel][position], rows of v_stride
-        const size_t k_halfs = ((size_t)c.n_kv_heads * c.max_seq + kAttnPass) * c.head_dim;
+        const size_t k_halfs = ((size_t)c.n_kv_heads * c.max_seq + 64) * c.head_dim;
         const size_t v_halfs = (size_t)c.n_kv_heads * c.head_dim * attn_v_stride(c.max_seq);
         const int G = c.n_q_heads / c.n_kv_heads;
         int rc = HIPC_OK;

@@ -250,12 +250,12 @@ struct GemvPrologue {
     int group = 0, head_dim = 0, window = 0;
 };
 // Decode attention splits the visible context of a kv head over kAttnSplits workgroups. The split
-// starts at attn_base: the first visible position rounded down to 16 (a wavefront's 16 positions are
-// then 32-byte aligned in the transposed value cache; positions before the first visible one are
-// masked). Each workgroup takes attn_chunk(span) consecutive positions of the span from there to the
-// end, kAttnPass at a time: one pass while span <= kAttnPass * kAttnSplits = 4096 positions. The first
+// starts at attn_base: the first visible position rounded down to 16 (16 positions are then 32 bytes,
+// aligned, in the transposed value cache; positions before the first visible one are masked). Each
+// workgroup takes attn_chunk(span) consecutive positions of the span from there to the end,
+// kAttnPass at a time: one pass while span <= kAttnPass * kAttnSplits = 2048 positions. The first
 // attn_live_chunks(span) splits hold at least one position and only those write a partial.
-constexpr int kAttnPass = 64;
+constexpr int kAttnPass = 32;
 constexpr int kAttnSplits = 64;
 // first visible position of a step that sees `total` positions through a window (<= 0: no window)
 __host__ __device__ inline int attn_first(int total, int window) { return window > 0 && total > window ? total - window : 0; }
@@ -269,8 +269,8 @@ __host__ __device__ inline int attn_live_chunks(int span) {
     const int c = attn_chunk(span);
     return (span + c - 1) / c;
 }
-// the transposed value cache's row length: max_seq rounded up to a pass
-__host__ __device__ inline int attn_v_stride(int max_seq) { return (max_seq + kAttnPass - 1) / kAttnPass * kAttnPass; }
+// the transposed value cache's row length: max_seq rounded up to 64
+__host__ __device__ inline int attn_v_stride(int max_seq) { return (max_seq + 63) / 64 * 64; }
 int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
                const GemvPrologue *pro = nullptr);
 
