@@ -111,6 +111,7 @@ const OptionName kOptions[] = {
     {"HIPC_DEC_FUSED_ATTN", &Tuning::dec_fused_attn},
     {"HIPC_GEMV_LEAN", &Tuning::gemv_lean},
     {"HIPC_DEC_LEAN", &Tuning::dec_lean},
+    {"HIPC_DEC_PREFETCH", &Tuning::dec_prefetch},
 };
 
 int create(int device, void *stream, bool adopt, hipc_ctx **out) {

@@ -24,6 +24,7 @@
 
 #include "internal.h"
 #include "lanes.h"
+#include "prefetch.h"
 
 namespace hipc {
 
@@ -347,7 +348,7 @@ __global__ void __launch_bounds__(256)
 dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
                        const float *__restrict__ k_norm, int n_q, int n_kv, float eps, const float *__restrict__ rope,
                        int max_seq, int v_stride, float scale, int window, __half *__restrict__ k_cache, __half *__restrict__ v_cache,
-                       float *__restrict__ part_ml, float *__restrict__ part_o) {
+                       float *__restrict__ part_ml, float *__restrict__ part_o, const PrefetchArgs pf) {
     constexpr int GH = G * HD, NK = HD / 64, HALF = HD / 2;
     constexpr int KS = HD / 64;                // 32-channel steps of a wavefront's half of the score product
     constexpr int NB = HD / 64;                // 16-channel blocks of a wavefront's quarter of the output product
@@ -365,6 +366,11 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
     __shared__ __attribute__((aligned(16))) float vn[HD];             // the step's value
     __shared__ float sown[2 * HL];                                      // the step's own scores
 
+    if ((int)blockIdx.y >= n_kv) {   // a helper row: read ahead for the next launch, nothing else
+        prefetch_for_next(pf, ((int)blockIdx.y - n_kv) * (int)gridDim.x + (int)blockIdx.x, pf.rows * (int)gridDim.x,
+                          (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x, pf.sink);
+        return;
+    }
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -401,21 +407,21 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
     const bool is_last = !dead && t_end == total;           // this workgroup owns the step's own position
     const int hist_end = min(t_end, pos);                   // positions below come from the cache
 
-    //    K: lane (position i16 of block pb, quarter g4) reads HD/8 channels of half dh, 16 bytes per
-    //    step (the query operand takes the same channel order); V: lane (channel i16 of a block,
-    //    quarter g4) reads positions 8 g4 .. + 8 of the pass. Rows past the end of the cache are
+    //    K: step u of lane (position i16 of block pb, quarter g4) reads channels 32 u + 8 g4 .. + 8 of
+    //    half dh: the four quarters of a position ask for 64 consecutive bytes in one instruction;
+    //    V: lane (channel i16 of a block, quarter g4) reads positions 8 g4 .. + 8 of the pass. Rows past the end of the cache are
     //    padding; positions that do not count are masked below.
     const __amdgpu_buffer_rsrc_t r_k = __builtin_amdgcn_make_buffer_rsrc(
         k_cache, 0, dead ? 0 : (int)(((uint32_t)n_kv * (uint32_t)max_seq + 64u) * HD * 2u), 0x00020000);
     const __amdgpu_buffer_rsrc_t r_v = __builtin_amdgcn_make_buffer_rsrc(
         v_cache, 0, dead ? 0 : (int)((uint32_t)n_kv * HD * (uint32_t)v_stride * 2u), 0x00020000);
-    const uint32_t v_k = (uint32_t)((pb * 16 + i16) * HD + dh * HALF + g4 * (HD / 8)) * 2u;
+    const uint32_t v_k = (uint32_t)((pb * 16 + i16) * HD + dh * HALF + g4 * 8) * 2u;
     const uint32_t v_v = ((uint32_t)(wave * (HD / 4) + i16) * (uint32_t)v_stride + (uint32_t)(g4 * 8)) * 2u;
     uint4 kreg[KS], vreg[NB];
     auto load_k = [&](int t0) {
         const uint32_t s_k = ((uint32_t)kvh * (uint32_t)max_seq + (uint32_t)t0) * HD * 2u;
 #pragma unroll
-        for (int u = 0; u < KS; u++) kreg[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r_k, (int)(v_k + u * 16u), (int)s_k, 0));
+        for (int u = 0; u < KS; u++) kreg[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r_k, (int)(v_k + u * 64u), (int)s_k, 0));
     };
     auto load_v = [&](int t0) {
 #pragma unroll
@@ -495,7 +501,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 #pragma unroll
     for (int u = 0; u < KS; u++) {
         uint4 raw = make_uint4(0, 0, 0, 0);
-        if (i16 < R) raw = *reinterpret_cast<const uint4 *>(qa + i16 * QS + dh * HALF + g4 * (HD / 8) + u * 8);
+        if (i16 < R) raw = *reinterpret_cast<const uint4 *>(qa + i16 * QS + dh * HALF + u * 32 + g4 * 8);
         aq[u] = __builtin_bit_cast(dh16x8, raw);
     }
 
@@ -694,6 +700,7 @@ struct hipc_decoder {
     float *yo = nullptr, *yd = nullptr;      // [o_slices][hidden], [down_slices][hidden] partial rows
     uint4 *h_split = nullptr;                // the gated row in operand order (see LeanArgs)
     int nsplit = 0;
+    uint32_t *pf_sink = nullptr;   // where a helper workgroup would write (it never does: keeps its loads alive)
     bool one_launch_attn = false;  // head_dim and group size have an instance of dec_attn_chunks_kernel
     std::vector<void *> owned;
 };
@@ -710,30 +717,31 @@ int dev_alloc(hipc_ctx *ctx, hipc_decoder *d, T **p, size_t count) {
 }
 
 template <int HD, int G>
-void attn_chunks_launch(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale) {
+void attn_chunks_launch(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale, const PrefetchArgs &pf) {
     const hipc_decoder_config &c = d->cfg;
-    dec_attn_chunks_kernel<HD, G><<<dim3(kAttnSplits, c.n_kv_heads), 256, 0, ctx->stream>>>(
+    dec_attn_chunks_kernel<HD, G><<<dim3(kAttnSplits, c.n_kv_heads + (pf.kind ? pf.rows : 0)), 256, 0, ctx->stream>>>(
         d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.rms_eps,
         d->rope + (size_t)l.rope_table * c.head_dim, c.max_seq, attn_v_stride(c.max_seq), scale, l.window, l.k_cache, l.v_cache,
-        d->part_ml, d->part_o);
+        d->part_ml, d->part_o, pf);
 }
 
 template <int HD>
-void attn_chunks_launch_g(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale, int G) {
+void attn_chunks_launch_g(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale, int G, const PrefetchArgs &pf) {
     switch (G) {
-        case 1: attn_chunks_launch<HD, 1>(ctx, d, l, scale); break;
-        case 2: attn_chunks_launch<HD, 2>(ctx, d, l, scale); break;
-        case 4: attn_chunks_launch<HD, 4>(ctx, d, l, scale); break;
-        default: attn_chunks_launch<HD, 8>(ctx, d, l, scale); break;
+        case 1: attn_chunks_launch<HD, 1>(ctx, d, l, scale, pf); break;
+        case 2: attn_chunks_launch<HD, 2>(ctx, d, l, scale, pf); break;
+        case 4: attn_chunks_launch<HD, 4>(ctx, d, l, scale, pf); break;
+        default: attn_chunks_launch<HD, 8>(ctx, d, l, scale, pf); break;
     }
 }
 
-int launch_attn_chunks(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale) {
+// pf: what the launch's helper rows read ahead for the launch after it (kind 0: no helper rows)
+int launch_attn_chunks(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale, const PrefetchArgs &pf = PrefetchArgs()) {
     const int G = d->cfg.n_q_heads / d->cfg.n_kv_heads;
     switch (d->cfg.head_dim) {
-        case 64: attn_chunks_launch_g<64>(ctx, d, l, scale, G); break;
-        case 128: attn_chunks_launch_g<128>(ctx, d, l, scale, G); break;
-        default: attn_chunks_launch_g<256>(ctx, d, l, scale, G); break;
+        case 64: attn_chunks_launch_g<64>(ctx, d, l, scale, G, pf); break;
+        case 128: attn_chunks_launch_g<128>(ctx, d, l, scale, G, pf); break;
+        default: attn_chunks_launch_g<256>(ctx, d, l, scale, G, pf); break;
     }
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
@@ -774,7 +782,9 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         // keys [kv head][position][channel] with a pass of padding rows behind the last head (the one-launch
         // attention reads whole passes); values transposed, [kv head][channel][position], rows of v_stride
         const size_t k_halfs = ((size_t)c.n_kv_heads * c.max_seq + 64) * c.head_dim;
-        const size_t v_halfs = (size_t)c.n_kv_heads * c.head_dim * attn_v_stride(c.max_seq);
+        // (+ a pass: a chunk that starts less than a pass before the end of a row reads on into the next row,
+        // the last row's into this padding; those positions are masked)
+        const size_t v_halfs = (size_t)c.n_kv_heads * c.head_dim * attn_v_stride(c.max_seq) + 2 * kAttnPass;
         const int G = c.n_q_heads / c.n_kv_heads;
         int rc = HIPC_OK;
         auto A = [&](auto **p, size_t n) { if (rc == HIPC_OK) rc = dev_alloc(ctx, d, p, n); };
@@ -789,6 +799,7 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         const size_t parts = (size_t)c.n_kv_heads * std::max(d->nsplit, kAttnSplits) * G;
         A(&d->part_ml, parts * 2), A(&d->part_o, parts * c.head_dim);
         A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
+        A(&d->pf_sink, 4);
         A(&d->rope, (size_t)2 * c.head_dim), A(&d->x2, c.hidden);
         // options read when the decoder is created: dec_fused_glue = 0 keeps the separate norm / GELU
         // kernels, dec_fused_attn = 0 the three-kernel attention (tests of those paths)
@@ -985,20 +996,41 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
         // branch into the stream reads one and (its first workgroup) writes the other.
         float *xc = d->x, *xo = d->x2;
+        // Every launch of a layer carries helper rows that read ahead what the NEXT launch will read
+        // (its weights, or the attention's cache rows) into the L2 of the XCD that will ask for it.
+        // Off unless the dec_prefetch option is set to 1: the first version read past the end of a weight (the
+        // hardware's range check of a buffer load does not cover the scalar offset) and faulted; the
+        // corrected version has not run on a GPU yet.
+        const bool ahead = ctx->tune.dec_prefetch > 0;
+        auto rows_for = [](int64_t gx) { return (int)std::max<int64_t>(1, std::min<int64_t>(8, (192 + gx - 1) / gx)); };   // about 200 helper workgroups
         for (int li = 0; li < c.n_layers && d->lean; li++) {
             DecLayer &l = d->layers[li];
-            LeanPlan pl;
+            LeanPlan pl_qkv, pl_o, pl_gu, pl_down, pl_next;
+            HIPC_REQUIRE(ctx, lean_plan(ctx, l.qkv, 1, 1, &pl_qkv), "decoder: no launch plan for the qkv projection");
+            pl_o = LeanPlan{1, (int)ceil_div(l.o->n_cg, d->o_slices), 4, d->o_slices};   // four wavefronts, each all k tiles of the slice: no sum over wavefronts
+            HIPC_REQUIRE(ctx, lean_plan(ctx, l.gate_up, 1, 2, &pl_gu), "decoder: no launch plan for the gate | up projection");
+            HIPC_REQUIRE(ctx, lean_plan(ctx, l.down, d->down_slices, 1, &pl_down, 8), "decoder: no launch plan for the down projection");
+            auto gx_of = [](const hipc_nbits_weight *w, const LeanPlan &p) { return ceil_div(w->n_tiles, p.WN); };
             // qkv: row = rmsnorm(x', w_input), x' = x + rmsnorm(sum of the down projection's partial rows, w_post_ffn of the layer before)
             {
                 LeanArgs a{};
                 a.x = xc, a.w_in = l.norm[HIPC_DEC_NORM_INPUT], a.x_out = xo, a.eps = c.rms_eps;
                 if (li > 0) a.yparts = d->yd, a.y_slices = d->down_slices, a.w_post = d->layers[li - 1].norm[HIPC_DEC_NORM_POST_FFN];
                 a.Y = d->qkv;
-                HIPC_REQUIRE(ctx, lean_plan(ctx, l.qkv, 1, 1, &pl), "decoder: no launch plan for the qkv projection");
-                if ((rc = lean_gemv(ctx, l.qkv, pl, a, 2, 0, terms)) != HIPC_OK) return rc;
+                if (ahead) {   // the attention's cache rows
+                    PrefetchArgs &pf = a.pf;
+                    pf.kind = 2, pf.rows = rows_for(gx_of(l.qkv, pl_qkv)), pf.sink = d->pf_sink;
+                    pf.pos = &d->state->pos, pf.k = l.k_cache, pf.v = l.v_cache, pf.window = l.window, pf.max_seq = c.max_seq;
+                    pf.v_stride = attn_v_stride(c.max_seq), pf.hd = c.head_dim, pf.n_kv = c.n_kv_heads;
+                }
+                if ((rc = lean_gemv(ctx, l.qkv, pl_qkv, a, 2, 0, terms)) != HIPC_OK) return rc;
                 std::swap(xc, xo);
             }
-            if ((rc = launch_attn_chunks(ctx, d, l, scale)) != HIPC_OK) return rc;
+            {
+                PrefetchArgs pf;
+                if (ahead) pf = lean_prefetch_of(l.o, pl_o, rows_for(kAttnSplits), d->pf_sink);
+                if ((rc = launch_attn_chunks(ctx, d, l, scale, pf)) != HIPC_OK) return rc;
+            }
             // output projection: a k slice per head, joined from the attention partials; partial rows out
             {
                 LeanArgs a{};
@@ -1006,9 +1038,8 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 a.lg_group = __builtin_ctz((unsigned)(c.n_q_heads / c.n_kv_heads)), a.lg_hd = __builtin_ctz((unsigned)c.head_dim);   // powers of two where the one-launch attention runs
                 a.n_kv = c.n_kv_heads, a.window = l.window;
                 a.Y = d->yo;
-                const int per_slice = (int)ceil_div(l.o->n_cg, d->o_slices);
-                pl = LeanPlan{1, per_slice, 4, d->o_slices};   // four wavefronts, each all k tiles of the slice: no sum over wavefronts
-                if ((rc = lean_gemv(ctx, l.o, pl, a, 3, 0, terms)) != HIPC_OK) return rc;
+                if (ahead) a.pf = lean_prefetch_of(l.gate_up, pl_gu, rows_for(gx_of(l.o, pl_o)), d->pf_sink);
+                if ((rc = lean_gemv(ctx, l.o, pl_o, a, 3, 0, terms)) != HIPC_OK) return rc;
             }
             // gate | up: row = rmsnorm(x'', w_pre_ffn), x'' = x' + rmsnorm(sum of the output projection's partial rows, w_post_attn);
             // epilogue gelu_tanh(gate) * up in operand order
@@ -1017,8 +1048,8 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 a.x = xc, a.w_in = l.norm[HIPC_DEC_NORM_PRE_FFN], a.x_out = xo, a.eps = c.rms_eps;
                 a.yparts = d->yo, a.y_slices = d->o_slices, a.w_post = l.norm[HIPC_DEC_NORM_POST_ATTN];
                 a.h_split = d->h_split;
-                HIPC_REQUIRE(ctx, lean_plan(ctx, l.gate_up, 1, 2, &pl), "decoder: no launch plan for the gate | up projection");
-                if ((rc = lean_gemv(ctx, l.gate_up, pl, a, 2, 1, terms)) != HIPC_OK) return rc;
+                if (ahead) a.pf = lean_prefetch_of(l.down, pl_down, rows_for(gx_of(l.gate_up, pl_gu)), d->pf_sink);
+                if ((rc = lean_gemv(ctx, l.gate_up, pl_gu, a, 2, 1, terms)) != HIPC_OK) return rc;
                 std::swap(xc, xo);
             }
             // down: the gated row straight into the operand registers; partial rows out
@@ -1026,9 +1057,9 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 LeanArgs a{};
                 a.a_split = d->h_split;
                 a.Y = d->yd;
-                HIPC_REQUIRE(ctx, lean_plan(ctx, l.down, d->down_slices, 1, &pl, 8),
-                             "decoder: no launch plan for the down projection");
-                if ((rc = lean_gemv(ctx, l.down, pl, a, 4, 0, terms)) != HIPC_OK) return rc;
+                if (ahead && li + 1 < c.n_layers && lean_plan(ctx, d->layers[li + 1].qkv, 1, 1, &pl_next))
+                    a.pf = lean_prefetch_of(d->layers[li + 1].qkv, pl_next, rows_for(gx_of(l.down, pl_down)), d->pf_sink);
+                if ((rc = lean_gemv(ctx, l.down, pl_down, a, 4, 0, terms)) != HIPC_OK) return rc;
             }
         }
         for (int li = 0; li < c.n_layers && !d->lean; li++) {

@@ -36,6 +36,7 @@
 
 #include "internal.h"
 #include "lanes.h"
+#include "prefetch.h"
 
 namespace hipc {
 
@@ -82,7 +83,8 @@ __device__ __forceinline__ float lean_gelu_tanh(float v) {
 
 // ---- buffer loads: a uniform descriptor, a per-lane byte offset computed once and a SCALAR offset per
 // load, so that asking for a tile, a partial row or a context chunk costs the vector unit nothing;
-// a load past the end of the descriptor's range returns zeros (no clamping, no zero filling)
+// a load whose per-lane offset lies past the end of the descriptor's range returns zeros (no clamping,
+// no zero filling); the scalar offset is NOT part of that check and must stay inside the buffer
 typedef unsigned int lu32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t lean_rsrc(const void *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
@@ -144,6 +146,11 @@ template <int SG, int NT, int PRO, int EPI, int KT>
 __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const LeanArgs p) {
     extern __shared__ uint4 lean_smem[];
     constexpr int CPG = 4 / SG;  // 32-k chunks per scale group
+    if ((int)blockIdx.y >= p.slices) {   // a helper row: read ahead for the next launch, nothing else
+        prefetch_for_next(p.pf, ((int)blockIdx.y - p.slices) * (int)gridDim.x + (int)blockIdx.x, p.pf.rows * (int)gridDim.x,
+                          (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x, p.pf.sink);
+        return;
+    }
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // wave = wn * WK + wk without a division: WK is at most 16 and WN at most 4
@@ -502,6 +509,15 @@ bool hipc::lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int 
     return true;
 }
 
+PrefetchArgs hipc::lean_prefetch_of(const hipc_nbits_weight *w, const LeanPlan &pl, int rows, uint32_t *sink) {
+    PrefetchArgs pf;
+    pf.kind = 1, pf.rows = rows, pf.sink = sink;
+    pf.wq = w->Wq, pf.sc = w->Sc, pf.zb = w->Zb;
+    pf.gx = (int)ceil_div(w->n_tiles, pl.WN), pf.gy = pl.slices, pf.WN = pl.WN, pf.slice_tiles = pl.WK * pl.KT;
+    pf.n_cg = w->n_cg, pf.n_tiles = w->n_tiles, pf.SG = w->SG;
+    return pf;
+}
+
 int hipc::lean_gemv(hipc_ctx *ctx, const hipc_nbits_weight *w, const LeanPlan &pl, LeanArgs a, int pro, int epi, int NT) {
     a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb;
     a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
@@ -522,7 +538,8 @@ int hipc::lean_gemv(hipc_ctx *ctx, const hipc_nbits_weight *w, const LeanPlan &p
     size_t lds = (size_t)slice_tiles * 4 * NT * 4 * 16;
     lds += (size_t)pl.WN * 16 * 16 * 4;   // reduction area [WN][16][16]; the norm's partial sums [16][4][4] fit its first KiB
     HIPC_REQUIRE(ctx, lds <= 64 * 1024, "MatMulNBits lean gemv: LDS plan of %zu bytes does not fit", lds);
-    const dim3 grid((unsigned)ceil_div(w->n_tiles, pl.WN), (unsigned)pl.slices);
+    if (a.pf.kind == 0) a.pf.rows = 0;
+    const dim3 grid((unsigned)ceil_div(w->n_tiles, pl.WN), (unsigned)(pl.slices + a.pf.rows));
     const dim3 block((unsigned)threads);
     switch (w->SG) {
         case 4: return NT == 3 ? lean_launch_pro<4, 3>(ctx, a, pro, epi, grid, block, lds) : lean_launch_pro<4, 2>(ctx, a, pro, epi, grid, block, lds);

@@ -47,6 +47,7 @@ struct Tuning {
     int dec_fused_attn = -1;  // HIPC_DEC_FUSED_ATTN 0 keeps the three-kernel attention (read when a decoder is created)
     int gemv_lean = -1;       // HIPC_GEMV_LEAN      0: one-row products keep the streaming GEMV kernel
     int dec_lean = -1;        // HIPC_DEC_LEAN       0: the decoder keeps the streaming GEMV and its prologues (read when a decoder is created)
+    int dec_prefetch = -1;    // HIPC_DEC_PREFETCH   1: launches of the decode step carry helper rows that read ahead for the next launch (off by default)
 };
 
 // Pinned staging ring of hipc_upload: the bytes are copied into a slot and travel from there, so the
@@ -279,6 +280,21 @@ int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weigh
 // major -- split[(c * NT + term) * 4 + group] -- so that a lane's matrix-core A operand is one
 // 16-byte load. (The sums over a quantisation block's activations, which take the +128 bias of the
 // weights out again, are formed by the consumer on the matrix cores: a product against ones.)
+// What the helper rows of a launch read ahead for the launch that follows it (prefetch.h).
+struct PrefetchArgs {
+    int kind = 0;          // 0 nothing; 1 the weight tiles of a one-row product; 2 the cache rows of an attention launch
+    int rows = 0;          // helper rows appended to the producer's grid (gridDim.x workgroups each)
+    uint32_t *sink = nullptr;
+    // kind 1: the consumer's weight and launch shape
+    const uint4 *wq = nullptr;
+    const float *sc = nullptr;
+    const uint8_t *zb = nullptr;
+    int gx = 0, gy = 0, WN = 0, slice_tiles = 0, n_cg = 0, n_tiles = 0, SG = 0;
+    // kind 2: the attention launch's cache
+    const int *pos = nullptr;
+    const void *k = nullptr, *v = nullptr;
+    int window = 0, max_seq = 0, v_stride = 0, hd = 0, n_kv = 0;
+};
 struct LeanArgs {
     const uint4 *Wq;
     const float *Sc;
@@ -302,6 +318,7 @@ struct LeanArgs {
     float *Y;                    // EPI 0: [slices][N] partial rows (the row itself when slices == 1)
     // EPI 1: gelu_tanh(gate) * up of the interleaved (gate, up) tile pairs, in operand order
     uint4 *h_split;
+    PrefetchArgs pf;             // helper rows behind the `slices` rows of the grid
 };
 struct LeanPlan {
     int WK, KT, WN, slices;
@@ -310,6 +327,8 @@ struct LeanPlan {
 bool lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int WN, LeanPlan *out, int max_waves = 16);
 // `a` carries the prologue / epilogue operands; weight and launch-shape fields are filled in here
 int lean_gemv(hipc_ctx *ctx, const hipc_nbits_weight *w, const LeanPlan &pl, LeanArgs a, int pro, int epi, int NT);
+// the prefetch description of a one-row product launched with plan `pl` (for the launch before it)
+PrefetchArgs lean_prefetch_of(const hipc_nbits_weight *w, const LeanPlan &pl, int rows, uint32_t *sink);
 
 int64_t nbits_cols(const hipc_nbits_weight *w);
 int64_t nbits_depth(const hipc_nbits_weight *w);

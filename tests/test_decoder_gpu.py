@@ -47,7 +47,13 @@ DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / 
     (128, 4, 2, 130),    # three live chunks only
     (192, 2, 1, 100),    # no instance for this head_dim: the three-kernel path
 ]
-PATHS = [{}, {"HIPC_DEC_LEAN": 0}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
+# The read-ahead route (helper workgroups that warm the L2 for the next launch) faulted on the GPU at the
+# full decoder shape: a buffer load's scalar offset is outside the hardware's range check, and the helper
+# read up to 96 KiB past the end of a weight. The corrected helper (per-lane offsets only) has not run on
+# a GPU since; until it has, the route is off by default and its cases are skipped.
+READ_AHEAD = pytest.param({"HIPC_DEC_PREFETCH": 1}, marks=pytest.mark.skip(
+    reason="read-ahead helper rows: faulted before the range-check fix, not yet re-run on a GPU"))
+PATHS = [{}, READ_AHEAD, {"HIPC_DEC_LEAN": 0}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
 
 
 @pytest.fixture
@@ -64,7 +70,7 @@ def route(ctx):
         ctx.set_option(k, -1)
 
 
-@pytest.mark.parametrize("env", PATHS, ids=["default", "streaming-gemv", "separate-glue", "three-kernel-attention"])
+@pytest.mark.parametrize("env", PATHS, ids=["default", "read-ahead", "streaming-gemv", "separate-glue", "three-kernel-attention"])
 @pytest.mark.parametrize("hd,nq,nkv,p0", DEEP)
 def test_attention_over_a_long_filled_cache(ctx, pkg, oracle, route, hd, nq, nkv, p0, env):
     """Steps taken deep into a context whose cache rows hold random f16 values on both sides: the
@@ -109,7 +115,7 @@ WINDOWS = [  # (head_dim, query heads, kv heads, first position, window of layer
 ]
 
 
-@pytest.mark.parametrize("env", PATHS, ids=["default", "streaming-gemv", "separate-glue", "three-kernel-attention"])
+@pytest.mark.parametrize("env", PATHS, ids=["default", "read-ahead", "streaming-gemv", "separate-glue", "three-kernel-attention"])
 @pytest.mark.parametrize("hd,nq,nkv,p0,w0,w1", WINDOWS)
 def test_sliding_windows_and_a_second_rotary_base(ctx, pkg, oracle, route, hd, nq, nkv, p0, w0, w1, env):
     """Local layers: the last `window` positions only, the step's own included (the reference's
