@@ -295,6 +295,24 @@ struct PrefetchArgs {
     const void *k = nullptr, *v = nullptr;
     int window = 0, max_seq = 0, v_stride = 0, hd = 0, n_kv = 0;
 };
+// The tiles consumer j (= y * gx + x of the consumer's grid) reads for its column tile wn: a run of
+// `count` consecutive tiles from `*tile0` in all three weight arrays (0: nothing).
+__host__ __device__ inline int pf_tile_run(const PrefetchArgs &pf, int j, int wn, size_t *tile0) {
+    int x = j, y = 0;
+    while (x >= pf.gx) x -= pf.gx, y++;
+    const int kt0 = y * pf.slice_tiles;
+    const int cnt = pf.slice_tiles < pf.n_cg - kt0 ? pf.slice_tiles : pf.n_cg - kt0;
+    const int nt = x * pf.WN + wn;
+    if (y >= pf.gy || nt >= pf.n_tiles || cnt <= 0) return 0;
+    *tile0 = (size_t)nt * pf.n_cg + kt0;
+    return cnt;
+}
+// Helper h of H (linear workgroup id b in its launch) serves the consumers j = first, first + step, ...:
+// those of its own XCD class (j = b mod 8), dealt round robin to the helpers of that class.
+__host__ __device__ inline void pf_consumers_of(int h, int H, int b, int *first, int *step) {
+    *first = (b & 7) + 8 * (h >> 3);
+    *step = 8 * ((H + 7) >> 3);
+}
 struct LeanArgs {
     const uint4 *Wq;
     const float *Sc;

@@ -38,23 +38,21 @@ __device__ __forceinline__ uint32_t pf_span(uint32_t acc, const void *base, uint
 
 // h: this helper's index among the H helpers of the launch; b: its linear workgroup id in the launch
 __device__ inline void prefetch_for_next(const PrefetchArgs &pf, int h, int H, int b, uint32_t *sink) {
-    const int cls = b & 7, rank = h >> 3, per_cls = (H + 7) >> 3;
+    int first, step;
+    pf_consumers_of(h, H, b, &first, &step);
     const int tid = threadIdx.x, nthreads = blockDim.x;
     uint32_t acc = 0;
     if (pf.kind == 1) {
-        // consumer j = (x, y) of a one-row product's grid reads, for each of its WN column tiles, the
-        // tiles [kt0, kt0 + cnt) of that column: contiguous in all three arrays
+        // consumer j of a one-row product's grid reads, for each of its WN column tiles, a run of tiles
+        // that is contiguous in all three arrays
         const int n_cons = pf.gx * pf.gy;
-        for (int j = cls + 8 * rank; j < n_cons; j += 8 * per_cls) {
-            int x = j, y = 0;
-            while (x >= pf.gx) x -= pf.gx, y++;
-            const int kt0 = y * pf.slice_tiles;
-            const int cnt = min(pf.slice_tiles, pf.n_cg - kt0);
+        for (int j = first; j < n_cons; j += step) {
             for (int wn = 0; wn < pf.WN; wn++) {
-                const int nt = x * pf.WN + wn;
-                if (nt >= pf.n_tiles || cnt <= 0) break;
-                const size_t tile0 = (size_t)nt * pf.n_cg + kt0;
-                // at most 16 tiles a slice: 16 KiB of weights (6 rounds of >= 192 threads), 4 KiB of scales, 1 KiB of zero points
+                size_t tile0;
+                const int cnt = pf_tile_run(pf, j, wn, &tile0);
+                if (cnt == 0) break;
+                // six rounds of >= 192 threads cover a run of 18 tiles (18 KiB of weights, 4.5 KiB of scales, 1.1 KiB of
+                // zero points); of a longer run only that much is read ahead
                 acc = pf_span<6>(acc, pf.wq + tile0 * 64, (uint32_t)cnt * 1024u, tid, nthreads);
                 acc = pf_span<2>(acc, pf.sc + tile0 * 16 * pf.SG, (uint32_t)cnt * 64u * pf.SG, tid, nthreads);
                 acc = pf_span<1>(acc, pf.zb + tile0 * 16 * pf.SG, (uint32_t)cnt * 16u * pf.SG, tid, nthreads);
@@ -67,7 +65,7 @@ __device__ inline void prefetch_for_next(const PrefetchArgs &pf, int h, int H, i
         const int base = attn_base(total, pf.window);
         const int chunk = attn_chunk(total - base);
         const int n_cons = kAttnSplits * pf.n_kv;
-        for (int j = cls + 8 * rank; j < n_cons; j += 8 * per_cls) {
+        for (int j = first; j < n_cons; j += step) {
             const int split = j & (kAttnSplits - 1), kvh = j / kAttnSplits;
             const int t0 = base + split * chunk;
             if (pos >= pf.max_seq || t0 >= total) continue;

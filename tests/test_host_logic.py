@@ -139,3 +139,19 @@ def test_missing_gpu_is_an_error_not_a_fallback(pkg):
         return
     c.close()
     pytest.skip("a GPU is present")
+
+
+def test_shared_index_arithmetic_on_the_host(tmp_path):
+    """The chunk split of the decode attention and the read-ahead helpers' tile runs are plain index
+    arithmetic in headers that host and device code share: tests/host/geometry_checks.cpp compiles
+    them for the host alone and checks their invariants (chunks cover the visible context, every tile
+    is read ahead once, from inside its array, by a helper of the consumer's XCD class)."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = str(tmp_path / "geometry_checks")
+    subprocess.run([hipcc, "--cuda-host-only", "-x", "hip", "-std=c++17", "-O1", "-I", os.path.join(root, "onnx-vulkan-rs_amd", "csrc"),
+                    os.path.join(root, "tests", "host", "geometry_checks.cpp"), "-o", exe], check=True, capture_output=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
