@@ -7,9 +7,13 @@ Prints ONE JSON line. The headline `value` is the HBM throughput of the int4 Mat
 GEMV over the linears of one gemma3-1b-shaped decode step (26 layers x 7 projections + lm_head,
 block 32 with zero points, M = 1): every weight is distinct and resident in HBM (640 MB per
 step, far beyond the 256 MB last-level cache), a step is replayed from a captured graph, and
-the clock is the host's around K steps with a flush on both sides. `roofline` is the dominant
-kernel (the lm_head GEMV) timed with device events on the library's stream; `extras` carries the
-other configurations (int8 GEMM TOPS, QLinearConv, single-op GEMVs hot and cold);
+the clock is the host's around K steps with a flush on both sides. `roofline` is the kernel that
+owns that step -- the narrow one-row MatMulNBits kernel of the 104 per-layer launches -- timed with
+device events on the library's stream over a graph of exactly those launches; the lm_head launch
+(one launch, 30 % of the bytes) is a labelled entry of `extras`, as are the same figures at
+accuracy_level = 1 (three bf16 terms per activation), the launch floor (a one-word fill kernel
+replayed in the same graph shape) and the other configurations (int8 GEMM TOPS, QLinearConv,
+single-op GEMVs hot and cold, the full decoder);
 `cpu_baseline` is the restated CPU oracle on this box's host cores (ONNX Runtime is not
 installed), on a bounded sample.
 """
@@ -57,8 +61,9 @@ def log(*a):
 class GemvSet:
     """Prepacked weights + device vectors of a list of (K, N) GEMVs, and a graph replaying them."""
 
-    def __init__(self, pkg, ctx, shapes, seed):
+    def __init__(self, pkg, ctx, shapes, seed, accuracy_level=0):
         self.pkg, self.ctx, self.items = pkg, ctx, []
+        self.accuracy_level = accuracy_level
         self.bytes = 0
         for i, (K, N) in enumerate(shapes):
             B, scales, zp = pkg.synth.fast_nbits_weight(N, K, BS, seed + i)
@@ -71,9 +76,12 @@ class GemvSet:
 
     def enqueue(self):
         for (w, a, y, K, N) in self.items:
-            self.pkg.ops.matmul_nbits_packed_device(self.ctx, a, self.pkg.F32, w, y, 1)
+            self.pkg.ops.matmul_nbits_packed_device(self.ctx, a, self.pkg.F32, w, y, 1, self.accuracy_level)
 
     def capture(self):
+        if self.graph:
+            self.ctx.graph_destroy(self.graph)
+            self.graph = None
         self.enqueue()  # warm every launch shape (scratch sizing) before recording
         self.ctx.flush()
         self.ctx.capture_begin()
@@ -99,34 +107,85 @@ def median_ns(ctx, graph, launches_per_graph=1, samples=20, reps=10):
     return float(np.median(ns)) / launches_per_graph, float(ns.min()) / launches_per_graph
 
 
+def host_timed_steps(ctx, graph, steps, warmup):
+    """Milliseconds per replay of `graph`: the host's clock around `steps` replays, a flush on both sides."""
+    for _ in range(warmup):
+        ctx.graph_launch(graph)
+    ctx.flush()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ctx.graph_launch(graph)
+    ctx.flush()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
 def bench_decode_linears(pkg, ctx, steps, warmup):
+    """The headline step (104 per-layer GEMVs + lm_head, host clock), then on the same weights: the
+    104 narrow launches alone under device events (the `roofline` block), and both again at
+    accuracy_level = 1. Returns (head, roofline, extras)."""
     shapes = []
     for _ in range(N_LAYERS):
         for (K, N, c) in LAYER_LINEARS:
             shapes += [(K, N)] * c
+    n_narrow = len(shapes)
     shapes.append(LM_HEAD)
     t0 = time.time()
     s = GemvSet(pkg, ctx, shapes, seed=5000)
     log(f"[bench] decode linears: {len(shapes)} weights, {s.bytes / 1e6:.1f} MB algorithmic, built in {time.time() - t0:.1f}s")
-    g = s.capture()
-    for _ in range(warmup):
-        ctx.graph_launch(g)
-    ctx.flush()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        ctx.graph_launch(g)
-    ctx.flush()
-    dt = time.perf_counter() - t0
-    ms = dt / steps * 1e3
-    res = dict(bytes_per_step=s.bytes, launches=len(shapes), ms_per_step=ms, gbs=s.bytes / (ms * 1e-3) / 1e9)
+    ms = host_timed_steps(ctx, s.capture(), steps, warmup)
+    head = dict(bytes_per_step=s.bytes, launches=len(shapes), ms_per_step=ms, gbs=s.bytes / (ms * 1e-3) / 1e9)
+    roof, extra = None, {}
+    every, narrow_bytes = s.items, s.bytes - gemv_bytes(*LM_HEAD)
+    try:
+        # the step at accuracy_level = 1 (f32 activations as three bf16 terms instead of two)
+        s.accuracy_level = 1
+        ms1 = host_timed_steps(ctx, s.capture(), steps, warmup)
+        extra["decode_linears_accuracy_level_1"] = dict(ms_per_step=ms1, gbs=s.bytes / (ms1 * 1e-3) / 1e9)
+        # the 104 narrow launches alone, device events on the library's stream around whole replays
+        s.items = every[:n_narrow]
+        per = narrow_bytes / n_narrow
+        med1, _ = median_ns(ctx, s.capture(), n_narrow, samples=15, reps=4)
+        s.accuracy_level = 0
+        med, mn = median_ns(ctx, s.capture(), n_narrow, samples=15, reps=4)
+        s.items = every
+        roof = dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS, traffic=None,
+                    kernel="mmnb_lean_kernel, PRO 0 (the 104 per-layer one-row MatMulNBits launches of the step: q|k|v, o, gate|up, down x 26)",
+                    bytes_per_launch=per, avg_launch_us=med / 1e3, min_launch_us=mn / 1e3, launches_per_replay=n_narrow,
+                    timing="device events around whole graph replays / launches per replay: launch gaps included",
+                    accuracy_level_1=dict(avg_launch_us=med1 / 1e3, achieved=per / med1, frac=per / med1 / HBM_PEAK_GBS))
+    except Exception as e:  # the headline above stands on its own
+        log(f"[bench] narrow-GEMV roofline failed: {e!r}")
+    s.items = every
     s.destroy()
-    return res
+    return head, roof, extra
 
 
-def bench_lm_head_roofline(pkg, ctx, copies=3):
-    """The dominant kernel: lm_head GEMV rotating over `copies` distinct weights (~200 MB each)."""
+def bench_launch_floor(ctx, launches=105):
+    """What a launch costs when the kernel does nothing: a one-word fill (one workgroup) replayed in a
+    graph of the headline step's shape, device events around whole replays."""
+    buf = ctx.alloc(4096)
+
+    def enqueue():
+        for i in range(launches):
+            ctx.fill(buf, 4 * (i % 64), 4, i)
+
+    enqueue()
+    ctx.flush()
+    ctx.capture_begin()
+    enqueue()
+    g = ctx.capture_end()
+    med, mn = median_ns(ctx, g, launches, samples=20, reps=4)
+    ctx.graph_destroy(g)
+    buf.free()
+    ctx.flush()
+    return dict(us_per_launch=med / 1e3, min_us_per_launch=mn / 1e3, launches_per_graph=launches,
+                kernel="one-word fill, one workgroup; every launch depends on the one before (one in-order stream)")
+
+
+def bench_lm_head(pkg, ctx, copies=3, accuracy_level=0):
+    """The widest launch of the step: lm_head GEMV rotating over `copies` distinct weights (~200 MB each)."""
     K, N = LM_HEAD
-    s = GemvSet(pkg, ctx, [LM_HEAD] * copies, seed=7000)
+    s = GemvSet(pkg, ctx, [LM_HEAD] * copies, seed=7000, accuracy_level=accuracy_level)
     s.items = s.items * 4                     # 4 passes over the ring per graph
     g = s.capture()
     med, mn = median_ns(ctx, g, launches_per_graph=copies * 4, samples=15, reps=2)
@@ -135,7 +194,7 @@ def bench_lm_head_roofline(pkg, ctx, copies=3):
     s.destroy()
     return dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS,
                 traffic=LM_HEAD_TRAFFIC_BYTES, kernel="mmnb_gemv_kernel (lm_head 1152->262144, M=1)", bytes_per_launch=per,
-                avg_launch_us=med / 1e3, min_launch_us=mn / 1e3)
+                avg_launch_us=med / 1e3, min_launch_us=mn / 1e3, accuracy_level=accuracy_level)
 
 
 def bench_single_gemv(pkg, ctx, K, N, cold_copies):
@@ -402,7 +461,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", default="", help="comma list of sections to run (decode, lm_head, gemv, int8, conv, prefill, "
+    ap.add_argument("--only", default="", help="comma list of sections to run (decode, floor, lm_head, gemv, int8, conv, prefill, "
                     "decoder, cpu; copy = counter calibration, only on request); default all. Used to profile "
                     "one kernel at a time.")
     args = ap.parse_args()
@@ -417,13 +476,26 @@ def main():
     ctx = pkg.Context(0)
     head = dict(gbs=None, ms_per_step=None, bytes_per_step=None, launches=None)
     roof = None
-    if want("decode"):
-        head = bench_decode_linears(pkg, ctx, args.steps, args.warmup)
-        log(f"[bench] decode linears: {head['ms_per_step']:.3f} ms/step, {head['gbs']:.0f} GB/s")
-    if want("lm_head"):
-        roof = bench_lm_head_roofline(pkg, ctx)
-        log(f"[bench] lm_head gemv: {roof['avg_launch_us']:.1f} us, {roof['achieved']:.0f} GB/s")
     extras = {}
+    if want("decode"):
+        head, roof, more = bench_decode_linears(pkg, ctx, args.steps, args.warmup)
+        extras.update(more)
+        log(f"[bench] decode linears: {head['ms_per_step']:.3f} ms/step, {head['gbs']:.0f} GB/s")
+        if roof:
+            log(f"[bench] narrow gemv: {roof['avg_launch_us']:.2f} us per launch, {roof['achieved']:.0f} GB/s")
+    if want("floor"):
+        try:
+            extras["launch_floor"] = bench_launch_floor(ctx)
+            log("[bench] launch floor:", json.dumps(extras["launch_floor"]))
+        except Exception as e:
+            log(f"[bench] launch floor failed: {e!r}")
+    if want("lm_head"):
+        extras["lm_head_gemv"] = bench_lm_head(pkg, ctx)
+        log(f"[bench] lm_head gemv: {extras['lm_head_gemv']['avg_launch_us']:.1f} us, {extras['lm_head_gemv']['achieved']:.0f} GB/s")
+        try:
+            extras["lm_head_gemv_accuracy_level_1"] = bench_lm_head(pkg, ctx, accuracy_level=1)
+        except Exception as e:
+            log(f"[bench] lm_head at accuracy_level 1 failed: {e!r}")
     if want("gemv"):
         extras["gemv_up_1152x6912"] = bench_single_gemv(pkg, ctx, 1152, 6912, cold_copies=104)
         extras["gemv_down_6912x1152"] = bench_single_gemv(pkg, ctx, 6912, 1152, cold_copies=104)
