@@ -155,3 +155,18 @@ def test_shared_index_arithmetic_on_the_host(tmp_path):
                     os.path.join(root, "tests", "host", "geometry_checks.cpp"), "-o", exe], check=True, capture_output=True)
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
+
+
+def test_the_rust_binding_declares_every_entry_point():
+    """crates/hip-compute/src/sys.rs cannot be compiled here (no Rust toolchain); at least it must name
+    exactly the functions the header declares, with as many parameters each."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(root, "include", "hipcompute.h")).read(), flags=re.S)
+    rust = re.sub(r"//[^\n]*", "", open(os.path.join(root, "crates", "hip-compute", "src", "sys.rs")).read())
+    c_protos = {m.group(1): m.group(2) for m in re.finditer(r"\b(hipc_\w+)\(([^;{]*)\);", header)}
+    r_protos = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (hipc_\w+)\(([^;{]*?)\)\s*(?:->[^;]*)?;", rust, flags=re.S)}
+    assert sorted(c_protos) == sorted(r_protos)
+    for name, args in c_protos.items():
+        n_c = 0 if args.strip() in ("", "void") else args.count(",") + 1
+        n_r = len([a for a in r_protos[name].split(",") if a.strip()])
+        assert n_c == n_r, (name, n_c, n_r)
