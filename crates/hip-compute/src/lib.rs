@@ -568,6 +568,69 @@ pub fn same_pads(input: i64, kernel: i64, stride: i64, dilation: i64, upper: boo
     (b, e)
 }
 
+/// One initializer of a model file: what `tensor_to_initializer` yields (`convert.rs:247-300`).
+#[derive(Clone, Debug, PartialEq, Eq)]
+pub struct Initializer {
+    pub name: String,
+    /// `TensorProto.DataType`
+    pub dtype: i32,
+    pub shape: Vec<i64>,
+    /// little-endian, row-major
+    pub data: Vec<u8>,
+}
+
+fn host_error(rc: c_int) -> Error {
+    let message = unsafe { CStr::from_ptr(sys::hipc_host_error()) }.to_string_lossy().into_owned();
+    Error { kind: kind_of(rc), message }
+}
+
+/// A serialized `TensorProto` -> its payload, whatever the storage form (`raw_data`, typed fields, or a
+/// slice of a file beside the model: `base_dir` is the model's directory, `None` refuses external data).
+pub fn read_initializer(tensor: &[u8], base_dir: Option<&std::path::Path>) -> Result<Initializer> {
+    let base = match base_dir {
+        Some(p) => Some(CString::new(p.to_string_lossy().as_bytes()).map_err(|_| Error { kind: ErrorKind::Invalid, message: "model directory holds a NUL".into() })?),
+        None => None,
+    };
+    let base_ptr = base.as_ref().map_or(ptr::null(), |c| c.as_ptr());
+    let mut info: sys::hipc_initializer_info = unsafe { std::mem::zeroed() };
+    let rc = unsafe { sys::hipc_initializer_read(tensor.as_ptr() as *const c_void, tensor.len(), base_ptr, &mut info, ptr::null_mut(), 0) };
+    if rc != sys::HIPC_OK {
+        return Err(host_error(rc));
+    }
+    let mut data = vec![0u8; info.bytes];
+    let rc = unsafe { sys::hipc_initializer_read(tensor.as_ptr() as *const c_void, tensor.len(), base_ptr, &mut info, data.as_mut_ptr() as *mut c_void, data.len()) };
+    if rc != sys::HIPC_OK {
+        return Err(host_error(rc));
+    }
+    let name = unsafe { CStr::from_ptr(info.name.as_ptr()) }.to_string_lossy().into_owned();
+    Ok(Initializer { name, dtype: info.data_type, shape: info.dims[..info.n_dims as usize].to_vec(), data })
+}
+
+/// Every initializer of a serialized `ModelProto`, in file order (`model_to_ir`, `convert.rs:51-76`):
+/// unnamed initializers and sparse initializers are refused as there.
+pub fn model_initializers(model: &[u8], base_dir: Option<&std::path::Path>) -> Result<Vec<Initializer>> {
+    let mut count = 0i64;
+    let rc = unsafe { sys::hipc_model_initializers(model.as_ptr() as *const c_void, model.len(), ptr::null_mut(), ptr::null_mut(), 0, &mut count) };
+    if rc != sys::HIPC_OK {
+        return Err(host_error(rc));
+    }
+    let n = count as usize;
+    let (mut offsets, mut sizes) = (vec![0usize; n], vec![0usize; n]);
+    let rc = unsafe { sys::hipc_model_initializers(model.as_ptr() as *const c_void, model.len(), offsets.as_mut_ptr(), sizes.as_mut_ptr(), count, &mut count) };
+    if rc != sys::HIPC_OK {
+        return Err(host_error(rc));
+    }
+    let mut out = Vec::with_capacity(n);
+    for i in 0..n {
+        let t = read_initializer(&model[offsets[i]..offsets[i] + sizes[i]], base_dir)?;
+        if t.name.is_empty() {
+            return Err(Error { kind: ErrorKind::Invalid, message: "unnamed initializer".into() });
+        }
+        out.push(t);
+    }
+    Ok(out)
+}
+
 /// Which linear of a layer (`q|k|v` and `gate|up` are given concatenated along N).
 #[derive(Clone, Copy, Debug, PartialEq, Eq)]
 #[repr(i32)]

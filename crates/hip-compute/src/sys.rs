@@ -65,6 +65,22 @@ pub struct hipc_decoder_config {
     pub embed_scale: f32,
 }
 
+pub const HIPC_INITIALIZER_MAX_DIMS: usize = 8;
+
+/// what `hipc_initializer_read` reports about a TensorProto
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct hipc_initializer_info {
+    /// `TensorProto.DataType` (the `HIPC_*` element types use the same numbers)
+    pub data_type: i32,
+    pub n_dims: i32,
+    pub dims: [i64; HIPC_INITIALIZER_MAX_DIMS],
+    /// length of the little-endian payload
+    pub bytes: usize,
+    /// NUL-terminated
+    pub name: [c_char; 256],
+}
+
 pub const HIPC_DEC_QKV: c_int = 0;
 pub const HIPC_DEC_O: c_int = 1;
 pub const HIPC_DEC_GATE_UP: c_int = 2;
@@ -180,6 +196,16 @@ unsafe extern "C" {
         w_scale: *const f32, n_w_scale: i64, w_zp: i32, y_scale: f32, y_zp: i32, y_dtype: c_int, bias: *const c_void,
         g: *const hipc_conv_geom, y: *mut c_void,
     ) -> c_int;
+
+    // ---- ONNX initializers (host code only)
+    pub fn hipc_initializer_read(
+        tensor: *const c_void, len: usize, base_dir: *const c_char, info: *mut hipc_initializer_info, data: *mut c_void,
+        data_cap: usize,
+    ) -> c_int;
+    pub fn hipc_model_initializers(
+        model: *const c_void, len: usize, offsets: *mut usize, sizes: *mut usize, cap: i64, count: *mut i64,
+    ) -> c_int;
+    pub fn hipc_host_error() -> *const c_char;
 
     // ---- decode step
     pub fn hipc_decoder_create(ctx: *mut hipc_ctx, cfg: *const hipc_decoder_config, out: *mut *mut hipc_decoder) -> c_int;

@@ -322,6 +322,40 @@ int hipc_qlinear_conv(hipc_ctx *ctx, const void *X, int x_dtype, float x_scale, 
                       float y_scale, int32_t y_zp, int y_dtype, const void *bias,
                       const hipc_conv_geom *g, void *Y);
 
+/* ------------------------------------------------------- ONNX initializers */
+
+/*
+ * The data format in front of the prepack calls: a weight as the model file holds it. Host code only
+ * (no context, no GPU); a failed call leaves its message in `hipc_host_error` (per thread).
+ *
+ * `tensor_to_initializer` + `read_external` (crates/onnx-vulkan-frontend/src/convert.rs:247-384):
+ * `tensor` is a serialized TensorProto. Its payload is, in this order of precedence, the slice
+ * [offset, offset + length) of the file `location` beside the model (data_location EXTERNAL; the path
+ * must be relative without "." or ".." components, `base_dir` NULL refuses it), `raw_data` as it is,
+ * or the typed repeated fields narrowed to the width `data_type` says (ONNX packs every narrow
+ * dtype into int32_data). Fills *info; with data != NULL also copies the little-endian payload
+ * (HIPC_ERR_INVALID when data_cap < info->bytes). Call once with data == NULL to size the buffer.
+ * A dtype with no readable field is HIPC_ERR_UNSUPPORTED, a malformed message HIPC_ERR_INVALID.
+ */
+#define HIPC_INITIALIZER_MAX_DIMS 8
+typedef struct {
+    int32_t data_type; /* TensorProto.DataType (the HIPC_* element types use the same numbers) */
+    int32_t n_dims;
+    int64_t dims[HIPC_INITIALIZER_MAX_DIMS];
+    size_t bytes;      /* length of the payload */
+    char name[256];
+} hipc_initializer_info;
+int hipc_initializer_read(const void *tensor, size_t len, const char *base_dir, hipc_initializer_info *info,
+                          void *data, size_t data_cap);
+/* `model_to_ir`'s walk over graph.initializer (convert.rs:51-76): `model` is a serialized ModelProto;
+ * writes the number of initializers to *count and, for the first `cap` of them, where each one's
+ * TensorProto lies inside `model` (offsets / sizes may be NULL to count only). A model without a
+ * graph is HIPC_ERR_INVALID, one with sparse initializers HIPC_ERR_UNSUPPORTED, as in the reference. */
+int hipc_model_initializers(const void *model, size_t len, size_t *offsets, size_t *sizes, int64_t cap,
+                            int64_t *count);
+/* message of the last failed host-only call (the two above) on the calling thread */
+const char *hipc_host_error(void);
+
 /* ------------------------------------------------------------ decode step */
 
 /*

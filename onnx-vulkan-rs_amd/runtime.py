@@ -52,6 +52,12 @@ class DecoderConfig(C.Structure):
                [(n, C.c_float) for n in ("rms_eps", "rope_theta", "attn_scale", "embed_scale")]
 
 
+class InitializerInfo(C.Structure):
+    """``hipc_initializer_info``."""
+    _fields_ = [("data_type", C.c_int32), ("n_dims", C.c_int32), ("dims", C.c_int64 * 8), ("bytes", C.c_size_t),
+                ("name", C.c_char * 256)]
+
+
 _lib = None
 
 # name -> (restype, argtypes); every symbol include/hipcompute.h declares
@@ -64,6 +70,9 @@ SIGNATURES = {
     "hipc_version": (C.c_char_p, []),
     "hipc_stream": (_vp, [_vp]),
     "hipc_set_option": (_int, [_vp, C.c_char_p, _int]),
+    "hipc_initializer_read": (_int, [_vp, _sz, C.c_char_p, C.POINTER(InitializerInfo), _vp, _sz]),
+    "hipc_model_initializers": (_int, [_vp, _sz, C.POINTER(_sz), C.POINTER(_sz), _i64, C.POINTER(_i64)]),
+    "hipc_host_error": (C.c_char_p, []),
     "hipc_pool_stats": (_int, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "hipc_alloc": (_int, [_vp, _sz, C.POINTER(_vp)]),
     "hipc_free_deferred": (_int, [_vp, _vp]),
