@@ -9,8 +9,11 @@ crates/onnx-vulkan-core/src in the reference tree):
   GatherBlockQuantized          shaders/gather_block_quantized.rs:26-57
   MatMulNBits                   oracle.matmul_nbits (the C oracle)
 All arithmetic is float32; the KV cache is rounded to float16 as the configuration asks.
-Pin status: composition of operators pinned elsewhere; the glue itself (norm, rotary, softmax,
-gelu) is checked in tests/test_oracle_pins.py against float64 closed forms.
+Pin status: the glue pieces (norm, rotary, masked softmax, gelu, gather) are checked in
+tests/test_oracle_pins.py against float64 closed forms; the step's composition (which norm feeds which
+product, residual order, gate before up, head to kv-head map, cache write before attention, the state
+rule) against an independent float64 route written from the operator definitions and against a
+closed form with silenced branches. No reference vector exists for a whole step.
 """
 from __future__ import annotations
 
