@@ -18,4 +18,4 @@ from .runtime import (  # noqa: F401
     load_library,
     F32, F16, U8, I8, I32,
 )
-from . import ops, synth, graph, decoder, initializers  # noqa: F401
+from . import ops, synth, graph, decoder, initializers, runtime  # noqa: F401

@@ -133,6 +133,7 @@ int create(int device, void *stream, bool adopt, hipc_ctx **out) {
         ctx->owns_stream = true;
     }
     for (const OptionName &o : kOptions) ctx->tune.*(o.field) = env_int(o.name);
+    if (!kReadAheadVerified) ctx->tune.dec_prefetch = -1;   // not reachable from the environment either
     if (hipMalloc(&ctx->params, kParamBytes) != hipSuccess ||
         hipMemsetAsync(ctx->params, 0, kParamBytes, ctx->stream) != hipSuccess ||
         dql_static_init(ctx) != HIPC_OK) {
@@ -219,7 +220,11 @@ using namespace hipc;
 
 extern "C" {
 
-const char *hipc_version(void) { return "hipcompute 0.2 (gfx950)"; }
+#ifndef HIPC_BUILD_ID
+#define HIPC_BUILD_ID "unknown"
+#endif
+// "... build <id>": the id is a hash over the sources and headers the library was compiled from (csrc/Makefile)
+const char *hipc_version(void) { return "hipcompute 0.3 (gfx950) build " HIPC_BUILD_ID; }
 
 int hipc_ctx_create(int device, hipc_ctx **out) {
     try {
@@ -275,6 +280,8 @@ int hipc_set_option(hipc_ctx *ctx, const char *name, int value) {
         HIPC_REQUIRE(ctx, name, "hipc_set_option: null name");
         for (const OptionName &o : kOptions)
             if (strcmp(o.name, name) == 0) {
+                HIPC_REFUSE(ctx, !kReadAheadVerified && o.field == &Tuning::dec_prefetch && value > 0,
+                            "HIPC_DEC_PREFETCH: the read-ahead route is switched off in this build");
                 ctx->tune.*(o.field) = value < 0 ? -1 : value;
                 return HIPC_OK;
             }

@@ -998,10 +998,10 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         float *xc = d->x, *xo = d->x2;
         // Every launch of a layer carries helper rows that read ahead what the NEXT launch will read
         // (its weights, or the attention's cache rows) into the L2 of the XCD that will ask for it.
-        // Off unless the dec_prefetch option is set to 1: the first version read past the end of a weight (the
-        // hardware's range check of a buffer load does not cover the scalar offset) and faulted; the
-        // corrected version has not run on a GPU yet.
-        const bool ahead = ctx->tune.dec_prefetch > 0;
+        // Off unless the dec_prefetch option is set to 1, and unreachable while kReadAheadVerified is
+        // false: the first version read past the end of a weight (the hardware's range check of a buffer
+        // load does not cover the scalar offset) and faulted.
+        const bool ahead = kReadAheadVerified && ctx->tune.dec_prefetch > 0;
         auto rows_for = [](int64_t gx) { return (int)std::max<int64_t>(1, std::min<int64_t>(8, (192 + gx - 1) / gx)); };   // about 200 helper workgroups
         for (int li = 0; li < c.n_layers && d->lean; li++) {
             DecLayer &l = d->layers[li];

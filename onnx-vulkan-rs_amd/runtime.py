@@ -127,8 +127,28 @@ SIGNATURES = {
 }
 
 
+def source_build_id():
+    """The build id of the sources in this tree, as csrc/Makefile computes it: sha256 over the sorted
+    ``*.hip`` and ``*.h`` of csrc/, the public header and the Makefile (first 16 hex digits).
+    None when the sources are not there (a library deployed on its own)."""
+    import glob
+    import hashlib
+    csrc = os.path.join(_HERE, "csrc")
+    names = sorted(os.path.basename(f) for f in glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.h")))
+    files = [os.path.join(csrc, n) for n in names] + [os.path.join(_HERE, "..", "include", "hipcompute.h"),
+                                                      os.path.join(csrc, "Makefile")]
+    if not names or not all(os.path.exists(f) for f in files):
+        return None
+    h = hashlib.sha256()
+    for f in files:
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def load_library():
-    """Load libhipcompute.so and declare its signatures. Raises if it has not been built."""
+    """Load libhipcompute.so and declare its signatures. Raises if it has not been built, or if it
+    was built from other sources than the ones beside it (a stale library must not run)."""
     global _lib
     if _lib is None:
         path = library_path()
@@ -140,6 +160,10 @@ def load_library():
             fn = getattr(lib, name)  # AttributeError here means the header and the library disagree
             fn.restype = res
             fn.argtypes = args
+        built, want = lib.hipc_version().decode().rsplit(" ", 1)[-1], source_build_id()
+        if want is not None and built != want:
+            raise HipComputeError(3, f"{path} is stale: built from sources with id {built}, the tree has {want}; "
+                                     f"rebuild it (make -C onnx-vulkan-rs_amd/csrc)")
         _lib = lib
     return _lib
 

@@ -52,7 +52,7 @@ DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / 
 # read up to 96 KiB past the end of a weight. The corrected helper (per-lane offsets only) has not run on
 # a GPU since; until it has, the route is off by default and its cases are skipped.
 READ_AHEAD = pytest.param({"HIPC_DEC_PREFETCH": 1}, marks=pytest.mark.skip(
-    reason="read-ahead helper rows: faulted before the range-check fix, not yet re-run on a GPU"))
+    reason="read-ahead helper rows: faulted before the range-check fix, not yet re-run on a GPU; the library refuses the option"))
 PATHS = [{}, READ_AHEAD, {"HIPC_DEC_LEAN": 0}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
 
 
@@ -68,6 +68,15 @@ def route(ctx):
     yield apply
     for k in touched:
         ctx.set_option(k, -1)
+
+
+def test_the_read_ahead_route_cannot_be_switched_on(ctx, pkg):
+    """While the helper rows are unverified the option is refused (and the environment variable is not read)."""
+    with pytest.raises(pkg.HipComputeError) as e:
+        ctx.set_option("HIPC_DEC_PREFETCH", 1)
+    assert e.value.code == 2 and "switched off" in e.value.message
+    ctx.set_option("HIPC_DEC_PREFETCH", 0)
+    ctx.set_option("HIPC_DEC_PREFETCH", -1)
 
 
 @pytest.mark.parametrize("env", PATHS, ids=["default", "read-ahead", "streaming-gemv", "separate-glue", "three-kernel-attention"])

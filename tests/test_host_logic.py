@@ -170,3 +170,22 @@ def test_the_rust_binding_declares_every_entry_point():
         n_c = 0 if args.strip() in ("", "void") else args.count(",") + 1
         n_r = len([a for a in r_protos[name].split(",") if a.strip()])
         assert n_c == n_r, (name, n_c, n_r)
+
+
+def test_the_library_carries_the_build_id_of_the_sources_beside_it(pkg):
+    """hipc_version() ends in a hash over the sources and headers the library was compiled from, and
+    load_library() refuses a library whose id is not the tree's (a stale object once hid a fix)."""
+    rt = pkg.runtime
+    lib = rt.load_library()
+    built = lib.hipc_version().decode().rsplit(" ", 1)[-1]
+    assert re.fullmatch(r"[0-9a-f]{16}", built), built
+    assert built == rt.source_build_id()
+
+
+def test_a_stale_library_is_refused(pkg, monkeypatch):
+    rt = pkg.runtime
+    rt.load_library()
+    monkeypatch.setattr(rt, "_lib", None)
+    monkeypatch.setattr(rt, "source_build_id", lambda: "0123456789abcdef")
+    with pytest.raises(rt.HipComputeError, match="stale"):
+        rt.load_library()
