@@ -44,7 +44,12 @@ BS = 32
 # scaled by its reading for a 256 MiB copy; profiles/mmnb_gemv_lm_head_1152x262144.txt). A counter
 # run cannot happen inside this program, so the figure is carried over from that profile.
 LM_HEAD_TRAFFIC_BYTES = 199.6e6
+# The same for the average of the 104 narrow launches (a layer's q|k|v, o, gate|up, down: 18.408 MB of traffic for
+# 17.304 MB algorithmic; profiles/mmnb_lean_decode_linears_gemma3_1b.txt)
+NARROW_TRAFFIC_BYTES = 4.602e6
 IN_GRAPH = 16   # instances of a small operator per captured graph: amortises the graph launch
+LIGHT = False   # --light: a third of the timing samples (runs under a profiler, which a process that replays
+                # graphs for more than ~12 k kernel dispatches brings down)
 
 
 def gemv_bytes(K, N, bs=BS, with_zp=True, elt=4):
@@ -103,6 +108,8 @@ def min_bound_us(byts, ops, peak_tops):
 
 
 def median_ns(ctx, graph, launches_per_graph=1, samples=20, reps=10):
+    if LIGHT:
+        samples = max(3, samples // 3)
     ns = ctx.measure_graph(graph, samples, reps)
     return float(np.median(ns)) / launches_per_graph, float(ns.min()) / launches_per_graph
 
@@ -147,7 +154,7 @@ def bench_decode_linears(pkg, ctx, steps, warmup):
         s.accuracy_level = 0
         med, mn = median_ns(ctx, s.capture(), n_narrow, samples=15, reps=4)
         s.items = every
-        roof = dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS, traffic=None,
+        roof = dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS, traffic=NARROW_TRAFFIC_BYTES,
                     kernel="mmnb_lean_kernel, PRO 0 (the 104 per-layer one-row MatMulNBits launches of the step: q|k|v, o, gate|up, down x 26)",
                     bytes_per_launch=per, avg_launch_us=med / 1e3, min_launch_us=mn / 1e3, launches_per_replay=n_narrow,
                     timing="device events around whole graph replays / launches per replay: launch gaps included",
@@ -463,7 +470,10 @@ def main():
     ap.add_argument("--only", default="", help="comma list of sections to run (decode, floor, lm_head, gemv, int8, conv, prefill, "
                     "decoder, cpu; copy = counter calibration, only on request); default all. Used to profile "
                     "one kernel at a time.")
+    ap.add_argument("--light", action="store_true", help="a third of the timing samples per figure (for runs under rocprofv3)")
     args = ap.parse_args()
+    global LIGHT
+    LIGHT = args.light
     only = set(filter(None, args.only.split(",")))
     want = lambda name: not only or name in only  # noqa: E731
     if args.gpus != 1:

@@ -373,7 +373,11 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
     const uint32_t nib_mask = p.nib_mask;
     uint32_t magic;
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(p.magic));
+    // (with three terms and four tiles the sixteen operands read ahead do not fit the 128 registers a
+    // wavefront of a 1024-thread workgroup may hold: that instance reads a tile's operands when it multiplies it)
+    constexpr bool kOperandsAhead = !(NT == 3 && KT == 4);
     uint4 aop[KT][4];
+    const uint4 *a_lane = As + term * 4 + g4;
     if (PRO == 4) {
         const __amdgpu_buffer_rsrc_t r_a = lean_rsrc(p.a_split, (uint32_t)p.n_cg * 4u * NT * 64u);
         const uint32_t v_a = (uint32_t)(term * 4 + g4) * 16u;
@@ -381,8 +385,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
         for (int i = 0; i < KT; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) aop[i][j] = lean_ld16(r_a, v_a, (uint32_t)((kt0 + tile_in_slice[i]) * 4 + j) * (NT * 64u));
-    } else {
-        const uint4 *a_lane = As + term * 4 + g4;
+    } else if (kOperandsAhead) {
 #pragma unroll
         for (int i = 0; i < KT; i++)
 #pragma unroll
@@ -391,8 +394,8 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
     const uint32_t one2 = 0x3f803f80u;   // bf16 1.0 twice
     const lbf16x8 ones = __builtin_bit_cast(lbf16x8, make_uint4(one2, one2, one2, one2));
     lf32x4 d[KT][SG], e[KT][SG];
-#pragma unroll
-    for (int i = 0; i < KT; i++) {
+    float acc = 0.f;
+    auto multiply_tile = [&](int i) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const uint32_t word = j == 0 ? wq[i].x : j == 1 ? wq[i].y : j == 2 ? wq[i].z : wq[i].w;
@@ -404,16 +407,33 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
             d[i][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(lbf16x8, bw), first ? lf32x4{0.f, 0.f, 0.f, 0.f} : d[i][g], 0, 0, 0);
             e[i][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ones, first ? lf32x4{0.f, 0.f, 0.f, 0.f} : e[i][g], 0, 0, 0);
         }
-    }
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < KT; i++) {
+    };
+    auto fold_tile = [&](int i) {
 #pragma unroll
         for (int g = 0; g < SG; g++) {
             const float dsum = NT == 3 ? (d[i][g][0] + d[i][g][1]) + d[i][g][2] : d[i][g][0] + d[i][g][1];
             const float asg = NT == 3 ? (e[i][g][0] + e[i][g][1]) + e[i][g][2] : e[i][g][0] + e[i][g][1];
             const float zb = (float)((sv[i].z >> (8 * g)) & 0xffu);
             acc = fmaf(sv[i].s[g] * tile_live[i], fmaf(-zb, asg, dsum), acc);
+        }
+    };
+    if (kOperandsAhead) {
+#pragma unroll
+        for (int i = 0; i < KT; i++) multiply_tile(i);
+#pragma unroll
+        for (int i = 0; i < KT; i++) fold_tile(i);
+    } else {
+        // one tile after the other, and nothing moved across a tile's end: a tile's operands and its 32
+        // result registers are dead before the next tile's are live
+#pragma unroll
+        for (int i = 0; i < KT; i++) {
+            if (PRO != 4) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) aop[i][j] = a_lane[(size_t)(tile_in_slice[i] * 4 + j) * NT * 4];
+            }
+            multiply_tile(i);
+            fold_tile(i);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
