@@ -719,8 +719,7 @@ int dev_alloc(hipc_ctx *ctx, hipc_decoder *d, T **p, size_t count) {
 template <int HD, int G>
 void attn_chunks_launch(hipc_ctx *ctx, hipc_decoder *d, DecLayer &l, float scale, const PrefetchArgs &pf) {
     const hipc_decoder_config &c = d->cfg;
-    dec_attn_chunks_kernel<HD, G><<<dim3(kAttnSplits, c.n_kv_heads + (pf.kind ? pf.rows : 0)), 256, 0, ctx->stream>>>(
-        d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.rms_eps,
+    hipLaunchKernelGGL((dec_attn_chunks_kernel<HD, G>), dim3(kAttnSplits, c.n_kv_heads + (pf.kind ? pf.rows : 0)), 256, 0, ctx->stream, d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads, c.n_kv_heads, c.rms_eps,
         d->rope + (size_t)l.rope_table * c.head_dim, c.max_seq, attn_v_stride(c.max_seq), scale, l.window, l.k_cache, l.v_cache,
         d->part_ml, d->part_o, pf);
 }
@@ -840,7 +839,7 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
                     hipMemsetAsync(l.v_cache, 0, v_halfs * 2, ctx->stream) != hipSuccess)
                     rc = fail(ctx, HIPC_ERR_BACKEND, "decoder: cannot clear the KV cache");
             }
-            dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, 0, 0);
+            hipLaunchKernelGGL((dec_set_state_kernel), 1, 64, 0, ctx->stream, d->state, 0, 0);
         }
         if (rc != HIPC_OK) {
             for (void *p : d->owned) (void)hipFree(p);
@@ -963,7 +962,7 @@ int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *d, int32_t token, int32_t po
     if (!d) return HIPC_ERR_INVALID;
     return entry(ctx, [&]() -> int {
         HIPC_REQUIRE(ctx, token >= 0 && token < d->cfg.vocab && pos >= 0 && pos < d->cfg.max_seq, "decoder: bad token %d or position %d", token, pos);
-        dec_set_state_kernel<<<1, 64, 0, ctx->stream>>>(d->state, token, pos);
+        hipLaunchKernelGGL((dec_set_state_kernel), 1, 64, 0, ctx->stream, d->state, token, pos);
         HIPC_LAUNCHED(ctx);
         return HIPC_OK;
     });
@@ -989,7 +988,7 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         const float scale = c.attn_scale > 0.f ? c.attn_scale : 1.f / sqrtf((float)c.head_dim);
         const int terms = 2;
         int rc;
-        dec_embed_kernel<<<1, 256, 0, s>>>(d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
+        hipLaunchKernelGGL((dec_embed_kernel), 1, 256, 0, s, d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
                                            d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn, c.head_dim, c.rope_theta,
                                            d->theta2, d->rope);
         HIPC_LAUNCHED(ctx);
@@ -1081,20 +1080,19 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                     merge.group = c.n_q_heads / c.n_kv_heads, merge.head_dim = c.head_dim, merge.window = l.window;
                     if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms, &merge)) != HIPC_OK) return rc;
                 } else {
-                    dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)kAttnSplits * sizeof(float), s>>>(
-                        d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads, c.head_dim, kAttnSplits, 1, l.window, d->attn);
+                    hipLaunchKernelGGL((dec_attn_merge_kernel), c.n_q_heads, 256, (size_t)kAttnSplits * sizeof(float), s, d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads, c.head_dim, kAttnSplits, 1, l.window, d->attn);
                     HIPC_LAUNCHED(ctx);
                     if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
                 }
             } else {
-                dec_qkv_kernel<<<heads, 256, 0, s>>>(d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
+                hipLaunchKernelGGL((dec_qkv_kernel), heads, 256, 0, s, d->state, d->qkv, l.norm[HIPC_DEC_NORM_Q], l.norm[HIPC_DEC_NORM_K], c.n_q_heads,
                                                      c.n_kv_heads, c.head_dim, c.rms_eps, l.rope_table ? d->theta2 : c.rope_theta, c.max_seq,
                                                      attn_v_stride(c.max_seq), d->q, l.k_cache, l.v_cache);
                 HIPC_LAUNCHED(ctx);
-                dec_attn_partial_kernel<<<dim3(d->nsplit, c.n_kv_heads), 256, 0, s>>>(d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
+                hipLaunchKernelGGL((dec_attn_partial_kernel), dim3(d->nsplit, c.n_kv_heads), 256, 0, s, d->state, d->q, l.k_cache, l.v_cache, c.n_q_heads, c.n_kv_heads,
                                                                                      c.head_dim, c.max_seq, attn_v_stride(c.max_seq), scale, l.window, d->part_ml, d->part_o);
                 HIPC_LAUNCHED(ctx);
-                dec_attn_merge_kernel<<<c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s>>>(d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
+                hipLaunchKernelGGL((dec_attn_merge_kernel), c.n_q_heads, 256, (size_t)d->nsplit * sizeof(float), s, d->state, d->part_ml, d->part_o, c.n_q_heads, c.n_kv_heads,
                                                                                                  c.head_dim, d->nsplit, 0, l.window, d->attn);
                 HIPC_LAUNCHED(ctx);
                 if ((rc = nbits_gemv(ctx, d->attn, HIPC_F32, l.o, d->y, 1, terms)) != HIPC_OK) return rc;
@@ -1109,29 +1107,29 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 gelu.mode = 1;
                 if ((rc = nbits_gemv(ctx, d->gu, HIPC_F32, l.down, d->y, 1, terms, &gelu)) != HIPC_OK) return rc;
             } else {
-                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, 1, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->x, d->xn);
+                hipLaunchKernelGGL((dec_norm_residual_kernel), 1, 256, 0, s, d->y, 1, l.norm[HIPC_DEC_NORM_POST_ATTN], l.norm[HIPC_DEC_NORM_PRE_FFN], c.hidden, c.rms_eps, d->x, d->x, d->xn);
                 HIPC_LAUNCHED(ctx);
                 if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, l.gate_up, d->gu, 1, terms)) != HIPC_OK) return rc;
-                dec_gelu_mul_kernel<<<(unsigned)ceil_div(c.ffn, 256), 256, 0, s>>>(d->gu, c.ffn, d->h);
+                hipLaunchKernelGGL((dec_gelu_mul_kernel), (unsigned)ceil_div(c.ffn, 256), 256, 0, s, d->gu, c.ffn, d->h);
                 HIPC_LAUNCHED(ctx);
                 if ((rc = nbits_gemv(ctx, d->h, HIPC_F32, l.down, d->y, 1, terms)) != HIPC_OK) return rc;
                 const float *next = li + 1 < c.n_layers ? d->layers[li + 1].norm[HIPC_DEC_NORM_INPUT] : d->final_norm;
-                dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->y, 1, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->x, d->xn);
+                hipLaunchKernelGGL((dec_norm_residual_kernel), 1, 256, 0, s, d->y, 1, l.norm[HIPC_DEC_NORM_POST_FFN], next, c.hidden, c.rms_eps, d->x, d->x, d->xn);
                 HIPC_LAUNCHED(ctx);
             }
         }
         if (d->fused_glue) {
             // the unembedding streams ~200 MB: its workgroups start on the weights at once and the
             // final norm stays a launch of its own
-            dec_norm_residual_kernel<<<1, 256, 0, s>>>(d->lean ? d->yd : d->y, d->lean ? d->down_slices : 1,
+            hipLaunchKernelGGL((dec_norm_residual_kernel), 1, 256, 0, s, d->lean ? d->yd : d->y, d->lean ? d->down_slices : 1,
                                                        d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], d->final_norm, c.hidden,
                                                        c.rms_eps, xc, xc, d->xn);
             HIPC_LAUNCHED(ctx);
         }
         if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;
-        dec_argmax_partial_kernel<<<kArgmaxParts, 256, 0, s>>>(d->logits, c.vocab, d->am_v, d->am_i);
+        hipLaunchKernelGGL((dec_argmax_partial_kernel), kArgmaxParts, 256, 0, s, d->logits, c.vocab, d->am_v, d->am_i);
         HIPC_LAUNCHED(ctx);
-        dec_argmax_final_kernel<<<1, 64, 0, s>>>(d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq, c.vocab);
+        hipLaunchKernelGGL((dec_argmax_final_kernel), 1, 64, 0, s, d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq, c.vocab);
         HIPC_LAUNCHED(ctx);
         return HIPC_OK;
     });

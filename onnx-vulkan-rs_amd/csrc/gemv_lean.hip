@@ -192,7 +192,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
     // Marks the point where values asked for in (wave-uniform) branches above are first needed: the
     // compiler may otherwise pull the arithmetic that consumes a load into the branch that issued it,
     // which turns one memory round trip into one per branch.
-#define LEAN_NEEDED_HERE(v) asm volatile("" : "+v"(v))
+#define LEAN_NEEDED_HERE(v) HIPC_PIN_VGPR(v)
 
     uint4 *As = lean_smem;                                                     // [nch][NT][4] operands
     float *red = reinterpret_cast<float *>(As + (size_t)slice_tiles * 4 * NT * 4);   // [WN][16 columns][16 k wavefronts]; before that the norm's partial sums
@@ -372,7 +372,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
     const int term = min(i16 & 3, NT - 1);
     const uint32_t nib_mask = p.nib_mask;
     uint32_t magic;
-    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(p.magic));
+    HIPC_VGPR_FROM_SGPR(magic, p.magic);
     // (with three terms and four tiles the sixteen operands read ahead do not fit the 128 registers a
     // wavefront of a 1024-thread workgroup may hold: that instance reads a tile's operands when it multiplies it)
     constexpr bool kOperandsAhead = !(NT == 3 && KT == 4);
@@ -491,10 +491,10 @@ namespace {
 template <int SG, int NT, int PRO, int EPI>
 void lean_launch_one(const LeanArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
     switch (a.KT) {
-        case 1: mmnb_lean_kernel<SG, NT, PRO, EPI, 1><<<grid, block, lds, s>>>(a); break;
-        case 2: mmnb_lean_kernel<SG, NT, PRO, EPI, 2><<<grid, block, lds, s>>>(a); break;
-        case 3: mmnb_lean_kernel<SG, NT, PRO, EPI, 3><<<grid, block, lds, s>>>(a); break;
-        default: mmnb_lean_kernel<SG, NT, PRO, EPI, 4><<<grid, block, lds, s>>>(a); break;
+        case 1: hipLaunchKernelGGL((mmnb_lean_kernel<SG, NT, PRO, EPI, 1>), grid, block, lds, s, a); break;
+        case 2: hipLaunchKernelGGL((mmnb_lean_kernel<SG, NT, PRO, EPI, 2>), grid, block, lds, s, a); break;
+        case 3: hipLaunchKernelGGL((mmnb_lean_kernel<SG, NT, PRO, EPI, 3>), grid, block, lds, s, a); break;
+        default: hipLaunchKernelGGL((mmnb_lean_kernel<SG, NT, PRO, EPI, 4>), grid, block, lds, s, a); break;
     }
 }
 

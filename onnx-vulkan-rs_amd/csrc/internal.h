@@ -17,6 +17,17 @@
 
 #include "../../include/hipcompute.h"
 
+// The inline assembly the kernels use sits behind macros, so that a host build of the kernel sources
+// (the address model under tests/host, which runs every thread of a launch on the CPU with checked
+// loads) can compile them: HIPC_HOST_MODEL is defined there and nowhere else.
+#ifndef HIPC_HOST_MODEL
+#define HIPC_PIN_VGPR(v) asm volatile("" : "+v"(v))                                              // the value is needed here, in a vector register
+#define HIPC_VGPR_FROM_SGPR(dst, src) asm volatile("v_mov_b32 %0, %1" : "=v"(dst) : "s"(src))   // a uniform value kept in a vector register
+#else
+#define HIPC_PIN_VGPR(v) ((void)0)
+#define HIPC_VGPR_FROM_SGPR(dst, src) ((dst) = (src))
+#endif
+
 namespace hipc {
 
 constexpr int kScratchSlots = 4;
@@ -50,11 +61,13 @@ struct Tuning {
     int dec_prefetch = -1;    // HIPC_DEC_PREFETCH   1: launches of the decode step carry helper rows that read ahead for the next launch (off by default; see kReadAheadVerified)
 };
 
-// The read-ahead helper rows (prefetch.h) once read past the end of a weight and faulted the GPU. The
-// route stays unreachable -- hipc_set_option refuses HIPC_DEC_PREFETCH > 0, the environment variable is
-// not read, the decoder ignores the field -- until the helper's byte addresses pass the host-side model
-// of tests/host/ (every load of every helper thread inside its allocation, scalar offset zero).
-constexpr bool kReadAheadVerified = false;
+// The read-ahead helper rows (prefetch.h) once read past the end of a weight and faulted the GPU (a buffer
+// load's scalar offset is outside the hardware's range check). While this constant is false the route is
+// unreachable: hipc_set_option refuses HIPC_DEC_PREFETCH > 0, the environment variable is not read, the
+// decoder ignores the field. It is true since the helper's byte addresses pass the host-side model of
+// tests/host (decoder_model.cpp: the kernel sources run thread by thread on the CPU, every load of every
+// helper thread inside its allocation, at every position of the cache).
+constexpr bool kReadAheadVerified = true;
 
 // Pinned staging ring of hipc_upload: the bytes are copied into a slot and travel from there, so the
 // call returns without waiting for the stream. A slot is reused once the copies that read it are done.

@@ -282,7 +282,7 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     // registers and each unpack step is one v_and_or_b32 instead of an and and an or with literals
     const uint32_t nib_mask = p.nib_mask;
     uint32_t magic;  // held in a vector register: only one scalar operand fits the constant bus
-    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(p.magic));
+    HIPC_VGPR_FROM_SGPR(magic, p.magic);
 
     // 32-bit byte offsets from uniform bases (the prepacked weight is below 4 GiB)
     const char *wq_base = reinterpret_cast<const char *>(p.Wq);
@@ -790,13 +790,10 @@ int launch_direct(hipc_ctx *ctx, const void *A, const void *B, const void *scale
         const AT *a = static_cast<const AT *>(A) + m_done * K;
         AT *y = static_cast<AT *>(Y) + m_done * N;
         if (rows == 1) {
-            mmnb_direct_kernel<AT, ST, 1><<<dim3((unsigned)ceil_div(N, 4), 1), block, 0, ctx->stream>>>(
-                a, static_cast<const uint32_t *>(B), static_cast<const ST *>(scales), static_cast<const uint8_t *>(zp),
+            hipLaunchKernelGGL((mmnb_direct_kernel<AT, ST, 1>), dim3((unsigned)ceil_div(N, 4), 1), block, 0, ctx->stream, a, static_cast<const uint32_t *>(B), static_cast<const ST *>(scales), static_cast<const uint8_t *>(zp),
                 y, (int)rows, (int)K, (int)N, bs_shift, n_blocks, row_words, zp_row);
         } else {
-            mmnb_direct_kernel<AT, ST, 4>
-                <<<dim3((unsigned)ceil_div(N, 4), (unsigned)ceil_div(rows, 4)), block, 0, ctx->stream>>>(
-                    a, static_cast<const uint32_t *>(B), static_cast<const ST *>(scales),
+            hipLaunchKernelGGL((mmnb_direct_kernel<AT, ST, 4>), dim3((unsigned)ceil_div(N, 4), (unsigned)ceil_div(rows, 4)), block, 0, ctx->stream, a, static_cast<const uint32_t *>(B), static_cast<const ST *>(scales),
                     static_cast<const uint8_t *>(zp), y, (int)rows, (int)K, (int)N, bs_shift, n_blocks, row_words,
                     zp_row);
         }
@@ -809,11 +806,11 @@ int launch_direct(hipc_ctx *ctx, const void *A, const void *B, const void *scale
 template <int T, int NR, int MC, int NT, int PRO = 0>
 void launch_gemv_sg(const GemvArgs &a, int SG, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
     if (SG == 4)
-        mmnb_gemv_kernel<T, NR, 4, MC, NT, PRO><<<grid, block, lds, s>>>(a);
+        hipLaunchKernelGGL((mmnb_gemv_kernel<T, NR, 4, MC, NT, PRO>), grid, block, lds, s, a);
     else if (SG == 2)
-        mmnb_gemv_kernel<T, NR, 2, MC, NT, PRO><<<grid, block, lds, s>>>(a);
+        hipLaunchKernelGGL((mmnb_gemv_kernel<T, NR, 2, MC, NT, PRO>), grid, block, lds, s, a);
     else
-        mmnb_gemv_kernel<T, NR, 1, MC, NT, PRO><<<grid, block, lds, s>>>(a);
+        hipLaunchKernelGGL((mmnb_gemv_kernel<T, NR, 1, MC, NT, PRO>), grid, block, lds, s, a);
 }
 
 template <int T, int NT>
@@ -938,8 +935,7 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
     HIPC_LAUNCHED(ctx);
     if (ksplit > 1) {
         const long total = (long)M * w->N;
-        mmnb_ksplit_reduce_kernel<<<dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream>>>(
-            a.Ypart, Y, total, ksplit, a.a_f16);
+        hipLaunchKernelGGL((mmnb_ksplit_reduce_kernel), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream, a.Ypart, Y, total, ksplit, a.a_f16);
         HIPC_LAUNCHED(ctx);
     }
     return HIPC_OK;
@@ -1028,12 +1024,10 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
     const long threads = (long)tiles * 64;
     const dim3 grid((unsigned)ceil_div(threads, 256)), block(256);
     if (scale_dtype == HIPC_F16)
-        mmnb_prepack_kernel<__half><<<grid, block, 0, ctx->stream>>>(
-            static_cast<const uint32_t *>(B), static_cast<const __half *>(scales), static_cast<const uint8_t *>(zp),
+        hipLaunchKernelGGL((mmnb_prepack_kernel<__half>), grid, block, 0, ctx->stream, static_cast<const uint32_t *>(B), static_cast<const __half *>(scales), static_cast<const uint8_t *>(zp),
             w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, interleave_half);
     else
-        mmnb_prepack_kernel<float><<<grid, block, 0, ctx->stream>>>(
-            static_cast<const uint32_t *>(B), static_cast<const float *>(scales), static_cast<const uint8_t *>(zp),
+        hipLaunchKernelGGL((mmnb_prepack_kernel<float>), grid, block, 0, ctx->stream, static_cast<const uint32_t *>(B), static_cast<const float *>(scales), static_cast<const uint8_t *>(zp),
             w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, interleave_half);
     e = hipGetLastError();
     if (e != hipSuccess) {

@@ -47,12 +47,8 @@ DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / 
     (128, 4, 2, 130),    # three live chunks only
     (192, 2, 1, 100),    # no instance for this head_dim: the three-kernel path
 ]
-# The read-ahead route (helper workgroups that warm the L2 for the next launch) faulted on the GPU at the
-# full decoder shape: a buffer load's scalar offset is outside the hardware's range check, and the helper
-# read up to 96 KiB past the end of a weight. The corrected helper (per-lane offsets only) has not run on
-# a GPU since; until it has, the route is off by default and its cases are skipped.
-READ_AHEAD = pytest.param({"HIPC_DEC_PREFETCH": 1}, marks=pytest.mark.skip(
-    reason="read-ahead helper rows: faulted before the range-check fix, not yet re-run on a GPU; the library refuses the option"))
+# The read-ahead route (helper workgroups of a launch that warm the L2 for the next launch); off by default.
+READ_AHEAD = {"HIPC_DEC_PREFETCH": 1}
 PATHS = [{}, READ_AHEAD, {"HIPC_DEC_LEAN": 0}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
 
 
@@ -68,15 +64,6 @@ def route(ctx):
     yield apply
     for k in touched:
         ctx.set_option(k, -1)
-
-
-def test_the_read_ahead_route_cannot_be_switched_on(ctx, pkg):
-    """While the helper rows are unverified the option is refused (and the environment variable is not read)."""
-    with pytest.raises(pkg.HipComputeError) as e:
-        ctx.set_option("HIPC_DEC_PREFETCH", 1)
-    assert e.value.code == 2 and "switched off" in e.value.message
-    ctx.set_option("HIPC_DEC_PREFETCH", 0)
-    ctx.set_option("HIPC_DEC_PREFETCH", -1)
 
 
 @pytest.mark.parametrize("env", PATHS, ids=["default", "read-ahead", "streaming-gemv", "separate-glue", "three-kernel-attention"])
@@ -249,7 +236,8 @@ def ctypes_state(ctx, dec):
     return tok.value, pos.value
 
 
-def test_gemma3_1b_shape_at_context_2040(ctx, pkg, oracle):
+@pytest.mark.parametrize("env", [{}, READ_AHEAD], ids=["default", "read-ahead"])
+def test_gemma3_1b_shape_at_context_2040(ctx, pkg, oracle, route, env):
     """The decoder configuration at its real size -- 26 layers, hidden 1152, ffn 6912, 4 query heads on
     1 kv head of 256, vocabulary 262144, 22 local layers (window 512, base 10000) and 4 global ones
     (base 1e6) -- three steps from position 2040 over a cache filled with random f16 rows on both
@@ -257,6 +245,7 @@ def test_gemma3_1b_shape_at_context_2040(ctx, pkg, oracle):
     second figure runs: the one-item-per-thread norm prologue, the gated-GELU prologue of a
     k-split down projection, the attention join of 64 chunks."""
     from oracle import decoder as od
+    route(env)
     D = pkg.decoder
     cfg = dict(D.GEMMA3_1B)
     p0, steps = 2040, 3

@@ -189,3 +189,19 @@ def test_a_stale_library_is_refused(pkg, monkeypatch):
     monkeypatch.setattr(rt, "source_build_id", lambda: "0123456789abcdef")
     with pytest.raises(rt.HipComputeError, match="stale"):
         rt.load_library()
+
+
+def test_decode_step_addresses_on_the_cpu_model(tmp_path):
+    """tests/host/decoder_model.cpp: the decode step's kernel sources compiled as plain C++ (buffer loads
+    replaced by a checker that applies the hardware's range rule, everything else under
+    AddressSanitizer) and run thread by thread with the read-ahead helper rows on: whole steps at the
+    positions around every chunk boundary for the shapes of the GPU tests and gemma3-1b's, and the
+    position-dependent launches of gemma3-1b's shape over the whole cache. (`decoder_model sweep` runs
+    every position of every shape; it takes a few minutes and is not part of this suite.)"""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = str(tmp_path / "model")
+    build = subprocess.run(["make", "-C", os.path.join(root, "tests", "host"), "-j", "4", "OUT=" + out], capture_output=True, text=True)
+    assert build.returncode == 0, build.stdout[-2000:] + build.stderr[-2000:]
+    run = subprocess.run([os.path.join(out, "decoder_model"), "quick", "8"], capture_output=True, text=True)
+    assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout[-2000:] + run.stderr[-2000:]
