@@ -375,14 +375,15 @@ def bench_decoder(pkg, ctx, steps, warmup, context=2048):
     out = dict(tok_s=tok_s, ms_per_token=dt / steps * 1e3, context=context, bytes_per_token=byts,
                hbm_bound_tok_s=HBM_PEAK_GBS * 1e9 / byts, frac_of_hbm_bound=tok_s * byts / (HBM_PEAK_GBS * 1e9),
                launches_per_token=1 + 5 * cfg["n_layers"] + 4, final_position=pos)
-    # the same step with the read-ahead helper rows (every launch of a layer carries extra workgroups that
-    # read what the next launch will read into the L2 of the XCD that will ask for it)
-    try:
-        with ctx.options(HIPC_DEC_PREFETCH=1):
-            dt_ra, _ = timed()
-        out["read_ahead"] = dict(tok_s=steps / dt_ra, ms_per_token=dt_ra / steps * 1e3)
-    except Exception as e:
-        log(f"[bench] decoder with read-ahead failed: {e!r}")
+    # the same step without the read-ahead helper rows (by default three of a layer's five launches carry extra
+    # workgroups that read what the next launch will read into the L2 of the XCD that will ask for it), and with all five
+    for name, mask in (("no_read_ahead", 0), ("read_ahead_all_five", 31)):
+        try:
+            with ctx.options(HIPC_DEC_PREFETCH=mask):
+                dt_ra, _ = timed()
+            out[name] = dict(tok_s=steps / dt_ra, ms_per_token=dt_ra / steps * 1e3)
+        except Exception as e:
+            log(f"[bench] decoder, {name}: {e!r}")
     # the layer pattern of the real gemma3-1b: five local layers (window 512, rotary base 10000) to one
     # global (base 1e6); the figure above keeps every layer global, as the byte model it is quoted against
     window, local = 512, 0

@@ -282,7 +282,7 @@ int hipc_set_option(hipc_ctx *ctx, const char *name, int value) {
             if (strcmp(o.name, name) == 0) {
                 HIPC_REFUSE(ctx, !kReadAheadVerified && o.field == &Tuning::dec_prefetch && value > 0,
                             "HIPC_DEC_PREFETCH: the read-ahead route is switched off in this build");
-                ctx->tune.*(o.field) = value < 0 ? -1 : value;
+                ctx->tune.*(o.field) = value < 0 ? -1 : value;   // (0 is a value of its own: HIPC_DEC_PREFETCH = 0 switches the helpers off)
                 return HIPC_OK;
             }
         return fail(ctx, HIPC_ERR_INVALID, "hipc_set_option: unknown option %s", name);

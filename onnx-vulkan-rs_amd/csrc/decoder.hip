@@ -995,13 +995,21 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
         // branch into the stream reads one and (its first workgroup) writes the other.
         float *xc = d->x, *xo = d->x2;
-        // Every launch of a layer carries helper rows that read ahead what the NEXT launch will read
-        // (its weights, or the attention's cache rows) into the L2 of the XCD that will ask for it.
-        // Off unless the dec_prefetch option is set to 1, and unreachable while kReadAheadVerified is
-        // false: the first version read past the end of a weight (the hardware's range check of a buffer
-        // load does not cover the scalar offset) and faulted.
-        const bool ahead = kReadAheadVerified && ctx->tune.dec_prefetch > 0;
-        auto rows_for = [](int64_t gx) { return (int)std::max<int64_t>(1, std::min<int64_t>(8, (192 + gx - 1) / gx)); };   // about 200 helper workgroups
+        // Launches of a layer may carry helper rows of workgroups that read ahead what the NEXT launch will read
+        // (its weights, or the attention's cache rows) into the L2 of the XCD that will ask for it (prefetch.h).
+        // The dec_prefetch option is a set of bits, one per producer: 1 q|k|v reads the attention's cache rows,
+        // 2 the attention reads o's weights, 4 o reads gate|up's, 8 gate|up reads down's, 16 down reads the next
+        // layer's q|k|v; 0 switches the helpers off. The default is 1 + 2 + 8: measured per producer on the
+        // gemma3-1b shape at context 2048, those three save 0.2-0.6 us per launch, the o launch (72 workgroups of
+        // its own) is lengthened by helpers that read gate|up's 10 MB, and the q|k|v launch hides its weights'
+        // arrival behind its norm prologue anyway.
+        const int ahead_mask = !kReadAheadVerified ? 0 : ctx->tune.dec_prefetch < 0 ? 11 : ctx->tune.dec_prefetch;
+        // helper rows of a producer whose grid is gx wide: about one helper workgroup per consumer workgroup (a helper
+        // that serves several consumers lasts longer than the launch it rides on), at least 192 and at most 512 in all
+        auto rows_for = [](int64_t gx, int64_t consumers) {
+            const int64_t want = std::min<int64_t>(512, std::max<int64_t>(192, consumers));
+            return (int)std::max<int64_t>(1, std::min<int64_t>(32, (want + gx - 1) / gx));
+        };
         for (int li = 0; li < c.n_layers && d->lean; li++) {
             DecLayer &l = d->layers[li];
             LeanPlan pl_qkv, pl_o, pl_gu, pl_down, pl_next;
@@ -1016,9 +1024,9 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 a.x = xc, a.w_in = l.norm[HIPC_DEC_NORM_INPUT], a.x_out = xo, a.eps = c.rms_eps;
                 if (li > 0) a.yparts = d->yd, a.y_slices = d->down_slices, a.w_post = d->layers[li - 1].norm[HIPC_DEC_NORM_POST_FFN];
                 a.Y = d->qkv;
-                if (ahead) {   // the attention's cache rows
+                if (ahead_mask & 1) {   // the attention's cache rows
                     PrefetchArgs &pf = a.pf;
-                    pf.kind = 2, pf.rows = rows_for(gx_of(l.qkv, pl_qkv)), pf.sink = d->pf_sink;
+                    pf.kind = 2, pf.rows = rows_for(gx_of(l.qkv, pl_qkv), (int64_t)kAttnSplits * c.n_kv_heads), pf.sink = d->pf_sink;
                     pf.pos = &d->state->pos, pf.k = l.k_cache, pf.v = l.v_cache, pf.window = l.window, pf.max_seq = c.max_seq;
                     pf.v_stride = attn_v_stride(c.max_seq), pf.hd = c.head_dim, pf.n_kv = c.n_kv_heads;
                 }
@@ -1027,7 +1035,12 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
             }
             {
                 PrefetchArgs pf;
-                if (ahead) pf = lean_prefetch_of(l.o, pl_o, rows_for(kAttnSplits), d->pf_sink);
+                if (ahead_mask & 2) {
+                    pf = lean_prefetch_of(l.o, pl_o, rows_for(kAttnSplits, gx_of(l.o, pl_o) * pl_o.slices), d->pf_sink);
+                    // only while the attention itself is long: behind a short one (a local layer's window, the first
+                    // positions of a context) the helpers would be what the launch waits for
+                    pf.pos = &d->state->pos, pf.gate_window = l.window, pf.gate_chunks = kAttnSplits / 2;
+                }
                 if ((rc = launch_attn_chunks(ctx, d, l, scale, pf)) != HIPC_OK) return rc;
             }
             // output projection: a k slice per head, joined from the attention partials; partial rows out
@@ -1037,7 +1050,7 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 a.lg_group = __builtin_ctz((unsigned)(c.n_q_heads / c.n_kv_heads)), a.lg_hd = __builtin_ctz((unsigned)c.head_dim);   // powers of two where the one-launch attention runs
                 a.n_kv = c.n_kv_heads, a.window = l.window;
                 a.Y = d->yo;
-                if (ahead) a.pf = lean_prefetch_of(l.gate_up, pl_gu, rows_for(gx_of(l.o, pl_o)), d->pf_sink);
+                if (ahead_mask & 4) a.pf = lean_prefetch_of(l.gate_up, pl_gu, rows_for(gx_of(l.o, pl_o), gx_of(l.gate_up, pl_gu) * pl_gu.slices), d->pf_sink);
                 if ((rc = lean_gemv(ctx, l.o, pl_o, a, 3, 0, terms)) != HIPC_OK) return rc;
             }
             // gate | up: row = rmsnorm(x'', w_pre_ffn), x'' = x' + rmsnorm(sum of the output projection's partial rows, w_post_attn);
@@ -1047,7 +1060,7 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 a.x = xc, a.w_in = l.norm[HIPC_DEC_NORM_PRE_FFN], a.x_out = xo, a.eps = c.rms_eps;
                 a.yparts = d->yo, a.y_slices = d->o_slices, a.w_post = l.norm[HIPC_DEC_NORM_POST_ATTN];
                 a.h_split = d->h_split;
-                if (ahead) a.pf = lean_prefetch_of(l.down, pl_down, rows_for(gx_of(l.gate_up, pl_gu)), d->pf_sink);
+                if (ahead_mask & 8) a.pf = lean_prefetch_of(l.down, pl_down, rows_for(gx_of(l.gate_up, pl_gu), gx_of(l.down, pl_down) * pl_down.slices), d->pf_sink);
                 if ((rc = lean_gemv(ctx, l.gate_up, pl_gu, a, 2, 1, terms)) != HIPC_OK) return rc;
                 std::swap(xc, xo);
             }
@@ -1056,8 +1069,8 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 LeanArgs a{};
                 a.a_split = d->h_split;
                 a.Y = d->yd;
-                if (ahead && li + 1 < c.n_layers && lean_plan(ctx, d->layers[li + 1].qkv, 1, 1, &pl_next))
-                    a.pf = lean_prefetch_of(d->layers[li + 1].qkv, pl_next, rows_for(gx_of(l.down, pl_down)), d->pf_sink);
+                if ((ahead_mask & 16) && li + 1 < c.n_layers && lean_plan(ctx, d->layers[li + 1].qkv, 1, 1, &pl_next))
+                    a.pf = lean_prefetch_of(d->layers[li + 1].qkv, pl_next, rows_for(gx_of(l.down, pl_down), gx_of(d->layers[li + 1].qkv, pl_next)), d->pf_sink);
                 if ((rc = lean_gemv(ctx, l.down, pl_down, a, 4, 0, terms)) != HIPC_OK) return rc;
             }
         }

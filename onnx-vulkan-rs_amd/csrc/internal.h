@@ -58,7 +58,7 @@ struct Tuning {
     int dec_fused_attn = -1;  // HIPC_DEC_FUSED_ATTN 0 keeps the three-kernel attention (read when a decoder is created)
     int gemv_lean = -1;       // HIPC_GEMV_LEAN      0: one-row products keep the streaming GEMV kernel
     int dec_lean = -1;        // HIPC_DEC_LEAN       0: the decoder keeps the streaming GEMV and its prologues (read when a decoder is created)
-    int dec_prefetch = -1;    // HIPC_DEC_PREFETCH   1: launches of the decode step carry helper rows that read ahead for the next launch (off by default; see kReadAheadVerified)
+    int dec_prefetch = -1;    // HIPC_DEC_PREFETCH   bits: which launches of a layer carry helper rows that read ahead for the next launch (0 none, 31 all; see hipc_decoder_step)
 };
 
 // The read-ahead helper rows (prefetch.h) once read past the end of a weight and faulted the GPU (a buffer
@@ -309,6 +309,9 @@ struct PrefetchArgs {
     const float *sc = nullptr;
     const uint8_t *zb = nullptr;
     int gx = 0, gy = 0, WN = 0, slice_tiles = 0, n_cg = 0, n_tiles = 0, SG = 0;
+    // kind 1 behind an attention launch: the helpers read only when the step's context is at least gate_chunks
+    // chunks long (attn_live_chunks; a short attention launch would be lengthened by them); pos as for kind 2
+    int gate_chunks = 0, gate_window = 0;
     // kind 2: the attention launch's cache
     const int *pos = nullptr;
     const void *k = nullptr, *v = nullptr;

@@ -84,7 +84,7 @@ struct Model {
         return p;
     }
     void build(const Shape &s) {
-        ctx.tune.dec_prefetch = 1;   // the helper rows are what is being verified
+        ctx.tune.dec_prefetch = 31;   // the helper rows are what is being verified
         cfg.n_layers = s.layers, cfg.hidden = s.hidden, cfg.ffn = s.ffn, cfg.n_q_heads = s.nq, cfg.n_kv_heads = s.nkv;
         cfg.head_dim = s.hd, cfg.vocab = s.vocab, cfg.max_seq = s.max_seq, cfg.block_size = 32;
         cfg.rms_eps = 1e-6f, cfg.rope_theta = 10000.f, cfg.attn_scale = 0.f, cfg.embed_scale = 1.f;

@@ -47,8 +47,10 @@ DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / 
     (128, 4, 2, 130),    # three live chunks only
     (192, 2, 1, 100),    # no instance for this head_dim: the three-kernel path
 ]
-# The read-ahead route (helper workgroups of a launch that warm the L2 for the next launch); off by default.
-READ_AHEAD = {"HIPC_DEC_PREFETCH": 1}
+# The read-ahead route (helper workgroups of a launch that warm the L2 for the next launch): one bit per producer
+# launch of a layer. By default three of the five producers carry helpers; the other cases run all five and none.
+READ_AHEAD = {"HIPC_DEC_PREFETCH": 31}
+NO_READ_AHEAD = {"HIPC_DEC_PREFETCH": 0}
 PATHS = [{}, READ_AHEAD, {"HIPC_DEC_LEAN": 0}, {"HIPC_DEC_FUSED_GLUE": 0}, {"HIPC_DEC_FUSED_ATTN": 0}]
 
 
@@ -236,7 +238,7 @@ def ctypes_state(ctx, dec):
     return tok.value, pos.value
 
 
-@pytest.mark.parametrize("env", [{}, READ_AHEAD], ids=["default", "read-ahead"])
+@pytest.mark.parametrize("env", [{}, READ_AHEAD, NO_READ_AHEAD], ids=["default", "read-ahead-everywhere", "no-read-ahead"])
 def test_gemma3_1b_shape_at_context_2040(ctx, pkg, oracle, route, env):
     """The decoder configuration at its real size -- 26 layers, hidden 1152, ffn 6912, 4 query heads on
     1 kv head of 256, vocabulary 262144, 22 local layers (window 512, base 10000) and 4 global ones
