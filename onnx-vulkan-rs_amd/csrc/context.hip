@@ -103,7 +103,6 @@ const OptionName kOptions[] = {
     {"HIPC_GEMM_TILE", &Tuning::gemm_tile},
     {"HIPC_GEMM_BIG", &Tuning::gemm_big},
     {"HIPC_GEMM_SMALL", &Tuning::gemm_small},
-    {"HIPC_GEMM_SPLITK", &Tuning::gemm_splitk},
     {"HIPC_CONV_ROW", &Tuning::conv_row},
     {"HIPC_PREFILL_TILE", &Tuning::prefill_tile},
     {"HIPC_PREFILL_SPLIT", &Tuning::prefill_split},

@@ -4,7 +4,8 @@
 //     C[i][j] = sum_k P[i][k] * Q[j][k]          (both operands k-contiguous, signed bytes)
 //
 // One 256-thread workgroup owns a 128x128 tile of C; its four wavefronts own
-// 64x64 each as 2x2 v_mfma_i32_32x32x32_i8 accumulators. Each k stage moves a
+// 64x64 each as 2x2 v_mfma_i32_32x32x32_i8 accumulators (this file's LDS-staged kernel; the
+// kernels for products with hundreds of tiles keep the constant operand out of LDS: int8_gemm_bdirect.h). Each k stage moves a
 // 128x128-byte slab of P and of Q through LDS with 128-bit accesses (row pitch
 // 144 bytes, conflict-free for ds_read_b128); two further stages are on their
 // way from memory while one is multiplied.
@@ -1097,202 +1098,6 @@ __global__ void __launch_bounds__(256, 3) int8_conv_row_kernel(const GemmArgs p)
         }
     __syncthreads();   // the hand-over reuses the slab's LDS
     conv_small_finish<EPI, DYN>(p, acc, dsum, chan, lds_acc, lds_sum, i0, j0, img, zd, zc);
-}
-
-// ---- the large-problem variant (MODE_MM, aligned A) --------------------------------------
-// A 128x128 tile needs 64 bytes of operand per clock per CU to keep the matrix cores busy,
-// which is all the vector memory path delivers. Large products therefore run on 256x256 tiles:
-// four wavefronts as 2 x 2, one per SIMD, 128x128 of C each as 4x4 accumulators (all 256
-// accumulation registers), which also halves the LDS bytes read per product against 64x64.
-// Per k stage of 128 a thread moves eight 16-byte chunks of each operand; a stage is about 2048
-// matrix-core cycles per SIMD, long enough that one stage in flight (loaded at the start of a
-// stage, stored to the other LDS buffer at its end) covers the memory latency, with one barrier
-// per stage.
-constexpr int kBigTile = 256;
-#ifndef HIPC_BIG_WM
-#define HIPC_BIG_WM 2
-#define HIPC_BIG_WN 2
-#endif
-constexpr int kBigWM = HIPC_BIG_WM, kBigWN = HIPC_BIG_WN;        // wavefronts over rows x columns
-constexpr int kBigThreads = 64 * kBigWM * kBigWN;
-constexpr int kBigFI = kBigTile / kBigWM / 32, kBigFJ = kBigTile / kBigWN / 32;  // 32x32 accumulators per wavefront
-constexpr int kBigChunks = kBigTile * (kBK / 16) / kBigThreads;  // 16-byte chunks of a slab per thread
-constexpr size_t kBigLds = 2 * (2 * kBigTile) * kPitch + kBigTile * sizeof(int);
-
-// DYN: the row sums of A are needed (the constant operand's zero point, in the signed domain, is not 0)
-template <int EPI, bool DYN>
-__global__ void __launch_bounds__(kBigThreads) int8_gemm_big_kernel(const GemmArgs p) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    uint8_t *lds_p = lds_raw;                                 // [2][256 * kPitch]
-    uint8_t *lds_q = lds_raw + 2 * kBigTile * kPitch;         // [2][256 * kPitch]
-    int *lds_sum = reinterpret_cast<int *>(lds_raw + 4 * kBigTile * kPitch);  // [256]
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / kBigWN, wn = wave % kBigWN;
-    const int r32 = lane & 31, kg = lane >> 5;
-
-    const int tiles_x = (p.J + kBigTile - 1) / kBigTile, tiles_y = (p.I + kBigTile - 1) / kBigTile;
-    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
-    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
-    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
-    const int i0 = ty * kBigTile, j0 = tx * kBigTile;
-
-    const int zd = (p.host_zp ? p.dyn_zp_value : zp_byte(p.dyn_zp, p.dyn_signed)) - p.dyn_shift;
-    const int zc = (p.host_zp ? p.const_zp_value : zp_byte(p.const_zp, p.const_signed)) - p.const_shift;
-    const uint32_t flip = p.dyn_shift ? 0x80808080u : 0u;
-
-    // chunk c = tid + kBigThreads u of a 256-row slab: row c / 8, 16-byte column c % 8
-    const int j_last = (p.J + kBN - 1) / kBN * kBN - 1;  // B is packed in whole 128-column tiles
-    // (the fragment-major B is read with consecutive lanes on consecutive columns instead: 16 bytes apart)
-    uint32_t p_off[kBigChunks], q_off[kBigChunks], l_off[kBigChunks], lq_off[kBigChunks];
-#pragma unroll
-    for (int u = 0; u < kBigChunks; u++) {
-        const int c = tid + kBigThreads * u, row = c >> 3, kc = c & 7;
-        const int qrow = c % kBigTile, qkc = c / kBigTile;
-        p_off[u] = (uint32_t)min(i0 + row, p.I - 1) * (uint32_t)p.K + kc * 16;  // rows past I: clamped, never stored
-        q_off[u] = qfrag_offset(min(j0 + qrow, j_last), qkc * 16, p.K_pad);
-        l_off[u] = row * kPitch + kc * 16;
-        lq_off[u] = qrow * kPitch + qkc * 16;
-    }
-    // Buffer loads: a uniform descriptor, the k offset in a scalar register and a fixed 32-bit
-    // offset per chunk, so a stage costs no address arithmetic. The descriptors carry the true
-    // sizes; the offsets are clamped into them anyway.
-    const __amdgpu_buffer_rsrc_t rsrc_p = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t *>(p.P), 0, (int)((uint32_t)p.I * (uint32_t)p.K), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t *>(p.Q), 0, (int)((uint32_t)(j_last + 1) * (uint32_t)p.K_pad), 0x00020000);
-    u32x4 rp[kBigChunks], rq[kBigChunks];
-    auto load_p = [&](int stage) {
-#pragma unroll
-        for (int u = 0; u < kBigChunks; u++) rp[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, p_off[u], stage * kBK, 0);
-    };
-    auto load_q = [&](int stage) {
-#pragma unroll
-        for (int u = 0; u < kBigChunks; u++) rq[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, q_off[u], stage * kBK * 32, 0);
-    };
-    auto store_regs = [&](int buf) {
-#pragma unroll
-        for (int u = 0; u < kBigChunks; u++) {
-            *reinterpret_cast<u32x4 *>(lds_p + buf * kBigTile * kPitch + l_off[u]) = rp[u] ^ flip;
-            *reinterpret_cast<u32x4 *>(lds_q + buf * kBigTile * kPitch + lq_off[u]) = rq[u];
-        }
-    };
-
-    i32x16 acc[kBigFI][kBigFJ];
-#pragma unroll
-    for (int i = 0; i < kBigFI; i++)
-#pragma unroll
-        for (int j = 0; j < kBigFJ; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
-    int dsum[kBigFI] = {};
-
-    // Operand fragments of one 32-wide k step. Two sets alternate: the reads of the next step are
-    // issued before the products of the current one, and nothing is allowed to move across a step
-    // boundary, which keeps the live fragments at two sets instead of a whole stage.
-    struct Frags {
-        uint4 pf[kBigFI], qf[kBigFJ];
-    };
-    const uint32_t frag_p = (wm * kBigFI * 32 + r32) * kPitch + kg * 16;
-    const uint32_t frag_q = (wn * kBigFJ * 32 + r32) * kPitch + kg * 16;
-    auto read_frags = [&](Frags &f, int buf, int step) {
-        const uint8_t *bp = lds_p + buf * kBigTile * kPitch + frag_p + step * 32;
-        const uint8_t *bq = lds_q + buf * kBigTile * kPitch + frag_q + step * 32;
-#pragma unroll
-        for (int j = 0; j < kBigFJ; j++) f.qf[j] = *reinterpret_cast<const uint4 *>(bq + j * 32 * kPitch);
-#pragma unroll
-        for (int i = 0; i < kBigFI; i++) f.pf[i] = *reinterpret_cast<const uint4 *>(bp + i * 32 * kPitch);
-    };
-    // The products of one k step, issued in a fixed pattern with the memory operations that
-    // were written next to them: a burst of loads or LDS writes would stall the wavefront (the
-    // only one on its SIMD) in the issue queues while the matrix core runs dry, so every memory
-    // instruction is followed by one or two products. `reads`/`loads`/`writes` say how many LDS
-    // reads, buffer loads and LDS writes share the step.
-    auto multiply = [&](const Frags &f, int reads, int loads, int writes) {
-#pragma unroll
-        for (int i = 0; i < kBigFI; i++)
-            if (DYN) dsum[i] += dot_ones(f.pf[i]);
-#pragma unroll
-        for (int i = 0; i < kBigFI; i++)
-#pragma unroll
-            for (int j = 0; j < kBigFJ; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, f.pf[i]),
-                                                                  __builtin_bit_cast(i32x4, f.qf[j]), acc[i][j], 0, 0, 0);
-        constexpr int kProducts = kBigFI * kBigFJ, kReads = kBigFI + kBigFJ;
-        if (writes) {
-            constexpr int kWrites = 2 * kBigChunks, kPer = kProducts / kWrites > 0 ? kProducts / kWrites : 1;
-#pragma unroll
-            for (int g = 0; g < kWrites; g++) {
-                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
-            }
-        } else {
-            constexpr int kPer = kProducts / kReads;
-#pragma unroll
-            for (int g = 0; g < kReads; g++) {
-                if (reads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                if (loads && g < kBigChunks) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    // Stage s is multiplied out of LDS buffer s % 2 while stage s + 1 travels memory -> registers
-    // (k steps 0 and 1) -> the other buffer (k step 3); one barrier per stage.
-    const int nk = p.K_pad / kBK;
-    Frags f0, f1;
-    load_p(0);
-    load_q(0);
-    store_regs(0);
-    __syncthreads();
-    for (int ks = 0; ks < nk; ks++) {
-        const int cur = ks & 1, next = min(ks + 1, nk - 1);  // the last trip reloads its own stage; nobody reads that copy
-        read_frags(f0, cur, 0);
-        read_frags(f1, cur, 1);
-        load_p(next);
-        multiply(f0, 1, 1, 0);
-        read_frags(f0, cur, 2);
-        load_q(next);
-        multiply(f1, 1, 1, 0);
-        read_frags(f1, cur, 3);
-        multiply(f0, 1, 0, 0);
-        store_regs(cur ^ 1);
-        multiply(f1, 0, 0, 1);
-        __syncthreads();
-    }
-
-    // row sums of A: the two k halves of a row sit in lanes l and l + 32; the wavefronts of a
-    // row group hold the same sums, one of them publishes
-#pragma unroll
-    for (int i = 0; i < kBigFI; i++) dsum[i] += __shfl_xor(dsum[i], 32, 64);
-    if (wn == 0 && kg == 0) {
-#pragma unroll
-        for (int i = 0; i < kBigFI; i++) lds_sum[wm * kBigFI * 32 + i * 32 + r32] = dsum[i];
-    }
-    __syncthreads();
-
-    const int kzz = p.K * zd * zc;
-    float fmn = 0.f, fmx = 0.f;
-#pragma unroll
-    for (int i = 0; i < kBigFI; i++) {
-#pragma unroll
-        for (int j = 0; j < kBigFJ; j++) {
-            const int gj = j0 + wn * kBigFJ * 32 + j * 32 + r32;
-            const int csum = gj < p.J ? p.const_sum[gj] : 0;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);
-                const int gi = i0 + wm * kBigFI * 32 + i * 32 + rf;
-                if (gi >= p.I || gj >= p.J) continue;
-                const int v = acc[i][j][r] - zd * csum + kzz - zc * lds_sum[wm * kBigFI * 32 + i * 32 + rf];
-                gemm_emit<MODE_MM, EPI>(p, 0, gi, gj, v, fmn, fmx);
-            }
-        }
-    }
-    if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
 }
 
 }  // namespace hipc

@@ -48,9 +48,8 @@ struct Tuning {
     int gemv_waves = -1;      // HIPC_GEMV_WAVES     wavefronts the GEMV aims for when it splits k inside a workgroup
     int gemv_per_cu = -1;     // HIPC_GEMV_PER_CU    resident GEMV wavefronts per CU of the persistent grid
     int gemm_tile = -1;       // HIPC_GEMM_TILE      LDS-staged int8 tiles: 64 or 128
-    int gemm_big = -1;        // HIPC_GEMM_BIG       256x256 int8 tiles: 0 never, 1 whenever A allows
+    int gemm_big = -1;        // HIPC_GEMM_BIG       the int8 kernels that keep B out of LDS: 0 never, 1 / 2 the 256x256 / 128x128 tile whenever A allows
     int gemm_small = -1;      // HIPC_GEMM_SMALL     the k-split 64x64 kernels: 0 never, 1 whenever A allows
-    int gemm_splitk = -1;     // HIPC_GEMM_SPLITK    the k-split-over-workgroups 128x128 kernel: 0 never, n >= 1 forces n ways
     int conv_row = -1;        // HIPC_CONV_ROW       0: convolutions along one axis take the general route
     int prefill_tile = -1;    // HIPC_PREFILL_TILE   64 or 128
     int prefill_split = -1;   // HIPC_PREFILL_SPLIT  0 never splits k, n forces n ways

@@ -7,6 +7,7 @@
 #include <algorithm>
 
 #include "int8_gemm.h"
+#include "int8_gemm_bdirect.h"
 
 namespace hipc {
 
@@ -160,30 +161,35 @@ int fill_common(hipc_ctx *ctx, const MmOperands &o, GemmArgs &g) {
     return HIPC_OK;
 }
 
-template <int EPI, bool DYN>
-int launch_mm_big_dyn(hipc_ctx *ctx, GemmArgs g) {
+template <int EPI, bool DYN, int T, int W>
+int launch_mm_bdirect_dyn(hipc_ctx *ctx, GemmArgs g) {
     static bool lds_allowed[kMaxDevices] = {};
-    if (int rc = allow_dynamic_lds(ctx, int8_gemm_big_kernel<EPI, DYN>, kBigLds, lds_allowed)) return rc;
-    const dim3 grid(gemm_grid(g, kBigTile), 1, 1);
-    int8_gemm_big_kernel<EPI, DYN><<<grid, kBigThreads, kBigLds, ctx->stream>>>(g);
+    if (int rc = allow_dynamic_lds(ctx, int8_gemm_bdirect_kernel<EPI, DYN, T, W>, bd_lds(T), lds_allowed)) return rc;
+    const dim3 grid(gemm_grid(g, T), 1, 1);
+    int8_gemm_bdirect_kernel<EPI, DYN, T, W><<<grid, 64 * W, bd_lds(T), ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }
 
+// The kernels that keep B out of LDS (int8_gemm_bdirect.h): 256x256 tiles once they fill most of the chip's
+// 256 CUs, 128x128 tiles once those do; 0 neither. The gemm_big option overrides (0 never, 1 / 2 the
+// 256 / 128 tile whenever A allows; tuning, tests).
+int big_tile_choice(hipc_ctx *ctx, const GemmArgs &g) {
+    const int forced = ctx->tune.gemm_big;
+    if (!g.p_aligned) return 0;
+    if (forced >= 0) return forced <= 2 ? forced : 0;
+    if (ceil_div(g.I, kBigTile) * ceil_div(g.J, kBigTile) >= 192) return 1;
+    if (ceil_div(g.I, kBM) * ceil_div(g.J, kBN) >= 192) return 2;
+    return 0;
+}
+
 template <int EPI>
-int launch_mm_big(hipc_ctx *ctx, const GemmArgs &g) {
+int launch_mm_big(hipc_ctx *ctx, const GemmArgs &g, int choice) {
     // the row sums of A only matter when the weight's zero point, shifted to the signed domain, is
     // not zero; the host knows that it is zero when the weight is int8 and carries no zero point
     const bool zero_known = g.const_shift == 0 && (g.host_zp ? g.const_zp_value == 0 : g.const_zp == nullptr);
-    return zero_known ? launch_mm_big_dyn<EPI, false>(ctx, g) : launch_mm_big_dyn<EPI, true>(ctx, g);
-}
-
-// 256x256 tiles once they fill most of the chip's 256 CUs; the gemm_big option (0 / 1) overrides (tuning, tests)
-bool wants_big_tiles(hipc_ctx *ctx, const GemmArgs &g) {
-    const int forced = ctx->tune.gemm_big;
-    if (!g.p_aligned) return false;
-    if (forced >= 0) return forced != 0;
-    return ceil_div(g.I, kBigTile) * ceil_div(g.J, kBigTile) >= 192;
+    if (choice == 1) return zero_known ? launch_mm_bdirect_dyn<EPI, false, 256, 8>(ctx, g) : launch_mm_bdirect_dyn<EPI, true, 256, 8>(ctx, g);
+    return zero_known ? launch_mm_bdirect_dyn<EPI, false, 128, 8>(ctx, g) : launch_mm_bdirect_dyn<EPI, true, 128, 8>(ctx, g);
 }
 
 // Products of a few 64x64 tiles per CU and a long enough k run on the kernel that keeps B out of LDS
@@ -212,7 +218,7 @@ int launch_mm_small(hipc_ctx *ctx, const GemmArgs &g) {
 template <int EPI>
 int launch_mm(hipc_ctx *ctx, const GemmArgs &g) {
     if (g.I == 0 || g.J == 0) return HIPC_OK;
-    if (wants_big_tiles(ctx, g)) return launch_mm_big<EPI>(ctx, g);
+    if (const int big = big_tile_choice(ctx, g)) return launch_mm_big<EPI>(ctx, g, big);
     if (wants_small_tiles(ctx, g)) return launch_mm_small<EPI>(ctx, g);
     return g.p_aligned ? gemm_launch<MODE_MM, EPI, true>(ctx, g, 1) : gemm_launch<MODE_MM, EPI, false>(ctx, g, 1);
 }

@@ -75,9 +75,9 @@ def test_ffn_pair_shapes(ctx, pkg, oracle, shape):
 
 @pytest.mark.parametrize("a_dt,b_dt", [(np.uint8, np.int8), (np.int8, np.uint8)])
 def test_large_products_take_the_256x256_tiles(ctx, pkg, oracle, a_dt, b_dt):
-    """Enough 256x256 tiles to fill the chip switches to the large-tile kernel: ragged edges in
-    both directions, an odd number of k stages, both zero points non-zero, then the same product
-    through the float epilogue."""
+    """Enough 256x256 tiles to fill the chip switches to the large tile of the kernel that keeps B out of
+    LDS: ragged edges in both directions, an odd number of k stages, both zero points non-zero, then the
+    same product through the float epilogue."""
     m, k, n = 3601, 384, 3585
     a = rc.pseudo_plus1(m * k, 31).view(a_dt).reshape(m, k)
     b = rc.pseudo_plus1(k * n, 32).view(b_dt).reshape(k, n)
@@ -251,10 +251,10 @@ def _mm_three_epilogues(ctx, pkg, oracle, m, k, n, a_dt, b_dt, seed):
 @pytest.mark.parametrize("a_dt,b_dt", SIGNS)
 @pytest.mark.parametrize("shape", [(2048, 384, 4096), (2017, 200, 4001), (3000, 256, 3000)], ids=lambda s: "M%d_K%d_N%d" % s)
 def test_many_tiles_take_the_128x128_kernel(ctx, pkg, oracle, shape, a_dt, b_dt):
-    """512 or more 128x128 tiles but fewer than 192 of 256x256 (or an A the large-tile kernel does not
-    take): the LDS-staged 128x128 kernel, in its aligned form (k a multiple of 128), its unaligned
-    form (k = 200, ragged rows and columns) and with an even stage count; every sign combination,
-    both zero points non-zero, all three epilogues."""
+    """192 or more 128x128 tiles but fewer than 192 of 256x256: with whole 128-byte k stages the 128x128
+    tile of the kernel that keeps B out of LDS (three stages, then an even count), with k = 200 and
+    ragged rows and columns the LDS-staged 128x128 kernel in its unaligned form; every sign
+    combination, both zero points non-zero, all three epilogues."""
     m, k, n = shape
     _mm_three_epilogues(ctx, pkg, oracle, m, k, n, a_dt, b_dt, seed=61)
 
@@ -262,7 +262,9 @@ def test_many_tiles_take_the_128x128_kernel(ctx, pkg, oracle, shape, a_dt, b_dt)
 ROUTES = [  # (options, M, K, N): every alternative route of the integer product once, forced in process
     ({"HIPC_GEMM_TILE": 128, "HIPC_GEMM_BIG": 0, "HIPC_GEMM_SMALL": 0}, 300, 640, 260),
     ({"HIPC_GEMM_TILE": 64, "HIPC_GEMM_BIG": 0, "HIPC_GEMM_SMALL": 0}, 1000, 1024, 520),
-    ({"HIPC_GEMM_BIG": 1}, 700, 384, 520),
+    ({"HIPC_GEMM_BIG": 1}, 700, 384, 520),                  # B out of LDS, 256x256 tiles: ragged, three stages
+    ({"HIPC_GEMM_BIG": 2}, 333, 128, 390),                  # ... 128x128 tiles: ragged, a single stage
+    ({"HIPC_GEMM_BIG": 2}, 1000, 1024, 4096),               # ... the first product of the dynamic int8 FFN
     ({"HIPC_GEMM_SMALL": 1, "HIPC_GEMM_BIG": 0}, 2100, 256, 1030),
     ({"HIPC_GEMM_SMALL": 0, "HIPC_GEMM_BIG": 0}, 1000, 1024, 1024),
 ]
