@@ -59,7 +59,7 @@ __device__ __forceinline__ __half from_f32<__half>(float v) {
 template <typename AT, typename ST, int MR>
 __global__ void __launch_bounds__(256)
 mmnb_direct_kernel(const AT *__restrict__ A, const uint32_t *__restrict__ B, const ST *__restrict__ scales,
-                   const uint8_t *__restrict__ zp, AT *__restrict__ Y, int M, int K, int N, int bs_shift,
+                   const uint8_t *__restrict__ zp, AT *__restrict__ Y, int M, int K, int N, int bs_shift, int block_size,
                    int n_blocks, int row_words, int zp_row) {
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -74,7 +74,8 @@ mmnb_direct_kernel(const AT *__restrict__ A, const uint32_t *__restrict__ B, con
         const int k0 = w * 8;
         if (k0 >= K) break;
         const uint32_t q = brow[w];
-        const int b = k0 >> bs_shift;
+        // a word's eight values lie in one block (block_size is a multiple of 8); a shift when it is a power of two
+        const int b = bs_shift >= 0 ? k0 >> bs_shift : k0 / block_size;
         const float s = to_f32<ST>(scales[(size_t)n * n_blocks + b]);
         const int z = zp ? (zp[(size_t)n * zp_row + (b >> 1)] >> (4 * (b & 1))) & 15 : 8;
         const float zf = (float)z;
@@ -760,7 +761,9 @@ int check_nbits_shape(hipc_ctx *ctx, int64_t M, int64_t K, int64_t N, int64_t bl
                       size_t scales_len, const void *zp, size_t zp_len, int scale_dtype) {
     HIPC_REQUIRE(ctx, M >= 0 && K > 0 && N >= 0, "MatMulNBits: bad dimensions M=%ld K=%ld N=%ld", (long)M, (long)K,
                  (long)N);
-    HIPC_REQUIRE(ctx, is_pow2(block_size) && block_size >= 16, "MatMulNBits: block_size %ld is not a power of two >= 16",
+    // the reference's envelope (interp.rs:447-464): any positive multiple of 8, "so a packed u32 never straddles
+    // two blocks"; the operator's own definition asks for a power of two >= 16
+    HIPC_REQUIRE(ctx, block_size > 0 && block_size % 8 == 0, "MatMulNBits: block_size %ld is not a positive multiple of 8",
                  (long)block_size);
     HIPC_REQUIRE(ctx, K < (int64_t(1) << 30) && N < (int64_t(1) << 30) && M < (int64_t(1) << 30),
                  "MatMulNBits: dimension too large");
@@ -782,7 +785,7 @@ int launch_direct(hipc_ctx *ctx, const void *A, const void *B, const void *scale
     const int n_blocks = (int)ceil_div(K, block_size);
     const int row_words = (int)(n_blocks * block_size / 8);
     const int zp_row = (n_blocks + 1) / 2;
-    const int bs_shift = log2i(block_size);
+    const int bs_shift = is_pow2(block_size) ? log2i(block_size) : -1;
     const dim3 block(256);
     int64_t m_done = 0;
     while (m_done < M) {  // grid.y is limited to 65535 row groups
@@ -791,10 +794,10 @@ int launch_direct(hipc_ctx *ctx, const void *A, const void *B, const void *scale
         AT *y = static_cast<AT *>(Y) + m_done * N;
         if (rows == 1) {
             hipLaunchKernelGGL((mmnb_direct_kernel<AT, ST, 1>), dim3((unsigned)ceil_div(N, 4), 1), block, 0, ctx->stream, a, static_cast<const uint32_t *>(B), static_cast<const ST *>(scales), static_cast<const uint8_t *>(zp),
-                y, (int)rows, (int)K, (int)N, bs_shift, n_blocks, row_words, zp_row);
+                y, (int)rows, (int)K, (int)N, bs_shift, (int)block_size, n_blocks, row_words, zp_row);
         } else {
             hipLaunchKernelGGL((mmnb_direct_kernel<AT, ST, 4>), dim3((unsigned)ceil_div(N, 4), (unsigned)ceil_div(rows, 4)), block, 0, ctx->stream, a, static_cast<const uint32_t *>(B), static_cast<const ST *>(scales),
-                    static_cast<const uint8_t *>(zp), y, (int)rows, (int)K, (int)N, bs_shift, n_blocks, row_words,
+                    static_cast<const uint8_t *>(zp), y, (int)rows, (int)K, (int)N, bs_shift, (int)block_size, n_blocks, row_words,
                     zp_row);
         }
         HIPC_LAUNCHED(ctx);
@@ -988,8 +991,8 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
     if (rc != HIPC_OK) return rc;
     HIPC_REQUIRE(ctx, N > 0 && B && scales, "MatMulNBits prepack: empty weight");
     HIPC_REQUIRE(ctx, aligned(B, 4), "MatMulNBits: packed weight must be 4-byte aligned");
-    HIPC_REFUSE(ctx, block_size < 32, "MatMulNBits prepack: block_size %ld < 32 only runs on the direct path",
-                (long)block_size);
+    HIPC_REFUSE(ctx, block_size < 32 || !is_pow2(block_size),
+                "MatMulNBits prepack: block_size %ld (below 32, or not a power of two) only runs on the direct path", (long)block_size);
     hipc_nbits_weight *w = new hipc_nbits_weight();
     w->K = K, w->N = N, w->block_size = block_size;
     w->interleave_half = interleave_half;

@@ -51,6 +51,10 @@ def is_implemented_node(node: NodeIr) -> bool:
             return False
         if int(node.attrs.get("bits", 4)) != 4:
             return False
+        # "block_size must be a multiple of 8 so a packed u32 never straddles two blocks"; K and N positive
+        bs = int(node.attrs.get("block_size", 0))
+        if bs <= 0 or bs % 8 != 0 or int(node.attrs.get("K", 0)) <= 0 or int(node.attrs.get("N", 0)) <= 0:
+            return False
     return True
 
 

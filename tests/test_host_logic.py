@@ -89,6 +89,8 @@ def test_matmul_nbits_node_forms(pkg):
     assert not g.is_implemented_node(g.NodeIr("MatMulNBits", ["a", "q", "s", "zp", "g_idx"], ["y"], dict(node.attrs)))
     assert not g.is_implemented_node(g.NodeIr("MatMulNBits", ["a", "q", "s", "zp", "", "bias"], ["y"], dict(node.attrs)))
     assert not g.is_implemented_node(g.NodeIr("MatMulNBits", ["a", "q", "s"], ["y"], dict(node.attrs, bits=8)))
+    for bs, ok in ((8, True), (24, True), (40, True), (20, False), (0, False)):   # any positive multiple of 8
+        assert g.is_implemented_node(g.NodeIr("MatMulNBits", ["a", "q", "s", "zp"], ["y"], dict(node.attrs, block_size=bs))) == ok
     assert not g.is_implemented_node(g.NodeIr("Softmax", ["a"], ["y"]))
 
 

@@ -83,8 +83,12 @@ def test_seeded_shapes_both_paths(ctx, pkg, oracle, shape):
     assert close(got, want, RTOL32), ("gemv", worst(got, want))
 
 
-def test_block_size_16_runs_direct_and_refuses_prepack(ctx, pkg, oracle):
-    k, n, bs = 208, 50, 16   # 13 blocks: odd, zero-point rows off word boundaries
+@pytest.mark.parametrize("k,n,bs", [(208, 50, 16), (200, 33, 8), (240, 50, 24), (1000, 64, 40), (330, 17, 48)],
+                         ids=lambda v: str(v))
+def test_small_and_odd_block_sizes_run_direct_and_refuse_prepack(ctx, pkg, oracle, k, n, bs):
+    """The reference accepts every block_size that is a positive multiple of 8 (interp.rs:447-464); those
+    below 32 or not a power of two run on the kernel that reads the ONNX layout. 13 blocks of 16: odd,
+    zero-point rows off word boundaries; 8, 24, 40, 48: blocks that are no power of two, partial last block."""
     B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=3)
     a = pkg.synth.normal_f32(3 * k, 8).reshape(3, k)
     got = pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs)
@@ -168,8 +172,8 @@ def test_refusals_and_short_buffers(ctx, pkg):
     with pytest.raises(pkg.HipComputeError) as e:   # the weight is short for N (interp.rs:6465-6472)
         pkg.ops.matmul_nbits(ctx, a, B[: n - 1], scales, zp, k, n, bs)
     assert e.value.code == 1 and "short" in e.value.message
-    with pytest.raises(pkg.HipComputeError) as e:
-        pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, 24)
+    with pytest.raises(pkg.HipComputeError) as e:   # not a multiple of 8: a packed word would straddle two blocks
+        pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, 20)
     assert e.value.code == 1
     y = pkg.ops.matmul_nbits(ctx, np.zeros((0, k), np.float32), B, scales, zp, k, n, bs)   # no rows: a no-op
     assert y.shape == (0, n)
