@@ -48,6 +48,7 @@ struct PrefillArgs {
     // weight tiles are not cut) and writes f32 partials [split][M][N] that a second launch adds up
     int ksplit, split_stages;
     float *Ypart;
+    float *Yf32;   // when set, the result is written here as f32 and Y is not used (rows of f32 activations, see nbits_prefill_f32)
 };
 
 // eight nibbles (order k0 k2 k4 k6 k1 k3 k5 k7) -> eight f16 values q - zp in k order, as four words of pairs
@@ -253,6 +254,8 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
                 if (gi < p.M && gj < p.N) {
                     if (p.ksplit > 1)
                         p.Ypart[((size_t)blockIdx.y * p.M + gi) * p.N + gj] = total[i][j][r];
+                    else if (p.Yf32)
+                        p.Yf32[(size_t)gi * p.N + gj] = total[i][j][r];
                     else
                         p.Y[(size_t)gi * p.N + gj] = __float2half(total[i][j][r]);
                 }
@@ -261,24 +264,17 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
     }
 }
 
-// Y = f16(sum over splits of the f32 partials), in split order (static: this file is compiled twice)
+// Y = f16(sum over splits of the f32 partials), in split order; or the f32 sum itself into Yf32
+// (static: this file is compiled twice)
 static __global__ void __launch_bounds__(256)
-mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ Y, long total, int ksplit) {
+mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ Y, float *__restrict__ Yf32, long total, int ksplit) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= total) return;
-    if (i + 4 <= total && (total & 3) == 0) {
-        float4 v = *reinterpret_cast<const float4 *>(part + i);
-        for (int s = 1; s < ksplit; s++) {
-            const float4 w = *reinterpret_cast<const float4 *>(part + (size_t)s * total + i);
-            v.x += w.x, v.y += w.y, v.z += w.z, v.w += w.w;
-        }
-        Y[i] = __float2half(v.x), Y[i + 1] = __float2half(v.y), Y[i + 2] = __float2half(v.z), Y[i + 3] = __float2half(v.w);
-    } else {
-        for (long j = i; j < min(i + 4, total); j++) {
-            float v = part[j];
-            for (int s = 1; s < ksplit; s++) v += part[(size_t)s * total + j];
-            Y[j] = __float2half(v);
-        }
+    for (long j = i; j < min(i + 4, total); j++) {
+        float v = part[j];
+        for (int s = 1; s < ksplit; s++) v += part[(size_t)s * total + j];
+        if (Yf32) Yf32[j] = v;
+        else Y[j] = __float2half(v);
     }
 }
 
@@ -329,7 +325,7 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
     HIPC_LAUNCHED(ctx);
     if (a.ksplit > 1) {
         const long total = (long)a.M * a.N;
-        mmnb_prefill_reduce_kernel<<<dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream>>>(a.Ypart, a.Y, total, a.ksplit);
+        mmnb_prefill_reduce_kernel<<<dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream>>>(a.Ypart, a.Y, a.Yf32, total, a.ksplit);
         HIPC_LAUNCHED(ctx);
     }
     return HIPC_OK;
@@ -387,6 +383,77 @@ int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void
         case 2: return prefill_launch<2>(ctx, a);
         default: return prefill_launch<1>(ctx, a);
     }
+}
+
+// Rows of f32 activations for the f16 matrix cores: row m becomes two f16 rows, hi = f16(a 2^-e) and
+// lo = f16(a 2^-e - hi) (22 significant bits), with 2^e the row's own power of two that brings its
+// largest magnitude into [2^14, 2^15) -- exact, and no value of the row leaves the f16 range. The rows
+// are stored as A2[m] = hi, A2[M + m] = lo; one workgroup per row.
+static __global__ void __launch_bounds__(256)
+mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half *__restrict__ A2, int *__restrict__ exps) {
+    __shared__ float red[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const float *row = A + (size_t)m * K;
+    float mx = 0.f;
+    for (int k = tid; k < K; k += 256) mx = fmaxf(mx, fabsf(row[k]));   // (a NaN does not raise the maximum: it passes through below)
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    // bits of mx: exponent field - 127 = floor(log2 mx) for a normal number; zero, subnormal or infinite rows are not scaled
+    const int ef = (int)((__float_as_uint(mx) >> 23) & 0xffu);
+    const int e = (ef == 0 || ef == 255) ? 0 : ef - 127 - 14;
+    if (tid == 0) exps[m] = e;
+    const float down = __uint_as_float((uint32_t)(127 - e) << 23);   // 2^-e: e is in [-140, 113], 2^-e a normal number
+    for (int k = tid; k < K; k += 256) {
+        const float a = row[k] * down;
+        const __half hi = __float2half(a);
+        A2[(size_t)m * K + k] = hi;
+        A2[(size_t)(M + m) * K + k] = __float2half(a - __half2float(hi));
+    }
+}
+// Y[m] = (P[m] + P[M + m]) 2^e[m]
+static __global__ void __launch_bounds__(256)
+mmnb_prefill_join_rows_kernel(const float *__restrict__ P, const int *__restrict__ exps, int M, int N, float *__restrict__ Y) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)M * N) return;
+    const int m = (int)(i / N);
+    Y[i] = ldexpf(P[i] + P[i + (long)M * N], exps[m]);
+}
+
+// Many rows of f32 activations: each row as two f16 rows (22 bits) through the same tiled kernel, 2 M rows
+// of f32 results, and a last launch that adds the pairs and puts the rows' powers of two back. Twice the
+// products of the f16 case, against one pass over the whole weight per 16 rows on the decode kernel.
+bool nbits_prefill_f32_takes(const void *A, const hipc_nbits_weight *w, int64_t M) {
+    return M > 32 && w->K % 8 == 0 && aligned(A, 16) && 2 * M * w->K < (int64_t(1) << 31) && 2 * M * w->N < (int64_t(1) << 31);
+}
+
+int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M) {
+    HIPC_REFUSE(ctx, !nbits_prefill_f32_takes(A, w, M), "MatMulNBits prefill: shape or alignment not taken by the tiled kernel");
+    const size_t a2_bytes = (size_t)2 * M * w->K * sizeof(__half), e_bytes = ((size_t)M * sizeof(int) + 255) & ~(size_t)255;
+    void *split = nullptr, *sums = nullptr;
+    if (int rc = scratch_get(ctx, 2, a2_bytes + e_bytes, &split)) return rc;
+    if (int rc = scratch_get(ctx, 3, (size_t)2 * M * w->N * sizeof(float), &sums)) return rc;
+    __half *A2 = reinterpret_cast<__half *>(static_cast<char *>(split) + e_bytes);
+    int *exps = static_cast<int *>(split);
+    mmnb_prefill_split_rows_kernel<<<dim3((unsigned)M), dim3(256), 0, ctx->stream>>>(static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
+    HIPC_LAUNCHED(ctx);
+    PrefillArgs a{};
+    a.A = A2, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = nullptr, a.Yf32 = static_cast<float *>(sums);
+    a.M = (int)(2 * M), a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
+    int rc;
+    switch (w->SG) {
+        case 4: rc = prefill_launch<4>(ctx, a); break;
+        case 2: rc = prefill_launch<2>(ctx, a); break;
+        default: rc = prefill_launch<1>(ctx, a); break;
+    }
+    if (rc != HIPC_OK) return rc;
+    const long total = (long)M * w->N;
+    mmnb_prefill_join_rows_kernel<<<dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream>>>(static_cast<const float *>(sums), exps, (int)M, (int)w->N,
+                                                                                                      static_cast<float *>(Y));
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
 }
 
 #endif  // HIPC_PREFILL_WIDE

@@ -132,6 +132,41 @@ def test_f16_rows_beyond_sixteen_run_the_tiled_kernel(ctx, pkg, oracle, shape):
     assert got.dtype == np.float16 and close(got, want, RTOL16), worst(got, want)
 
 
+F32_PREFILL = [  # (M, K, N, block_size, zero points)
+    (100, 1000, 200, 32, True), (130, 384, 131, 64, True), (257, 640, 96, 128, False), (33, 72, 16, 32, True),
+    (512, 2048, 2560, 128, False),
+]
+
+
+@pytest.mark.parametrize("shape", F32_PREFILL, ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_f32_rows_beyond_thirty_two_run_the_tiled_kernel(ctx, pkg, oracle, shape):
+    """More than 32 rows of f32 activations (the reference's own element type, interp.rs:6455-6472) go through
+    the tiled matrix-core kernel as two f16 rows each, scaled per row by a power of two: against the oracle at
+    the operator's f32 tolerance, against the float64 product at 2e-5 of the row's largest output, and equal
+    in quality to the decode kernel's route (the same rows, 16 at a time)."""
+    m, k, n, bs, with_zp = shape
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=45, with_zp=with_zp)
+    a = pkg.synth.normal_f32(m * k, 46).reshape(m, k)
+    a[0] *= np.float32(3.0e7)      # a row far beyond the f16 range, one far below it, one of zeros
+    a[1] *= np.float32(1.0e-9)
+    a[2] = 0
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    by_rows = np.concatenate([pkg.ops.matmul_nbits(ctx, a[i:i + 16], None, None, None, k, n, bs, weight=w) for i in range(0, m, 16)])
+    w.destroy()
+    assert got.dtype == np.float32 and got.shape == (m, n)
+    # rows 0 and 1 are out of the absolute tolerance's scale: compare them relative to their own size
+    scale = np.maximum(np.abs(want).max(axis=1, keepdims=True), 1e-30)
+    assert np.all(np.abs(got - want) <= (1e-3 + 1e-4 * np.abs(want)) * np.maximum(scale / np.abs(want[3:]).max(), 1e-30) + 1e-4 * scale), worst(got, want)
+    nib, z = _unpack(B, zp if zp is not None else np.full((n, (-(-k // bs) + 1) // 2), 0x88, np.uint8), k, n, bs)
+    f64 = rc.matmul_nbits_f64(a, nib, z, scales.reshape(n, -1), bs)
+    big = np.abs(f64).max(axis=1, keepdims=True)
+    assert np.all(np.abs(got - f64) <= 2e-5 * np.maximum(big, 1e-300)), float(np.max(np.abs(got - f64) / np.maximum(big, 1e-300)))
+    assert np.all(np.abs(got - f64) <= np.abs(by_rows - f64).max(axis=1, keepdims=True) * 1.5 + 2e-6 * big)
+    assert np.all(got[2] == 0)
+
+
 @pytest.mark.parametrize("kn", [(2048, 11008), (11008, 2048), (2048, 2560)], ids=lambda s: "K%d_N%d" % s)
 def test_prefill_configuration_full_size(ctx, pkg, oracle, kn):
     """512 rows of f16 activations against block-128 symmetric weights with f16 scales (no zero
