@@ -131,6 +131,23 @@ pub struct Graph {
     raw: *mut sys::hipc_graph,
 }
 
+/// Which scalar of a recorded call a replay changes (`HIPC_SCALAR_*`).
+#[derive(Clone, Copy, Debug, PartialEq, Eq)]
+#[repr(i32)]
+pub enum Scalar {
+    AZeroPoint = 1,
+    BZeroPoint = 2,
+    YZeroPoint = 3,
+    Relu = 4,
+}
+/// One patch of a replay: recorded call `op` (in call order, from 0), its scalar `which`, the new value.
+#[derive(Clone, Copy, Debug)]
+pub struct ScalarPatch {
+    pub op: usize,
+    pub which: Scalar,
+    pub value: i32,
+}
+
 /// Prepacked MatMulNBits weight (the role `packed_b` plays for MatMulInteger, `interp.rs:2712-2768`).
 pub struct NBitsWeight {
     raw: *mut sys::hipc_nbits_weight,
@@ -353,10 +370,25 @@ impl HipContext {
         self.check(unsafe { sys::hipc_capture_end(self.raw, &mut raw) })?;
         Ok(Graph { raw })
     }
-    /// `replay` (stream.rs:572). Nothing is patched between replays: every quantity that changes (token,
-    /// position, zero points, quantisation ranges) is read from device memory by the kernels.
+    /// `replay` (stream.rs:572) of a graph as recorded: most quantities that change between replays (token,
+    /// position, the zero points and ranges of the dynamic operators) are read from device memory by the kernels.
     pub fn replay(&self, graph: &Graph) -> Result<()> {
         self.check(unsafe { sys::hipc_graph_launch(self.raw, graph.raw) })
+    }
+    /// `replay` with patches (the reference's `PushPatch`, onnx-vulkan-core/src/plan.rs:52-68): the scalars that were
+    /// given by value when the graph was recorded -- the zero points of QLinearMatMul / QLinearConv, the relu
+    /// attribute of the fused rescale -- are changed in the instantiated graph first, then it is launched.
+    pub fn replay_patched(&self, graph: &Graph, patches: &[ScalarPatch]) -> Result<()> {
+        for p in patches {
+            self.check(unsafe { sys::hipc_graph_set_scalar(self.raw, graph.raw, p.op as c_int, p.which as c_int, p.value) })?;
+        }
+        self.replay(graph)
+    }
+    /// how many calls recorded work while the capture of `graph` was open (the `op` of a `ScalarPatch` counts them from 0)
+    pub fn graph_op_count(&self, graph: &Graph) -> Result<usize> {
+        let mut n: c_int = 0;
+        self.check(unsafe { sys::hipc_graph_op_count(self.raw, graph.raw, &mut n) })?;
+        Ok(n as usize)
     }
     pub fn destroy_graph(&self, graph: Graph) {
         unsafe { sys::hipc_graph_destroy(self.raw, graph.raw) }

@@ -119,6 +119,8 @@ unsafe extern "C" {
     pub fn hipc_capture_end(ctx: *mut hipc_ctx, out: *mut *mut hipc_graph) -> c_int;
     pub fn hipc_graph_launch(ctx: *mut hipc_ctx, graph: *mut hipc_graph) -> c_int;
     pub fn hipc_graph_destroy(ctx: *mut hipc_ctx, graph: *mut hipc_graph);
+    pub fn hipc_graph_op_count(ctx: *mut hipc_ctx, graph: *mut hipc_graph, count: *mut c_int) -> c_int;
+    pub fn hipc_graph_set_scalar(ctx: *mut hipc_ctx, graph: *mut hipc_graph, op: c_int, which: c_int, value: i32) -> c_int;
     pub fn hipc_measure_graph(ctx: *mut hipc_ctx, graph: *mut hipc_graph, samples: c_int, launches_per_sample: c_int, ns_out: *mut f64) -> c_int;
     pub fn hipc_probe_int8_mfma(ctx: *mut hipc_ctx, random_operands: c_int, waves_per_simd: c_int, iterations: c_int, tops: *mut f64) -> c_int;
 

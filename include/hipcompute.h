@@ -117,6 +117,25 @@ int hipc_capture_end(hipc_ctx *ctx, hipc_graph **out);
 int hipc_graph_launch(hipc_ctx *ctx, hipc_graph *graph);
 void hipc_graph_destroy(hipc_ctx *ctx, hipc_graph *graph);
 
+/* The reference patches push-constant words of a recorded step between replays (`PushPatch`,
+ * crates/onnx-vulkan-core/src/plan.rs:52-68: "a push-constant word that moves with the step"). Here a graph
+ * keeps, for every call that recorded work while the capture was open (numbered from 0 in call order,
+ * `hipc_graph_op_count` of them), the scalars of that call a replay may change without recording again:
+ *   QLinearMatMul, QLinearConv        the three zero points given by value
+ *   MatMulIntegerScaleBias            the relu attribute (0 / 1)
+ * `hipc_graph_set_scalar` changes one (a kernel-node parameter update of the instantiated graph); the next
+ * `hipc_graph_launch` uses it. Everything that decides a launch's grid (M, the conv geometry) and everything
+ * the library keeps in device memory (requantisation ratios, weights) is fixed at recording time, as in the
+ * reference ("step-invariant grids and sizes", plan.rs:21-29); MatMulNBits, MatMulInteger and
+ * DynamicQuantizeLinear read their zero points, scales and ranges from device memory and carry no such scalar
+ * (asking for one is HIPC_ERR_UNSUPPORTED). The decoder needs none: token and position live in device memory. */
+#define HIPC_SCALAR_A_ZERO_POINT 1
+#define HIPC_SCALAR_B_ZERO_POINT 2
+#define HIPC_SCALAR_Y_ZERO_POINT 3
+#define HIPC_SCALAR_RELU 4
+int hipc_graph_op_count(hipc_ctx *ctx, hipc_graph *graph, int *count);
+int hipc_graph_set_scalar(hipc_ctx *ctx, hipc_graph *graph, int op, int which, int32_t value);
+
 /* `measure_dispatch_gpu` (crates/vk-compute/src/pipeline.rs:246): time `samples`
  * groups of `launches_per_sample` launches of a recorded graph with device
  * events on the context's stream; writes nanoseconds PER LAUNCH to ns_out[samples]. */

@@ -398,6 +398,7 @@ int hipc_capture_begin(hipc_ctx *ctx) {
         HIPC_REQUIRE(ctx, !ctx->capturing, "hipc_capture_begin: a capture is already open");
         HIPC_TRY(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
         ctx->capturing = true;
+        ctx->cap_ops.clear();
         return HIPC_OK;
     });
 }
@@ -419,6 +420,7 @@ int hipc_capture_end(hipc_ctx *ctx, hipc_graph **out) {
         hipc_graph *gr = new hipc_graph();
         gr->graph = graph;
         gr->exec = exec;
+        gr->ops.swap(ctx->cap_ops);
         ctx->live_graphs++;
         *out = gr;
         return HIPC_OK;
@@ -447,6 +449,35 @@ void hipc_graph_destroy(hipc_ctx *ctx, hipc_graph *graph) {
             for (void *p : ctx->retained) ctx->deferred.push_back(p);
             ctx->retained.clear();
         }
+    });
+}
+
+int hipc_graph_op_count(hipc_ctx *ctx, hipc_graph *graph, int *count) {
+    if (!graph || !count) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        *count = (int)graph->ops.size();
+        return HIPC_OK;
+    });
+}
+
+int hipc_graph_set_scalar(hipc_ctx *ctx, hipc_graph *graph, int op, int which, int32_t value) {
+    if (!graph) return HIPC_ERR_INVALID;
+    return entry(ctx, [&]() -> int {
+        HIPC_REQUIRE(ctx, !ctx->capturing, "hipc_graph_set_scalar while a capture is open");
+        HIPC_REQUIRE(ctx, op >= 0 && op < (int)graph->ops.size(), "hipc_graph_set_scalar: the graph recorded %zu operator calls, not %d", graph->ops.size(), op + 1);
+        int changed = 0;
+        for (const ScalarPatch &sp : graph->ops[(size_t)op].patches) {
+            if (sp.which != which) continue;
+            hipKernelNodeParams params{};
+            HIPC_TRY(ctx, hipGraphKernelNodeGetParams(sp.node, &params));
+            HIPC_REQUIRE(ctx, params.kernelParams && params.kernelParams[0], "hipc_graph_set_scalar: the kernel node carries no arguments");
+            memcpy(static_cast<char *>(params.kernelParams[0]) + sp.offset, &value, sizeof value);
+            HIPC_TRY(ctx, hipGraphKernelNodeSetParams(sp.node, &params));           // the graph itself, for later instantiations
+            HIPC_TRY(ctx, hipGraphExecKernelNodeSetParams(graph->exec, sp.node, &params));
+            changed++;
+        }
+        HIPC_REFUSE(ctx, changed == 0, "hipc_graph_set_scalar: operator call %d of the graph has no scalar %d that a replay can change", op, which);
+        return HIPC_OK;
     });
 }
 

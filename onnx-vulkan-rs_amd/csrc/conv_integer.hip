@@ -273,6 +273,7 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
                 else int8_conv_row_kernel<EPI_I32, true><<<grid, 256, lds, ctx->stream>>>(ga);
             }
             HIPC_LAUNCHED(ctx);
+            gemm_note_scalars(ctx, ga, !zero_known);
             return HIPC_OK;
         }
 
@@ -302,6 +303,7 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
                 else int8_conv_small_kernel<EPI_I32, true><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
             }
             HIPC_LAUNCHED(ctx);
+            gemm_note_scalars(ctx, ga, !zero_known);
             return HIPC_OK;
         }
         return ep.requant ? gemm_launch<MODE_CONV, EPI_REQUANT, true>(ctx, ga, (unsigned)g->n)
@@ -322,6 +324,11 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
     d.out_signed = ep.out_signed;
     conv_direct_kernel<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, ctx->stream>>>(d);
     HIPC_LAUNCHED(ctx);
+    if (host_zp) {
+        note_scalar(ctx, HIPC_SCALAR_A_ZERO_POINT, offsetof(DirectConvArgs, x_zp_value));
+        note_scalar(ctx, HIPC_SCALAR_B_ZERO_POINT, offsetof(DirectConvArgs, w_zp_value));
+    }
+    if (ep.requant) note_scalar(ctx, HIPC_SCALAR_Y_ZERO_POINT, offsetof(DirectConvArgs, y_zp));
     return HIPC_OK;
 }
 

@@ -21,6 +21,7 @@
 // point is not 0.
 #pragma once
 
+#include <cstddef>
 #include <cstdlib>
 
 #include "internal.h"
@@ -447,6 +448,20 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
     if (EPI == EPI_SCALE_BIAS) gemm_emit_range(p, lane, fmn, fmx);
 }
 
+// After a launch whose argument is a GemmArgs: the scalars of it that a replay of a recorded graph may change
+// (hipc_graph_set_scalar). Zero points only when they were given by value (the QLinear operators).
+// `sums`: the launched instance forms the dynamic operand's sums over k, which a non-zero zero point of the
+// constant operand needs (an instance chosen because that zero point was known to be zero cannot take another).
+inline void gemm_note_scalars(hipc_ctx *ctx, const GemmArgs &g, bool sums) {
+    if (!ctx->capturing) return;
+    if (g.host_zp) {
+        note_scalar(ctx, HIPC_SCALAR_A_ZERO_POINT, offsetof(GemmArgs, dyn_zp_value));
+        if (sums) note_scalar(ctx, HIPC_SCALAR_B_ZERO_POINT, offsetof(GemmArgs, const_zp_value));
+    }
+    if (g.ratio) note_scalar(ctx, HIPC_SCALAR_Y_ZERO_POINT, offsetof(GemmArgs, y_zp));
+    if (g.scale) note_scalar(ctx, HIPC_SCALAR_RELU, offsetof(GemmArgs, relu));
+}
+
 // ---- host side: tile choice and launch of the kernel above ---------------------------------
 // 64x64 tiles until 128x128 ones would give every CU at least two workgroups;
 // the gemm_tile option (64 / 128) overrides (tuning, tests).
@@ -464,6 +479,7 @@ int gemm_launch_tile(hipc_ctx *ctx, GemmArgs g, unsigned batch) {
     const dim3 grid(gemm_grid(g, T), 1, batch);
     int8_gemm_kernel<MODE, EPI, ALIGNED, T><<<grid, 256, gemm_lds(T), ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);
+    gemm_note_scalars(ctx, g, true);
     return HIPC_OK;
 }
 

@@ -80,6 +80,17 @@ struct StageRing {
     size_t used = 0;                    // bytes of the current slot handed out
 };
 
+// What a recorded operator call left in the graph: the scalars of it that a replay may change
+// (hipc_graph_set_scalar), each a 32-bit word inside the first argument of one kernel node.
+struct ScalarPatch {
+    int which;              // HIPC_SCALAR_*
+    hipGraphNode_t node;
+    size_t offset;          // byte offset of the word inside the kernel's argument struct
+};
+struct RecordedOp {
+    std::vector<ScalarPatch> patches;
+};
+
 }  // namespace hipc
 
 struct hipc_ctx {
@@ -99,6 +110,8 @@ struct hipc_ctx {
     void *params = nullptr;              // small device block: range slot, scalars, range partials
     void *dql_static = nullptr;          // this device's address of the static range-partials array (see dynamic_quantize.hip)
     int cu_count = 256;
+    std::vector<hipc::RecordedOp> cap_ops;     // while a capture is open: the calls that recorded work so far
+    std::vector<hipc::ScalarPatch> cap_patches;   // ... the patchable scalars the current call has noted
     hipc::Tuning tune;
     hipc::StageRing stage;
     // hipc_alloc's blocks by size class (the reference's pooled scratch buffers,
@@ -112,6 +125,7 @@ struct hipc_ctx {
 struct hipc_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    std::vector<hipc::RecordedOp> ops;   // the entry-point calls that recorded work, in call order
 };
 
 // A MatMulNBits weight repacked for the matrix cores: 1 KiB tiles of 16 columns x 128 k. Lane l
@@ -149,13 +163,38 @@ struct Guard {
 // The body of an entry point: takes the context's lock, makes its device current and keeps C++
 // exceptions (a failed host allocation, a length error) from crossing the C ABI -- they become
 // HIPC_ERR_BACKEND with a message, under the same lock.
+// The kernel node a launch on the capturing stream has just added (null when nothing is being captured).
+inline hipGraphNode_t last_captured_node(hipc_ctx *ctx) {
+    if (!ctx->capturing) return nullptr;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    const hipGraphNode_t *deps = nullptr;
+    size_t n = 0;
+    if (hipStreamGetCaptureInfo_v2(ctx->stream, &status, nullptr, nullptr, &deps, &n) != hipSuccess || status != hipStreamCaptureStatusActive || n == 0)
+        return nullptr;
+    return deps[n - 1];
+}
+// called right after the launch whose argument struct holds the scalar: the word at `offset` of that struct may be
+// changed in the instantiated graph later (hipc_graph_set_scalar)
+inline void note_scalar(hipc_ctx *ctx, int which, size_t offset) {
+    if (hipGraphNode_t node = last_captured_node(ctx)) ctx->cap_patches.push_back(ScalarPatch{which, node, offset});
+}
+
 template <typename F>
 int entry(hipc_ctx *ctx, F &&body) noexcept {
     if (!ctx) return HIPC_ERR_INVALID;
     try {
         Guard g(ctx);
         try {
-            return body();
+            if (!ctx->capturing) return body();
+            // while a capture is open every call that records work becomes an entry of the graph's operator list
+            const hipGraphNode_t before = last_captured_node(ctx);
+            ctx->cap_patches.clear();
+            const int rc = body();
+            if (ctx->capturing && rc == HIPC_OK && last_captured_node(ctx) != before) {
+                ctx->cap_ops.emplace_back();
+                ctx->cap_ops.back().patches.swap(ctx->cap_patches);
+            }
+            return rc;
         } catch (const std::bad_alloc &) {
             return fail(ctx, HIPC_ERR_BACKEND, "out of host memory");
         } catch (const std::exception &e) {

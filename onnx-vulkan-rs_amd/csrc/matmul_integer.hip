@@ -168,6 +168,7 @@ int launch_mm_bdirect_dyn(hipc_ctx *ctx, GemmArgs g) {
     const dim3 grid(gemm_grid(g, T), 1, 1);
     int8_gemm_bdirect_kernel<EPI, DYN, T, W><<<grid, 64 * W, bd_lds(T), ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);
+    gemm_note_scalars(ctx, g, DYN);
     return HIPC_OK;
 }
 
@@ -208,6 +209,7 @@ int launch_mm_small_dyn(hipc_ctx *ctx, GemmArgs g) {
     const dim3 grid(gemm_grid(g, 64));
     int8_gemm_small_kernel<EPI, DYN><<<grid, 256, kSmallLds, ctx->stream>>>(g);
     HIPC_LAUNCHED(ctx);
+    gemm_note_scalars(ctx, g, DYN);
     return HIPC_OK;
 }
 template <int EPI>

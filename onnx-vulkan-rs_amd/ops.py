@@ -268,6 +268,13 @@ def requantize(ctx: Context, acc, bias, ratio, inner, y_zp, out_signed=False):
     return out
 
 
+def qlinear_matmul_device(ctx, A, a_dtype, a_scale, a_zp, weight: Int8Weight, b_scale, b_zp, y_scale, y_zp, y_dtype, Y, M):
+    bs = np.ascontiguousarray(np.atleast_1d(b_scale), np.float32)
+    ctx._check(ctx.lib.hipc_qlinear_matmul(
+        ctx.handle, _ptr(A), a_dtype, float(a_scale), int(a_zp), weight.handle, bs.ctypes.data_as(C.POINTER(C.c_float)),
+        bs.size, int(b_zp), float(y_scale), int(y_zp), y_dtype, _ptr(Y), M))
+
+
 def qlinear_matmul(ctx: Context, A, a_scale, a_zp, B, b_scale, b_zp, y_scale, y_zp, y_signed=False,
                    weight: Int8Weight = None):
     A = np.ascontiguousarray(A)

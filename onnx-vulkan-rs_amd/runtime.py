@@ -12,6 +12,7 @@ import os
 import numpy as np
 
 F32, U8, I8, I32, F16 = 1, 2, 3, 6, 10
+SCALAR_A_ZERO_POINT, SCALAR_B_ZERO_POINT, SCALAR_Y_ZERO_POINT, SCALAR_RELU = 1, 2, 3, 4
 _NP_TO_HIPC = {np.dtype(np.float32): F32, np.dtype(np.uint8): U8, np.dtype(np.int8): I8,
                np.dtype(np.int32): I32, np.dtype(np.float16): F16}
 
@@ -86,6 +87,8 @@ SIGNATURES = {
     "hipc_graph_launch": (_int, [_vp, _vp]),
     "hipc_graph_destroy": (None, [_vp, _vp]),
     "hipc_measure_graph": (_int, [_vp, _vp, _int, _int, C.POINTER(C.c_double)]),
+    "hipc_graph_op_count": (_int, [_vp, _vp, C.POINTER(_int)]),
+    "hipc_graph_set_scalar": (_int, [_vp, _vp, _int, _int, C.c_int32]),
     "hipc_probe_int8_mfma": (_int, [_vp, _int, _int, _int, C.POINTER(C.c_double)]),
     "hipc_matmul_nbits": (_int, [_vp, _vp, _int, _vp, _sz, _vp, _int, _sz, _vp, _sz, _vp, _i64, _i64, _i64,
                                  _i64, _int]),
@@ -285,6 +288,16 @@ class Context:
 
     def graph_destroy(self, graph):
         self.lib.hipc_graph_destroy(self.handle, graph)
+
+    def graph_op_count(self, graph) -> int:
+        """How many calls recorded work while the capture of `graph` was open."""
+        n = _int()
+        self._check(self.lib.hipc_graph_op_count(self.handle, graph, C.byref(n)))
+        return n.value
+
+    def graph_set_scalar(self, graph, op: int, which: int, value: int):
+        """Change a scalar of recorded call `op` for the replays that follow (the reference's ``PushPatch``)."""
+        self._check(self.lib.hipc_graph_set_scalar(self.handle, graph, op, which, value))
 
     def probe_int8_mfma(self, random_operands: bool, waves_per_simd: int = 2, iterations: int = 4096) -> float:
         """Sustained int8 matrix-core rate (TOPS) of a register-only MFMA loop."""

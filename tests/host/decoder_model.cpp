@@ -48,6 +48,10 @@ const char *hipGetErrorString(hipError_t) { return "model"; }
 hipError_t hipMemcpy(void *d, const void *s, size_t n, hipMemcpyKind) { std::memcpy(d, s, n); return hipSuccess; }
 hipError_t hipSetDevice(int) { return hipSuccess; }
 hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+hipError_t hipStreamGetCaptureInfo_v2(hipStream_t, hipStreamCaptureStatus *status, unsigned long long *, hipGraph_t *, const hipGraphNode_t **, size_t *n) {
+    *status = hipStreamCaptureStatusNone, *n = 0;
+    return hipSuccess;
+}
 }
 
 #define MUST(call)                                                                    \

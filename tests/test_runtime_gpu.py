@@ -147,3 +147,73 @@ def test_unknown_options_are_refused(ctx, pkg):
     assert e.value.code == 1
     ctx.set_option("HIPC_GEMM_TILE", 128)
     ctx.set_option("HIPC_GEMM_TILE", -1)
+
+
+def test_scalars_of_a_recorded_graph_can_be_patched(ctx, pkg, oracle):
+    """The reference patches push-constant words of a recorded step between replays
+    (crates/onnx-vulkan-core/src/plan.rs:52-68). Here: a graph of QLinearMatMul, QLinearConv and the fused
+    rescale is recorded once and replayed with other zero points / the relu attribute, every replay against
+    the oracle; a scalar the recorded call does not carry is refused."""
+    ops, rt = pkg.ops, pkg.runtime
+    rng = np.random.default_rng(5)
+    m, k, n = 70, 256, 96
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(0, 256, (k, n), dtype=np.uint8)
+    w = ops.Int8Weight(ctx, b)
+    dA, dY = ctx.upload(a), ctx.alloc(m * n)
+    ys = 0.9
+    qmm = lambda a_zp, b_zp, y_zp: ops.qlinear_matmul_device(ctx, dA, pkg.U8, 0.02, a_zp, w, np.float32(0.01), b_zp, ys, y_zp, pkg.U8, dY, m)  # noqa: E731
+    # conv: 1-D, grouped (the direct kernel) and dense (the slab kernel)
+    X = rng.integers(0, 256, (1, 32, 1, 64), dtype=np.uint8)
+    W = rng.integers(-127, 128, (32, 32, 1, 3), dtype=np.int8)
+    geom = pkg.ConvGeom.make(X.shape, W.shape, pads=(0, 1, 0, 1))
+    og = oracle.conv_geom(X.shape, W.shape, pads=(0, 1, 0, 1))
+    cw = ops.ConvWeight(ctx, W, geom)
+    dX, dC = ctx.upload(X), ctx.alloc(X.size)
+    wsc = np.full(32, 0.01, np.float32)
+    qconv = lambda x_zp, y_zp: ops.qlinear_conv_device(ctx, dX, pkg.U8, 0.02, x_zp, cw, wsc, 0, 0.3, y_zp, pkg.U8, None, geom, dC)  # noqa: E731
+    # fused rescale
+    dS = ctx.upload(np.array([0.003], np.float32))
+    dZ = ctx.upload(np.array([131, 0, 0, 0], np.uint8))
+    dF = ctx.alloc(m * n * 4)
+    resc = lambda relu: ops.matmul_integer_scale_bias_device(ctx, dA, pkg.U8, w, dZ, None, dS, 0, None, 0, None, 0, relu, None, dF, m)  # noqa: E731
+    qmm(128, 121, 7), qconv(128, 10), resc(False)      # once eagerly: ratios uploaded, scratch sized
+    ctx.flush()
+    ctx.capture_begin()
+    qmm(128, 121, 7), qconv(128, 10), resc(False)
+    g = ctx.capture_end()
+    assert ctx.graph_op_count(g) == 3
+
+    def check(a_zp, b_zp, y_zp, x_zp, cy_zp, relu):
+        ctx.graph_launch(g)
+        got = ctx.download(dY, np.uint8, (m, n))
+        assert np.array_equal(got, oracle.qlinear_matmul(a, 0.02, a_zp, b, np.float32(0.01), b_zp, ys, y_zp, False))
+        gotc = ctx.download(dC, np.uint8, X.shape)
+        assert np.array_equal(gotc, oracle.qlinear_conv(X, 0.02, x_zp, W, wsc, 0, 0.3, cy_zp, None, og))
+        acc = oracle.matmul_integer(a, b, 131, 0)
+        want = oracle.rescale(acc, np.float32(0.003), None)
+        gotf = ctx.download(dF, np.float32, (m, n))
+        assert np.array_equal(gotf.view(np.uint32), (np.maximum(want, 0) if relu else want).view(np.uint32))
+
+    check(128, 121, 7, 128, 10, False)
+    ctx.graph_set_scalar(g, 0, rt.SCALAR_A_ZERO_POINT, 90)
+    ctx.graph_set_scalar(g, 0, rt.SCALAR_B_ZERO_POINT, 3)
+    ctx.graph_set_scalar(g, 0, rt.SCALAR_Y_ZERO_POINT, 200)
+    ctx.graph_set_scalar(g, 1, rt.SCALAR_A_ZERO_POINT, 77)
+    ctx.graph_set_scalar(g, 1, rt.SCALAR_Y_ZERO_POINT, 130)
+    ctx.graph_set_scalar(g, 2, rt.SCALAR_RELU, 1)
+    check(90, 3, 200, 77, 130, True)
+    check(90, 3, 200, 77, 130, True)                   # a patch holds for every later replay
+    with pytest.raises(pkg.HipComputeError) as e:      # the int8 weight's zero point was known to be zero when the conv was recorded
+        ctx.graph_set_scalar(g, 1, rt.SCALAR_B_ZERO_POINT, 5)
+    assert e.value.code == 2
+    with pytest.raises(pkg.HipComputeError) as e:
+        ctx.graph_set_scalar(g, 2, rt.SCALAR_Y_ZERO_POINT, 5)
+    assert e.value.code == 2
+    with pytest.raises(pkg.HipComputeError) as e:
+        ctx.graph_set_scalar(g, 3, rt.SCALAR_RELU, 1)
+    assert e.value.code == 1
+    ctx.graph_destroy(g)
+    w.destroy(), cw.destroy()
+    for buf in (dA, dY, dX, dC, dS, dZ, dF):
+        buf.free()
