@@ -812,14 +812,17 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
             const int n_cg_f = (int)ceil_div(c.ffn, 128);
             d->lean = d->fused_glue && d->one_launch_attn && ctx->tune.dec_lean != 0 && c.ffn % 16 == 0 && n_cg_h <= 32 &&
                       c.hidden % 8 == 0;
-            // output projection: a k slice is one head (or one 128-k tile when heads are shorter), at most 8 slices
+            // output projection: a k slice is one head (or one 128-k tile when heads are shorter), at most 4 slices
+            // (the consumer's norm prologue adds up at most four partial rows: every row is code it has to fetch)
             int o_tiles = std::max(1, c.head_dim / 128);
-            while (ceil_div(n_cg_o, o_tiles) > 8 && o_tiles < 4) o_tiles *= 2;
+            while (ceil_div(n_cg_o, o_tiles) > 4 && o_tiles < 4) o_tiles *= 2;
             d->o_slices = (int)ceil_div(n_cg_o, o_tiles);
-            if (d->o_slices > 8 || o_tiles > 4) d->lean = false;
-            // down projection: 18 k tiles per slice (six wavefronts of three tiles), at most 8 slices
+            if (d->o_slices > 4 || o_tiles > 4) d->lean = false;
+            // down projection: 18 k tiles per slice (six wavefronts of three tiles); a longer row in four slices of
+            // up to 32 tiles (eight wavefronts of four)
             d->down_slices = (int)std::max<int64_t>(1, ceil_div(n_cg_f, 18));
-            if (d->down_slices > 8) d->lean = false;
+            if (d->down_slices > 4) d->down_slices = 4;
+            if (ceil_div(n_cg_f, d->down_slices) > 32) d->lean = false;
             if (d->lean) {
                 A(&d->yo, (size_t)d->o_slices * c.hidden), A(&d->yd, (size_t)d->down_slices * c.hidden);
                 const size_t chunks = (size_t)n_cg_f * 4;

@@ -130,7 +130,20 @@ __device__ __forceinline__ void lean_split1(float v, uint16_t (&t)[3]) {
     }
 }
 
-constexpr int kLeanMaxSlices = 8;   // partial rows a norm prologue adds up at most
+#ifdef HIPC_LEAN_STAMPS
+__device__ unsigned long long lean_stamps[5 * 1024 * 8 * 12];
+#define LEAN_STAMP(ph)                                                                                       \
+    do {                                                                                                     \
+        const unsigned long long t_ = (unsigned long long)wall_clock64();                                    \
+        if ((threadIdx.x & 63) == 0 && st_wg < 1024 && (threadIdx.x >> 6) < 8)                               \
+            lean_stamps[((st_slot * 1024 + st_wg) * 8 + (threadIdx.x >> 6)) * 12 + (ph)] = t_;                \
+    } while (0)
+#define LEAN_STAMP_AFTER(v, ph) do { asm volatile("" ::"v"(v)); LEAN_STAMP(ph); } while (0)
+#else
+#define LEAN_STAMP(ph)
+#define LEAN_STAMP_AFTER(v, ph)
+#endif
+constexpr int kLeanMaxSlices = 4;   // partial rows a norm prologue adds up at most
 
 // PRO: 0 plain row, 2 norm, 3 attention join, 4 row already split by the producer
 // EPI: 0 store (a partial row per k slice), 1 gated GELU of a (gate, up) tile pair -> split row
@@ -146,13 +159,55 @@ template <int SG, int NT, int PRO, int EPI, int KT>
 __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const LeanArgs p) {
     extern __shared__ uint4 lean_smem[];
     constexpr int CPG = 4 / SG;  // 32-k chunks per scale group
-    if ((int)blockIdx.y >= p.slices) {   // a helper row: read ahead for the next launch, nothing else
+#ifdef HIPC_LEAN_STAMPS
+    const int st_slot = PRO + (EPI ? -1 : 0), st_wg = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+#endif
+    // Every argument this instance uses is read here, in one batch: left to itself the compiler reads an argument
+    // next to its first use, and each such group is a round trip of its own to memory (the scalar cache starts
+    // every launch empty) in the middle of the kernel -- five of them before the norm prologue's first load.
+    HIPC_ARG_NOW(p.Wq); HIPC_ARG_NOW(p.Sc); HIPC_ARG_NOW(p.Zb);
+    HIPC_ARG_NOW(p.K); HIPC_ARG_NOW(p.N); HIPC_ARG_NOW(p.n_tiles); HIPC_ARG_NOW(p.n_cg);
+    HIPC_ARG_NOW(p.WK); HIPC_ARG_NOW(p.WN); HIPC_ARG_NOW(p.slices); HIPC_ARG_NOW(p.nib_mask); HIPC_ARG_NOW(p.magic);
+    if (PRO == 0) { HIPC_ARG_NOW(p.A); }
+    if (PRO == 2) {
+        HIPC_ARG_NOW(p.x); HIPC_ARG_NOW(p.yparts); HIPC_ARG_NOW(p.w_post); HIPC_ARG_NOW(p.w_in); HIPC_ARG_NOW(p.x_out);
+        HIPC_ARG_NOW(p.y_slices); HIPC_ARG_NOW(p.eps);
+    }
+    if (PRO == 3) {
+        HIPC_ARG_NOW(p.part_o); HIPC_ARG_NOW(p.part_ml); HIPC_ARG_NOW(p.pos);
+        HIPC_ARG_NOW(p.lg_group); HIPC_ARG_NOW(p.lg_hd); HIPC_ARG_NOW(p.n_kv); HIPC_ARG_NOW(p.window);
+    }
+    if (PRO == 4) { HIPC_ARG_NOW(p.a_split); }
+    if (EPI == 0) { HIPC_ARG_NOW(p.Y); }
+    if (EPI == 1) { HIPC_ARG_NOW(p.h_split); }
+    LEAN_STAMP(0);
+    if (__builtin_expect((int)blockIdx.y >= p.slices, 0)) {   // a helper row: read ahead for the next launch, nothing else
         prefetch_for_next(p.pf, ((int)blockIdx.y - p.slices) * (int)gridDim.x + (int)blockIdx.x, p.pf.rows * (int)gridDim.x,
                           (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x, p.pf.sink);
+        LEAN_STAMP(7);
         return;
     }
+    LEAN_STAMP(8);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // PRO 2: the row's operands are asked for before anything else is worked out. They come from the launch
+    // before this one, i.e. from memory and not from this XCD's L2, and the instructions between here and their
+    // first use (index arithmetic, descriptors, the weight loads) take about as long to arrive as they do.
+    // Every wavefront asks; a thread past the end of the row reads zeros and causes no traffic, and so does a
+    // partial row that does not exist (an empty descriptor).
+    float x8[8], w8[8], wp8[8], part[kLeanMaxSlices][8];
+    if (PRO == 2) {
+        const uint32_t row_bytes = (uint32_t)p.K * 4u, voff = (uint32_t)tid * 32u;
+        const bool has_y = p.yparts != nullptr;
+        const int ys = has_y ? p.y_slices : 0;
+        lean_ld8f(lean_rsrc(p.x, row_bytes), voff, 0, x8);
+        lean_ld8f(lean_rsrc(p.w_in, row_bytes), voff, 0, w8);
+        lean_ld8f(lean_rsrc(has_y ? p.w_post : p.w_in, row_bytes), voff, 0, wp8);
+#pragma unroll
+        for (int s = 0; s < kLeanMaxSlices; s++) lean_ld8f(lean_rsrc(p.yparts + (size_t)s * p.K, s < ys ? row_bytes : 0u), voff, 0, part[s]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    LEAN_STAMP(9);
     // wave = wn * WK + wk without a division: WK is at most 16 and WN at most 4
     int wn = 0, wk = wave;
     while (wk >= p.WK) wk -= p.WK, wn++;
@@ -230,30 +285,16 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
         // Every load is issued before the first sum: one memory round trip. Only the partial rows that
         // exist are asked for; items past K read zeros.
         const int pw = (nitems + 63) >> 6;  // wavefronts that hold items
-        float x8[8], yw8[8], w8[8];
+        float yw8[8];
         float4 *red4 = reinterpret_cast<float4 *>(red);
-        const uint32_t row_bytes = (uint32_t)p.K * 4u, voff = (uint32_t)tid * 32u;
+        load_weights();
         if (wave < pw) {
-            float part[kLeanMaxSlices][8], wp8[8];
-            const bool has_y = p.yparts != nullptr;
-            const int ys = has_y ? p.y_slices : 0;
-            lean_ld8f(lean_rsrc(p.x, row_bytes), voff, 0, x8);
-            lean_ld8f(lean_rsrc(p.w_in, row_bytes), voff, 0, w8);
-            lean_ld8f(lean_rsrc(has_y ? p.w_post : p.w_in, row_bytes), voff, 0, wp8);
-#pragma unroll
-            for (int s = 0; s < kLeanMaxSlices; s++) {
-                if (s < ys) {   // wave-uniform; a descriptor per partial row, so that an item past K reads zeros and not the next row
-                    lean_ld8f(lean_rsrc(p.yparts + (size_t)s * p.K, row_bytes), voff, 0, part[s]);
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 8; i++) part[s][i] = 0.f;
-                }
-            }
-            load_weights();
+            LEAN_STAMP(1);
 #pragma unroll
             for (int s = 0; s < kLeanMaxSlices; s++)
 #pragma unroll
                 for (int i = 0; i < 8; i++) LEAN_NEEDED_HERE(part[s][i]);
+            LEAN_STAMP(2);
             float s_yy = 0.f, s_xx = 0.f, s_xyw = 0.f, s_ywyw = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -266,8 +307,6 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
             }
             s_yy = lean_row_sum(s_yy), s_xx = lean_row_sum(s_xx), s_xyw = lean_row_sum(s_xyw), s_ywyw = lean_row_sum(s_ywyw);
             if (i16 == 0) red4[wave * 4 + g4] = make_float4(s_yy, s_xx, s_xyw, s_ywyw);
-        } else {
-            load_weights();
         }
         __syncthreads();
         if (wave < pw) {
@@ -293,6 +332,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
             if (tid < nitems) put_item(tid, av);
         }
         __syncthreads();  // also: `red` is free for the k reduction
+        LEAN_STAMP(3);
     } else if (PRO == 3) {
         // The channels of this workgroup's k slice, joined over the live context chunks of their
         // head: sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m). A wavefront's 64 channels
@@ -332,10 +372,12 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
                 }
             }
             if (!weights_asked) load_weights(), weights_asked = true;
+            LEAN_STAMP(1);
             float mx = __uint_as_float(ml_raw.x), ls = __uint_as_float(ml_raw.y);
             LEAN_NEEDED_HERE(mx);
 #pragma unroll
             for (int j = 0; j < kAttnSplits; j++) LEAN_NEEDED_HERE(f[j]);
+            LEAN_STAMP(2);
             const bool on = lane < live;
             const float m = lean_wave_max(on ? mx : -3.0e38f);
             const float e = on ? __expf(mx - m) : 0.f;
@@ -359,8 +401,10 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
         }
         if (!weights_asked) load_weights();
         __syncthreads();
+        LEAN_STAMP(3);
     } else {
         load_weights();
+        LEAN_STAMP(1);
     }
 
     // ---- products, phase by phase so that nothing waits for its neighbour: every operand first
@@ -391,6 +435,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
 #pragma unroll
             for (int j = 0; j < 4; j++) aop[i][j] = a_lane[(size_t)(tile_in_slice[i] * 4 + j) * NT * 4];
     }
+    LEAN_STAMP_AFTER(aop[KT - 1][3].x, 4);
     const uint32_t one2 = 0x3f803f80u;   // bf16 1.0 twice
     const lbf16x8 ones = __builtin_bit_cast(lbf16x8, make_uint4(one2, one2, one2, one2));
     lf32x4 d[KT][SG], e[KT][SG];
@@ -439,11 +484,13 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
 
     // ---- the sum over the wavefronts that split k: column n's partials sit side by side, and every
     // lane of the finishing wavefront reads its column's slots and adds the first WK in order
+    LEAN_STAMP_AFTER(acc, 5);
     const bool through_lds = p.WK > 1 || EPI == 1;   // the gated epilogue's two tiles meet in LDS even when k is not split
     if (through_lds) {
         if (g4 == 0) red[(wn * 16 + i16) * 16 + wk] = acc;
         __syncthreads();
     }
+    LEAN_STAMP(6);
     const bool reducer = wk == 0 && (EPI == 0 || wn == 0);
     if (!reducer) return;
     auto reduce_tile = [&](int tile_wn, float own) {
@@ -480,9 +527,16 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
             for (int q = 0; q < NT; q++) dst[32 * q] = t[q];
         }
     }
+    LEAN_STAMP(7);
 }
 
 }  // namespace hipc
+
+#ifdef HIPC_LEAN_STAMPS
+extern "C" int hipc_debug_lean_stamps(void *dst, size_t bytes) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(hipc::lean_stamps), bytes, 0, hipMemcpyDeviceToHost);
+}
+#endif
 
 using namespace hipc;
 

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
+#include <cstddef>
 #include <cstdint>
 #include <cstdio>
 #include <exception>
@@ -23,7 +24,9 @@
 #ifndef HIPC_HOST_MODEL
 #define HIPC_PIN_VGPR(v) asm volatile("" : "+v"(v))                                              // the value is needed here, in a vector register
 #define HIPC_VGPR_FROM_SGPR(dst, src) asm volatile("v_mov_b32 %0, %1" : "=v"(dst) : "s"(src))   // a uniform value kept in a vector register
+#define HIPC_ARG_NOW(v) asm volatile("" ::"s"(v))                                                // the kernel argument is read here
 #else
+#define HIPC_ARG_NOW(v) ((void)0)
 #define HIPC_PIN_VGPR(v) ((void)0)
 #define HIPC_VGPR_FROM_SGPR(dst, src) ((dst) = (src))
 #endif
@@ -373,31 +376,43 @@ __host__ __device__ inline void pf_consumers_of(int h, int H, int b, int *first,
     *first = (b & 7) + 8 * (h >> 3);
     *step = 8 * ((H + 7) >> 3);
 }
+// The first 120 bytes -- two lines of the scalar cache -- hold everything a workgroup of the product itself reads, and
+// the kernel reads them in one batch at its entry: the scalar cache starts every launch empty, every line is a trip to
+// memory of its own, and an argument read where it is first used puts that trip into the middle of the kernel. The
+// operands of the prologues share their bytes (a launch has one prologue); the read-ahead description behind them is read
+// by the helper rows only.
 struct LeanArgs {
     const uint4 *Wq;
     const float *Sc;
     const uint8_t *Zb;
+    union {
+        float *Y;        // EPI 0: [slices][N] partial rows (the row itself when slices == 1)
+        uint4 *h_split;  // EPI 1: gelu_tanh(gate) * up of the interleaved (gate, up) tile pairs, in operand order
+    };
     int K, N, n_tiles, n_cg;
     int WK, KT, WN, slices;      // wavefronts along k, k tiles per wavefront (<= 4), column tiles per workgroup, k slices (gridDim.y)
     uint32_t nib_mask, magic;    // 0x000f000f and 0x43004300 (bf16 128.0 in both halves)
-    const float *A;              // PRO 0: the row
-    // PRO 2: row = rmsnorm(x', w_in), x' = x + rmsnorm(sum of y_slices rows of yparts, w_post) (x' = x when yparts is null);
-    //        workgroup (0, 0) also writes x' to x_out
-    const float *x, *yparts, *w_post, *w_in;
-    float *x_out;
-    int y_slices;
-    float eps;
-    // PRO 3: the attention output joined from the flash-decoding partials (see GemvPrologue mode 3)
-    const float *part_o, *part_ml;
-    const int *pos;
-    int lg_group, lg_hd, n_kv, window;   // log2 of the query heads per kv head and of head_dim (both powers of two), kv heads
-    // PRO 4: the row in operand order
-    const uint4 *a_split;
-    float *Y;                    // EPI 0: [slices][N] partial rows (the row itself when slices == 1)
-    // EPI 1: gelu_tanh(gate) * up of the interleaved (gate, up) tile pairs, in operand order
-    uint4 *h_split;
+    union {
+        // PRO 2: row = rmsnorm(x', w_in), x' = x + rmsnorm(sum of y_slices rows of yparts, w_post) (x' = x when yparts is null);
+        //        workgroup (0, 0) also writes x' to x_out
+        struct {
+            const float *x, *yparts, *w_post, *w_in;
+            float *x_out;
+            int y_slices;
+            float eps;
+        };
+        // PRO 3: the attention output joined from the flash-decoding partials (see GemvPrologue mode 3)
+        struct {
+            const float *part_o, *part_ml;
+            const int *pos;
+            int lg_group, lg_hd, n_kv, window;   // log2 of the query heads per kv head and of head_dim (both powers of two), kv heads
+        };
+        const float *A;          // PRO 0: the row
+        const uint4 *a_split;    // PRO 4: the row in operand order
+    };
     PrefetchArgs pf;             // helper rows behind the `slices` rows of the grid
 };
+static_assert(offsetof(LeanArgs, pf) == 120, "the arguments of the product fill two 64-byte lines");
 struct LeanPlan {
     int WK, KT, WN, slices;
 };

@@ -211,7 +211,7 @@ void sweep(const Shape &s, int threads) {
     // the output projection's own rows: its k slices, as hipc_decoder_create cuts them (one head per slice, at most 8)
     const int n_cg_o = (s.nq * s.hd + 127) / 128;
     int o_tiles = std::max(1, s.hd / 128);
-    while ((n_cg_o + o_tiles - 1) / o_tiles > 8 && o_tiles < 4) o_tiles *= 2;
+    while ((n_cg_o + o_tiles - 1) / o_tiles > 4 && o_tiles < 4) o_tiles *= 2;
     const unsigned o_slices = (unsigned)((n_cg_o + o_tiles - 1) / o_tiles);
     for (int w : windows_of(s)) {
         std::vector<std::thread> pool;
