@@ -403,6 +403,86 @@ def bench_decoder(pkg, ctx, steps, warmup, context=2048):
     return out
 
 
+LEAN_PHASES = {0: "first instruction (arguments read)", 8: "helper rows branched off", 9: "prologue loads issued", 1: "weight loads issued",
+               2: "prologue operands arrived", 3: "row in LDS (norm or join done)", 4: "operands read from LDS",
+               5: "products and block folds done (weights arrived)", 6: "sum over wavefronts in LDS", 7: "result stored"}
+ATTN_PHASES = {0: "first instruction (arguments read)", 1: "position arrived", 2: "cache loads issued", 3: "own rows normed and rotated",
+               4: "workgroup barrier", 5: "query operand read", 6: "first pass: scores (keys arrived)", 7: "first pass: softmax weights in LDS",
+               8: "first pass: value product", 9: "all passes done", 10: "partials stored"}
+
+
+def bench_phases(pkg, ctx, context=2048):
+    """Where the time of a decode step's launches goes: the library built by `make stamps` (load it with
+    HIPC_LIBRARY=libhipcompute_stamps.so) records the device clock (10 ns ticks) at fixed points of the one-row kernels
+    and of the attention kernel; this reads the stamps the LAST layer's launches left after a replayed step and
+    reports, per launch, the median / 90th percentile / maximum over its wavefronts of the time since the launch's
+    first wavefront started, and the gaps between the launches."""
+    import ctypes
+    lib = pkg.runtime.load_library()
+    if not hasattr(lib, "hipc_debug_lean_stamps"):
+        raise RuntimeError("this library records no phase stamps: make -C onnx-vulkan-rs_amd/csrc stamps, then run with "
+                           "HIPC_LIBRARY=libhipcompute_stamps.so")
+    D = pkg.decoder
+    cfg = dict(D.GEMMA3_1B)
+    dec = D.Decoder(ctx, cfg, context + 64)
+    dec.load(D.build_weights(cfg, seed=9))
+    rng = np.random.default_rng(1)
+    filler = (rng.standard_normal((cfg["n_kv_heads"], context, cfg["head_dim"])) * 0.5).astype(np.float16)
+    for li in range(cfg["n_layers"]):
+        dec.fill_cache(li, filler, filler)
+    dec.reset(1234, context - 1)
+    dec.step()
+    ctx.flush()
+    ctx.capture_begin()
+    dec.step()
+    g = ctx.capture_end()
+    for _ in range(20):
+        ctx.graph_launch(g)
+    ctx.flush()
+    lean = np.zeros(5 * 1024 * 8 * 12, dtype=np.uint64)
+    attn = np.zeros(64 * 4 * 12, dtype=np.uint64)
+    for fn, buf in ((lib.hipc_debug_lean_stamps, lean), (lib.hipc_debug_attn_stamps, attn)):
+        fn.restype, fn.argtypes = ctypes.c_int, [ctypes.c_void_p, ctypes.c_size_t]
+        if fn(buf.ctypes.data_as(ctypes.c_void_p), buf.nbytes) != 0:
+            raise RuntimeError("reading the stamps failed")
+    lean = lean.reshape(5, 1024, 8, 12).astype(np.int64)
+    attn = attn.reshape(1, 64, 4, 12).astype(np.int64)
+    launches = [("q|k|v (norm prologue)", lean[2], LEAN_PHASES, 5), ("attention", attn[0], ATTN_PHASES, 9),
+                ("o (attention join prologue)", lean[3], LEAN_PHASES, 5), ("gate|up (norm prologue, gated GELU)", lean[1], LEAN_PHASES, 5),
+                ("down (row in operand order)", lean[4], LEAN_PHASES, 5)]
+    out, prev_end = {}, None
+    for name, st, phases, work_phase in launches:
+        begun = st[:, :, 0] > 0
+        start = int(st[:, :, 0][begun].min())
+        # wavefronts of the product itself: they reached `work_phase` in this replay (stamps of helper rows, and of
+        # workgroups that had no positions, are older or absent)
+        main = begun & (st[:, :, work_phase] >= start)
+        rec = {"wavefronts": int(main.sum()), "phases_ns": {}}
+        end = start
+        for ph, label in phases.items():
+            v = st[:, :, ph][main]
+            v = v[v >= start]
+            if v.size == 0:
+                continue
+            d = (v - start) * 10
+            rec["phases_ns"][label] = dict(median=int(np.median(d)), p90=int(np.percentile(d, 90)), max=int(d.max()))
+            end = max(end, int(v.max()))
+        helpers = begun & ~main & (st[:, :, 7] >= start) if phases is LEAN_PHASES else None
+        if helpers is not None and helpers.any():
+            h0, h7 = (st[:, :, 0][helpers] - start) * 10, (st[:, :, 7][helpers] - start) * 10
+            rec["helper_rows_ns"] = dict(wavefronts=int(helpers.sum()), start_median=int(np.median(h0)), end_median=int(np.median(h7)), end_max=int(h7.max()))
+            end = max(end, int(st[:, :, 7][helpers].max()))
+        rec["duration_ns"] = (end - start) * 10
+        if prev_end is not None:
+            rec["gap_from_previous_launch_ns"] = (start - prev_end) * 10
+        prev_end = end
+        out[name] = rec
+    ctx.graph_destroy(g)
+    dec.destroy()
+    ctx.flush()
+    return out
+
+
 F16_PEAK_TFLOPS = 2500.0    # MI355X dense f16 MFMA, published
 
 
@@ -492,7 +572,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma list of sections to run (decode, floor, lm_head, gemv, int8, conv, prefill, "
-                    "decoder, cpu; copy = counter calibration, only on request); default all. Used to profile "
+                    "decoder, cpu; copy = counter calibration and phases = time stamps inside the decode step's kernels, only on request); default all. Used to profile "
                     "one kernel at a time.")
     ap.add_argument("--light", action="store_true", help="a third of the timing samples per figure (for runs under rocprofv3)")
     args = ap.parse_args()
@@ -546,6 +626,14 @@ def main():
     if want("decoder"):
         extras["gemma3_1b_int4_decode"] = bench_decoder(pkg, ctx, max(args.steps, 20), args.warmup)
         log("[bench] decoder:", json.dumps(extras["gemma3_1b_int4_decode"]))
+    if "phases" in only:
+        extras["decode_step_phases_last_layer"] = bench_phases(pkg, ctx)
+        for name, rec in extras["decode_step_phases_last_layer"].items():
+            log(f"[bench] {name}: {rec['wavefronts']} wavefronts, {rec['duration_ns']} ns" +
+                (f", {rec['gap_from_previous_launch_ns']} ns after the launch before it ended" if "gap_from_previous_launch_ns" in rec else "") +
+                (f"; helper rows {json.dumps(rec['helper_rows_ns'])}" if "helper_rows_ns" in rec else ""))
+            for label, v in rec["phases_ns"].items():
+                log(f"[bench]     {label:52s} median {v['median']:6d}  p90 {v['p90']:6d}  max {v['max']:6d} ns")
     if "copy" in only:
         extras["copy_256MiB"] = bench_copy(ctx)
         log("[bench] copy:", json.dumps(extras["copy_256MiB"]))

@@ -58,6 +58,10 @@ dec_embed_kernel(const DecState *st, const uint8_t *__restrict__ q, const float 
                  const float *__restrict__ w, float eps, float *__restrict__ x, float *__restrict__ xn, int hd, float theta,
                  float theta2, float *__restrict__ rope) {
     __shared__ float red[4];
+    // (arguments in one batch at entry: see dec_attn_chunks_kernel)
+    HIPC_ARG_NOW(st); HIPC_ARG_NOW(q); HIPC_ARG_NOW(scales); HIPC_ARG_NOW(zp); HIPC_ARG_NOW(hidden); HIPC_ARG_NOW(bs); HIPC_ARG_NOW(n_blocks);
+    HIPC_ARG_NOW(embed_scale); HIPC_ARG_NOW(w); HIPC_ARG_NOW(eps); HIPC_ARG_NOW(x); HIPC_ARG_NOW(xn); HIPC_ARG_NOW(hd); HIPC_ARG_NOW(theta);
+    HIPC_ARG_NOW(theta2); HIPC_ARG_NOW(rope);
     for (int j = threadIdx.x; j < hd / 2; j += 256) {
         const float ang = (float)st->pos * powf(theta, -2.f * (float)j / (float)hd);
         rope[j] = cosf(ang), rope[hd / 2 + j] = sinf(ang);
@@ -89,6 +93,8 @@ __global__ void __launch_bounds__(256)
 dec_norm_residual_kernel(const float *__restrict__ y, int y_slices, const float *__restrict__ w_post, const float *__restrict__ w_next,
                          int hidden, float eps, const float *__restrict__ x_in, float *__restrict__ x, float *__restrict__ xn) {
     __shared__ float red[4];
+    HIPC_ARG_NOW(y); HIPC_ARG_NOW(y_slices); HIPC_ARG_NOW(w_post); HIPC_ARG_NOW(w_next); HIPC_ARG_NOW(hidden); HIPC_ARG_NOW(eps);
+    HIPC_ARG_NOW(x_in); HIPC_ARG_NOW(x); HIPC_ARG_NOW(xn);
     float yv[kNormPer], xv[kNormPer], wp[kNormPer], wn[kNormPer];
 #pragma unroll
     for (int e = 0; e < kNormPer; e++) {
@@ -343,6 +349,20 @@ dec_attn_merge_kernel(const DecState *st, const float *__restrict__ part_ml, con
 typedef _Float16 dh16x8 __attribute__((ext_vector_type(8)));
 typedef float df32x4 __attribute__((ext_vector_type(4)));
 
+// phase time stamps of the attention launch (library built with `make stamps` only; see gemv_lean.hip):
+// attn_stamps[split][wavefront][phase] of kv head 0, read out by hipc_debug_attn_stamps
+#ifdef HIPC_PHASE_STAMPS
+__device__ unsigned long long attn_stamps[64 * 4 * 12];
+#define ATTN_STAMP(ph)                                                                                          \
+    do {                                                                                                        \
+        const unsigned long long t_ = (unsigned long long)wall_clock64();                                       \
+        if ((threadIdx.x & 63) == 0 && blockIdx.y == 0) attn_stamps[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 12 + (ph)] = t_; \
+    } while (0)
+#define ATTN_STAMP_AFTER(v, ph) do { asm volatile("" ::"v"(v)); ATTN_STAMP(ph); } while (0)
+#else
+#define ATTN_STAMP(ph)
+#define ATTN_STAMP_AFTER(v, ph)
+#endif
 template <int HD, int G>
 __global__ void __launch_bounds__(256)
 dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const float *__restrict__ q_norm,
@@ -366,11 +386,17 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
     __shared__ __attribute__((aligned(16))) float vn[HD];             // the step's value
     __shared__ float sown[2 * HL];                                      // the step's own scores
 
-    if ((int)blockIdx.y >= n_kv) {   // a helper row: read ahead for the next launch, nothing else
+    // every argument is read here, in one batch (left to the compiler, each is read next to its first use: a trip to
+    // memory of its own in the middle of the kernel, since the scalar cache starts every launch empty)
+    HIPC_ARG_NOW(st); HIPC_ARG_NOW(qkv); HIPC_ARG_NOW(q_norm); HIPC_ARG_NOW(k_norm); HIPC_ARG_NOW(n_q); HIPC_ARG_NOW(n_kv);
+    HIPC_ARG_NOW(eps); HIPC_ARG_NOW(rope); HIPC_ARG_NOW(max_seq); HIPC_ARG_NOW(v_stride); HIPC_ARG_NOW(scale); HIPC_ARG_NOW(window);
+    HIPC_ARG_NOW(k_cache); HIPC_ARG_NOW(v_cache); HIPC_ARG_NOW(part_ml); HIPC_ARG_NOW(part_o);
+    if (__builtin_expect((int)blockIdx.y >= n_kv, 0)) {   // a helper row: read ahead for the next launch, nothing else
         prefetch_for_next(pf, ((int)blockIdx.y - n_kv) * (int)gridDim.x + (int)blockIdx.x, pf.rows * (int)gridDim.x,
                           (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x, pf.sink);
         return;
     }
+    ATTN_STAMP(0);
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -430,8 +456,10 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
             vreg[b] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r_v, (int)v_v, (int)s_v, 0));
         }
     };
+    ATTN_STAMP(1);
     load_k(t_begin);
     load_v(t_begin);
+    ATTN_STAMP(2);
 
     // 2. per-head RMS norm and half-split rotary embedding (pairs d, d + HD/2), one wavefront per
     //    row and no workgroup barrier: with HD = 128 or 256 both members of a pair sit in one lane
@@ -477,7 +505,9 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
         }
     }
     if (is_last && tid < HD) vn[tid] = __half2float(__float2half(pv_own));
+    ATTN_STAMP(3);
     __syncthreads();
+    ATTN_STAMP(4);
     if (is_last) {
         if (tid < HD) {
             k_cache[((size_t)kvh * max_seq + pos) * HD + tid] = __float2half(kn[tid]);
@@ -510,6 +540,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 #pragma unroll
     for (int b = 0; b < NB; b++) o[b] = df32x4{0.f, 0.f, 0.f, 0.f};
 
+    ATTN_STAMP_AFTER(aq[KS - 1], 5);
     for (int t0 = t_begin; t0 < t_end; t0 += kAttnPass) {   // (a workgroup without positions: not once)
         const bool more = t0 + kAttnPass < t_end;
         // 3a. this wavefront's half of the scores of its 16 positions, all heads
@@ -517,6 +548,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
 #pragma unroll
         for (int u = 0; u < KS; u++) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(aq[u], __builtin_bit_cast(dh16x8, kreg[u]), acc, 0, 0, 0);
         sp[wave][lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        if (t0 == t_begin) ATTN_STAMP_AFTER(acc[0], 6);
         if (more) load_k(t0 + kAttnPass);
         __syncthreads();
         // 3b. all 32 positions' scores (block b: wavefronts b and b + 2), the pass's max and sum
@@ -553,6 +585,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
         uint4 praw = make_uint4(0, 0, 0, 0);
         if (i16 < R) praw = *reinterpret_cast<const uint4 *>(pa[wave] + i16 * PS + g4 * 8);
         const dh16x8 ap = __builtin_bit_cast(dh16x8, praw);
+        if (t0 == t_begin) ATTN_STAMP_AFTER(praw.x, 7);
         // 3c. unnormalised outputs of this wavefront's channels: a lane's result registers are rows
         //     4 g4 .. + 3, the heads whose factors it holds
 #pragma unroll
@@ -560,11 +593,13 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
             o[b][0] *= f0, o[b][1] *= f0, o[b][2] *= f1, o[b][3] *= f1;
             o[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ap, __builtin_bit_cast(dh16x8, vreg[b]), o[b], 0, 0, 0);
         }
+        if (t0 == t_begin) ATTN_STAMP_AFTER(o[NB - 1][0], 8);
         if (more) {
             load_v(t0 + kAttnPass);
             __syncthreads();   // the next pass's scores must not overtake this pass's reads of sp
         }
     }
+    ATTN_STAMP_AFTER(o[0][0], 9);
 
     // 4. the step's own position joins in the workgroup that owns it; then the partial goes out
     float e0 = 1.f, e1 = 1.f, eo0 = 0.f, eo1 = 0.f;
@@ -591,6 +626,7 @@ dec_attn_chunks_kernel(const DecState *st, const float *__restrict__ qkv, const 
             if (2 * g4 + 1 < G) ml[4 * g4 + 2] = m_run1, ml[4 * g4 + 3] = l_run1;
         }
     }
+    ATTN_STAMP(10);
 }
 
 
@@ -636,6 +672,7 @@ dec_argmax_partial_kernel(const float *__restrict__ logits, int n, float *__rest
 __global__ void __launch_bounds__(64)
 dec_argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int nparts, DecState *st,
                         int32_t *__restrict__ history, int max_hist, int vocab) {
+    HIPC_ARG_NOW(pv); HIPC_ARG_NOW(pi); HIPC_ARG_NOW(nparts); HIPC_ARG_NOW(st); HIPC_ARG_NOW(history); HIPC_ARG_NOW(max_hist); HIPC_ARG_NOW(vocab);
     float best = -3.4e38f;
     int bi = 0x7fffffff;
     for (int i = threadIdx.x; i < nparts; i += 64) {
@@ -667,6 +704,12 @@ __global__ void dec_set_state_kernel(DecState *st, int token, int pos) {
 }  // namespace hipc
 
 using namespace hipc;
+
+#ifdef HIPC_PHASE_STAMPS
+extern "C" int hipc_debug_attn_stamps(void *dst, size_t bytes) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(hipc::attn_stamps), bytes, 0, hipMemcpyDeviceToHost);
+}
+#endif
 
 struct DecLayer {
     hipc_nbits_weight *qkv = nullptr, *o = nullptr, *gate_up = nullptr, *down = nullptr;
@@ -1006,7 +1049,7 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         // gemma3-1b shape at context 2048, those three save 0.2-0.6 us per launch, the o launch (72 workgroups of
         // its own) is lengthened by helpers that read gate|up's 10 MB, and the q|k|v launch hides its weights'
         // arrival behind its norm prologue anyway.
-        const int ahead_mask = !kReadAheadVerified ? 0 : ctx->tune.dec_prefetch < 0 ? 11 : ctx->tune.dec_prefetch;
+        const int ahead_mask = !kReadAheadVerified ? 0 : ctx->tune.dec_prefetch < 0 ? 9 : ctx->tune.dec_prefetch;
         // helper rows of a producer whose grid is gx wide: about one helper workgroup per consumer workgroup (a helper
         // that serves several consumers lasts longer than the launch it rides on), at least 192 and at most 512 in all
         auto rows_for = [](int64_t gx, int64_t consumers) {
@@ -1016,9 +1059,9 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         for (int li = 0; li < c.n_layers && d->lean; li++) {
             DecLayer &l = d->layers[li];
             LeanPlan pl_qkv, pl_o, pl_gu, pl_down, pl_next;
-            HIPC_REQUIRE(ctx, lean_plan(ctx, l.qkv, 1, 1, &pl_qkv), "decoder: no launch plan for the qkv projection");
+            HIPC_REQUIRE(ctx, lean_plan(ctx, l.qkv, 1, 1, &pl_qkv, 8), "decoder: no launch plan for the qkv projection");
             pl_o = LeanPlan{1, (int)ceil_div(l.o->n_cg, d->o_slices), 4, d->o_slices};   // four wavefronts, each all k tiles of the slice: no sum over wavefronts
-            HIPC_REQUIRE(ctx, lean_plan(ctx, l.gate_up, 1, 2, &pl_gu), "decoder: no launch plan for the gate | up projection");
+            HIPC_REQUIRE(ctx, lean_plan(ctx, l.gate_up, 1, 2, &pl_gu, 8), "decoder: no launch plan for the gate | up projection");
             HIPC_REQUIRE(ctx, lean_plan(ctx, l.down, d->down_slices, 1, &pl_down, 8), "decoder: no launch plan for the down projection");
             auto gx_of = [](const hipc_nbits_weight *w, const LeanPlan &p) { return ceil_div(w->n_tiles, p.WN); };
             // qkv: row = rmsnorm(x', w_input), x' = x + rmsnorm(sum of the down projection's partial rows, w_post_ffn of the layer before)
@@ -1072,7 +1115,7 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 LeanArgs a{};
                 a.a_split = d->h_split;
                 a.Y = d->yd;
-                if ((ahead_mask & 16) && li + 1 < c.n_layers && lean_plan(ctx, d->layers[li + 1].qkv, 1, 1, &pl_next))
+                if ((ahead_mask & 16) && li + 1 < c.n_layers && lean_plan(ctx, d->layers[li + 1].qkv, 1, 1, &pl_next, 8))
                     a.pf = lean_prefetch_of(d->layers[li + 1].qkv, pl_next, rows_for(gx_of(l.down, pl_down), gx_of(d->layers[li + 1].qkv, pl_next)), d->pf_sink);
                 if ((rc = lean_gemv(ctx, l.down, pl_down, a, 4, 0, terms)) != HIPC_OK) return rc;
             }

@@ -130,13 +130,18 @@ __device__ __forceinline__ void lean_split1(float v, uint16_t (&t)[3]) {
     }
 }
 
-#ifdef HIPC_LEAN_STAMPS
+// Phase time stamps (only in the library built with `make stamps`, which defines HIPC_PHASE_STAMPS): wavefront w of
+// workgroup g of the last launch of an instance leaves the 100 MHz device clock at up to twelve points of the kernel in
+// lean_stamps[slot][g][w][phase] (slot = PRO, or 1 for the gated epilogue); LEAN_STAMP_AFTER first waits for the value it
+// names. hipc_debug_lean_stamps copies the table out. This is how the kernel's time was found to go into instruction
+// issue, argument fetches and the first trip to memory rather than into moving the weights.
+#ifdef HIPC_PHASE_STAMPS
 __device__ unsigned long long lean_stamps[5 * 1024 * 8 * 12];
 #define LEAN_STAMP(ph)                                                                                       \
     do {                                                                                                     \
         const unsigned long long t_ = (unsigned long long)wall_clock64();                                    \
         if ((threadIdx.x & 63) == 0 && st_wg < 1024 && (threadIdx.x >> 6) < 8)                               \
-            lean_stamps[((st_slot * 1024 + st_wg) * 8 + (threadIdx.x >> 6)) * 12 + (ph)] = t_;                \
+            lean_stamps[((st_slot * 1024 + st_wg) * 8 + (threadIdx.x >> 6)) * 12 + (ph)] = t_;               \
     } while (0)
 #define LEAN_STAMP_AFTER(v, ph) do { asm volatile("" ::"v"(v)); LEAN_STAMP(ph); } while (0)
 #else
@@ -159,7 +164,7 @@ template <int SG, int NT, int PRO, int EPI, int KT>
 __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const LeanArgs p) {
     extern __shared__ uint4 lean_smem[];
     constexpr int CPG = 4 / SG;  // 32-k chunks per scale group
-#ifdef HIPC_LEAN_STAMPS
+#ifdef HIPC_PHASE_STAMPS
     const int st_slot = PRO + (EPI ? -1 : 0), st_wg = (int)(blockIdx.y * gridDim.x + blockIdx.x);
 #endif
     // Every argument this instance uses is read here, in one batch: left to itself the compiler reads an argument
@@ -193,10 +198,10 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
     // PRO 2: the row's operands are asked for before anything else is worked out. They come from the launch
     // before this one, i.e. from memory and not from this XCD's L2, and the instructions between here and their
     // first use (index arithmetic, descriptors, the weight loads) take about as long to arrive as they do.
-    // Every wavefront asks; a thread past the end of the row reads zeros and causes no traffic, and so does a
-    // partial row that does not exist (an empty descriptor).
+    // The wavefronts that hold items ask (the others would only spend issue slots); a thread past the end of the
+    // row reads zeros and causes no traffic, and so does a partial row that does not exist (an empty descriptor).
     float x8[8], w8[8], wp8[8], part[kLeanMaxSlices][8];
-    if (PRO == 2) {
+    if (PRO == 2 && wave < ((min(p.WK * KT, p.n_cg) * 16 + 63) >> 6)) {
         const uint32_t row_bytes = (uint32_t)p.K * 4u, voff = (uint32_t)tid * 32u;
         const bool has_y = p.yparts != nullptr;
         const int ys = has_y ? p.y_slices : 0;
@@ -532,7 +537,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
 
 }  // namespace hipc
 
-#ifdef HIPC_LEAN_STAMPS
+#ifdef HIPC_PHASE_STAMPS
 extern "C" int hipc_debug_lean_stamps(void *dst, size_t bytes) {
     return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(hipc::lean_stamps), bytes, 0, hipMemcpyDeviceToHost);
 }
@@ -574,8 +579,8 @@ bool hipc::lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int 
     // slice is short (a workgroup of three wavefronts then holds the row and all of them prepare it)
     const int max_wk = max_waves / WN;
     int KT = (per_slice + max_wk - 1) / max_wk;
-    if (per_slice <= 12 && per_slice >= 3) KT = std::max(KT, 3);
     if (ctx->tune.gemv_t >= 1 && ctx->tune.gemv_t <= 4) KT = std::max(KT, ctx->tune.gemv_t);
+    else if (per_slice <= 12 && per_slice >= 3) KT = std::max(KT, 3);
     if (KT > 4) return false;
     LeanPlan pl{};
     pl.KT = KT, pl.WK = (per_slice + KT - 1) / KT, pl.WN = WN, pl.slices = slices;

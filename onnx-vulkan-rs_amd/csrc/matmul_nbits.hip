@@ -260,6 +260,11 @@ __device__ __forceinline__ uint32_t bf16_rne(float v) {  // bits of the nearest 
 template <int T, int NR, int SG, int MC, int NT, int PRO>
 __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel(const GemvArgs p) {
     extern __shared__ uint4 smem[];
+    // the arguments every instance uses are read here, in one batch (left to the compiler, each is read next to its first
+    // use: a trip to memory of its own in the middle of the kernel, since the scalar cache starts every launch empty)
+    HIPC_ARG_NOW(p.A); HIPC_ARG_NOW(p.Wq); HIPC_ARG_NOW(p.Sc); HIPC_ARG_NOW(p.Zb); HIPC_ARG_NOW(p.Y); HIPC_ARG_NOW(p.Ypart);
+    HIPC_ARG_NOW(p.M); HIPC_ARG_NOW(p.K); HIPC_ARG_NOW(p.N); HIPC_ARG_NOW(p.n_tiles); HIPC_ARG_NOW(p.n_cg); HIPC_ARG_NOW(p.WK); HIPC_ARG_NOW(p.WN);
+    HIPC_ARG_NOW(p.slice_tiles); HIPC_ARG_NOW(p.ksplit); HIPC_ARG_NOW(p.a_f16); HIPC_ARG_NOW(p.a_vec); HIPC_ARG_NOW(p.nib_mask); HIPC_ARG_NOW(p.magic);
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int M = MC > 0 ? MC : p.M;
@@ -851,7 +856,10 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
     if (M == 1 && a_dtype == HIPC_F32 && !(pro && pro->mode) && aligned(A, 16) && aligned(Y, 4) && w->n_tiles < 2048 &&
         ctx->tune.gemv_lean != 0) {
         LeanPlan pl;
-        if (lean_plan(ctx, w, 1, 1, &pl)) {
+        // several column tiles per workgroup once that still leaves a workgroup for most CUs: the row is then prepared
+        // (read, split into terms, written to LDS) by a half or a quarter as many workgroups (1152 -> 13824: 5.4 -> 5.0 us)
+        const int WN = w->n_tiles >= 768 ? 4 : w->n_tiles >= 384 ? 2 : 1;
+        if (lean_plan(ctx, w, 1, WN, &pl)) {
             LeanArgs la{};
             la.A = static_cast<const float *>(A), la.Y = static_cast<float *>(Y);
             return lean_gemv(ctx, w, pl, la, 0, 0, NT);

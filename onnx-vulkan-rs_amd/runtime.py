@@ -43,7 +43,9 @@ class ConvGeom(C.Structure):
 
 
 def library_path() -> str:
-    return os.path.join(_HERE, "libhipcompute.so")
+    """The library beside this package; HIPC_LIBRARY names another build of the same sources there (the one with phase
+    time stamps, libhipcompute_stamps.so, for ``bench.py --only phases``)."""
+    return os.path.join(_HERE, os.environ.get("HIPC_LIBRARY", "libhipcompute.so"))
 
 
 class DecoderConfig(C.Structure):
