@@ -48,41 +48,100 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
     return s;
 }
 
-// x = embed_scale * dequant(table[token]); xn = rmsnorm(x, w). One workgroup. It also leaves the
+// x = embed_scale * dequant(table[token]); xn = rmsnorm(x, w). One workgroup of 256. It also leaves the
 // step's rotary table behind: rope[j] = cos(pos * theta^(-2j/hd)), rope[hd/2 + j] = the sine, which
 // every layer's attention reads instead of evaluating the functions again; a second table for the
-// layers that rotate with another base follows at rope[hd...] when theta2 > 0.
-__global__ void __launch_bounds__(256)
-dec_embed_kernel(const DecState *st, const uint8_t *__restrict__ q, const float *__restrict__ scales,
-                 const uint8_t *__restrict__ zp, int hidden, int bs, int n_blocks, float embed_scale,
-                 const float *__restrict__ w, float eps, float *__restrict__ x, float *__restrict__ xn, int hd, float theta,
-                 float theta2, float *__restrict__ rope) {
-    __shared__ float red[4];
-    // (arguments in one batch at entry: see dec_attn_chunks_kernel)
-    HIPC_ARG_NOW(st); HIPC_ARG_NOW(q); HIPC_ARG_NOW(scales); HIPC_ARG_NOW(zp); HIPC_ARG_NOW(hidden); HIPC_ARG_NOW(bs); HIPC_ARG_NOW(n_blocks);
-    HIPC_ARG_NOW(embed_scale); HIPC_ARG_NOW(w); HIPC_ARG_NOW(eps); HIPC_ARG_NOW(x); HIPC_ARG_NOW(xn); HIPC_ARG_NOW(hd); HIPC_ARG_NOW(theta);
-    HIPC_ARG_NOW(theta2); HIPC_ARG_NOW(rope);
-    for (int j = threadIdx.x; j < hd / 2; j += 256) {
-        const float ang = (float)st->pos * powf(theta, -2.f * (float)j / (float)hd);
-        rope[j] = cosf(ang), rope[hd / 2 + j] = sinf(ang);
-        if (theta2 > 0.f) {
-            const float ang2 = (float)st->pos * powf(theta2, -2.f * (float)j / (float)hd);
-            rope[hd + j] = cosf(ang2), rope[hd + hd / 2 + j] = sinf(ang2);
+// layers that rotate with another base follows at rope[hd...] when theta2 > 0. The table is the work of
+// the upper two wavefronts (powers and range reductions: hundreds of instructions), the row of the lower two.
+struct EmbedArgs {
+    const uint8_t *q;
+    const float *scales;
+    const uint8_t *zp;
+    const float *w;   // the first layer's input norm
+    float *x, *xn, *rope;
+    int hidden, bs, n_blocks, hd;
+    float embed_scale, eps, theta, theta2;
+};
+// the rotary table of position `pos`: the work of threads 128 .. 255
+__device__ __forceinline__ void dec_rope_table(const EmbedArgs &e, int pos) {
+    if (threadIdx.x >= 128) {
+        for (int j = threadIdx.x - 128; j < e.hd / 2; j += 128) {
+            const float ang = (float)pos * powf(e.theta, -2.f * (float)j / (float)e.hd);
+            e.rope[j] = cosf(ang), e.rope[e.hd / 2 + j] = sinf(ang);
+            if (e.theta2 > 0.f) {
+                const float ang2 = (float)pos * powf(e.theta2, -2.f * (float)j / (float)e.hd);
+                e.rope[e.hd + j] = cosf(ang2), e.rope[e.hd + e.hd / 2 + j] = sinf(ang2);
+            }
         }
     }
-    const size_t row = (size_t)st->token;
-    const size_t row_bytes = (size_t)n_blocks * bs / 2, zp_row = (n_blocks + 1) / 2;
-    float sq = 0.f;
-    for (int c = threadIdx.x; c < hidden; c += 256) {
-        const int b = c / bs;
-        const int nib = (q[row * row_bytes + c / 2] >> (4 * (c & 1))) & 15;
-        const int z = zp ? (zp[row * zp_row + b / 2] >> (4 * (b & 1))) & 15 : 8;
-        const float v = ((float)nib - (float)z) * scales[row * n_blocks + b] * embed_scale;
-        x[c] = v;
-        sq += v * v;
+}
+// ROPE: the table is worked out here, between asking for the row and using it (else the caller has done it)
+template <bool ROPE>
+__device__ __forceinline__ void dec_embed_token(const EmbedArgs &e, int token, int pos, float *red) {
+    const size_t row = (size_t)token;
+    const size_t row_bytes = (size_t)e.n_blocks * e.bs / 2, zp_row = (e.n_blocks + 1) / 2;
+    // The row comes from a table far larger than any cache: every load of it is a trip to memory, so all of them are
+    // asked for at once -- a thread takes eight consecutive elements (one word of nibbles, one scale, one zero-point
+    // byte) of up to two places of the row -- and the rotary table is worked out while they are on their way.
+    constexpr int kPlaces = 2;
+    const bool wide = e.hidden % 8 == 0 && e.bs % 8 == 0 && e.hidden <= 256 * 8 * kPlaces;
+    uint32_t word[kPlaces];
+    float sc[kPlaces], v[kPlaces][8];
+    float4 w_lo[kPlaces], w_hi[kPlaces];
+    int zq[kPlaces];
+    if (wide) {
+#pragma unroll
+        for (int u = 0; u < kPlaces; u++) {
+            const int k0 = min(((int)threadIdx.x + 256 * u) * 8, e.hidden - 8), b = k0 / e.bs;
+            word[u] = *reinterpret_cast<const uint32_t *>(e.q + row * row_bytes + k0 / 2);
+            sc[u] = e.scales[row * e.n_blocks + b];
+            zq[u] = e.zp ? (e.zp[row * zp_row + b / 2] >> (4 * (b & 1))) & 15 : 8;
+            w_lo[u] = *reinterpret_cast<const float4 *>(e.w + k0), w_hi[u] = *reinterpret_cast<const float4 *>(e.w + k0 + 4);
+        }
     }
-    const float inv = rsqrtf(block_sum(sq, red) / (float)hidden + eps);
-    for (int c = threadIdx.x; c < hidden; c += 256) xn[c] = x[c] * inv * w[c];
+    if (ROPE) dec_rope_table(e, pos);
+    float sq = 0.f;
+    if (wide) {
+#pragma unroll
+        for (int u = 0; u < kPlaces; u++) {
+            const int k0 = ((int)threadIdx.x + 256 * u) * 8;
+            if (k0 < e.hidden) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    v[u][i] = ((float)((word[u] >> (4 * i)) & 15u) - (float)zq[u]) * sc[u] * e.embed_scale;
+                    sq += v[u][i] * v[u][i];
+                }
+                reinterpret_cast<float4 *>(e.x + k0)[0] = make_float4(v[u][0], v[u][1], v[u][2], v[u][3]);
+                reinterpret_cast<float4 *>(e.x + k0)[1] = make_float4(v[u][4], v[u][5], v[u][6], v[u][7]);
+            }
+        }
+    } else {
+        for (int c = threadIdx.x; c < e.hidden; c += 256) {
+            const int b = c / e.bs;
+            const int nib = (e.q[row * row_bytes + c / 2] >> (4 * (c & 1))) & 15;
+            const int z = e.zp ? (e.zp[row * zp_row + b / 2] >> (4 * (b & 1))) & 15 : 8;
+            const float val = ((float)nib - (float)z) * e.scales[row * e.n_blocks + b] * e.embed_scale;
+            e.x[c] = val;
+            sq += val * val;
+        }
+    }
+    const float inv = rsqrtf(block_sum(sq, red) / (float)e.hidden + e.eps);
+    if (wide) {
+#pragma unroll
+        for (int u = 0; u < kPlaces; u++) {
+            const int k0 = ((int)threadIdx.x + 256 * u) * 8;
+            if (k0 < e.hidden) {
+                reinterpret_cast<float4 *>(e.xn + k0)[0] = make_float4(v[u][0] * inv * w_lo[u].x, v[u][1] * inv * w_lo[u].y, v[u][2] * inv * w_lo[u].z, v[u][3] * inv * w_lo[u].w);
+                reinterpret_cast<float4 *>(e.xn + k0)[1] = make_float4(v[u][4] * inv * w_hi[u].x, v[u][5] * inv * w_hi[u].y, v[u][6] * inv * w_hi[u].z, v[u][7] * inv * w_hi[u].w);
+            }
+        }
+    } else {
+        for (int c = threadIdx.x; c < e.hidden; c += 256) e.xn[c] = e.x[c] * inv * e.w[c];   // (x[c] is this thread's own store)
+    }
+}
+__global__ void __launch_bounds__(256) dec_embed_kernel(const DecState *st, const EmbedArgs e) {
+    __shared__ float red[4];
+    dec_embed_token<true>(e, st->token, st->pos, red);
 }
 
 // x += rmsnorm(y, w_post); xn = rmsnorm(x, w_next). One workgroup of 256; every operand is read once,
@@ -131,7 +190,7 @@ dec_qkv_kernel(const DecState *st, const float *__restrict__ qkv, const float *_
     __shared__ float buf[512];
     const int head = blockIdx.x;
     const int pos = st->pos;
-    if (pos >= max_seq) return;  // the cache is full: the step is a no-op (dec_argmax_final_kernel reports it)
+    if (pos >= max_seq) return;  // the cache is full: the step is a no-op (dec_pick_embed_kernel reports it)
     const float *src = qkv + (size_t)head * hd;
     const bool is_q = head < n_q, is_k = !is_q && head < n_q + n_kv;
     if (!is_q && !is_k) {  // a value head: straight into the cache
@@ -646,10 +705,17 @@ dec_argmax_partial_kernel(const float *__restrict__ logits, int n, float *__rest
     __shared__ int si[4];
     float best = -3.4e38f;
     int bi = 0x7fffffff;
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
-        const float v = logits[i];
+    auto take = [&](float v, int i) {
         if (v > best || (v == best && i < bi)) best = v, bi = i;
+    };
+    // four logits per load (the logits buffer is the library's own allocation: 16-byte aligned); with a vocabulary of
+    // 2^18 that is one load per thread, in flight together with every other thread's
+    const int n4 = n >> 2;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n4; i += gridDim.x * 256) {
+        const float4 v = reinterpret_cast<const float4 *>(logits)[i];
+        take(v.x, 4 * i), take(v.y, 4 * i + 1), take(v.z, 4 * i + 2), take(v.w, 4 * i + 3);
     }
+    for (int i = 4 * n4 + blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) take(logits[i], i);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
         const float ov = __shfl_xor(best, off, 64);
@@ -669,32 +735,45 @@ dec_argmax_partial_kernel(const float *__restrict__ logits, int n, float *__rest
 // The state only ever holds a token inside the vocabulary and a position inside the cache: a
 // candidate outside [0, vocab) (every logit NaN: no comparison succeeds) becomes token 0, and a step
 // taken with the cache full (pos == max_seq) changes nothing and raises the sticky overflow flag.
-__global__ void __launch_bounds__(64)
-dec_argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int nparts, DecState *st,
-                        int32_t *__restrict__ history, int max_hist, int vocab) {
-    HIPC_ARG_NOW(pv); HIPC_ARG_NOW(pi); HIPC_ARG_NOW(nparts); HIPC_ARG_NOW(st); HIPC_ARG_NOW(history); HIPC_ARG_NOW(max_hist); HIPC_ARG_NOW(vocab);
-    float best = -3.4e38f;
-    int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < nparts; i += 64) {
-        if (pv[i] > best || (pv[i] == best && pi[i] < bi)) best = pv[i], bi = pi[i];
-    }
+// The same launch then embeds the chosen token for the next step (x, xn and the rotary table of the new
+// position): a step begins with its q|k|v product, not with a launch of its own for the embedding.
+__global__ void __launch_bounds__(256)
+dec_pick_embed_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int nparts, DecState *st,
+                      int32_t *__restrict__ history, int max_hist, int vocab, const EmbedArgs e) {
+    __shared__ float red[4];
+    __shared__ int next[2];
+    // the upper two wavefronts work out the next position's rotary table (it follows from the position alone) while
+    // the first picks the token
+    const int pos_now = st->pos;
+    dec_rope_table(e, pos_now >= max_hist ? pos_now : pos_now + 1);
+    if (threadIdx.x < 64) {
+        float best = -3.4e38f;
+        int bi = 0x7fffffff;
+        for (int i = threadIdx.x; i < nparts; i += 64) {
+            if (pv[i] > best || (pv[i] == best && pi[i] < bi)) best = pv[i], bi = pi[i];
+        }
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        const float ov = __shfl_xor(best, off, 64);
-        const int oi = __shfl_xor(bi, off, 64);
-        if (ov > best || (ov == best && oi < bi)) best = ov, bi = oi;
-    }
-    if (threadIdx.x == 0) {
-        const int pos = st->pos;
-        if (pos >= max_hist) {
-            st->overflow = 1;
-        } else {
-            if (bi < 0 || bi >= vocab) bi = 0;
-            history[pos] = bi;
-            st->token = bi;
-            st->pos = pos + 1;
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(best, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (ov > best || (ov == best && oi < bi)) best = ov, bi = oi;
+        }
+        if (threadIdx.x == 0) {
+            const int pos = st->pos;
+            int token = st->token, new_pos = pos;
+            if (pos >= max_hist) {
+                st->overflow = 1;
+            } else {
+                if (bi < 0 || bi >= vocab) bi = 0;
+                history[pos] = bi;
+                st->token = token = bi;
+                st->pos = new_pos = pos + 1;
+            }
+            next[0] = token, next[1] = new_pos;
         }
     }
+    __syncthreads();
+    dec_embed_token<false>(e, next[0], next[1], red);
 }
 
 __global__ void dec_set_state_kernel(DecState *st, int token, int pos) {
@@ -744,6 +823,9 @@ struct hipc_decoder {
     uint4 *h_split = nullptr;                // the gated row in operand order (see LeanArgs)
     int nsplit = 0;
     uint32_t *pf_sink = nullptr;   // where a helper workgroup would write (it never does: keeps its loads alive)
+    // x, xn and the rotary table hold the state's token and position (left by the reset or by the step before);
+    // anything that changes what they are made of clears it, and a step that finds it cleared embeds first
+    bool x_ready = false;
     bool one_launch_attn = false;  // head_dim and group size have an instance of dec_attn_chunks_kernel
     std::vector<void *> owned;
 };
@@ -959,6 +1041,7 @@ int hipc_decoder_set_norm(hipc_ctx *ctx, hipc_decoder *d, int layer, int which, 
             if (rc != HIPC_OK) return rc;
         }
         HIPC_TRY(ctx, hipMemcpyAsync(*slot, w, n * 4, hipMemcpyDeviceToDevice, ctx->stream));
+        d->x_ready = false;
         return HIPC_OK;
     });
 }
@@ -980,6 +1063,7 @@ int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *d, const void *B, si
         HIPC_TRY(ctx, hipMemcpyAsync(d->emb_q, B, qb, hipMemcpyDeviceToDevice, ctx->stream));
         HIPC_TRY(ctx, hipMemcpyAsync(d->emb_scales, scales, sb * 4, hipMemcpyDeviceToDevice, ctx->stream));
         if (zp) HIPC_TRY(ctx, hipMemcpyAsync(d->emb_zp, zp, zb, hipMemcpyDeviceToDevice, ctx->stream));
+        d->x_ready = false;
         return HIPC_OK;
     });
 }
@@ -1000,9 +1084,26 @@ int hipc_decoder_set_layer_attention(hipc_ctx *ctx, hipc_decoder *d, int layer, 
         }
         l.window = window > 0 ? window : 0;
         l.rope_table = table;
+        d->x_ready = false;   // the rotary table may need its second half
         return HIPC_OK;
     });
 }
+
+namespace {
+
+bool can_embed(const hipc_decoder *d) { return d->emb_q && d->emb_scales && d->layers[0].norm[HIPC_DEC_NORM_INPUT]; }
+
+EmbedArgs embed_args(const hipc_decoder *d) {
+    const hipc_decoder_config &c = d->cfg;
+    EmbedArgs e{};
+    e.q = d->emb_q, e.scales = d->emb_scales, e.zp = d->emb_zp, e.w = d->layers[0].norm[HIPC_DEC_NORM_INPUT];
+    e.x = d->x, e.xn = d->xn, e.rope = d->rope;
+    e.hidden = c.hidden, e.bs = c.block_size, e.n_blocks = (int)ceil_div(c.hidden, c.block_size), e.hd = c.head_dim;
+    e.embed_scale = c.embed_scale, e.eps = c.rms_eps, e.theta = c.rope_theta, e.theta2 = d->theta2;
+    return e;
+}
+
+}  // namespace
 
 int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *d, int32_t token, int32_t pos) {
     if (!d) return HIPC_ERR_INVALID;
@@ -1010,6 +1111,14 @@ int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *d, int32_t token, int32_t po
         HIPC_REQUIRE(ctx, token >= 0 && token < d->cfg.vocab && pos >= 0 && pos < d->cfg.max_seq, "decoder: bad token %d or position %d", token, pos);
         hipLaunchKernelGGL((dec_set_state_kernel), 1, 64, 0, ctx->stream, d->state, token, pos);
         HIPC_LAUNCHED(ctx);
+        // the step expects the token embedded (x, xn, the position's rotary table): every step leaves that behind for
+        // the next one, the reset does it for the first
+        d->x_ready = false;
+        if (can_embed(d)) {
+            hipLaunchKernelGGL((dec_embed_kernel), 1, 256, 0, ctx->stream, d->state, embed_args(d));
+            HIPC_LAUNCHED(ctx);
+            d->x_ready = !ctx->capturing;   // a recorded launch has not run yet
+        }
         return HIPC_OK;
     });
 }
@@ -1029,15 +1138,14 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
         HIPC_REQUIRE(ctx, complete(d), "decoder: not every weight has been set");
         const hipc_decoder_config &c = d->cfg;
         hipStream_t s = ctx->stream;
-        const int nb = (int)ceil_div(c.hidden, c.block_size);
         const int heads = c.n_q_heads + 2 * c.n_kv_heads;
         const float scale = c.attn_scale > 0.f ? c.attn_scale : 1.f / sqrtf((float)c.head_dim);
         const int terms = 2;
         int rc;
-        hipLaunchKernelGGL((dec_embed_kernel), 1, 256, 0, s, d->state, d->emb_q, d->emb_scales, d->emb_zp, c.hidden, c.block_size, nb, c.embed_scale,
-                                           d->layers[0].norm[HIPC_DEC_NORM_INPUT], c.rms_eps, d->x, d->xn, c.head_dim, c.rope_theta,
-                                           d->theta2, d->rope);
-        HIPC_LAUNCHED(ctx);
+        if (!d->x_ready) {   // nothing has embedded the state's token yet (no reset since the weights changed)
+            hipLaunchKernelGGL((dec_embed_kernel), 1, 256, 0, s, d->state, embed_args(d));
+            HIPC_LAUNCHED(ctx);
+        }
         // The residual stream alternates between two buffers: a GEMV whose prologue folds the previous
         // branch into the stream reads one and (its first workgroup) writes the other.
         float *xc = d->x, *xo = d->x2;
@@ -1178,18 +1286,20 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
             }
         }
         if (d->fused_glue) {
-            // the unembedding streams ~200 MB: its workgroups start on the weights at once and the
-            // final norm stays a launch of its own
-            hipLaunchKernelGGL((dec_norm_residual_kernel), 1, 256, 0, s, d->lean ? d->yd : d->y, d->lean ? d->down_slices : 1,
-                                                       d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], d->final_norm, c.hidden,
-                                                       c.rms_eps, xc, xc, d->xn);
-            HIPC_LAUNCHED(ctx);
+            // the unembedding's prologue adds the last branch to the stream and applies the final norm (every workgroup
+            // for itself, while its first weight tiles are on their way)
+            GemvPrologue pro;
+            pro.mode = 2, pro.x = xc, pro.y = d->lean ? d->yd : d->y, pro.y_slices = d->lean ? d->down_slices : 1;
+            pro.w_post = d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], pro.w_in = d->final_norm, pro.eps = c.rms_eps;
+            if ((rc = nbits_gemv(ctx, xc, HIPC_F32, d->lm_head, d->logits, 1, terms, &pro)) != HIPC_OK) return rc;
+        } else {
+            if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;
         }
-        if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;
         hipLaunchKernelGGL((dec_argmax_partial_kernel), kArgmaxParts, 256, 0, s, d->logits, c.vocab, d->am_v, d->am_i);
         HIPC_LAUNCHED(ctx);
-        hipLaunchKernelGGL((dec_argmax_final_kernel), 1, 64, 0, s, d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq, c.vocab);
+        hipLaunchKernelGGL((dec_pick_embed_kernel), 1, 256, 0, s, d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq, c.vocab, embed_args(d));
         HIPC_LAUNCHED(ctx);
+        if (!ctx->capturing) d->x_ready = true;
         return HIPC_OK;
     });
 }

@@ -304,6 +304,7 @@ void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
 struct GemvPrologue {
     int mode = 0;
     const float *x = nullptr, *y = nullptr, *w_post = nullptr, *w_in = nullptr;
+    int y_slices = 1;   // y is the sum of this many partial rows, K floats apart
     float *x_out = nullptr;
     float eps = 0.f;
     const float *part_o = nullptr, *part_ml = nullptr;

@@ -180,6 +180,7 @@ struct GemvArgs {
     const int *npos;
     int ngroup, nhd, nwindow;
     int nparts;   // ways the live chunks are divided among threads that share four channels
+    int ny_slices; // norm prologue: ny is this many partial rows, K floats apart, that add up to y
     int pro_off;  // byte offset of the prologue's own LDS area
 };
 
@@ -361,6 +362,12 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     // from them -- one memory round trip where the general path below makes three.
     const bool row_once = PRO == 2 && tile0 == 0 && tile1 * 128 >= p.K && nitems <= nthreads;
     float av_row[8];
+    // PRO 2: element c of y, which may arrive as ny_slices partial rows
+    auto y_at = [&](int c) {
+        float v = p.ny[c];
+        for (int s = 1; s < p.ny_slices; s++) v += p.ny[(size_t)s * p.K + c];
+        return v;
+    };
     if (PRO == 2) {
         __shared__ float nred[16];
         const int nw = nthreads >> 6;
@@ -384,7 +391,15 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
             };
             float x8[8], y8[8], p8[8], w8[8];
             ld8(p.nx, x8), ld8(p.nw_in, w8);
-            if (p.ny) ld8(p.ny, y8), ld8(p.nw_post, p8);
+            if (p.ny) {
+                ld8(p.ny, y8), ld8(p.nw_post, p8);
+                for (int s = 1; s < p.ny_slices; s++) {   // y arrives as partial rows
+                    float t8[8];
+                    ld8(p.ny + (size_t)s * p.K, t8);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) y8[i] += t8[i];
+                }
+            }
             load_first();  // the first weight tiles travel while the row is normalised
             if (p.ny) {
                 float sq = 0.f;
@@ -408,12 +423,12 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
             load_first();
             if (p.ny) {
                 float sq = 0.f;
-                for (int c = tid; c < p.K; c += nthreads) sq += p.ny[c] * p.ny[c];
+                for (int c = tid; c < p.K; c += nthreads) sq += y_at(c) * y_at(c);
                 inv1 = rsqrtf(block_total(sq) / (float)p.K + p.eps);
             }
             float sq2 = 0.f;
             for (int c = tid; c < p.K; c += nthreads) {
-                const float xp = p.ny ? p.nx[c] + p.ny[c] * inv1 * p.nw_post[c] : p.nx[c];
+                const float xp = p.ny ? p.nx[c] + y_at(c) * inv1 * p.nw_post[c] : p.nx[c];
                 sq2 += xp * xp;
                 if (writer) p.nx_out[c] = xp;
             }
@@ -494,7 +509,15 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
             };
             float x8[8], y8[8], p8[8], w8[8];
             ld8(p.nx, x8), ld8(p.nw_in, w8);
-            if (p.ny) ld8(p.ny, y8), ld8(p.nw_post, p8);
+            if (p.ny) {
+                ld8(p.ny, y8), ld8(p.nw_post, p8);
+                for (int s = 1; s < p.ny_slices; s++) {
+                    float t8[8];
+                    ld8(p.ny + (size_t)s * p.K, t8);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) y8[i] += t8[i];
+                }
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 const float xp = p.ny ? x8[i] + y8[i] * inv1 * p8[i] : x8[i];
@@ -920,6 +943,7 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
             HIPC_REQUIRE(ctx, aligned(pro->x, 16) && aligned(pro->w_in, 16) && (!pro->y || (aligned(pro->y, 16) && aligned(pro->w_post, 16))),
                          "MatMulNBits gemv: norm prologue operands must be 16-byte aligned");
             a.nx = pro->x, a.ny = pro->y, a.nw_post = pro->w_post, a.nw_in = pro->w_in, a.nx_out = pro->x_out, a.eps = pro->eps;
+            a.ny_slices = std::max(1, pro->y_slices);
             a.a_vec = 1;
         }
         if (mode == 3) {
