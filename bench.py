@@ -44,9 +44,9 @@ BS = 32
 # scaled by its reading for a 256 MiB copy; profiles/mmnb_gemv_lm_head_1152x262144.txt). A counter
 # run cannot happen inside this program, so the figure is carried over from that profile.
 LM_HEAD_TRAFFIC_BYTES = 199.6e6
-# The same for the average of the 104 narrow launches (a layer's q|k|v, o, gate|up, down: 18.408 MB of traffic for
+# The same for the average of the 104 narrow launches (a layer's q|k|v, o, gate|up, down: 18.257 MB of traffic for
 # 17.304 MB algorithmic; profiles/mmnb_lean_decode_linears_gemma3_1b.txt)
-NARROW_TRAFFIC_BYTES = 4.602e6
+NARROW_TRAFFIC_BYTES = 4.564e6
 IN_GRAPH = 16   # instances of a small operator per captured graph: amortises the graph launch
 LIGHT = False   # --light: a third of the timing samples (runs under a profiler, which a process that replays
                 # graphs for more than ~12 k kernel dispatches brings down)
