@@ -440,7 +440,10 @@ int hipc_decoder_set_embedding(hipc_ctx *ctx, hipc_decoder *dec, const void *B, 
  * (gemma3's local layers rotate with another base than its global ones; the reference gets the
  * tables as the operator's cos / sin cache inputs); at most two distinct bases per decoder. */
 int hipc_decoder_set_layer_attention(hipc_ctx *ctx, hipc_decoder *dec, int layer, int32_t window, float rope_theta);
-/* the token the next step consumes and its position (= tokens already in the cache) */
+/* the token the next step consumes and its position (= tokens already in the cache). When the embedding table and
+ * the first layer's input norm are set, the reset also embeds the token: a step expects the embedded row of the
+ * state's token (every step leaves the one of the token it picked behind; a step that finds none -- no reset since
+ * the embedding, a norm or a layer's rotary base changed -- embeds first). */
 int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *dec, int32_t token, int32_t pos);
 /* Device pointers of one layer's resident f16 cache. Keys: [n_kv_heads, max_seq, head_dim]. Values are
  * kept transposed, [n_kv_heads, head_dim, v_stride] with v_stride = max_seq rounded up to a multiple of
@@ -448,7 +451,8 @@ int hipc_decoder_reset(hipc_ctx *ctx, hipc_decoder *dec, int32_t token, int32_t 
  * one 16-byte load). A caller that fills the cache itself (a prefill) writes position t of channel c of
  * kv head h at v_cache[(h * head_dim + c) * v_stride + t]. */
 int hipc_decoder_kv_cache(hipc_ctx *ctx, hipc_decoder *dec, int layer, void **k_cache, void **v_cache);
-/* enqueue one decode step (capturable) */
+/* enqueue one decode step (capturable; record it after a reset or a step has run, so that the recorded launches do
+ * not include an embedding launch of their own) */
 int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *dec);
 /* flush, then read the state: next token, next position, the last step's logits [vocab] (or NULL),
  * and the tokens chosen at positions 0..n_history-1 (or NULL). Returns HIPC_ERR_INVALID (outputs
