@@ -190,6 +190,42 @@ def test_a_captured_step_replays_without_patching(ctx, pkg):
     assert np.array_equal(runs[0], runs[1])
 
 
+def test_the_embedded_row_follows_the_weights_it_is_made_of(ctx, pkg, oracle):
+    """Every step leaves the embedded row of the token it picked for the next one. When the embedding table or the
+    first layer's input norm is replaced between steps, the next step must embed again -- with the new weights -- and
+    a decoder that was never reset steps from token 0 at position 0."""
+    from oracle import decoder as od
+    w = pkg.decoder.build_weights(SMALL, seed=6)
+    w2 = pkg.decoder.build_weights(SMALL, seed=7)
+    for env in ({}, {"HIPC_DEC_LEAN": 0}):
+        with ctx.options(**env):
+            dec = pkg.decoder.Decoder(ctx, SMALL, 24)
+            dec.load(w)
+            ref = od.Decoder(w, 24)
+            token = 0                       # no reset: the state a new decoder starts from
+            for pos in range(8):
+                if pos == 3:                # a new embedding table and input norm, the other weights stay
+                    w.embedding = w2.embedding
+                    w.norms[(0, pkg.decoder.NORM_INPUT)] = w2.norms[(0, pkg.decoder.NORM_INPUT)]
+                    B, scales, zp = w.embedding
+                    dB, dS, dZ = ctx.upload(B), ctx.upload(scales), ctx.upload(zp)
+                    ctx._check(ctx.lib.hipc_decoder_set_embedding(ctx.handle, dec.handle, dB.ptr, B.size, dS.ptr, scales.size, dZ.ptr, zp.size))
+                    dV = ctx.upload(w.norms[(0, pkg.decoder.NORM_INPUT)])
+                    ctx._check(ctx.lib.hipc_decoder_set_norm(ctx.handle, dec.handle, 0, pkg.decoder.NORM_INPUT, dV.ptr))
+                    ctx.flush()
+                    for buf in (dB, dS, dZ, dV):
+                        buf.free()
+                dec.step()
+                got_tok, got_pos, logits, _ = dec.read(want_logits=True)
+                want_logits, want_tok = ref.step(token, pos)
+                assert got_pos == pos + 1
+                err = np.abs(logits - want_logits)
+                assert np.all(err <= 2e-3 + 2e-3 * np.abs(want_logits)), (env, pos, float(err.max()))
+                token = got_tok
+            dec.destroy()
+        w = pkg.decoder.build_weights(SMALL, seed=6)   # the first route's replacements do not carry over
+
+
 def test_refuses_incomplete_models_and_bad_shapes(ctx, pkg):
     dec = pkg.decoder.Decoder(ctx, SMALL, 16)
     with pytest.raises(pkg.HipComputeError) as e:
