@@ -266,11 +266,11 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
             const size_t lds = std::max(kSmallLds, slab_bytes);
             const dim3 grid(gemm_grid(ga, 64), 1, (unsigned)g->n);
             if (ep.requant) {
-                if (zero_known) int8_conv_row_kernel<EPI_REQUANT, false><<<grid, 256, lds, ctx->stream>>>(ga);
-                else int8_conv_row_kernel<EPI_REQUANT, true><<<grid, 256, lds, ctx->stream>>>(ga);
+                if (zero_known) hipLaunchKernelGGL((int8_conv_row_kernel<EPI_REQUANT, false>), grid, 256, lds, ctx->stream, ga);
+                else hipLaunchKernelGGL((int8_conv_row_kernel<EPI_REQUANT, true>), grid, 256, lds, ctx->stream, ga);
             } else {
-                if (zero_known) int8_conv_row_kernel<EPI_I32, false><<<grid, 256, lds, ctx->stream>>>(ga);
-                else int8_conv_row_kernel<EPI_I32, true><<<grid, 256, lds, ctx->stream>>>(ga);
+                if (zero_known) hipLaunchKernelGGL((int8_conv_row_kernel<EPI_I32, false>), grid, 256, lds, ctx->stream, ga);
+                else hipLaunchKernelGGL((int8_conv_row_kernel<EPI_I32, true>), grid, 256, lds, ctx->stream, ga);
             }
             HIPC_LAUNCHED(ctx);
             gemm_note_scalars(ctx, ga, !zero_known);
@@ -284,23 +284,21 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
         if (rc != HIPC_OK) return rc;
         const int HW = (int)(g->h * g->w);
         if (g->c_in % 4 == 0 && HW % 4 == 0 && aligned(X, 4))
-            nchw_to_nhwc4_kernel<<<dim3((unsigned)ceil_div(HW, 64), (unsigned)ceil_div(g->c_in, 64), (unsigned)g->n), 256, 0,
-                                   ctx->stream>>>(static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
+            hipLaunchKernelGGL((nchw_to_nhwc4_kernel), dim3((unsigned)ceil_div(HW, 64), (unsigned)ceil_div(g->c_in, 64), (unsigned)g->n), 256, 0, ctx->stream, static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
                                                   x_dtype == HIPC_U8 ? 0x80808080u : 0u);
         else
-            nchw_to_nhwc_kernel<<<dim3((unsigned)ceil_div(HW, 32), (unsigned)ceil_div(g->c_in, 32), (unsigned)g->n), 256, 0,
-                                  ctx->stream>>>(static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
+            hipLaunchKernelGGL((nchw_to_nhwc_kernel), dim3((unsigned)ceil_div(HW, 32), (unsigned)ceil_div(g->c_in, 32), (unsigned)g->n), 256, 0, ctx->stream, static_cast<const uint8_t *>(X), static_cast<uint8_t *>(xt), (int)g->c_in, HW,
                                                  x_dtype == HIPC_U8 ? 0x80 : 0);
         HIPC_LAUNCHED(ctx);
         ga.Q = static_cast<const uint8_t *>(xt);
         if (small) {
             const dim3 grid(gemm_grid(ga, 64), 1, (unsigned)g->n);
             if (ep.requant) {
-                if (zero_known) int8_conv_small_kernel<EPI_REQUANT, false><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
-                else int8_conv_small_kernel<EPI_REQUANT, true><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
+                if (zero_known) hipLaunchKernelGGL((int8_conv_small_kernel<EPI_REQUANT, false>), grid, 256, kSmallLds, ctx->stream, ga);
+                else hipLaunchKernelGGL((int8_conv_small_kernel<EPI_REQUANT, true>), grid, 256, kSmallLds, ctx->stream, ga);
             } else {
-                if (zero_known) int8_conv_small_kernel<EPI_I32, false><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
-                else int8_conv_small_kernel<EPI_I32, true><<<grid, 256, kSmallLds, ctx->stream>>>(ga);
+                if (zero_known) hipLaunchKernelGGL((int8_conv_small_kernel<EPI_I32, false>), grid, 256, kSmallLds, ctx->stream, ga);
+                else hipLaunchKernelGGL((int8_conv_small_kernel<EPI_I32, true>), grid, 256, kSmallLds, ctx->stream, ga);
             }
             HIPC_LAUNCHED(ctx);
             gemm_note_scalars(ctx, ga, !zero_known);
@@ -322,7 +320,7 @@ int run_conv(hipc_ctx *ctx, const void *X, int x_dtype, const hipc_conv_weight *
     d.Y = Y;
     d.requant = ep.requant, d.ratio = ep.ratio, d.ratio_step = ep.ratio_step, d.qbias = ep.qbias, d.y_zp = ep.y_zp,
     d.out_signed = ep.out_signed;
-    conv_direct_kernel<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, ctx->stream>>>(d);
+    hipLaunchKernelGGL((conv_direct_kernel), dim3((unsigned)ceil_div(total, 256)), 256, 0, ctx->stream, d);
     HIPC_LAUNCHED(ctx);
     if (host_zp) {
         note_scalar(ctx, HIPC_SCALAR_A_ZERO_POINT, offsetof(DirectConvArgs, x_zp_value));
@@ -379,8 +377,7 @@ int hipc_prepack_conv_w(hipc_ctx *ctx, const void *W, int w_dtype, const hipc_co
             e = hipMalloc(reinterpret_cast<void **>(&w->Wp), (size_t)w->O_pad * w->K_pad);
             if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&w->rowsum), (size_t)w->O_pad * 4);
             if (e == hipSuccess) {
-                pack_conv_w_kernel<<<dim3((unsigned)w->O_pad), 256, 0, ctx->stream>>>(
-                    static_cast<const uint8_t *>(W), w->Wp, w->rowsum, (int)g->c_out, (int)g->c_in, (int)g->kh, (int)g->kw,
+                hipLaunchKernelGGL((pack_conv_w_kernel), dim3((unsigned)w->O_pad), 256, 0, ctx->stream, static_cast<const uint8_t *>(W), w->Wp, w->rowsum, (int)g->c_out, (int)g->c_in, (int)g->kh, (int)g->kw,
                     w->O_pad, w->K_pad, w_dtype == HIPC_I8, w_dtype == HIPC_U8 ? 128 : 0);
                 e = hipGetLastError();
             }

@@ -477,7 +477,7 @@ int gemm_launch_tile(hipc_ctx *ctx, GemmArgs g, unsigned batch) {
     static bool lds_allowed[kMaxDevices] = {};
     if (int rc = allow_dynamic_lds(ctx, int8_gemm_kernel<MODE, EPI, ALIGNED, T>, gemm_lds(T), lds_allowed)) return rc;
     const dim3 grid(gemm_grid(g, T), 1, batch);
-    int8_gemm_kernel<MODE, EPI, ALIGNED, T><<<grid, 256, gemm_lds(T), ctx->stream>>>(g);
+    hipLaunchKernelGGL((int8_gemm_kernel<MODE, EPI, ALIGNED, T>), grid, 256, gemm_lds(T), ctx->stream, g);
     HIPC_LAUNCHED(ctx);
     gemm_note_scalars(ctx, g, true);
     return HIPC_OK;

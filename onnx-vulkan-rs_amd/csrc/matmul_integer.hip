@@ -126,10 +126,9 @@ namespace {
 int pack_into(hipc_ctx *ctx, const void *B, int b_dtype, int64_t K, int64_t N, int K_pad, int N_pad, uint8_t *Bp,
               int32_t *colsum) {
     const uint32_t flip = b_dtype == HIPC_U8 ? 0x80808080u : 0u;
-    pack_b_kernel<<<dim3((unsigned)ceil_div(N_pad, 64), (unsigned)ceil_div(K_pad / 4, 4)), 256, 0, ctx->stream>>>(
-        static_cast<const uint8_t *>(B), reinterpret_cast<uint32_t *>(Bp), (int)K, (int)N, K_pad, N_pad, flip);
+    hipLaunchKernelGGL((pack_b_kernel), dim3((unsigned)ceil_div(N_pad, 64), (unsigned)ceil_div(K_pad / 4, 4)), 256, 0, ctx->stream, static_cast<const uint8_t *>(B), reinterpret_cast<uint32_t *>(Bp), (int)K, (int)N, K_pad, N_pad, flip);
     HIPC_LAUNCHED(ctx);
-    col_sum_kernel<<<dim3((unsigned)ceil_div(N_pad, 4)), 256, 0, ctx->stream>>>(Bp, colsum, K_pad, N_pad);
+    hipLaunchKernelGGL((col_sum_kernel), dim3((unsigned)ceil_div(N_pad, 4)), 256, 0, ctx->stream, Bp, colsum, K_pad, N_pad);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }
@@ -166,7 +165,7 @@ int launch_mm_bdirect_dyn(hipc_ctx *ctx, GemmArgs g) {
     static bool lds_allowed[kMaxDevices] = {};
     if (int rc = allow_dynamic_lds(ctx, int8_gemm_bdirect_kernel<EPI, DYN, T, W>, bd_lds(T), lds_allowed)) return rc;
     const dim3 grid(gemm_grid(g, T), 1, 1);
-    int8_gemm_bdirect_kernel<EPI, DYN, T, W><<<grid, 64 * W, bd_lds(T), ctx->stream>>>(g);
+    hipLaunchKernelGGL((int8_gemm_bdirect_kernel<EPI, DYN, T, W>), grid, 64 * W, bd_lds(T), ctx->stream, g);
     HIPC_LAUNCHED(ctx);
     gemm_note_scalars(ctx, g, DYN);
     return HIPC_OK;
@@ -207,7 +206,7 @@ bool wants_small_tiles(hipc_ctx *ctx, const GemmArgs &g) {
 template <int EPI, bool DYN>
 int launch_mm_small_dyn(hipc_ctx *ctx, GemmArgs g) {
     const dim3 grid(gemm_grid(g, 64));
-    int8_gemm_small_kernel<EPI, DYN><<<grid, 256, kSmallLds, ctx->stream>>>(g);
+    hipLaunchKernelGGL((int8_gemm_small_kernel<EPI, DYN>), grid, 256, kSmallLds, ctx->stream, g);
     HIPC_LAUNCHED(ctx);
     gemm_note_scalars(ctx, g, DYN);
     return HIPC_OK;
@@ -240,9 +239,9 @@ int hipc_probe_int8_mfma(hipc_ctx *ctx, int random_operands, int waves_per_simd,
         HIPC_TRY(ctx, hipEventCreate(&t1));
         int *sink = reinterpret_cast<int *>(static_cast<char *>(ctx->params) + 128);
         const unsigned grid = (unsigned)(ctx->cu_count * waves_per_simd);  // 4 wavefronts per workgroup, one per SIMD
-        int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(64, 1u, random_operands, sink);  // warm the clocks and the code
+        hipLaunchKernelGGL((int8_mfma_probe_kernel), grid, 256, 0, ctx->stream, 64, 1u, random_operands, sink);  // warm the clocks and the code
         hipError_t e = hipEventRecord(t0, ctx->stream);
-        int8_mfma_probe_kernel<<<grid, 256, 0, ctx->stream>>>(iterations, 7u, random_operands, sink);
+        hipLaunchKernelGGL((int8_mfma_probe_kernel), grid, 256, 0, ctx->stream, iterations, 7u, random_operands, sink);
         if (e == hipSuccess) e = hipGetLastError();
         if (e == hipSuccess) e = hipEventRecord(t1, ctx->stream);
         if (e == hipSuccess) e = hipEventSynchronize(t1);
@@ -381,8 +380,7 @@ int hipc_requantize(hipc_ctx *ctx, const void *acc, const void *bias, const void
         if (n == 0) return HIPC_OK;
         HIPC_REQUIRE(ctx, acc && ratio && out, "Requantize: null operand");
         const long words = ceil_div(n, 4);
-        requantize_kernel<<<dim3((unsigned)ceil_div(words, 256)), 256, 0, ctx->stream>>>(
-            static_cast<const int32_t *>(acc), static_cast<const int32_t *>(bias), static_cast<const float *>(ratio), (long)n,
+        hipLaunchKernelGGL((requantize_kernel), dim3((unsigned)ceil_div(words, 256)), 256, 0, ctx->stream, static_cast<const int32_t *>(acc), static_cast<const int32_t *>(bias), static_cast<const float *>(ratio), (long)n,
             (long)std::max<int64_t>(inner, 1), (long)axis_len, y_zp, out_dtype == HIPC_I8, static_cast<uint8_t *>(out));
         HIPC_LAUNCHED(ctx);
         return HIPC_OK;

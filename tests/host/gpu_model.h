@@ -136,6 +136,13 @@ inline void gpu_model_nt_store(U v, T *p) { *p = v; }
 #define __builtin_amdgcn_update_dpp gpu_model_dpp
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16 gpu_model_mfma
 #define __builtin_amdgcn_mfma_f32_16x16x32_f16 gpu_model_mfma
+#define __builtin_amdgcn_mfma_i32_32x32x32_i8 gpu_model_mfma
+inline int gpu_model_sdot4(int, int, int c, bool) { return c; }
+#define __builtin_amdgcn_sdot4 gpu_model_sdot4
+inline uint32_t gpu_model_perm(uint32_t a, uint32_t, uint32_t) { return a; }
+#define __builtin_amdgcn_perm gpu_model_perm
+template <typename T>
+inline T atomicMax(T *p, T v) { const T old = *p; if (v > old) *p = v; return old; }
 #define __builtin_amdgcn_sched_barrier gpu_model_nothing
 #define __builtin_amdgcn_sched_group_barrier gpu_model_nothing
 #define __builtin_amdgcn_fence gpu_model_nothing

@@ -193,7 +193,7 @@ def test_a_stale_library_is_refused(pkg, monkeypatch):
         rt.load_library()
 
 
-def test_decode_step_addresses_on_the_cpu_model(tmp_path):
+def test_kernel_addresses_on_the_cpu_model(tmp_path):
     """tests/host/decoder_model.cpp: the decode step's kernel sources compiled as plain C++ (buffer loads
     replaced by a checker that applies the hardware's range rule, everything else under
     AddressSanitizer) and run thread by thread with the read-ahead helper rows on: whole steps at the
@@ -206,4 +206,10 @@ def test_decode_step_addresses_on_the_cpu_model(tmp_path):
     build = subprocess.run(["make", "-C", os.path.join(root, "tests", "host"), "-j", "4", "OUT=" + out], capture_output=True, text=True)
     assert build.returncode == 0, build.stdout[-2000:] + build.stderr[-2000:]
     run = subprocess.run([os.path.join(out, "decoder_model"), "quick", "8"], capture_output=True, text=True)
+    assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout[-2000:] + run.stderr[-2000:]
+    # the same build holds the int8 operators' model (tests/host/int8_model.cpp): every matrix-product route -- the
+    # kernels that step along k in a buffer load's scalar offset among them -- and the convolution routes, on tiny,
+    # ragged and aligned shapes and on the benchmark's, with operands of exactly the operator's size
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
+    run = subprocess.run([os.path.join(out, "int8_model")], capture_output=True, text=True, env=env)
     assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout[-2000:] + run.stderr[-2000:]
