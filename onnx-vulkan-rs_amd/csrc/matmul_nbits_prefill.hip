@@ -66,6 +66,41 @@ __device__ __forceinline__ uint4 dequant8(uint32_t w, uint32_t zb) {
     return make_uint4(out[0], out[1], out[2], out[3]);
 }
 
+// the wavefront's accumulators (F x F blocks of 32x32, first row i0, first column j0) to Y, to the f32 result or to
+// the k split's partials. Which of the three, and whether the wavefront's square lies inside the matrix, is decided
+// once (asked per element, the same questions made 3000 instructions of this and 5 of the kernel's 45 us).
+template <int F, bool CHECKED, typename OUT>
+__device__ __forceinline__ void prefill_store_as(OUT *__restrict__ dst, int M, int N, const f32x16 (&total)[F][F], int i0, int j0, int r32, int kg) {
+#pragma unroll
+    for (int i = 0; i < F; i++) {
+#pragma unroll
+        for (int j = 0; j < F; j++) {
+            const int gj = j0 + j * 32 + r32;
+            OUT *at = dst + (size_t)(i0 + i * 32 + kg * 4) * N + gj;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int rf = (r >> 2) * 8 + (r & 3);   // (+ kg * 4, which is in `at`)
+                if (!CHECKED || (i0 + i * 32 + kg * 4 + rf < M && gj < N)) {
+                    if constexpr (sizeof(OUT) == 2) at[(size_t)rf * N] = __float2half(total[i][j][r]);
+                    else at[(size_t)rf * N] = total[i][j][r];
+                }
+            }
+        }
+    }
+}
+template <int F>
+__device__ __forceinline__ void prefill_store(const PrefillArgs &p, const f32x16 (&total)[F][F], int i0, int j0, int r32, int kg) {
+    const bool inside = i0 + F * 32 <= p.M && j0 + F * 32 <= p.N;
+    float *f32_to = p.ksplit > 1 ? p.Ypart + (size_t)blockIdx.y * p.M * p.N : p.Yf32;
+    if (f32_to) {
+        if (inside) prefill_store_as<F, false>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
+        else prefill_store_as<F, true>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
+    } else {
+        if (inside) prefill_store_as<F, false>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
+        else prefill_store_as<F, true>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
+    }
+}
+
 // FULL: K is a multiple of 128, so no stage is partial or missing and nothing needs masking.
 template <int SG, int T, bool FULL>
 __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) {
@@ -242,27 +277,231 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
         __syncthreads();
     }
 
+    prefill_store<kF>(p, total, i0 + wm * kWT, j0 + wn * kWT, r32, kg);
+}
+
+#ifdef HIPC_PREFILL_WIDE
+
+// ---- the weight never enters LDS --------------------------------------------------------------------------------
+// The B operand of v_mfma_f32_32x32x16_f16 is eight k values of one column per lane, and a 32-bit word of the
+// prepacked weight is eight k values of one column: tile lane (c, q) of a 128-k weight tile holds, in its word j,
+// k = 32 j + 8 q + 0..7 of column c. The wavefront that multiplies a 32-column block reads the words itself (lane
+// (r32, kg) takes tile lanes q = 2 kg and 2 kg + 1 of its column: two 16-byte loads per 128 k), turns a word into
+// the operand in registers (nine instructions) and uses it for every 32-row block it owns. A k step (j, h) then
+// covers k = 32 j + 16 kg + 8 h + 0..7 -- an order of its own, which only has to be the same for both operands: A
+// is read from LDS at that offset. LDS carries A alone (half the traffic and half the writes of the kernel above,
+// and no conversion ahead of a barrier).
+
+// 1024 + zp and 64 + zp as f16 in both halves of a word (zb carries 128 + zp)
+struct ZeroPair {
+    f16x2 unit, sixteenth;
+};
+__device__ __forceinline__ ZeroPair zero_pair(uint32_t zb) {
+    const uint32_t zp = zb - 128u, a = 0x6400u + zp, b = 0x5400u + (zp << 4);
+    return {__builtin_bit_cast(f16x2, a | (a << 16)), __builtin_bit_cast(f16x2, b | (b << 16))};
+}
+// eight nibbles (k0 k2 k4 k6 in the low half, k1 k3 k5 k7 in the high half) -> the f16 values q - zp in k order.
+// Nibbles 0 and 2 of each half sit where the low mantissa bits are: or-ed with the exponent of 1024 that is
+// 1024 + q. Nibbles 1 and 3 sit four bits higher: 1024 + 16 q, and one fused multiply-add by 1/16 makes q - zp
+// of it ((1024 + 16 q) / 16 = 64 + q is exact). One shift instead of three.
+// (x & mask) | 0x64006400 as one instruction: v_and_or_b32 can take one scalar operand only, so the compiler, which
+// keeps both constants in scalar registers, emits two; the exponent pattern is handed over in a vector register
+__device__ __forceinline__ uint32_t and_or_1024(uint32_t x, uint32_t mask, uint32_t ones) {
+#ifdef HIPC_HOST_MODEL
+    return (x & mask) | ones;
+#else
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(ones));
+    return r;
+#endif
+}
+__device__ __forceinline__ f16x8 dequant_operand(uint32_t w, const ZeroPair &z, uint32_t ones) {
+    const f16x2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const uint32_t w8 = w >> 8;
+    const f16x2 p0 = __builtin_bit_cast(f16x2, and_or_1024(w, 0x000f000fu, ones)) - z.unit;
+    const f16x2 p1 = __builtin_bit_cast(f16x2, and_or_1024(w, 0x00f000f0u, ones)) * sixteenth - z.sixteenth;
+    const f16x2 p2 = __builtin_bit_cast(f16x2, and_or_1024(w8, 0x000f000fu, ones)) - z.unit;
+    const f16x2 p3 = __builtin_bit_cast(f16x2, and_or_1024(w8, 0x00f000f0u, ones)) * sixteenth - z.sixteenth;
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+__device__ __forceinline__ uint32_t word_of(const uint4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
+
+template <int SG, bool FULL>
+__global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const PrefillArgs p) {
+    constexpr int T = 128, kChunks = T / 32, kF = 2, kWT = 64;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    uint8_t *lds_a = lds_raw;  // [2][T * kPPitch]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r32 = lane & 31, kg = lane >> 5;
+
+    const int tiles_x = (p.N + T - 1) / T, tiles_y = (p.M + T - 1) / T;
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
+    const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
+    if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
+    const int i0 = ty * T, j0 = tx * T;
+
+    // A: chunk c = tid + 256 u -> slab row c / 8, 16-byte column c % 8 (8 halves)
+    uint32_t a_off[kChunks], a_lds[kChunks];
+    int a_k[kChunks];
 #pragma unroll
-    for (int i = 0; i < kF; i++) {
+    for (int u = 0; u < kChunks; u++) {
+        const int c = tid + 256 * u, row = c >> 3, kc = c & 7;
+        a_off[u] = ((uint32_t)min(i0 + row, p.M - 1) * (uint32_t)p.K + kc * 8) * 2;  // rows past M: clamped, never stored
+        a_lds[u] = row * kPPitch + kc * 16;
+        a_k[u] = kc * 8;
+    }
+    struct ARegs {
+        uint4 a[kChunks];
+    };
+    const char *a_base = reinterpret_cast<const char *>(p.A);
+    auto load_a = [&](ARegs &r, int stage) {
+        const int k0 = stage * kPK;
+#pragma unroll
+        for (int u = 0; u < kChunks; u++) {
+            const uint4 v = *reinterpret_cast<const uint4 *>((a_base + (size_t)k0 * 2) + a_off[u]);   // (uniform part first: a scalar base and a 32-bit lane offset)
+            const bool in = FULL || k0 + a_k[u] < p.K;  // K is a multiple of 8: a chunk is inside or outside as a whole
+            r.a[u] = make_uint4(in ? v.x : 0u, in ? v.y : 0u, in ? v.z : 0u, in ? v.w : 0u);
+        }
+    };
+    // a stage past the end reads clamped addresses and stores zeros for A: it adds nothing
+    auto store_a = [&](const ARegs &r, int buf, bool live) {
+        const uint32_t keep = FULL || live ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int u = 0; u < kChunks; u++)
+            *reinterpret_cast<uint4 *>(lds_a + buf * T * kPPitch + a_lds[u]) =
+                make_uint4(r.a[u].x & keep, r.a[u].y & keep, r.a[u].z & keep, r.a[u].w & keep);
+    };
+
+    // B: column block j of the wavefront = 32 columns = two weight tiles; the lane's column is r32 of the block
+    uint32_t b_at[kF], sc_at[kF];
+#pragma unroll
+    for (int j = 0; j < kF; j++) {
+        const int nt = min(j0 / 16 + wn * 4 + j * 2 + (r32 >> 4), p.n_tiles - 1);  // tiles past N: clamped, never stored
+        b_at[j] = (uint32_t)nt * (uint32_t)p.n_cg * 64 + (r32 & 15) + 32 * kg;
+        sc_at[j] = ((uint32_t)nt * (uint32_t)p.n_cg * 16 + (r32 & 15)) * SG;
+    }
+    struct BRegs {
+        uint4 w[kF][2];
+        float s[kF][SG];
+        uint32_t z[kF];  // SG bytes of 128 + zp
+    };
+    auto load_b = [&](BRegs &b, int cg) {
 #pragma unroll
         for (int j = 0; j < kF; j++) {
-            const int gj = j0 + wn * kWT + j * 32 + r32;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int rf = (r >> 2) * 8 + kg * 4 + (r & 3);
-                const int gi = i0 + wm * kWT + i * 32 + rf;
-                if (gi < p.M && gj < p.N) {
-                    if (p.ksplit > 1)
-                        p.Ypart[((size_t)blockIdx.y * p.M + gi) * p.N + gj] = total[i][j][r];
-                    else if (p.Yf32)
-                        p.Yf32[(size_t)gi * p.N + gj] = total[i][j][r];
-                    else
-                        p.Y[(size_t)gi * p.N + gj] = __float2half(total[i][j][r]);
-                }
+            const uint4 *src = (p.Wq + (size_t)cg * 64) + b_at[j];
+            b.w[j][0] = src[0];
+            b.w[j][1] = src[16];
+            const float *sc = (p.Sc + (size_t)cg * 16 * SG) + sc_at[j];
+            const uint8_t *zb = (p.Zb + (size_t)cg * 16 * SG) + sc_at[j];
+            if (SG == 4) {
+                const float4 v = *reinterpret_cast<const float4 *>(sc);
+                b.s[j][0] = v.x, b.s[j][1 % SG] = v.y, b.s[j][2 % SG] = v.z, b.s[j][3 % SG] = v.w;
+                b.z[j] = *reinterpret_cast<const uint32_t *>(zb);
+            } else if (SG == 2) {
+                const float2 v = *reinterpret_cast<const float2 *>(sc);
+                b.s[j][0] = v.x, b.s[j][1 % SG] = v.y;
+                b.z[j] = *reinterpret_cast<const uint16_t *>(zb);
+            } else {
+                b.s[j][0] = sc[0];
+                b.z[j] = zb[0];
             }
         }
+    };
+
+    f32x16 total[kF][kF], raw[kF][kF];
+#pragma unroll
+    for (int i = 0; i < kF; i++)
+#pragma unroll
+        for (int j = 0; j < kF; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) total[i][j][r] = 0.f, raw[i][j][r] = 0.f;
+    f32x16 zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+
+    uint32_t ones = 0x64006400u;   // kept in a vector register (see and_or_1024)
+    asm volatile("" : "+v"(ones));
+    // One stage = 64 k = the k steps (j, h) with j = 2 half + 0 / 1 of the weight tile the stage lies in;
+    // scale groups end after every second step (SG 4), every stage (SG 2) or every odd stage (SG 1).
+    auto compute = [&](const BRegs &b, int buf, int half) {
+        const uint8_t *ba = lds_a + buf * T * kPPitch + (wm * kWT + r32) * kPPitch + kg * 32;
+        ZeroPair zp[kF][SG == 4 ? 2 : 1];
+#pragma unroll
+        for (int j = 0; j < kF; j++) {
+            if (SG == 4) {
+                zp[j][0] = zero_pair((b.z[j] >> (16 * half)) & 0xffu);
+                zp[j][SG == 4 ? 1 : 0] = zero_pair((b.z[j] >> (16 * half + 8)) & 0xffu);
+            } else {
+                zp[j][0] = zero_pair(SG == 2 ? (b.z[j] >> (8 * half)) & 0xffu : b.z[j]);
+            }
+        }
+#pragma unroll
+        for (int step = 0; step < 4; step++) {
+            const int word = half * 2 + (step >> 1), h = step & 1;
+            const bool opens = SG == 4 ? h == 0 : SG == 2 ? step == 0 : step == 0 && half == 0;
+            f16x8 af[kF], wf[kF];
+#pragma unroll
+            for (int i = 0; i < kF; i++) af[i] = *reinterpret_cast<const f16x8 *>(ba + i * 32 * kPPitch + (step >> 1) * 64 + h * 16);
+#pragma unroll
+            for (int j = 0; j < kF; j++) wf[j] = dequant_operand(word_of(b.w[j][h], word), zp[j][SG == 4 ? step >> 1 : 0], ones);
+#pragma unroll
+            for (int i = 0; i < kF; i++)
+#pragma unroll
+                for (int j = 0; j < kF; j++) raw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], opens ? zero : raw[i][j], 0, 0, 0);
+            const bool closes = SG == 4 ? h == 1 : SG == 2 ? step == 3 : step == 3 && half == 1;
+            if (closes) {
+                const int g = SG == 4 ? word : SG == 2 ? half : 0;
+#pragma unroll
+                for (int i = 0; i < kF; i++)
+#pragma unroll
+                    for (int j = 0; j < kF; j++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) total[i][j][r] = fmaf(raw[i][j][r], b.s[j][g % SG], total[i][j][r]);
+            }
+        }
+    };
+
+    const int nk_all = (p.K + kPK - 1) / kPK;
+    const int ks0 = blockIdx.y * p.split_stages, nk = min(nk_all, ks0 + p.split_stages);  // this workgroup's stages (ks0 is even)
+    const int cg_last = (nk - 1) >> 1;
+    ARegs r0, r1;
+    BRegs bc, bn;
+    load_b(bc, ks0 >> 1);
+    load_a(r0, ks0);
+    load_a(r1, min(ks0 + 1, nk - 1));
+    store_a(r0, 0, true);
+    __syncthreads();
+    // two stages = one weight tile per trip; with an odd stage count the second half of the last trip multiplies
+    // a stage whose A is all zeros. (The fences keep the order written here: left alone, the compiler moves the
+    // stores -- and with them the wait for the loads they store -- ahead of the products and the next loads behind
+    // them, and every half trip then waits out a whole trip to memory.)
+    auto trip = [&](const BRegs &bcur, BRegs &bnext, int ks) {
+        load_b(bnext, min((ks >> 1) + 1, cg_last));
+        load_a(r0, min(ks + 2, nk - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        compute(bcur, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        store_a(r1, 1, ks + 1 < nk);
+        __syncthreads();
+        load_a(r1, min(ks + 3, nk - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        compute(bcur, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_a(r0, 0, true);
+        __syncthreads();
+    };
+    for (int ks = ks0; ks < nk; ks += 4) {   // the two register sets of the weight take turns
+        trip(bc, bn, ks);
+        if (ks + 2 < nk) trip(bn, bc, ks + 2);
     }
+    prefill_store<kF>(p, total, i0 + wm * kWT, j0 + wn * kWT, r32, kg);
 }
+
+#endif  // HIPC_PREFILL_WIDE
 
 // Y = f16(sum over splits of the f32 partials), in split order; or the f32 sum itself into Yf32
 // (static: this file is compiled twice)
@@ -283,12 +522,13 @@ namespace {
 // the prefill_split option: 0 never splits k, n > 0 forces n ways (tuning, tests); unset: chosen by shape
 
 template <int SG, int T>
-int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
+int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a, bool direct = false) {
     const bool full = a.K % (2 * kPK) == 0;
     static bool lds_allowed[2][kMaxDevices] = {};
-    if (int rc = full ? allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, true>, prefill_lds(T), lds_allowed[1])
-                      : allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, false>, prefill_lds(T), lds_allowed[0]))
-        return rc;
+    if (!direct)
+        if (int rc = full ? allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, true>, prefill_lds(T), lds_allowed[1])
+                          : allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, false>, prefill_lds(T), lds_allowed[0]))
+            return rc;
     const int tiles_x = (int)ceil_div(a.N, T), tiles_y = (int)ceil_div(a.M, T);
     int best = 8, best_cost = 1 << 30;
     for (int r = 1; r <= 8; r *= 2) {
@@ -318,11 +558,22 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
         a.Ypart = static_cast<float *>(part);
     }
     const dim3 g2(grid, (unsigned)a.ksplit);
-    if (full)
-        mmnb_prefill_kernel<SG, T, true><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
-    else
-        mmnb_prefill_kernel<SG, T, false><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
-    HIPC_LAUNCHED(ctx);
+#ifdef HIPC_PREFILL_WIDE
+    if (direct) {   // A alone in LDS: 36 KB, inside the limit that needs no permission
+        if (full)
+            mmnb_prefill_direct_kernel<SG, true><<<g2, dim3(256), prefill_lds(T) / 2, ctx->stream>>>(a);
+        else
+            mmnb_prefill_direct_kernel<SG, false><<<g2, dim3(256), prefill_lds(T) / 2, ctx->stream>>>(a);
+        HIPC_LAUNCHED(ctx);
+    } else
+#endif
+    {
+        if (full)
+            mmnb_prefill_kernel<SG, T, true><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
+        else
+            mmnb_prefill_kernel<SG, T, false><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
+        HIPC_LAUNCHED(ctx);
+    }
     if (a.ksplit > 1) {
         const long total = (long)a.M * a.N;
         mmnb_prefill_reduce_kernel<<<dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream>>>(a.Ypart, a.Y, a.Yf32, total, a.ksplit);
@@ -343,10 +594,11 @@ int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG);
 #ifdef HIPC_PREFILL_WIDE
 
 int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG) {
+    const bool direct = ctx->tune.prefill_direct != 0;
     switch (SG) {
-        case 4: return prefill_launch_tile<4, 128>(ctx, a);
-        case 2: return prefill_launch_tile<2, 128>(ctx, a);
-        default: return prefill_launch_tile<1, 128>(ctx, a);
+        case 4: return prefill_launch_tile<4, 128>(ctx, a, direct);
+        case 2: return prefill_launch_tile<2, 128>(ctx, a, direct);
+        default: return prefill_launch_tile<1, 128>(ctx, a, direct);
     }
 }
 

@@ -132,6 +132,29 @@ def test_f16_rows_beyond_sixteen_run_the_tiled_kernel(ctx, pkg, oracle, shape):
     assert got.dtype == np.float16 and close(got, want, RTOL16), worst(got, want)
 
 
+WIDE_ROUTES = [  # the 128x128 tiles, forced on shapes that would take 64x64: each kernel, alone and with k split over workgroups
+    {"HIPC_PREFILL_TILE": 128}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2},
+    {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_DIRECT": 0}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_DIRECT": 0, "HIPC_PREFILL_SPLIT": 3},
+]
+
+
+@pytest.mark.parametrize("options", WIDE_ROUTES, ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("shape", PREFILL + [(300, 1152, 392, 32, True), (129, 512, 260, 64, False)], ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_both_wide_tile_kernels_on_ragged_shapes(ctx, pkg, oracle, shape, options):
+    """The kernel that dequantises the weight in the registers of the wavefront that multiplies it (its k order
+    inside a stage differs from memory order, for both operands alike) and the one that passes it through LDS:
+    ragged rows and columns, a partial last stage, an odd stage count, every scale grouping, zero points."""
+    m, k, n, bs, with_zp = shape
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=47, with_zp=with_zp, scale_dtype=np.float16)
+    a = pkg.synth.normal_f32(m * k, 48).reshape(m, k).astype(np.float16)
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    with ctx.options(**options):
+        got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    assert got.dtype == np.float16 and close(got, want, RTOL16), worst(got, want)
+
+
 F32_PREFILL = [  # (M, K, N, block_size, zero points)
     (100, 1000, 200, 32, True), (130, 384, 131, 64, True), (257, 640, 96, 128, False), (33, 72, 16, 32, True),
     (512, 2048, 2560, 128, False),
