@@ -54,9 +54,9 @@ struct Tuning {
     int gemm_big = -1;        // HIPC_GEMM_BIG       the int8 kernels that keep B out of LDS: 0 never, 1 / 2 the 256x256 / 128x128 tile whenever A allows
     int gemm_small = -1;      // HIPC_GEMM_SMALL     the k-split 64x64 kernels: 0 never, 1 whenever A allows
     int conv_row = -1;        // HIPC_CONV_ROW       0: convolutions along one axis take the general route
-    int prefill_tile = -1;    // HIPC_PREFILL_TILE   64 or 128
+    int prefill_tile = -1;    // HIPC_PREFILL_TILE   64, 128 or 192 (columns; 192 has 128 rows)
     int prefill_split = -1;   // HIPC_PREFILL_SPLIT  0 never splits k, n forces n ways
-    int prefill_direct = -1;  // HIPC_PREFILL_DIRECT 0: the 128x128 tiles keep the kernel that passes the weight through LDS
+    int prefill_direct = -1;  // HIPC_PREFILL_DIRECT 0: 128-row tiles keep the kernel that passes the weight through LDS (and are never 192 wide)
     int dec_fused_glue = -1;  // HIPC_DEC_FUSED_GLUE 0 keeps the separate norm / GELU kernels (read when a decoder is created)
     int dec_fused_attn = -1;  // HIPC_DEC_FUSED_ATTN 0 keeps the three-kernel attention (read when a decoder is created)
     int gemv_lean = -1;       // HIPC_GEMV_LEAN      0: one-row products keep the streaming GEMV kernel

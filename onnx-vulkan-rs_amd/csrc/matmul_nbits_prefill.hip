@@ -69,12 +69,12 @@ __device__ __forceinline__ uint4 dequant8(uint32_t w, uint32_t zb) {
 // the wavefront's accumulators (F x F blocks of 32x32, first row i0, first column j0) to Y, to the f32 result or to
 // the k split's partials. Which of the three, and whether the wavefront's square lies inside the matrix, is decided
 // once (asked per element, the same questions made 3000 instructions of this and 5 of the kernel's 45 us).
-template <int F, bool CHECKED, typename OUT>
-__device__ __forceinline__ void prefill_store_as(OUT *__restrict__ dst, int M, int N, const f32x16 (&total)[F][F], int i0, int j0, int r32, int kg) {
+template <int FM, int FN, bool CHECKED, typename OUT>
+__device__ __forceinline__ void prefill_store_as(OUT *__restrict__ dst, int M, int N, const f32x16 (&total)[FM][FN], int i0, int j0, int r32, int kg) {
 #pragma unroll
-    for (int i = 0; i < F; i++) {
+    for (int i = 0; i < FM; i++) {
 #pragma unroll
-        for (int j = 0; j < F; j++) {
+        for (int j = 0; j < FN; j++) {
             const int gj = j0 + j * 32 + r32;
             OUT *at = dst + (size_t)(i0 + i * 32 + kg * 4) * N + gj;
 #pragma unroll
@@ -88,16 +88,16 @@ __device__ __forceinline__ void prefill_store_as(OUT *__restrict__ dst, int M, i
         }
     }
 }
-template <int F>
-__device__ __forceinline__ void prefill_store(const PrefillArgs &p, const f32x16 (&total)[F][F], int i0, int j0, int r32, int kg) {
-    const bool inside = i0 + F * 32 <= p.M && j0 + F * 32 <= p.N;
+template <int FM, int FN>
+__device__ __forceinline__ void prefill_store(const PrefillArgs &p, const f32x16 (&total)[FM][FN], int i0, int j0, int r32, int kg) {
+    const bool inside = i0 + FM * 32 <= p.M && j0 + FN * 32 <= p.N;
     float *f32_to = p.ksplit > 1 ? p.Ypart + (size_t)blockIdx.y * p.M * p.N : p.Yf32;
     if (f32_to) {
-        if (inside) prefill_store_as<F, false>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
-        else prefill_store_as<F, true>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
+        if (inside) prefill_store_as<FM, FN, false>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
+        else prefill_store_as<FM, FN, true>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
     } else {
-        if (inside) prefill_store_as<F, false>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
-        else prefill_store_as<F, true>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
+        if (inside) prefill_store_as<FM, FN, false>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
+        else prefill_store_as<FM, FN, true>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
     }
 }
 
@@ -277,10 +277,8 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
         __syncthreads();
     }
 
-    prefill_store<kF>(p, total, i0 + wm * kWT, j0 + wn * kWT, r32, kg);
+    prefill_store<kF, kF>(p, total, i0 + wm * kWT, j0 + wn * kWT, r32, kg);
 }
-
-#ifdef HIPC_PREFILL_WIDE
 
 // ---- the weight never enters LDS --------------------------------------------------------------------------------
 // The B operand of v_mfma_f32_32x32x16_f16 is eight k values of one column per lane, and a 32-bit word of the
@@ -326,9 +324,12 @@ __device__ __forceinline__ f16x8 dequant_operand(uint32_t w, const ZeroPair &z, 
 }
 __device__ __forceinline__ uint32_t word_of(const uint4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
 
-template <int SG, bool FULL>
-__global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const PrefillArgs p) {
-    constexpr int T = 128, kChunks = T / 32, kF = 2, kWT = 64;
+// NJ: 32-column blocks per wavefront. 2: a 128x128 tile. 3: a 128x192 tile -- a third less LDS traffic per product,
+// and a matrix of 512 x 11008 becomes 232 workgroups for 256 CUs where 128x128 tiles make 344, two of them on every
+// third CU.
+template <int SG, int NJ, bool FULL>
+__global__ void __launch_bounds__(256, NJ == 2 ? 2 : 1) mmnb_prefill_direct_kernel(const PrefillArgs p) {
+    constexpr int T = 128, TN = 64 * NJ, kChunks = T / 32, kF = 2, kWT = 64, kWN = 32 * NJ;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     uint8_t *lds_a = lds_raw;  // [2][T * kPPitch]
 
@@ -337,12 +338,12 @@ __global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const Prefi
     const int wm = wave >> 1, wn = wave & 1;
     const int r32 = lane & 31, kg = lane >> 5;
 
-    const int tiles_x = (p.N + T - 1) / T, tiles_y = (p.M + T - 1) / T;
+    const int tiles_x = (p.N + TN - 1) / TN, tiles_y = (p.M + T - 1) / T;
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
     const int rows_per = (tiles_y + p.xcd_rows - 1) / p.xcd_rows, cols_per = (tiles_x + p.xcd_cols - 1) / p.xcd_cols;
     const int ty = (xcd / p.xcd_cols) * rows_per + idx / cols_per, tx = (xcd % p.xcd_cols) * cols_per + idx % cols_per;
     if (idx >= rows_per * cols_per || ty >= tiles_y || tx >= tiles_x) return;
-    const int i0 = ty * T, j0 = tx * T;
+    const int i0 = ty * T, j0 = tx * TN;
 
     // A: chunk c = tid + 256 u -> slab row c / 8, 16-byte column c % 8 (8 halves)
     uint32_t a_off[kChunks], a_lds[kChunks];
@@ -377,21 +378,21 @@ __global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const Prefi
     };
 
     // B: column block j of the wavefront = 32 columns = two weight tiles; the lane's column is r32 of the block
-    uint32_t b_at[kF], sc_at[kF];
+    uint32_t b_at[NJ], sc_at[NJ];
 #pragma unroll
-    for (int j = 0; j < kF; j++) {
-        const int nt = min(j0 / 16 + wn * 4 + j * 2 + (r32 >> 4), p.n_tiles - 1);  // tiles past N: clamped, never stored
+    for (int j = 0; j < NJ; j++) {
+        const int nt = min(j0 / 16 + wn * (2 * NJ) + j * 2 + (r32 >> 4), p.n_tiles - 1);  // tiles past N: clamped, never stored
         b_at[j] = (uint32_t)nt * (uint32_t)p.n_cg * 64 + (r32 & 15) + 32 * kg;
         sc_at[j] = ((uint32_t)nt * (uint32_t)p.n_cg * 16 + (r32 & 15)) * SG;
     }
     struct BRegs {
-        uint4 w[kF][2];
-        float s[kF][SG];
-        uint32_t z[kF];  // SG bytes of 128 + zp
+        uint4 w[NJ][2];
+        float s[NJ][SG];
+        uint32_t z[NJ];  // SG bytes of 128 + zp
     };
     auto load_b = [&](BRegs &b, int cg) {
 #pragma unroll
-        for (int j = 0; j < kF; j++) {
+        for (int j = 0; j < NJ; j++) {
             const uint4 *src = (p.Wq + (size_t)cg * 64) + b_at[j];
             b.w[j][0] = src[0];
             b.w[j][1] = src[16];
@@ -412,26 +413,55 @@ __global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const Prefi
         }
     };
 
-    f32x16 total[kF][kF], raw[kF][kF];
+    // One set of accumulators, kept in units of the scale of the quantisation block that is open: when the next
+    // block opens they are multiplied by (scale of the old block) / (scale of the new one), the products of the new
+    // block add to them as they are, and the store multiplies by the last scale. That is one multiplication per
+    // accumulator and block, like adding scale x (block sum) to a running total, without the second set of
+    // registers for the block sum (which is what lets a wavefront own three 32-column blocks). A scale of magnitude
+    // below 2^-64 (a block of zeros carries 0) counts as 2^-64: the quotient stays finite, and what such a block
+    // adds, at most 2^-64 x 15 x sum |a|, is far below one unit of the last place of any result that has a block
+    // with a real scale; a column without one is stored as 0.
+    f32x16 acc[kF][NJ];
 #pragma unroll
     for (int i = 0; i < kF; i++)
 #pragma unroll
-        for (int j = 0; j < kF; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) total[i][j][r] = 0.f, raw[i][j][r] = 0.f;
-    f32x16 zero;
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    float unit[NJ];   // the scale the accumulators of column block j are in
+    bool scaled[NJ];  // the lane's column of block j has met a scale of 2^-64 or more
 #pragma unroll
-    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+    for (int j = 0; j < NJ; j++) unit[j] = 1.f, scaled[j] = false;
+    // the scales of a weight tile's groups -> the factors that take the accumulators from each group to the next
+    // (worked out when the trip begins, next to the loads, not in front of the products that wait for them)
+    auto scales_to_ratios = [&](BRegs &b) {
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int g = 0; g < SG; g++) {
+                const bool real = !(fabsf(b.s[j][g]) < 0x1p-64f);
+                const float s = real ? b.s[j][g] : 0x1p-64f;
+                scaled[j] |= real;
+                b.s[j][g] = unit[j] * __builtin_amdgcn_rcpf(s);   // (1 ulp: a relative error of 1e-7 in what was added so far)
+                unit[j] = s;
+            }
+    };
+    auto reopen = [&](int j, float ratio) {
+#pragma unroll
+        for (int i = 0; i < kF; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] *= ratio;
+    };
 
     uint32_t ones = 0x64006400u;   // kept in a vector register (see and_or_1024)
     asm volatile("" : "+v"(ones));
     // One stage = 64 k = the k steps (j, h) with j = 2 half + 0 / 1 of the weight tile the stage lies in;
-    // scale groups end after every second step (SG 4), every stage (SG 2) or every odd stage (SG 1).
-    auto compute = [&](const BRegs &b, int buf, int half) {
+    // a scale group opens at every second step (SG 4), every stage (SG 2) or every even stage (SG 1).
+    auto compute = [&](const BRegs &b, int buf, int half) {   // (b.s holds ratios by now)
         const uint8_t *ba = lds_a + buf * T * kPPitch + (wm * kWT + r32) * kPPitch + kg * 32;
-        ZeroPair zp[kF][SG == 4 ? 2 : 1];
+        ZeroPair zp[NJ][SG == 4 ? 2 : 1];
 #pragma unroll
-        for (int j = 0; j < kF; j++) {
+        for (int j = 0; j < NJ; j++) {
             if (SG == 4) {
                 zp[j][0] = zero_pair((b.z[j] >> (16 * half)) & 0xffu);
                 zp[j][SG == 4 ? 1 : 0] = zero_pair((b.z[j] >> (16 * half + 8)) & 0xffu);
@@ -443,25 +473,20 @@ __global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const Prefi
         for (int step = 0; step < 4; step++) {
             const int word = half * 2 + (step >> 1), h = step & 1;
             const bool opens = SG == 4 ? h == 0 : SG == 2 ? step == 0 : step == 0 && half == 0;
-            f16x8 af[kF], wf[kF];
+            f16x8 af[kF], wf[NJ];
+            if (opens) {
+                const int g = SG == 4 ? word : SG == 2 ? half : 0;
+#pragma unroll
+                for (int j = 0; j < NJ; j++) reopen(j, b.s[j][g % SG]);
+            }
 #pragma unroll
             for (int i = 0; i < kF; i++) af[i] = *reinterpret_cast<const f16x8 *>(ba + i * 32 * kPPitch + (step >> 1) * 64 + h * 16);
 #pragma unroll
-            for (int j = 0; j < kF; j++) wf[j] = dequant_operand(word_of(b.w[j][h], word), zp[j][SG == 4 ? step >> 1 : 0], ones);
+            for (int j = 0; j < NJ; j++) wf[j] = dequant_operand(word_of(b.w[j][h], word), zp[j][SG == 4 ? step >> 1 : 0], ones);
 #pragma unroll
             for (int i = 0; i < kF; i++)
 #pragma unroll
-                for (int j = 0; j < kF; j++) raw[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], opens ? zero : raw[i][j], 0, 0, 0);
-            const bool closes = SG == 4 ? h == 1 : SG == 2 ? step == 3 : step == 3 && half == 1;
-            if (closes) {
-                const int g = SG == 4 ? word : SG == 2 ? half : 0;
-#pragma unroll
-                for (int i = 0; i < kF; i++)
-#pragma unroll
-                    for (int j = 0; j < kF; j++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++) total[i][j][r] = fmaf(raw[i][j][r], b.s[j][g % SG], total[i][j][r]);
-            }
+                for (int j = 0; j < NJ; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], wf[j], acc[i][j], 0, 0, 0);
         }
     };
 
@@ -479,9 +504,10 @@ __global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const Prefi
     // a stage whose A is all zeros. (The fences keep the order written here: left alone, the compiler moves the
     // stores -- and with them the wait for the loads they store -- ahead of the products and the next loads behind
     // them, and every half trip then waits out a whole trip to memory.)
-    auto trip = [&](const BRegs &bcur, BRegs &bnext, int ks) {
+    auto trip = [&](BRegs &bcur, BRegs &bnext, int ks) {
         load_b(bnext, min((ks >> 1) + 1, cg_last));
         load_a(r0, min(ks + 2, nk - 1));
+        scales_to_ratios(bcur);
         __builtin_amdgcn_sched_barrier(0);
         compute(bcur, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -498,10 +524,14 @@ __global__ void __launch_bounds__(256, 2) mmnb_prefill_direct_kernel(const Prefi
         trip(bc, bn, ks);
         if (ks + 2 < nk) trip(bn, bc, ks + 2);
     }
-    prefill_store<kF>(p, total, i0 + wm * kWT, j0 + wn * kWT, r32, kg);
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int i = 0; i < kF; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] *= scaled[j] ? unit[j] : 0.f;
+    prefill_store<kF, NJ>(p, acc, i0 + wm * kWT, j0 + wn * kWN, r32, kg);
 }
-
-#endif  // HIPC_PREFILL_WIDE
 
 // Y = f16(sum over splits of the f32 partials), in split order; or the f32 sum itself into Yf32
 // (static: this file is compiled twice)
@@ -519,24 +549,17 @@ mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ 
 
 namespace {
 
-// the prefill_split option: 0 never splits k, n > 0 forces n ways (tuning, tests); unset: chosen by shape
-
-template <int SG, int T>
-int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a, bool direct = false) {
-    const bool full = a.K % (2 * kPK) == 0;
-    static bool lds_allowed[2][kMaxDevices] = {};
-    if (!direct)
-        if (int rc = full ? allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, true>, prefill_lds(T), lds_allowed[1])
-                          : allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, false>, prefill_lds(T), lds_allowed[0]))
-            return rc;
-    const int tiles_x = (int)ceil_div(a.N, T), tiles_y = (int)ceil_div(a.M, T);
+// The tile grid cut into one rectangle per XCD, the k split (prefill_split option: 0 never splits k, n > 0 forces n
+// ways; unset: chosen by shape) with its partials in scratch memory; returns the launch grid in *grid.
+int prefill_plan(hipc_ctx *ctx, PrefillArgs &a, int TM, int TN, bool may_split, dim3 *grid) {
+    const int tiles_x = (int)ceil_div(a.N, TN), tiles_y = (int)ceil_div(a.M, TM);
     int best = 8, best_cost = 1 << 30;
     for (int r = 1; r <= 8; r *= 2) {
         const int cost = (int)(ceil_div(tiles_y, r) + ceil_div(tiles_x, 8 / r));
         if (cost < best_cost) best_cost = cost, best = r;
     }
     a.xcd_rows = best, a.xcd_cols = 8 / best;
-    const unsigned grid = 8u * (unsigned)(ceil_div(tiles_y, a.xcd_rows) * ceil_div(tiles_x, a.xcd_cols));
+    const unsigned gx = 8u * (unsigned)(ceil_div(tiles_y, a.xcd_rows) * ceil_div(tiles_x, a.xcd_cols));
     // Too few tiles for the chip: split k over workgroups, as many ways as gives every CU a
     // workgroup, at least 32 stages each (with fewer, the second launch and the partials cost more
     // than the idle CUs: 512 x 2048 x 2560 took 27 us split three ways, 21 us on 64x64 tiles). The
@@ -544,7 +567,7 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a, bool direct = false) {
     const int nk = (int)ceil_div(a.K, kPK);
     int ksplit = 1;
     const int g_prefill_split = ctx->tune.prefill_split;
-    if (T == 128 && g_prefill_split != 0) {
+    if (may_split && g_prefill_split != 0) {
         const int tiles = tiles_x * tiles_y;
         ksplit = g_prefill_split > 0 ? g_prefill_split : std::min(4, ctx->cu_count / std::max(1, tiles));
         ksplit = std::max(1, std::min(ksplit, g_prefill_split > 0 ? nk / 2 : nk / 32));
@@ -557,29 +580,49 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a, bool direct = false) {
         if (int rc = scratch_get(ctx, 0, (size_t)a.ksplit * a.M * a.N * sizeof(float), &part)) return rc;
         a.Ypart = static_cast<float *>(part);
     }
-    const dim3 g2(grid, (unsigned)a.ksplit);
-#ifdef HIPC_PREFILL_WIDE
-    if (direct) {   // A alone in LDS: 36 KB, inside the limit that needs no permission
-        if (full)
-            mmnb_prefill_direct_kernel<SG, true><<<g2, dim3(256), prefill_lds(T) / 2, ctx->stream>>>(a);
-        else
-            mmnb_prefill_direct_kernel<SG, false><<<g2, dim3(256), prefill_lds(T) / 2, ctx->stream>>>(a);
-        HIPC_LAUNCHED(ctx);
-    } else
-#endif
-    {
-        if (full)
-            mmnb_prefill_kernel<SG, T, true><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
-        else
-            mmnb_prefill_kernel<SG, T, false><<<g2, dim3(256), prefill_lds(T), ctx->stream>>>(a);
-        HIPC_LAUNCHED(ctx);
-    }
+    *grid = dim3(gx, (unsigned)a.ksplit);
+    return HIPC_OK;
+}
+// the second launch of a k split
+int prefill_join_splits(hipc_ctx *ctx, const PrefillArgs &a) {
     if (a.ksplit > 1) {
         const long total = (long)a.M * a.N;
-        mmnb_prefill_reduce_kernel<<<dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream>>>(a.Ypart, a.Y, a.Yf32, total, a.ksplit);
+        hipLaunchKernelGGL(mmnb_prefill_reduce_kernel, dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit);
         HIPC_LAUNCHED(ctx);
     }
     return HIPC_OK;
+}
+
+// both operands through LDS
+template <int SG, int T>
+int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
+    const bool full = a.K % (2 * kPK) == 0;
+    static bool lds_allowed[2][kMaxDevices] = {};
+    if (int rc = full ? allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, true>, prefill_lds(T), lds_allowed[1])
+                      : allow_dynamic_lds(ctx, mmnb_prefill_kernel<SG, T, false>, prefill_lds(T), lds_allowed[0]))
+        return rc;
+    dim3 grid;
+    if (int rc = prefill_plan(ctx, a, T, T, T == 128, &grid)) return rc;
+    if (full)
+        hipLaunchKernelGGL((mmnb_prefill_kernel<SG, T, true>), grid, dim3(256), prefill_lds(T), ctx->stream, a);
+    else
+        hipLaunchKernelGGL((mmnb_prefill_kernel<SG, T, false>), grid, dim3(256), prefill_lds(T), ctx->stream, a);
+    HIPC_LAUNCHED(ctx);
+    return prefill_join_splits(ctx, a);
+}
+
+// the weight from memory into the operand registers; A alone in LDS (36 KB: inside the limit that needs no permission)
+template <int SG, int NJ>
+int prefill_launch_direct(hipc_ctx *ctx, PrefillArgs a) {
+    const bool full = a.K % (2 * kPK) == 0;
+    dim3 grid;
+    if (int rc = prefill_plan(ctx, a, 128, 64 * NJ, true, &grid)) return rc;
+    if (full)
+        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, NJ, true>), grid, dim3(256), prefill_lds(128) / 2, ctx->stream, a);
+    else
+        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, NJ, false>), grid, dim3(256), prefill_lds(128) / 2, ctx->stream, a);
+    HIPC_LAUNCHED(ctx);
+    return prefill_join_splits(ctx, a);
 }
 
 }  // namespace
@@ -589,16 +632,25 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a, bool direct = false) {
 // scales then multiply them without copies out of the accumulation file: 48.5 -> 44.7 us for
 // 512 x 2048 x 11008); the 64x64 instances are faster with the accumulation file (80.6 against
 // 87.9 us for 512 x 11008 x 2048), and that is a switch of the whole compilation.
-int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG);
+int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG, int tile);
 
 #ifdef HIPC_PREFILL_WIDE
 
-int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG) {
-    const bool direct = ctx->tune.prefill_direct != 0;
+int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG, int tile) {
+    if (tile == 192) switch (SG) {
+            case 4: return prefill_launch_direct<4, 3>(ctx, a);
+            case 2: return prefill_launch_direct<2, 3>(ctx, a);
+            default: return prefill_launch_direct<1, 3>(ctx, a);
+        }
+    if (ctx->tune.prefill_direct != 0) switch (SG) {
+            case 4: return prefill_launch_direct<4, 2>(ctx, a);
+            case 2: return prefill_launch_direct<2, 2>(ctx, a);
+            default: return prefill_launch_direct<1, 2>(ctx, a);
+        }
     switch (SG) {
-        case 4: return prefill_launch_tile<4, 128>(ctx, a, direct);
-        case 2: return prefill_launch_tile<2, 128>(ctx, a, direct);
-        default: return prefill_launch_tile<1, 128>(ctx, a, direct);
+        case 4: return prefill_launch_tile<4, 128>(ctx, a);
+        case 2: return prefill_launch_tile<2, 128>(ctx, a);
+        default: return prefill_launch_tile<1, 128>(ctx, a);
     }
 }
 
@@ -609,14 +661,18 @@ namespace {
 template <int SG>
 int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
     const int forced = ctx->tune.prefill_tile, g_prefill_split = ctx->tune.prefill_split;
-    // 128x128 tiles when they give every CU a workgroup, directly or (long k) with k split over up
+    // 128-row tiles when they give every CU a workgroup, directly or (long k) with k split over up
     // to four workgroups per tile; else 64x64
-    const int64_t tiles128 = ceil_div(a.M, 128) * ceil_div(a.N, 128);
+    const int64_t rows128 = ceil_div(a.M, 128), tiles128 = rows128 * ceil_div(a.N, 128), tiles192 = rows128 * ceil_div(a.N, 192);
     const int nk = (int)ceil_div(a.K, kPK);
     const bool by_split = g_prefill_split != 0 && tiles128 * std::min<int64_t>(4, nk / 32) >= 192;
     int tile = tiles128 >= 256 || by_split ? 128 : 64;
-    if (forced == 64 || forced == 128) tile = forced;
-    return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_wide(ctx, a, SG);
+    // 128x192 where that shortens the longest queue of a SIMD: rounds of workgroups over the CUs times the wavefront's
+    // 32-column blocks (512 x 11008: 344 tiles of 128x128 are two rounds of 2, 232 of 128x192 one round of 3)
+    const int64_t cus = std::max(1, ctx->cu_count);
+    if (tile == 128 && tiles128 >= 256 && ctx->tune.prefill_direct != 0 && ceil_div(tiles192, cus) * 3 < ceil_div(tiles128, cus) * 2) tile = 192;
+    if (forced == 64 || forced == 128 || (forced == 192 && ctx->tune.prefill_direct != 0)) tile = forced;
+    return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_wide(ctx, a, SG, tile);
 }
 
 }  // namespace

@@ -132,8 +132,9 @@ def test_f16_rows_beyond_sixteen_run_the_tiled_kernel(ctx, pkg, oracle, shape):
     assert got.dtype == np.float16 and close(got, want, RTOL16), worst(got, want)
 
 
-WIDE_ROUTES = [  # the 128x128 tiles, forced on shapes that would take 64x64: each kernel, alone and with k split over workgroups
-    {"HIPC_PREFILL_TILE": 128}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2},
+WIDE_ROUTES = [  # the 128-row tiles, forced on shapes that would take 64x64: each kernel, alone and with k split over workgroups
+    {"HIPC_PREFILL_TILE": 192}, {"HIPC_PREFILL_TILE": 192, "HIPC_PREFILL_SPLIT": 2}, {"HIPC_PREFILL_TILE": 128},
+    {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2},
     {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_DIRECT": 0}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_DIRECT": 0, "HIPC_PREFILL_SPLIT": 3},
 ]
 
@@ -153,6 +154,42 @@ def test_both_wide_tile_kernels_on_ragged_shapes(ctx, pkg, oracle, shape, option
         got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
     w.destroy()
     assert got.dtype == np.float16 and close(got, want, RTOL16), worst(got, want)
+
+
+@pytest.mark.parametrize("options", [{"HIPC_PREFILL_TILE": 192}, {"HIPC_PREFILL_TILE": 128}, {"HIPC_PREFILL_TILE": 64}], ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("bs,dtype", [(32, np.float16), (128, np.float16), (64, np.float32)], ids=lambda v: str(getattr(v, "__name__", v)))
+def test_block_scales_of_zero_and_of_very_different_size(ctx, pkg, oracle, bs, dtype, options):
+    """The kernels that keep the weight out of LDS hold their accumulators in units of the open block's scale and
+    rescale them when the next block opens: blocks whose scale is 0 (a block of zeros), 1000 times larger or 10000
+    times smaller than their neighbours must come out as from the running total the other kernels keep (the
+    64x64 tiles are in the list as that control), first block and last block included."""
+    m, k, n = 96, 1024, 200
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=49, with_zp=True, scale_dtype=dtype)
+    sc = scales.reshape(n, -1).copy()
+    sc[:, ::3] = 0
+    sc[:, 1::7] *= dtype(1000)
+    sc[:, 2::5] *= dtype(1e-4)
+    sc[5] = 0                      # a column of zeros
+    sc[6, :-1] = 0                 # only the last block counts
+    sc[7, 1:] = 0                  # only the first
+    scales = sc.reshape(scales.shape)
+    a = pkg.synth.normal_f32(m * k, 50).reshape(m, k).astype(dtype)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    with ctx.options(**options):
+        got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    assert np.all(got[:, 5] == 0)
+    # Scales seven orders of magnitude apart make sums that cancel: against the float64 product, with the f32
+    # accumulation's share stated in units of the row's largest result (the oracle itself is 4e-4 of it away; a
+    # rescaled accumulator rounds once more per block than a running total does)
+    nib, z = _unpack(B, zp, k, n, bs)
+    f64 = rc.matmul_nbits_f64(a, nib, z, scales.reshape(n, -1), bs)
+    big = np.abs(f64).max(axis=1, keepdims=True)
+    err = np.abs(got.astype(np.float64) - f64)
+    if dtype is np.float16:
+        assert np.all(err <= 1e-3 + 1e-3 * np.abs(f64) + 1e-6 * big), float((err - 1e-3 * np.abs(f64)).max())
+    else:   # f32 rows travel as two f16 rows (22 bits): as in the test of that route
+        assert np.all(err <= 2e-5 * big + 1e-3), float((err / big).max())
 
 
 F32_PREFILL = [  # (M, K, N, block_size, zero points)
