@@ -327,9 +327,11 @@ __device__ __forceinline__ uint32_t word_of(const uint4 &v, int j) { return j ==
 // NJ: 32-column blocks per wavefront. 2: a 128x128 tile. 3: a 128x192 tile -- a third less LDS traffic per product,
 // and a matrix of 512 x 11008 becomes 232 workgroups for 256 CUs where 128x128 tiles make 344, two of them on every
 // third CU.
-template <int SG, int NJ, bool FULL>
-__global__ void __launch_bounds__(256, NJ == 2 ? 2 : 1) mmnb_prefill_direct_kernel(const PrefillArgs p) {
-    constexpr int T = 128, TN = 64 * NJ, kChunks = T / 32, kF = 2, kWT = 64, kWN = 32 * NJ;
+// MI: 32-row blocks per wavefront. 2 with the tiles above; 1 with NJ 1 is a 64x64 tile for matrices that have too few
+// of the large ones (four wavefronts of 32x32: a conversion per product, but many short wavefronts per SIMD).
+template <int SG, int MI, int NJ, bool FULL>
+__global__ void __launch_bounds__(256, MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) mmnb_prefill_direct_kernel(const PrefillArgs p) {
+    constexpr int T = 64 * MI, TN = 64 * NJ, kChunks = T / 32, kF = MI, kWT = 32 * MI, kWN = 32 * NJ;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     uint8_t *lds_a = lds_raw;  // [2][T * kPPitch]
 
@@ -533,12 +535,28 @@ __global__ void __launch_bounds__(256, NJ == 2 ? 2 : 1) mmnb_prefill_direct_kern
     prefill_store<kF, NJ>(p, acc, i0 + wm * kWT, j0 + wn * kWN, r32, kg);
 }
 
-// Y = f16(sum over splits of the f32 partials), in split order; or the f32 sum itself into Yf32
-// (static: this file is compiled twice)
+// Y = f16(sum over splits of the f32 partials), in split order; or the f32 sum itself into Yf32. Four results per
+// thread; VEC: the element count is a multiple of four and the rows are aligned for 16-byte loads and one 8- or
+// 16-byte store. (static: this file is compiled twice)
+template <bool VEC>
 static __global__ void __launch_bounds__(256)
 mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ Y, float *__restrict__ Yf32, long total, int ksplit) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= total) return;
+    if (VEC) {
+        float4 v = *reinterpret_cast<const float4 *>(part + i);
+        for (int s = 1; s < ksplit; s++) {
+            const float4 u = *reinterpret_cast<const float4 *>(part + (size_t)s * total + i);
+            v.x += u.x, v.y += u.y, v.z += u.z, v.w += u.w;
+        }
+        if (Yf32) {
+            *reinterpret_cast<float4 *>(Yf32 + i) = v;
+        } else {
+            const __half2 lo = __halves2half2(__float2half(v.x), __float2half(v.y)), hi = __halves2half2(__float2half(v.z), __float2half(v.w));
+            *reinterpret_cast<uint2 *>(Y + i) = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+        }
+        return;
+    }
     for (long j = i; j < min(i + 4, total); j++) {
         float v = part[j];
         for (int s = 1; s < ksplit; s++) v += part[(size_t)s * total + j];
@@ -587,7 +605,11 @@ int prefill_plan(hipc_ctx *ctx, PrefillArgs &a, int TM, int TN, bool may_split, 
 int prefill_join_splits(hipc_ctx *ctx, const PrefillArgs &a) {
     if (a.ksplit > 1) {
         const long total = (long)a.M * a.N;
-        hipLaunchKernelGGL(mmnb_prefill_reduce_kernel, dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit);
+        const bool vec = total % 4 == 0 && (a.Yf32 ? aligned(a.Yf32, 16) : aligned(a.Y, 8));
+        if (vec)
+            hipLaunchKernelGGL((mmnb_prefill_reduce_kernel<true>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit);
+        else
+            hipLaunchKernelGGL((mmnb_prefill_reduce_kernel<false>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit);
         HIPC_LAUNCHED(ctx);
     }
     return HIPC_OK;
@@ -611,16 +633,16 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
     return prefill_join_splits(ctx, a);
 }
 
-// the weight from memory into the operand registers; A alone in LDS (36 KB: inside the limit that needs no permission)
-template <int SG, int NJ>
+// the weight from memory into the operand registers; A alone in LDS (at most 36 KB: inside the limit that needs no permission)
+template <int SG, int MI, int NJ>
 int prefill_launch_direct(hipc_ctx *ctx, PrefillArgs a) {
     const bool full = a.K % (2 * kPK) == 0;
     dim3 grid;
-    if (int rc = prefill_plan(ctx, a, 128, 64 * NJ, true, &grid)) return rc;
+    if (int rc = prefill_plan(ctx, a, 64 * MI, 64 * NJ, MI == 2, &grid)) return rc;
     if (full)
-        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, NJ, true>), grid, dim3(256), prefill_lds(128) / 2, ctx->stream, a);
+        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, MI, NJ, true>), grid, dim3(256), prefill_lds(64 * MI) / 2, ctx->stream, a);
     else
-        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, NJ, false>), grid, dim3(256), prefill_lds(128) / 2, ctx->stream, a);
+        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, MI, NJ, false>), grid, dim3(256), prefill_lds(64 * MI) / 2, ctx->stream, a);
     HIPC_LAUNCHED(ctx);
     return prefill_join_splits(ctx, a);
 }
@@ -638,14 +660,19 @@ int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG, int tile);
 
 int prefill_launch_wide(hipc_ctx *ctx, const PrefillArgs &a, int SG, int tile) {
     if (tile == 192) switch (SG) {
-            case 4: return prefill_launch_direct<4, 3>(ctx, a);
-            case 2: return prefill_launch_direct<2, 3>(ctx, a);
-            default: return prefill_launch_direct<1, 3>(ctx, a);
+            case 4: return prefill_launch_direct<4, 2, 3>(ctx, a);
+            case 2: return prefill_launch_direct<2, 2, 3>(ctx, a);
+            default: return prefill_launch_direct<1, 2, 3>(ctx, a);
+        }
+    if (tile == 64) switch (SG) {
+            case 4: return prefill_launch_direct<4, 1, 1>(ctx, a);
+            case 2: return prefill_launch_direct<2, 1, 1>(ctx, a);
+            default: return prefill_launch_direct<1, 1, 1>(ctx, a);
         }
     if (ctx->tune.prefill_direct != 0) switch (SG) {
-            case 4: return prefill_launch_direct<4, 2>(ctx, a);
-            case 2: return prefill_launch_direct<2, 2>(ctx, a);
-            default: return prefill_launch_direct<1, 2>(ctx, a);
+            case 4: return prefill_launch_direct<4, 2, 2>(ctx, a);
+            case 2: return prefill_launch_direct<2, 2, 2>(ctx, a);
+            default: return prefill_launch_direct<1, 2, 2>(ctx, a);
         }
     switch (SG) {
         case 4: return prefill_launch_tile<4, 128>(ctx, a);
@@ -672,7 +699,7 @@ int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
     const int64_t cus = std::max(1, ctx->cu_count);
     if (tile == 128 && tiles128 >= 256 && ctx->tune.prefill_direct != 0 && ceil_div(tiles192, cus) * 3 < ceil_div(tiles128, cus) * 2) tile = 192;
     if (forced == 64 || forced == 128 || (forced == 192 && ctx->tune.prefill_direct != 0)) tile = forced;
-    return tile == 64 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_wide(ctx, a, SG, tile);
+    return tile == 64 && ctx->tune.prefill_direct == 0 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_wide(ctx, a, SG, tile);
 }
 
 }  // namespace
@@ -701,9 +728,21 @@ static __global__ void __launch_bounds__(256)
 mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half *__restrict__ A2, int *__restrict__ exps) {
     __shared__ float red[4];
     const int m = blockIdx.x, tid = threadIdx.x;
-    const float *row = A + (size_t)m * K;
+    const float4 *row = reinterpret_cast<const float4 *>(A + (size_t)m * K);   // (K is a multiple of 8 and A is aligned: see nbits_prefill_f32_takes)
+    const int nv = K / 4;
+    constexpr int kHeld = 4;   // 16-byte pieces a thread keeps between the two passes: rows up to 4096 values are read once
+    float4 held[kHeld];
     float mx = 0.f;
-    for (int k = tid; k < K; k += 256) mx = fmaxf(mx, fabsf(row[k]));   // (a NaN does not raise the maximum: it passes through below)
+#pragma unroll
+    for (int u = 0; u < kHeld; u++) {
+        const int c = tid + 256 * u;
+        held[u] = c < nv ? row[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(held[u].x), fabsf(held[u].y)), fmaxf(fabsf(held[u].z), fabsf(held[u].w))));   // (a NaN does not raise the maximum: it passes through below)
+    }
+    for (int c = tid + 256 * kHeld; c < nv; c += 256) {
+        const float4 v = row[c];
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
     if ((tid & 63) == 0) red[tid >> 6] = mx;
@@ -714,20 +753,33 @@ mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half
     const int e = (ef == 0 || ef == 255) ? 0 : ef - 127 - 14;
     if (tid == 0) exps[m] = e;
     const float down = __uint_as_float((uint32_t)(127 - e) << 23);   // 2^-e: e is in [-140, 113], 2^-e a normal number
-    for (int k = tid; k < K; k += 256) {
-        const float a = row[k] * down;
-        const __half hi = __float2half(a);
-        A2[(size_t)m * K + k] = hi;
-        A2[(size_t)(M + m) * K + k] = __float2half(a - __half2float(hi));
-    }
+    uint2 *hi_row = reinterpret_cast<uint2 *>(A2 + (size_t)m * K), *lo_row = reinterpret_cast<uint2 *>(A2 + (size_t)(M + m) * K);
+    auto split4 = [&](const float4 &v, int c) {
+        const float a[4] = {v.x * down, v.y * down, v.z * down, v.w * down};
+        __half hi[4], lo[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) hi[t] = __float2half(a[t]), lo[t] = __float2half(a[t] - __half2float(hi[t]));
+        hi_row[c] = make_uint2(__builtin_bit_cast(uint32_t, __halves2half2(hi[0], hi[1])), __builtin_bit_cast(uint32_t, __halves2half2(hi[2], hi[3])));
+        lo_row[c] = make_uint2(__builtin_bit_cast(uint32_t, __halves2half2(lo[0], lo[1])), __builtin_bit_cast(uint32_t, __halves2half2(lo[2], lo[3])));
+    };
+#pragma unroll
+    for (int u = 0; u < kHeld; u++)
+        if (tid + 256 * u < nv) split4(held[u], tid + 256 * u);
+    for (int c = tid + 256 * kHeld; c < nv; c += 256) split4(row[c], c);
 }
 // Y[m] = (P[m] + P[M + m]) 2^e[m]
+template <bool VEC>   // VEC: N is a multiple of four and Y is aligned for 16-byte stores
 static __global__ void __launch_bounds__(256)
 mmnb_prefill_join_rows_kernel(const float *__restrict__ P, const int *__restrict__ exps, int M, int N, float *__restrict__ Y) {
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * (VEC ? 4 : 1);
     if (i >= (long)M * N) return;
-    const int m = (int)(i / N);
-    Y[i] = ldexpf(P[i] + P[i + (long)M * N], exps[m]);
+    const int e = exps[(int)(i / N)];
+    if (VEC) {
+        const float4 a = *reinterpret_cast<const float4 *>(P + i), b = *reinterpret_cast<const float4 *>(P + i + (long)M * N);
+        *reinterpret_cast<float4 *>(Y + i) = make_float4(ldexpf(a.x + b.x, e), ldexpf(a.y + b.y, e), ldexpf(a.z + b.z, e), ldexpf(a.w + b.w, e));
+    } else {
+        Y[i] = ldexpf(P[i] + P[i + (long)M * N], e);
+    }
 }
 
 // Many rows of f32 activations: each row as two f16 rows (22 bits) through the same tiled kernel, 2 M rows
@@ -745,7 +797,7 @@ int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, 
     if (int rc = scratch_get(ctx, 3, (size_t)2 * M * w->N * sizeof(float), &sums)) return rc;
     __half *A2 = reinterpret_cast<__half *>(static_cast<char *>(split) + e_bytes);
     int *exps = static_cast<int *>(split);
-    mmnb_prefill_split_rows_kernel<<<dim3((unsigned)M), dim3(256), 0, ctx->stream>>>(static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
+    hipLaunchKernelGGL(mmnb_prefill_split_rows_kernel, dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
     HIPC_LAUNCHED(ctx);
     PrefillArgs a{};
     a.A = A2, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = nullptr, a.Yf32 = static_cast<float *>(sums);
@@ -758,8 +810,10 @@ int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, 
     }
     if (rc != HIPC_OK) return rc;
     const long total = (long)M * w->N;
-    mmnb_prefill_join_rows_kernel<<<dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream>>>(static_cast<const float *>(sums), exps, (int)M, (int)w->N,
-                                                                                                      static_cast<float *>(Y));
+    if (w->N % 4 == 0 && aligned(Y, 16))
+        hipLaunchKernelGGL((mmnb_prefill_join_rows_kernel<true>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, static_cast<const float *>(sums), exps, (int)M, (int)w->N, static_cast<float *>(Y));
+    else
+        hipLaunchKernelGGL((mmnb_prefill_join_rows_kernel<false>), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream, static_cast<const float *>(sums), exps, (int)M, (int)w->N, static_cast<float *>(Y));
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }
