@@ -51,6 +51,11 @@ struct PrefillArgs {
     float *Yf32;   // when set, the result is written here as f32 and Y is not used (rows of f32 activations, see nbits_prefill_f32)
 };
 
+// two f16 values as one word, the first in the low half
+__device__ __forceinline__ uint32_t two_halves(__half lo, __half hi) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+}
+
 // eight nibbles (order k0 k2 k4 k6 k1 k3 k5 k7) -> eight f16 values q - zp in k order, as four words of pairs
 __device__ __forceinline__ uint4 dequant8(uint32_t w, uint32_t zb) {
     // 1024 + zp in both halves; zb carries 128 + zp
@@ -456,7 +461,9 @@ __global__ void __launch_bounds__(256, MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) 
     };
 
     uint32_t ones = 0x64006400u;   // kept in a vector register (see and_or_1024)
+#ifndef HIPC_HOST_MODEL
     asm volatile("" : "+v"(ones));
+#endif
     // One stage = 64 k = the k steps (j, h) with j = 2 half + 0 / 1 of the weight tile the stage lies in;
     // a scale group opens at every second step (SG 4), every stage (SG 2) or every even stage (SG 1).
     auto compute = [&](const BRegs &b, int buf, int half) {   // (b.s holds ratios by now)
@@ -552,8 +559,7 @@ mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ 
         if (Yf32) {
             *reinterpret_cast<float4 *>(Yf32 + i) = v;
         } else {
-            const __half2 lo = __halves2half2(__float2half(v.x), __float2half(v.y)), hi = __halves2half2(__float2half(v.z), __float2half(v.w));
-            *reinterpret_cast<uint2 *>(Y + i) = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+            *reinterpret_cast<uint2 *>(Y + i) = make_uint2(two_halves(__float2half(v.x), __float2half(v.y)), two_halves(__float2half(v.z), __float2half(v.w)));
         }
         return;
     }
@@ -759,8 +765,8 @@ mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half
         __half hi[4], lo[4];
 #pragma unroll
         for (int t = 0; t < 4; t++) hi[t] = __float2half(a[t]), lo[t] = __float2half(a[t] - __half2float(hi[t]));
-        hi_row[c] = make_uint2(__builtin_bit_cast(uint32_t, __halves2half2(hi[0], hi[1])), __builtin_bit_cast(uint32_t, __halves2half2(hi[2], hi[3])));
-        lo_row[c] = make_uint2(__builtin_bit_cast(uint32_t, __halves2half2(lo[0], lo[1])), __builtin_bit_cast(uint32_t, __halves2half2(lo[2], lo[3])));
+        hi_row[c] = make_uint2(two_halves(hi[0], hi[1]), two_halves(hi[2], hi[3]));
+        lo_row[c] = make_uint2(two_halves(lo[0], lo[1]), two_halves(lo[2], lo[3]));
     };
 #pragma unroll
     for (int u = 0; u < kHeld; u++)

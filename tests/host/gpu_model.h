@@ -137,6 +137,9 @@ inline void gpu_model_nt_store(U v, T *p) { *p = v; }
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16 gpu_model_mfma
 #define __builtin_amdgcn_mfma_f32_16x16x32_f16 gpu_model_mfma
 #define __builtin_amdgcn_mfma_i32_32x32x32_i8 gpu_model_mfma
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16 gpu_model_mfma
+inline float gpu_model_rcp(float v) { return 1.f / v; }
+#define __builtin_amdgcn_rcpf gpu_model_rcp
 inline int gpu_model_sdot4(int, int, int c, bool) { return c; }
 #define __builtin_amdgcn_sdot4 gpu_model_sdot4
 inline uint32_t gpu_model_perm(uint32_t a, uint32_t, uint32_t) { return a; }

@@ -213,3 +213,7 @@ def test_kernel_addresses_on_the_cpu_model(tmp_path):
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
     run = subprocess.run([os.path.join(out, "int8_model")], capture_output=True, text=True, env=env)
     assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout[-2000:] + run.stderr[-2000:]
+    # and the tiled MatMulNBits kernels' (tests/host/prefill_model.cpp): every instance, scale grouping and k split,
+    # f16 and f32 rows, on ragged shapes with operands of exactly the operator's size
+    run = subprocess.run([os.path.join(out, "prefill_model")], capture_output=True, text=True, env=env)
+    assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout[-2000:] + run.stderr[-2000:]
