@@ -107,6 +107,7 @@ const OptionName kOptions[] = {
     {"HIPC_PREFILL_TILE", &Tuning::prefill_tile},
     {"HIPC_PREFILL_SPLIT", &Tuning::prefill_split},
     {"HIPC_PREFILL_DIRECT", &Tuning::prefill_direct},
+    {"HIPC_PREFILL_GROUPS", &Tuning::prefill_groups},
     {"HIPC_DEC_FUSED_GLUE", &Tuning::dec_fused_glue},
     {"HIPC_DEC_FUSED_ATTN", &Tuning::dec_fused_attn},
     {"HIPC_GEMV_LEAN", &Tuning::gemv_lean},

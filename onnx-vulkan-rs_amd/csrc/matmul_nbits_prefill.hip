@@ -334,13 +334,19 @@ __device__ __forceinline__ uint32_t word_of(const uint4 &v, int j) { return j ==
 // third CU.
 // MI: 32-row blocks per wavefront. 2 with the tiles above; 1 with NJ 1 is a 64x64 tile for matrices that have too few
 // of the large ones (four wavefronts of 32x32: a conversion per product, but many short wavefronts per SIMD).
-template <int SG, int MI, int NJ, bool FULL>
-__global__ void __launch_bounds__(256, MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) mmnb_prefill_direct_kernel(const PrefillArgs p) {
+// KG: groups of four wavefronts per workgroup. With 2 (512 threads; MI 2 only) each group takes half of the
+// workgroup's k range with LDS buffers of its own, and the two sets of accumulators are added through LDS at the end
+// (each group hands over the 32-row blocks the other one stores). For launches that put one workgroup on a CU: a
+// second wavefront per SIMD issues while the first waits for LDS, a barrier or the matrix core.
+template <int SG, int MI, int NJ, int KG, bool FULL>
+__global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) mmnb_prefill_direct_kernel(const PrefillArgs p) {
+    static_assert(KG == 1 || MI == 2, "two k groups hand over one of two row blocks");
     constexpr int T = 64 * MI, TN = 64 * NJ, kChunks = T / 32, kF = MI, kWT = 32 * MI, kWN = 32 * NJ;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    uint8_t *lds_a = lds_raw;  // [2][T * kPPitch]
+    const int grp = KG == 2 ? (int)(threadIdx.x >> 8) : 0;
+    uint8_t *lds_a = lds_raw + grp * 2 * T * kPPitch;  // [KG][2][T * kPPitch]
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x & 255;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int r32 = lane & 31, kg = lane >> 5;
@@ -377,7 +383,7 @@ __global__ void __launch_bounds__(256, MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) 
     };
     // a stage past the end reads clamped addresses and stores zeros for A: it adds nothing
     auto store_a = [&](const ARegs &r, int buf, bool live) {
-        const uint32_t keep = FULL || live ? 0xffffffffu : 0u;
+        const uint32_t keep = (FULL && KG == 1) || live ? 0xffffffffu : 0u;
 #pragma unroll
         for (int u = 0; u < kChunks; u++)
             *reinterpret_cast<uint4 *>(lds_a + buf * T * kPPitch + a_lds[u]) =
@@ -500,14 +506,19 @@ __global__ void __launch_bounds__(256, MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) 
     };
 
     const int nk_all = (p.K + kPK - 1) / kPK;
-    const int ks0 = blockIdx.y * p.split_stages, nk = min(nk_all, ks0 + p.split_stages);  // this workgroup's stages (ks0 is even)
-    const int cg_last = (nk - 1) >> 1;
+    const int wg_ks0 = blockIdx.y * p.split_stages, wg_nk = min(nk_all, wg_ks0 + p.split_stages);  // this workgroup's stages (wg_ks0 is even)
+    // ... and this group's: with two groups the first takes the larger half of the trips; both run as many trips as
+    // the first (the barriers are the workgroup's), the second's last one, if it has one less, on zeros
+    const int wg_trips = (wg_nk - wg_ks0 + 1) >> 1, my_trips = (wg_trips + KG - 1) / KG;
+    const int ks0 = wg_ks0 + grp * 2 * my_trips, nk = KG == 2 && grp == 0 ? min(wg_nk, ks0 + 2 * my_trips) : wg_nk;
+    const int last = min(wg_nk - 1, max(nk - 1, wg_ks0));   // the last stage whose addresses this group may form
+    const int cg_last = last >> 1;
     ARegs r0, r1;
     BRegs bc, bn;
-    load_b(bc, ks0 >> 1);
-    load_a(r0, ks0);
-    load_a(r1, min(ks0 + 1, nk - 1));
-    store_a(r0, 0, true);
+    load_b(bc, min(ks0, last) >> 1);
+    load_a(r0, min(ks0, last));
+    load_a(r1, min(ks0 + 1, last));
+    store_a(r0, 0, ks0 < nk);
     __syncthreads();
     // two stages = one weight tile per trip; with an odd stage count the second half of the last trip multiplies
     // a stage whose A is all zeros. (The fences keep the order written here: left alone, the compiler moves the
@@ -515,23 +526,23 @@ __global__ void __launch_bounds__(256, MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) 
     // them, and every half trip then waits out a whole trip to memory.)
     auto trip = [&](BRegs &bcur, BRegs &bnext, int ks) {
         load_b(bnext, min((ks >> 1) + 1, cg_last));
-        load_a(r0, min(ks + 2, nk - 1));
+        load_a(r0, min(ks + 2, last));
         scales_to_ratios(bcur);
         __builtin_amdgcn_sched_barrier(0);
         compute(bcur, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         store_a(r1, 1, ks + 1 < nk);
         __syncthreads();
-        load_a(r1, min(ks + 3, nk - 1));
+        load_a(r1, min(ks + 3, last));
         __builtin_amdgcn_sched_barrier(0);
         compute(bcur, 1, 1);
         __builtin_amdgcn_sched_barrier(0);
-        store_a(r0, 0, true);
+        store_a(r0, 0, ks + 2 < nk);
         __syncthreads();
     };
-    for (int ks = ks0; ks < nk; ks += 4) {   // the two register sets of the weight take turns
-        trip(bc, bn, ks);
-        if (ks + 2 < nk) trip(bn, bc, ks + 2);
+    for (int t = 0; t < my_trips; t += 2) {   // the two register sets of the weight take turns
+        trip(bc, bn, ks0 + 2 * t);
+        if (t + 1 < my_trips) trip(bn, bc, ks0 + 2 * t + 2);
     }
 #pragma unroll
     for (int j = 0; j < NJ; j++)
@@ -539,7 +550,35 @@ __global__ void __launch_bounds__(256, MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) 
         for (int i = 0; i < kF; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] *= scaled[j] ? unit[j] : 0.f;
-    prefill_store<kF, NJ>(p, acc, i0 + wm * kWT, j0 + wn * kWN, r32, kg);
+    if constexpr (KG == 2) {
+        // group g keeps row block g and hands the other one over: [group][16-byte piece][thread] in LDS (the A
+        // buffers are done with: the last barrier of the loop is behind every read of them)
+        float4 *mine = reinterpret_cast<float4 *>(lds_raw) + grp * (NJ * 4 * 256), *theirs = reinterpret_cast<float4 *>(lds_raw) + (grp ^ 1) * (NJ * 4 * 256);
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const f32x16 &v = grp == 0 ? acc[1][j] : acc[0][j];
+                mine[(j * 4 + q) * 256 + tid] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+            }
+        __syncthreads();
+        f32x16 sum[1][NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float4 o = theirs[(j * 4 + q) * 256 + tid];
+                const f32x16 &v = grp == 0 ? acc[0][j] : acc[1][j];
+                // (first group's share + second group's share, whichever of them adds)
+                sum[0][j][4 * q] = grp == 0 ? v[4 * q] + o.x : o.x + v[4 * q];
+                sum[0][j][4 * q + 1] = grp == 0 ? v[4 * q + 1] + o.y : o.y + v[4 * q + 1];
+                sum[0][j][4 * q + 2] = grp == 0 ? v[4 * q + 2] + o.z : o.z + v[4 * q + 2];
+                sum[0][j][4 * q + 3] = grp == 0 ? v[4 * q + 3] + o.w : o.w + v[4 * q + 3];
+            }
+        prefill_store<1, NJ>(p, sum, i0 + wm * kWT + grp * 32, j0 + wn * kWN, r32, kg);
+    } else {
+        prefill_store<kF, NJ>(p, acc, i0 + wm * kWT, j0 + wn * kWN, r32, kg);
+    }
 }
 
 // Y = f16(sum over splits of the f32 partials), in split order; or the f32 sum itself into Yf32. Four results per
@@ -639,17 +678,42 @@ int prefill_launch_tile(hipc_ctx *ctx, PrefillArgs a) {
     return prefill_join_splits(ctx, a);
 }
 
-// the weight from memory into the operand registers; A alone in LDS (at most 36 KB: inside the limit that needs no permission)
+// the weight from memory into the operand registers; A alone in LDS
+template <int SG, int MI, int NJ, int KG>
+int prefill_launch_direct_groups(hipc_ctx *ctx, const PrefillArgs &a, dim3 grid) {
+    const bool full = a.K % (2 * kPK) == 0;
+    // one group: at most 36 KB, inside the limit that needs no permission; two: their A buffers, then the hand-over
+    constexpr size_t lds = KG == 1 ? prefill_lds(64 * MI) / 2 : std::max(prefill_lds(64 * MI), (size_t)2 * NJ * 4 * 256 * 16);
+    if (KG == 2) {
+        static bool lds_allowed[2][kMaxDevices] = {};
+        if (int rc = full ? allow_dynamic_lds(ctx, mmnb_prefill_direct_kernel<SG, MI, NJ, KG, true>, lds, lds_allowed[1])
+                          : allow_dynamic_lds(ctx, mmnb_prefill_direct_kernel<SG, MI, NJ, KG, false>, lds, lds_allowed[0]))
+            return rc;
+    }
+    if (full)
+        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, MI, NJ, KG, true>), grid, dim3(256 * KG), lds, ctx->stream, a);
+    else
+        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, MI, NJ, KG, false>), grid, dim3(256 * KG), lds, ctx->stream, a);
+    HIPC_LAUNCHED(ctx);
+    return HIPC_OK;
+}
 template <int SG, int MI, int NJ>
 int prefill_launch_direct(hipc_ctx *ctx, PrefillArgs a) {
-    const bool full = a.K % (2 * kPK) == 0;
     dim3 grid;
     if (int rc = prefill_plan(ctx, a, 64 * MI, 64 * NJ, MI == 2, &grid)) return rc;
-    if (full)
-        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, MI, NJ, true>), grid, dim3(256), prefill_lds(64 * MI) / 2, ctx->stream, a);
-    else
-        hipLaunchKernelGGL((mmnb_prefill_direct_kernel<SG, MI, NJ, false>), grid, dim3(256), prefill_lds(64 * MI) / 2, ctx->stream, a);
-    HIPC_LAUNCHED(ctx);
+    if constexpr (MI == 2) {
+        // Two k groups per workgroup when the launch leaves the second wavefront slot of the SIMDs empty (no more
+        // workgroups than CUs) and every group gets two trips or more; prefill_groups 1 / 2 forces the choice.
+        const int trips = (a.split_stages + 1) / 2, forced = ctx->tune.prefill_groups;
+        const long wgs = (long)ceil_div(a.M, 64 * MI) * ceil_div(a.N, 64 * NJ) * a.ksplit;
+        // (three column blocks and two groups leave no register for more than one scale per weight tile)
+        const bool two = (NJ == 2 || SG == 1) && (forced == 1 ? false : forced == 2 ? true : wgs <= ctx->cu_count && trips >= 4);
+        if constexpr (NJ == 2 || SG == 1) if (two) {
+            if (int rc = prefill_launch_direct_groups<SG, MI, NJ, 2>(ctx, a, grid)) return rc;
+            return prefill_join_splits(ctx, a);
+        }
+    }
+    if (int rc = prefill_launch_direct_groups<SG, MI, NJ, 1>(ctx, a, grid)) return rc;
     return prefill_join_splits(ctx, a);
 }
 

@@ -6,7 +6,8 @@
 // Values are not checked here (the matrix cores are stubs): parity is the GPU tests' business.
 //
 //   prefill_model   every instance (64x64, 128x128 and 128x192 tiles with the weight read into operand registers,
-//                   64x64 and 128x128 with both operands through LDS), every scale grouping, k split 1 / 2 / 3 ways,
+//                   one or two groups of wavefronts per workgroup; 64x64 and 128x128 with both operands through LDS),
+//                   every scale grouping, k split 1 / 2 / 3 ways,
 //                   f16 rows and f32 rows, on ragged and aligned shapes.
 #include <cstdio>
 #include <cstring>
@@ -56,9 +57,10 @@ hipc_ctx ctx;
 size_t prefill_launches = 0;
 
 struct Route {
-    int tile, direct, split;   // HIPC_PREFILL_TILE, HIPC_PREFILL_DIRECT, HIPC_PREFILL_SPLIT (-1: the library's choice)
+    int tile, direct, split, groups;   // HIPC_PREFILL_TILE, _DIRECT, _SPLIT, _GROUPS (-1: the library's choice)
 };
-const Route kRoutes[] = {{-1, -1, -1}, {64, -1, -1}, {64, 0, -1}, {128, -1, 0}, {128, -1, 2}, {128, 0, 3}, {128, 0, 0}, {192, -1, 0}, {192, -1, 2}, {192, -1, 3}};
+const Route kRoutes[] = {{-1, -1, -1, -1}, {64, -1, -1, -1}, {64, 0, -1, -1},  {128, -1, 0, 1},  {128, -1, 2, 1}, {128, 0, 3, -1}, {128, 0, 0, -1},
+                         {192, -1, 0, 1},  {192, -1, 2, 1},  {192, -1, 3, 1},  {128, -1, 0, 2},  {128, -1, 2, 2}, {192, -1, 0, 2},  {192, -1, 3, 2}};
 
 void product(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dtype) {
     const int64_t nb = (K + bs - 1) / bs;
@@ -70,14 +72,14 @@ void product(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dt
     void *A = gpu_model::alloc((size_t)(M * K) * esz), *Y = gpu_model::alloc((size_t)(M * N) * esz);
     std::memset(A, 0, (size_t)(M * K) * esz);
     for (const Route &r : kRoutes) {
-        ctx.tune.prefill_tile = r.tile, ctx.tune.prefill_direct = r.direct, ctx.tune.prefill_split = r.split;
+        ctx.tune.prefill_tile = r.tile, ctx.tune.prefill_direct = r.direct, ctx.tune.prefill_split = r.split, ctx.tune.prefill_groups = r.groups;
         char where[160];
-        std::snprintf(where, sizeof where, "%lld x %lld x %lld block %lld %s, tile %d direct %d split %d", (long long)M, (long long)K, (long long)N, (long long)bs,
-                      a_dtype == HIPC_F16 ? "f16" : "f32", r.tile, r.direct, r.split);
+        std::snprintf(where, sizeof where, "%lld x %lld x %lld block %lld %s, tile %d direct %d split %d groups %d", (long long)M, (long long)K, (long long)N, (long long)bs,
+                      a_dtype == HIPC_F16 ? "f16" : "f32", r.tile, r.direct, r.split, r.groups);
         gpu_model::reg().where = where;
         MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 0));
     }
-    ctx.tune.prefill_tile = ctx.tune.prefill_direct = ctx.tune.prefill_split = -1;
+    ctx.tune.prefill_tile = ctx.tune.prefill_direct = ctx.tune.prefill_split = ctx.tune.prefill_groups = -1;
     gpu_model::release(A), gpu_model::release(Y);
     hipc_nbits_weight_destroy(&ctx, w);
     for (void *p : ctx.deferred) gpu_model::release(p);
@@ -103,7 +105,7 @@ int main() {
     }
     gpu_model::Registry &g = gpu_model::reg();
     std::printf("%zu launches (%zu of the tiled kernels and their helpers), %zu threads\n", g.launches, prefill_launches, g.threads);
-    if (prefill_launches < 200) {
+    if (prefill_launches < 300) {
         std::printf("FAILED: the tiled kernels were not reached\n");
         return 1;
     }

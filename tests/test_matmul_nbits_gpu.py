@@ -137,6 +137,9 @@ WIDE_ROUTES = [  # the 128-row tiles, forced on shapes that would take 64x64: ea
     {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2},
     {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_DIRECT": 0}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_DIRECT": 0, "HIPC_PREFILL_SPLIT": 3},
     {"HIPC_PREFILL_TILE": 64}, {"HIPC_PREFILL_TILE": 64, "HIPC_PREFILL_DIRECT": 0},
+    # two groups of four wavefronts per workgroup, each with half of k (a group without a trip of its own among them)
+    {"HIPC_PREFILL_TILE": 192, "HIPC_PREFILL_GROUPS": 2}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 2},
+    {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 2, "HIPC_PREFILL_SPLIT": 2}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 1},
 ]
 
 
@@ -157,7 +160,8 @@ def test_both_wide_tile_kernels_on_ragged_shapes(ctx, pkg, oracle, shape, option
     assert got.dtype == np.float16 and close(got, want, RTOL16), worst(got, want)
 
 
-@pytest.mark.parametrize("options", [{"HIPC_PREFILL_TILE": 192}, {"HIPC_PREFILL_TILE": 128}, {"HIPC_PREFILL_TILE": 64}, {"HIPC_PREFILL_TILE": 64, "HIPC_PREFILL_DIRECT": 0}], ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("options", [{"HIPC_PREFILL_TILE": 192}, {"HIPC_PREFILL_TILE": 128}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 2}, {"HIPC_PREFILL_TILE": 64},
+                                     {"HIPC_PREFILL_TILE": 64, "HIPC_PREFILL_DIRECT": 0}], ids=lambda v: str(v).replace(" ", ""))
 @pytest.mark.parametrize("bs,dtype", [(32, np.float16), (128, np.float16), (64, np.float32)], ids=lambda v: str(getattr(v, "__name__", v)))
 def test_block_scales_of_zero_and_of_very_different_size(ctx, pkg, oracle, bs, dtype, options):
     """The kernels that keep the weight out of LDS hold their accumulators in units of the open block's scale and
