@@ -183,7 +183,11 @@ void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w);
 size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w);
 /* MatMulNBits on a prepacked weight. `accuracy_level` as in the operator: 0 (unset), 2 or 3 let
  * f32 activations enter the matrix cores as two bf16 terms (16 significant bits, less error than
- * f32 accumulation over K adds); 1 pins f32 and uses three terms (all 24 bits); 4 is refused. */
+ * f32 accumulation over K adds); 1 pins f32 and uses three terms (all 24 bits); 4 is refused.
+ * More than 16 rows of f16 (32 of f32) run a tiled matrix-core kernel whose accumulators are kept in
+ * units of the open quantisation block's scale: there a scale of magnitude below 2^-64 counts as
+ * 2^-64 (what such a block adds is below 2^-64 x 15 x sum |a|), and a column whose scales are all
+ * below it is stored as 0. */
 int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w,
                              void *Y, int64_t M, int accuracy_level);
 
