@@ -382,12 +382,14 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI 
         }
     };
     // a stage past the end reads clamped addresses and stores zeros for A: it adds nothing
-    auto store_a = [&](const ARegs &r, int buf, bool live) {
-        const uint32_t keep = (FULL && KG == 1) || live ? 0xffffffffu : 0u;
+    auto store_a = [&](const ARegs &r, int buf, bool live) {   // (`live` is the same for the whole workgroup group: a branch, no masks)
+        if ((FULL && KG == 1) || live) {
 #pragma unroll
-        for (int u = 0; u < kChunks; u++)
-            *reinterpret_cast<uint4 *>(lds_a + buf * T * kPPitch + a_lds[u]) =
-                make_uint4(r.a[u].x & keep, r.a[u].y & keep, r.a[u].z & keep, r.a[u].w & keep);
+            for (int u = 0; u < kChunks; u++) *reinterpret_cast<uint4 *>(lds_a + buf * T * kPPitch + a_lds[u]) = r.a[u];
+        } else {
+#pragma unroll
+            for (int u = 0; u < kChunks; u++) *reinterpret_cast<uint4 *>(lds_a + buf * T * kPPitch + a_lds[u]) = make_uint4(0u, 0u, 0u, 0u);
+        }
     };
 
     // B: column block j of the wavefront = 32 columns = two weight tiles; the lane's column is r32 of the block
@@ -472,18 +474,25 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI 
 #endif
     // One stage = 64 k = the k steps (j, h) with j = 2 half + 0 / 1 of the weight tile the stage lies in;
     // a scale group opens at every second step (SG 4), every stage (SG 2) or every even stage (SG 1).
-    auto compute = [&](const BRegs &b, int buf, int half) {   // (b.s holds ratios by now)
-        const uint8_t *ba = lds_a + buf * T * kPPitch + (wm * kWT + r32) * kPPitch + kg * 32;
-        ZeroPair zp[NJ][SG == 4 ? 2 : 1];
+    // the zero points of a stage as f16 pairs (with one scale group per weight tile: of the whole tile, made once per trip)
+    struct ZeroPairs {
+        ZeroPair at[NJ][SG == 4 ? 2 : 1];
+    };
+    auto zero_pairs = [&](const BRegs &b, int half) {
+        ZeroPairs zp;
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
             if (SG == 4) {
-                zp[j][0] = zero_pair((b.z[j] >> (16 * half)) & 0xffu);
-                zp[j][SG == 4 ? 1 : 0] = zero_pair((b.z[j] >> (16 * half + 8)) & 0xffu);
+                zp.at[j][0] = zero_pair((b.z[j] >> (16 * half)) & 0xffu);
+                zp.at[j][SG == 4 ? 1 : 0] = zero_pair((b.z[j] >> (16 * half + 8)) & 0xffu);
             } else {
-                zp[j][0] = zero_pair(SG == 2 ? (b.z[j] >> (8 * half)) & 0xffu : b.z[j]);
+                zp.at[j][0] = zero_pair(SG == 2 ? (b.z[j] >> (8 * half)) & 0xffu : b.z[j]);
             }
         }
+        return zp;
+    };
+    auto compute = [&](const BRegs &b, const ZeroPairs &zp, int buf, int half) {   // (b.s holds ratios by now)
+        const uint8_t *ba = lds_a + buf * T * kPPitch + (wm * kWT + r32) * kPPitch + kg * 32;
 #pragma unroll
         for (int step = 0; step < 4; step++) {
             const int word = half * 2 + (step >> 1), h = step & 1;
@@ -497,7 +506,7 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI 
 #pragma unroll
             for (int i = 0; i < kF; i++) af[i] = *reinterpret_cast<const f16x8 *>(ba + i * 32 * kPPitch + (step >> 1) * 64 + h * 16);
 #pragma unroll
-            for (int j = 0; j < NJ; j++) wf[j] = dequant_operand(word_of(b.w[j][h], word), zp[j][SG == 4 ? step >> 1 : 0], ones);
+            for (int j = 0; j < NJ; j++) wf[j] = dequant_operand(word_of(b.w[j][h], word), zp.at[j][SG == 4 ? step >> 1 : 0], ones);
 #pragma unroll
             for (int i = 0; i < kF; i++)
 #pragma unroll
@@ -528,14 +537,16 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI 
         load_b(bnext, min((ks >> 1) + 1, cg_last));
         load_a(r0, min(ks + 2, last));
         scales_to_ratios(bcur);
+        ZeroPairs zp = zero_pairs(bcur, 0);
         __builtin_amdgcn_sched_barrier(0);
-        compute(bcur, 0, 0);
+        compute(bcur, zp, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         store_a(r1, 1, ks + 1 < nk);
         __syncthreads();
         load_a(r1, min(ks + 3, last));
+        if (SG != 1) zp = zero_pairs(bcur, 1);
         __builtin_amdgcn_sched_barrier(0);
-        compute(bcur, 1, 1);
+        compute(bcur, zp, 1, 1);
         __builtin_amdgcn_sched_barrier(0);
         store_a(r0, 0, ks + 2 < nk);
         __syncthreads();
