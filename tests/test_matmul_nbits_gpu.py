@@ -243,8 +243,13 @@ def test_prefill_configuration_full_size(ctx, pkg, oracle, kn):
     want = oracle.matmul_nbits(a, B, scales, None, k, n, bs)
     w = pkg.ops.NBitsWeight(ctx, B, scales, None, k, n, bs)
     got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    # linearity in A, a size-independent property: f(2a) == 2 f(a) exactly (a power of two scales every product, every
+    # partial sum and the rounding to a normal f16 alike)
+    got2 = pkg.ops.matmul_nbits(ctx, (2 * a).astype(np.float16), None, None, None, k, n, bs, weight=w)
     w.destroy()
     assert close(got, want, RTOL16), worst(got, want)
+    normal = np.abs(got.astype(np.float32)) >= 2.0 ** -13   # (a subnormal f16 result has no spare bit to double into)
+    assert np.array_equal(got2.astype(np.float32)[normal], 2 * got.astype(np.float32)[normal]) and normal.mean() > 0.99
 
 
 def test_unembedding_width_full_size(ctx, pkg, oracle):
