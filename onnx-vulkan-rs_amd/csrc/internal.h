@@ -56,7 +56,7 @@ struct Tuning {
     int conv_row = -1;        // HIPC_CONV_ROW       0: convolutions along one axis take the general route
     int prefill_tile = -1;    // HIPC_PREFILL_TILE   64, 128 or 192 (columns; 192 has 128 rows)
     int prefill_split = -1;   // HIPC_PREFILL_SPLIT  0 never splits k, n forces n ways
-    int prefill_groups = -1;  // HIPC_PREFILL_GROUPS 1 / 2: groups of four wavefronts per workgroup of the 128-row prefill tiles (2: each takes half of k)
+    int prefill_groups = -1;  // HIPC_PREFILL_GROUPS 1 / 2: groups of four wavefronts per workgroup of the prefill tiles (2: each takes half of k)
     int prefill_direct = -1;  // HIPC_PREFILL_DIRECT 0: 128-row tiles keep the kernel that passes the weight through LDS (and are never 192 wide)
     int dec_fused_glue = -1;  // HIPC_DEC_FUSED_GLUE 0 keeps the separate norm / GELU kernels (read when a decoder is created)
     int dec_fused_attn = -1;  // HIPC_DEC_FUSED_ATTN 0 keeps the three-kernel attention (read when a decoder is created)

@@ -334,16 +334,17 @@ __device__ __forceinline__ uint32_t word_of(const uint4 &v, int j) { return j ==
 // third CU.
 // MI: 32-row blocks per wavefront. 2 with the tiles above; 1 with NJ 1 is a 64x64 tile for matrices that have too few
 // of the large ones (four wavefronts of 32x32: a conversion per product, but many short wavefronts per SIMD).
-// KG: groups of four wavefronts per workgroup. With 2 (512 threads; MI 2 only) each group takes half of the
-// workgroup's k range with LDS buffers of its own, and the two sets of accumulators are added through LDS at the end
-// (each group hands over the 32-row blocks the other one stores). For launches that put one workgroup on a CU: a
-// second wavefront per SIMD issues while the first waits for LDS, a barrier or the matrix core.
+// KG: groups of four wavefronts per workgroup. With 2 (512 threads) each group takes half of the workgroup's k range
+// with LDS buffers of its own, and the two sets of accumulators are added through LDS at the end (128-row tiles: each
+// group hands over the 32-row blocks the other one stores; 64-row tiles: the second hands everything to the first).
+// For launches that leave wavefront slots of the SIMDs empty: a second wavefront issues while the first waits for
+// LDS, a barrier or the matrix core.
 template <int SG, int MI, int NJ, int KG, bool FULL>
-__global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) mmnb_prefill_direct_kernel(const PrefillArgs p) {
-    static_assert(KG == 1 || MI == 2, "two k groups hand over one of two row blocks");
+__global__ void __launch_bounds__(256 * KG, KG > 1 ? 1 : MI * NJ == 1 ? 4 : MI * NJ <= 4 ? 2 : 1) mmnb_prefill_direct_kernel(const PrefillArgs p) {
+    static_assert(KG == 1 || KG == 2, "one or two groups");
     constexpr int T = 64 * MI, TN = 64 * NJ, kChunks = T / 32, kF = MI, kWT = 32 * MI, kWN = 32 * NJ;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    const int grp = KG == 2 ? (int)(threadIdx.x >> 8) : 0;
+    const int grp = KG > 1 ? (int)(threadIdx.x >> 8) : 0;
     uint8_t *lds_a = lds_raw + grp * 2 * T * kPPitch;  // [KG][2][T * kPPitch]
 
     const int tid = threadIdx.x & 255;
@@ -519,7 +520,7 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI 
     // ... and this group's: with two groups the first takes the larger half of the trips; both run as many trips as
     // the first (the barriers are the workgroup's), the second's last one, if it has one less, on zeros
     const int wg_trips = (wg_nk - wg_ks0 + 1) >> 1, my_trips = (wg_trips + KG - 1) / KG;
-    const int ks0 = wg_ks0 + grp * 2 * my_trips, nk = KG == 2 && grp == 0 ? min(wg_nk, ks0 + 2 * my_trips) : wg_nk;
+    const int ks0 = wg_ks0 + grp * 2 * my_trips, nk = KG == 1 ? wg_nk : min(wg_nk, ks0 + 2 * my_trips);
     const int last = min(wg_nk - 1, max(nk - 1, wg_ks0));   // the last stage whose addresses this group may form
     const int cg_last = last >> 1;
     ARegs r0, r1;
@@ -561,7 +562,30 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : MI * NJ == 1 ? 4 : MI 
         for (int i = 0; i < kF; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] *= scaled[j] ? unit[j] : 0.f;
-    if constexpr (KG == 2) {
+    if constexpr (KG > 1 && MI == 1) {
+        // the later groups hand their accumulators to the first: [group - 1][16-byte piece][thread] in LDS (the A
+        // buffers are done with: the last barrier of the loop is behind every read of them), added in group order
+        float4 *slot = reinterpret_cast<float4 *>(lds_raw);
+        if (grp > 0) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    slot[((grp - 1) * NJ * 4 + j * 4 + q) * 256 + tid] = make_float4(acc[0][j][4 * q], acc[0][j][4 * q + 1], acc[0][j][4 * q + 2], acc[0][j][4 * q + 3]);
+        }
+        __syncthreads();
+        if (grp > 0) return;
+#pragma unroll
+        for (int g = 1; g < KG; g++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4 o = slot[((g - 1) * NJ * 4 + j * 4 + q) * 256 + tid];
+                    acc[0][j][4 * q] += o.x, acc[0][j][4 * q + 1] += o.y, acc[0][j][4 * q + 2] += o.z, acc[0][j][4 * q + 3] += o.w;
+                }
+        prefill_store<kF, NJ>(p, acc, i0 + wm * kWT, j0 + wn * kWN, r32, kg);
+    } else if constexpr (KG == 2) {
         // group g keeps row block g and hands the other one over: [group][16-byte piece][thread] in LDS (the A
         // buffers are done with: the last barrier of the loop is behind every read of them)
         float4 *mine = reinterpret_cast<float4 *>(lds_raw) + grp * (NJ * 4 * 256), *theirs = reinterpret_cast<float4 *>(lds_raw) + (grp ^ 1) * (NJ * 4 * 256);
@@ -694,8 +718,8 @@ template <int SG, int MI, int NJ, int KG>
 int prefill_launch_direct_groups(hipc_ctx *ctx, const PrefillArgs &a, dim3 grid) {
     const bool full = a.K % (2 * kPK) == 0;
     // one group: at most 36 KB, inside the limit that needs no permission; two: their A buffers, then the hand-over
-    constexpr size_t lds = KG == 1 ? prefill_lds(64 * MI) / 2 : std::max(prefill_lds(64 * MI), (size_t)2 * NJ * 4 * 256 * 16);
-    if (KG == 2) {
+    constexpr size_t lds = KG == 1 ? prefill_lds(64 * MI) / 2 : std::max(KG * prefill_lds(64 * MI) / 2, (size_t)(MI == 2 ? 2 : KG - 1) * NJ * 4 * 256 * 16);
+    if (KG > 1 && lds > 64 * 1024) {
         static bool lds_allowed[2][kMaxDevices] = {};
         if (int rc = full ? allow_dynamic_lds(ctx, mmnb_prefill_direct_kernel<SG, MI, NJ, KG, true>, lds, lds_allowed[1])
                           : allow_dynamic_lds(ctx, mmnb_prefill_direct_kernel<SG, MI, NJ, KG, false>, lds, lds_allowed[0]))
@@ -720,6 +744,17 @@ int prefill_launch_direct(hipc_ctx *ctx, PrefillArgs a) {
         // (three column blocks and two groups leave no register for more than one scale per weight tile)
         const bool two = (NJ == 2 || SG == 1) && (forced == 1 ? false : forced == 2 ? true : wgs <= ctx->cu_count && trips >= 4);
         if constexpr (NJ == 2 || SG == 1) if (two) {
+            if (int rc = prefill_launch_direct_groups<SG, MI, NJ, 2>(ctx, a, grid)) return rc;
+            return prefill_join_splits(ctx, a);
+        }
+    }
+    if constexpr (MI == 1) {
+        // 64-row tiles: two groups when the launch has too few wavefronts to hide one another's waits (no more than
+        // two workgroups per CU) and each group keeps two trips (512 x 2048 x 2560: 15.9 against 16.9 us; four
+        // groups, 18.3 us, cost more in prologues than they hide)
+        const int trips = (a.split_stages + 1) / 2, forced = ctx->tune.prefill_groups;
+        const long wgs = (long)ceil_div(a.M, 64) * ceil_div(a.N, 64 * NJ) * a.ksplit;
+        if (forced == 1 ? false : forced == 2 ? true : wgs <= 2 * ctx->cu_count && trips >= 4) {
             if (int rc = prefill_launch_direct_groups<SG, MI, NJ, 2>(ctx, a, grid)) return rc;
             return prefill_join_splits(ctx, a);
         }

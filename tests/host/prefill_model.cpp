@@ -60,7 +60,8 @@ struct Route {
     int tile, direct, split, groups;   // HIPC_PREFILL_TILE, _DIRECT, _SPLIT, _GROUPS (-1: the library's choice)
 };
 const Route kRoutes[] = {{-1, -1, -1, -1}, {64, -1, -1, -1}, {64, 0, -1, -1},  {128, -1, 0, 1},  {128, -1, 2, 1}, {128, 0, 3, -1}, {128, 0, 0, -1},
-                         {192, -1, 0, 1},  {192, -1, 2, 1},  {192, -1, 3, 1},  {128, -1, 0, 2},  {128, -1, 2, 2}, {192, -1, 0, 2},  {192, -1, 3, 2}};
+                         {192, -1, 0, 1},  {192, -1, 2, 1},  {192, -1, 3, 1},  {128, -1, 0, 2},  {128, -1, 2, 2}, {192, -1, 0, 2},  {192, -1, 3, 2},
+                         {64, -1, -1, 2},  {64, -1, -1, 1}};
 
 void product(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dtype) {
     const int64_t nb = (K + bs - 1) / bs;

@@ -140,6 +140,7 @@ WIDE_ROUTES = [  # the 128-row tiles, forced on shapes that would take 64x64: ea
     # two groups of four wavefronts per workgroup, each with half of k (a group without a trip of its own among them)
     {"HIPC_PREFILL_TILE": 192, "HIPC_PREFILL_GROUPS": 2}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 2},
     {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 2, "HIPC_PREFILL_SPLIT": 2}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 1},
+    {"HIPC_PREFILL_TILE": 64, "HIPC_PREFILL_GROUPS": 2}, {"HIPC_PREFILL_TILE": 64, "HIPC_PREFILL_GROUPS": 1},
 ]
 
 
