@@ -330,7 +330,7 @@ __global__ void __launch_bounds__(256) int8_gemm_kernel(const GemmArgs p) {
             const int ih = base_h[u] + r * p.dh, iw = base_w[u] + s * p.dw;
             const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
             const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
-            const uint4 v = *reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + c0);
+            const uint4 v = HIPC_LOAD_ALWAYS(reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + c0));
             const bool live = pos_ok[u] && gk < p.K;  // beyond the problem: zeros; padding taps: the zero point
             const uint32_t alt = live ? pad_word : 0u;
             const bool take = live && inside;
@@ -870,7 +870,7 @@ __global__ void __launch_bounds__(256) int8_conv_small_kernel(const GemmArgs p) 
             const int ih = base_h[u] + q_r[u] * p.dh, iw = base_w[u] + q_s[u] * p.dw;
             const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
             const int ihc = min(max(ih, 0), p.H - 1), iwc = min(max(iw, 0), p.W - 1);
-            const uint4 v = *reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + q_c[u]);
+            const uint4 v = HIPC_LOAD_ALWAYS(reinterpret_cast<const uint4 *>(q_img + ((size_t)ihc * p.W + iwc) * p.C + q_c[u]));
             const bool live = pos_ok[u] && q_k[u] < p.K;
             const uint32_t alt = live ? pad_word : 0u;
             const bool take = live && inside;

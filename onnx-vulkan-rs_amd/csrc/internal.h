@@ -25,7 +25,11 @@
 #define HIPC_PIN_VGPR(v) asm volatile("" : "+v"(v))                                              // the value is needed here, in a vector register
 #define HIPC_VGPR_FROM_SGPR(dst, src) asm volatile("v_mov_b32 %0, %1" : "=v"(dst) : "s"(src))   // a uniform value kept in a vector register
 #define HIPC_ARG_NOW(v) asm volatile("" ::"s"(v))                                                // the kernel argument is read here
+// A load whose value may go unused on some paths (it is masked afterwards): on the GPU it is issued whatever the mask
+// says, so the model must perform it too -- a plain load there may be moved under the condition and never be checked.
+#define HIPC_LOAD_ALWAYS(ptr) (*(ptr))
 #else
+#define HIPC_LOAD_ALWAYS(ptr) gpu_model_load_always(ptr)
 #define HIPC_ARG_NOW(v) ((void)0)
 #define HIPC_PIN_VGPR(v) ((void)0)
 #define HIPC_VGPR_FROM_SGPR(dst, src) ((dst) = (src))

@@ -160,8 +160,11 @@ __global__ void __launch_bounds__(256) mmnb_prefill_kernel(const PrefillArgs p) 
         const int k0 = stage * kPK;
 #pragma unroll
         for (int u = 0; u < kChunks; u++) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(a_base + a_off[u] + (size_t)k0 * 2);
-            const bool in = FULL || k0 + a_k[u] < p.K;  // K is a multiple of 8: a chunk is inside or outside as a whole
+            // K is a multiple of 8: a chunk is inside or outside as a whole; one outside is read from the row's last
+            // chunk instead (the load is issued whatever the mask says, and past the last row lies the end of A)
+            const bool in = FULL || k0 + a_k[u] < p.K;
+            const int back = FULL ? 0 : max(0, k0 + a_k[u] - (p.K - 8));
+            const uint4 v = HIPC_LOAD_ALWAYS(reinterpret_cast<const uint4 *>(a_base + a_off[u] + ((size_t)k0 - back) * 2));
             r.a[u] = make_uint4(in ? v.x : 0u, in ? v.y : 0u, in ? v.z : 0u, in ? v.w : 0u);
         }
         const int cg = stage >> 1, half = stage & 1;
@@ -377,8 +380,11 @@ __global__ void __launch_bounds__(256 * KG, KG > 1 ? 1 : MI * NJ == 1 ? 4 : MI *
         const int k0 = stage * kPK;
 #pragma unroll
         for (int u = 0; u < kChunks; u++) {
-            const uint4 v = *reinterpret_cast<const uint4 *>((a_base + (size_t)k0 * 2) + a_off[u]);   // (uniform part first: a scalar base and a 32-bit lane offset)
-            const bool in = FULL || k0 + a_k[u] < p.K;  // K is a multiple of 8: a chunk is inside or outside as a whole
+            // K is a multiple of 8: a chunk is inside or outside as a whole; one outside is read from the row's last
+            // chunk instead (the load is issued whatever the mask says, and past the last row lies the end of A)
+            const bool in = FULL || k0 + a_k[u] < p.K;
+            const uint32_t back = FULL ? 0u : (uint32_t)max(0, k0 + a_k[u] - (p.K - 8)) * 2u;
+            const uint4 v = HIPC_LOAD_ALWAYS(reinterpret_cast<const uint4 *>((a_base + (size_t)k0 * 2) + (a_off[u] - back)));   // (uniform part first: a scalar base and a 32-bit lane offset)
             r.a[u] = make_uint4(in ? v.x : 0u, in ? v.y : 0u, in ? v.z : 0u, in ? v.w : 0u);
         }
     };

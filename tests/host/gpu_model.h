@@ -128,7 +128,10 @@ template <typename A, typename B, typename C>
 inline C gpu_model_mfma(A, B, C c, int, int, int) { return c; }
 inline void gpu_model_nothing(...) {}
 template <typename T>
-inline T gpu_model_nt_load(const T *p) { return *p; }
+__attribute__((noinline)) T gpu_model_nt_load(const T *p) { return *p; }   // (never inlined: performed even where its value ends up unused)
+// a load that happens even if its value is dropped afterwards (never inlined: the optimizer cannot move it under a condition)
+template <typename T>
+__attribute__((noinline)) T gpu_model_load_always(const T *p) { return *p; }
 template <typename T, typename U>
 inline void gpu_model_nt_store(U v, T *p) { *p = v; }
 #define __builtin_amdgcn_readfirstlane gpu_model_same
