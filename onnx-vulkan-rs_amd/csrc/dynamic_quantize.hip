@@ -202,7 +202,7 @@ int dql_launch(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out
     HIPC_REQUIRE(ctx, scale_out && zp_out, "DynamicQuantizeLinear: null scale or zero-point output");
     HIPC_REQUIRE(ctx, aligned(scale_out, 4), "DynamicQuantizeLinear: scale output must be 4-byte aligned");
     if (n == 0) {  // empty input: y empty, scale 1, zero point 0 (interp.rs:1949-1966)
-        dql_empty_kernel<<<1, 64, 0, ctx->stream>>>(static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out));
+        hipLaunchKernelGGL((dql_empty_kernel), 1, 64, 0, ctx->stream, static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out));
         HIPC_LAUNCHED(ctx);
         return HIPC_OK;
     }
@@ -219,21 +219,20 @@ int dql_launch(hipc_ctx *ctx, const void *X, int64_t n, void *Y, void *scale_out
         // second pass -- no clearing launch and no atomics
         slot = parts ? parts : reinterpret_cast<uint32_t *>(static_cast<char *>(ctx->params) + kParamParts);
         nparts = (int)std::min<long>(std::max<long>(ceil_div(n, 256 * 16), 1), kParamPartsMax);
-        dql_range_kernel<<<(unsigned)nparts, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 1, gelu);
+        hipLaunchKernelGGL((dql_range_kernel), (unsigned)nparts, 256, 0, ctx->stream, x, (long)n, slot, vec_ok, 1, gelu);
         HIPC_LAUNCHED(ctx);
     } else if (!range_ready) {
-        dql_clear_range_kernel<<<1, 64, 0, ctx->stream>>>(slot);
+        hipLaunchKernelGGL((dql_clear_range_kernel), 1, 64, 0, ctx->stream, slot);
         HIPC_LAUNCHED(ctx);
         // enough workgroups to pull from every HBM channel, few enough that the atomics are noise
         const long want = ceil_div(n, 256 * 16);
         const unsigned grid = (unsigned)std::min<long>(std::max<long>(want, 1), 8L * ctx->cu_count);
-        dql_range_kernel<<<grid, 256, 0, ctx->stream>>>(x, (long)n, slot, vec_ok, 0, gelu);
+        hipLaunchKernelGGL((dql_range_kernel), grid, 256, 0, ctx->stream, x, (long)n, slot, vec_ok, 0, gelu);
         HIPC_LAUNCHED(ctx);
     }
     const long quads = ceil_div(n, 4);
     HIPC_REQUIRE(ctx, ceil_div(quads, 256) < (int64_t(1) << 31), "DynamicQuantizeLinear: tensor too large");
-    dql_quantize_kernel<<<(unsigned)ceil_div(quads, 256), 256, 0, ctx->stream>>>(
-        x, (long)n, slot, nparts, static_cast<uint8_t *>(Y), static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out),
+    hipLaunchKernelGGL((dql_quantize_kernel), (unsigned)ceil_div(quads, 256), 256, 0, ctx->stream, x, (long)n, slot, nparts, static_cast<uint8_t *>(Y), static_cast<float *>(scale_out), static_cast<uint8_t *>(zp_out),
         vec_ok, gelu);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
@@ -286,7 +285,7 @@ int hipc_decomposed_gelu(hipc_ctx *ctx, const void *X, int64_t n, float divisor,
         if (n == 0) return HIPC_OK;
         HIPC_REQUIRE(ctx, X && Y && aligned(X, 4) && aligned(Y, 4), "DecomposedGelu: null or unaligned tensor");
         HIPC_REQUIRE(ctx, ceil_div(n, 256) < (int64_t(1) << 31), "DecomposedGelu: tensor too large");
-        decomposed_gelu_kernel<<<(unsigned)ceil_div(n, 256), 256, 0, ctx->stream>>>(static_cast<const float *>(X), (long)n, gp,
+        hipLaunchKernelGGL((decomposed_gelu_kernel), (unsigned)ceil_div(n, 256), 256, 0, ctx->stream, static_cast<const float *>(X), (long)n, gp,
                                                                                     static_cast<float *>(Y));
         HIPC_LAUNCHED(ctx);
         return HIPC_OK;

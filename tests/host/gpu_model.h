@@ -164,6 +164,7 @@ inline uint32_t __float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); r
 inline float __expf(float v) { return std::exp(v); }
 inline float rsqrtf(float v) { return 1.f / std::sqrt(v); }
 inline float __fmul_rn(float a, float b) { return a * b; }
+inline float __fdiv_rn(float a, float b) { return a / b; }
 inline float __fadd_rn(float a, float b) { return a + b; }
 using std::max;
 using std::min;
@@ -174,6 +175,12 @@ using std::min;
 #define hipMemsetAsync gpu_model_hipMemsetAsync
 #define hipMemcpyAsync gpu_model_hipMemcpyAsync
 #define hipGetLastError gpu_model_hipGetLastError
+#ifndef __align__
+#define __align__(n) __attribute__((aligned(n)))
+#endif
+#undef HIP_SYMBOL
+#define HIP_SYMBOL(x) (x)   // a "device" array of the sources is a host array here
+#define hipGetSymbolAddress(pp, sym) (*(pp) = const_cast<void *>(static_cast<const void *>(sym)), hipSuccess)
 #define hipFuncSetAttribute(...) hipSuccess
 template <typename T>
 inline hipError_t gpu_model_hipMalloc(T **p, size_t bytes) { *p = static_cast<T *>(gpu_model::alloc(bytes)); return hipSuccess; }

@@ -1,12 +1,13 @@
-// Address model of the int8 operators: matmul_integer.hip and conv_integer.hip (with int8_gemm.h and
-// int8_gemm_bdirect.h) compiled as host code behind gpu_model.h and driven through the entry points a caller uses.
+// Address model of the int8 operators: dynamic_quantize.hip, matmul_integer.hip and conv_integer.hip (with int8_gemm.h
+// and int8_gemm_bdirect.h) compiled as host code behind gpu_model.h and driven through the entry points a caller uses.
 // Every launch runs thread by thread on the CPU; every buffer load is checked against the allocations the library
 // and this driver made (operands of exactly the operator's size, no slack), under the hardware's rule that the
 // descriptor's range check sees the per-lane offset only -- the kernels that read B straight from the prepacked
 // weight step along k in the SCALAR offset -- and every ordinary load and store is checked by AddressSanitizer.
 // Values are not checked here (the matrix cores are stubs): parity is the GPU tests' business.
 //
-//   int8_model [quick]   every matrix-product route (LDS-staged 64 / 128 tiles, the k-split 64x64 kernel, the two
+//   int8_model [quick]   DynamicQuantizeLinear (every entry point, aligned and unaligned, sizes around the vector and
+//                        workgroup boundaries); every matrix-product route (LDS-staged 64 / 128 tiles, the k-split 64x64 kernel, the two
 //                        B-direct kernels) on aligned, ragged and tiny shapes, u8 / i8 operands, zero points by
 //                        pointer and by value, the three epilogues; the convolution routes (row-resident, gathered,
 //                        tiled, grouped) on the shapes of the GPU tests. `quick` leaves out the largest shapes.
@@ -145,9 +146,33 @@ void conv(int64_t n, int64_t c_in, int64_t h, int64_t w, int64_t c_out, int64_t 
 
 }  // namespace
 
+// DynamicQuantizeLinear on n values: the context's range slot and a caller's, the variant that allocates nothing,
+// the fused GELU, the GELU alone -- X with the alignment given (vector loads need 16 bytes, the others take the
+// element path), Y and the two parameters of exactly their sizes
+void quantize(int64_t n, int misalign) {
+    uint8_t *xraw = static_cast<uint8_t *>(input((size_t)n * 4 + 16));
+    void *X = xraw + misalign;
+    void *Y = input((size_t)(n > 0 ? n : 1)), *scale = input(4), *zp = input(1), *range = input(8), *G = input((size_t)(n > 0 ? n : 1) * 4);
+    char where[96];
+    std::snprintf(where, sizeof where, "DynamicQuantizeLinear, %lld values, X at +%d", (long long)n, misalign);
+    gpu_model::reg().where = where;
+    MUST(hipc_dynamic_quantize_linear(&ctx, X, n, Y, scale, zp, nullptr, 0));
+    MUST(hipc_dynamic_quantize_linear(&ctx, X, n, Y, scale, zp, range, 0));
+    MUST(hipc_dynamic_quantize_linear(&ctx, X, n, Y, scale, zp, range, 1));
+    MUST(hipc_dynamic_quantize_linear_static(&ctx, X, n, Y, scale, zp));
+    MUST(hipc_dynamic_quantize_linear_gelu(&ctx, X, n, 1.41421356f, 1.f, 0.5f, 0, Y, scale, zp, nullptr));
+    MUST(hipc_decomposed_gelu(&ctx, X, n, 1.41421356f, 1.f, 0.5f, 1, G));
+    release_all();
+}
+
 int main(int argc, char **argv) {
     const bool quick = argc > 1 && std::strcmp(argv[1], "quick") == 0;
     ctx.params = gpu_model::alloc(hipc::kParamBytes);
+    ctx.cu_count = 256;
+    MUST(hipc::dql_static_init(&ctx));
+    for (int64_t n : {0, 1, 3, 4, 5, 255, 256, 257, 1000, 4096, 4099, 65536 + 7, 1000 * 1024})
+        for (int misalign : {0, 4}) quantize(n, misalign);
+    report("DynamicQuantizeLinear and the decomposed GELU");
     // matrix products: tiny, ragged in every direction, aligned, one tile more than a multiple, both signs
     const int64_t shapes[][3] = {{1, 8, 1}, {5, 7, 3}, {33, 100, 65}, {64, 128, 64}, {129, 257, 130}, {200, 512, 264}, {256, 1024, 512}, {300, 640, 520}};
     for (const auto &s : shapes) {
