@@ -160,7 +160,8 @@ int hipc_probe_int8_mfma(hipc_ctx *ctx, int random_operands, int waves_per_simd,
  *   scales [N * n_blocks]  f32 or f16 (scale_dtype)
  *   zp     [N, ceil(n_blocks/2)] u8, packed like B; NULL => 8 for every block
  *   Y      [M, N]  the dtype of A (crates/onnx-vulkan-frontend/src/shape.rs:497-512)
- * bits is fixed at 4; block_size is a power of two >= 16; g_idx and bias are
+ * bits is fixed at 4; block_size is any positive multiple of 8, the reference's envelope (the
+ * operator's own definition asks for a power of two >= 16); g_idx and bias are
  * refused as in the reference (interp.rs:447-464). `accuracy_level` must be 0
  * (unset) or 1..3: level 4 asks for int8 activations and is refused.
  * Buffer lengths are in elements and are checked against K, N and block_size

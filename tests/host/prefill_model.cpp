@@ -8,7 +8,8 @@
 //   prefill_model   every instance (64x64, 128x128 and 128x192 tiles with the weight read into operand registers,
 //                   one or two groups of wavefronts per workgroup; 64x64 and 128x128 with both operands through LDS),
 //                   every scale grouping, k split 1 / 2 / 3 ways,
-//                   f16 rows and f32 rows, on ragged and aligned shapes.
+//                   f16 rows and f32 rows, on ragged and aligned shapes; then the operator with few rows, on the ONNX
+//                   layout (block sizes 8, 24, 40 among them) and on the decode kernels.
 #include <cstdio>
 #include <cstring>
 #include <vector>
@@ -87,6 +88,38 @@ void product(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dt
     ctx.deferred.clear();
 }
 
+// the operator on the ONNX layout (no prepack: the kernel that takes every block size the reference takes) and, on a
+// prepacked weight, the row counts the decode kernels serve
+void rows(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dtype) {
+    const int64_t nb = (K + bs - 1) / bs;
+    const size_t b_len = (size_t)(N * nb * bs / 2), s_len = (size_t)(N * nb), z_len = (size_t)(N * ((nb + 1) / 2));
+    const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
+    void *B = gpu_model::alloc(b_len), *S = gpu_model::alloc(s_len * esz), *Z = gpu_model::alloc(z_len);
+    std::memset(B, 0x5a, b_len), std::memset(S, 0, s_len * esz), std::memset(Z, 0x88, z_len);
+    void *A = gpu_model::alloc((size_t)(M * K) * esz), *Y = gpu_model::alloc((size_t)(M * N) * esz);
+    std::memset(A, 0, (size_t)(M * K) * esz);
+    char where[160];
+    std::snprintf(where, sizeof where, "%lld x %lld x %lld block %lld %s, ONNX layout / decode kernels", (long long)M, (long long)K, (long long)N, (long long)bs,
+                  a_dtype == HIPC_F16 ? "f16" : "f32");
+    gpu_model::reg().where = where;
+    for (int level : {0, 1})
+        MUST(hipc_matmul_nbits(&ctx, A, a_dtype, B, b_len, S, a_dtype, s_len, with_zp ? Z : nullptr, with_zp ? z_len : 0, Y, M, K, N, bs, level));
+    if (bs >= 32 && (bs & (bs - 1)) == 0) {
+        hipc_nbits_weight *w = nullptr;
+        MUST(hipc_prepack_matmul_nbits(&ctx, B, b_len, S, a_dtype, s_len, with_zp ? Z : nullptr, with_zp ? z_len : 0, K, N, bs, &w));
+        for (int level : {0, 1}) MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, level));
+        for (int lean = 0; lean <= 1 && M == 1; lean++) {
+            ctx.tune.gemv_lean = lean;
+            MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 0));
+        }
+        ctx.tune.gemv_lean = -1;
+        hipc_nbits_weight_destroy(&ctx, w);
+    }
+    for (void *p : {A, Y, B, S, Z}) gpu_model::release(p);
+    for (void *p : ctx.deferred) gpu_model::release(p);
+    ctx.deferred.clear();
+}
+
 }  // namespace
 
 int main() {
@@ -104,6 +137,12 @@ int main() {
         product(s[0], s[1], s[2], s[3], s[4] != 0, HIPC_F16);
         if (s[0] > 32) product(s[0], s[1], s[2], s[3], s[4] != 0, HIPC_F32);
     }
+    // few rows: block sizes of the reference's envelope that only the ONNX-layout kernel takes (8, 24, 40), the
+    // prepacked ones on the decode kernels; one row, a partial 16-row group, a full one; ragged K and N
+    const int64_t few[][5] = {{1, 72, 16, 8, 1},   {3, 120, 50, 24, 1},  {16, 200, 33, 40, 0}, {1, 1000, 200, 32, 1}, {5, 384, 131, 64, 1},
+                              {16, 640, 96, 128, 0}, {1, 1152, 1536, 32, 1}, {2, 256, 1024, 256, 1}};
+    for (const auto &s : few)
+        for (int dt : {HIPC_F32, HIPC_F16}) rows(s[0], s[1], s[2], s[3], s[4] != 0, dt);
     gpu_model::Registry &g = gpu_model::reg();
     std::printf("%zu launches (%zu of the tiled kernels and their helpers), %zu threads\n", g.launches, prefill_launches, g.threads);
     if (prefill_launches < 300) {
