@@ -382,7 +382,9 @@ def bench_decoder(pkg, ctx, steps, warmup, context=2048):
     tok_s = steps / dt
     out = dict(tok_s=tok_s, ms_per_token=dt / steps * 1e3, context=context, bytes_per_token=byts,
                hbm_bound_tok_s=HBM_PEAK_GBS * 1e9 / byts, frac_of_hbm_bound=tok_s * byts / (HBM_PEAK_GBS * 1e9),
-               launches_per_token=5 * cfg["n_layers"] + 3, final_position=pos)
+               # five launches per layer, then the unembedding (whose workgroups leave the argmax candidates) and the
+               # launch that picks the token and embeds it for the next step
+               launches_per_token=5 * cfg["n_layers"] + 2, final_position=pos)
     # the same step without the read-ahead helper rows (by default three of a layer's five launches carry extra
     # workgroups that read what the next launch will read into the L2 of the XCD that will ask for it), and with all five
     for name, mask in (("no_read_ahead", 0), ("read_ahead_all_five", 31)):

@@ -75,7 +75,7 @@ void *hipc_stream(hipc_ctx *ctx);
  * (the reference keeps the same kind of switch in its tactic keys, crates/onnx-vulkan-core/src/tuning.rs).
  * `name` is one of HIPC_GEMV_T, HIPC_GEMV_WAVES, HIPC_GEMV_PER_CU, HIPC_GEMM_TILE, HIPC_GEMM_BIG,
  * HIPC_GEMM_SMALL, HIPC_CONV_ROW, HIPC_PREFILL_TILE, HIPC_PREFILL_SPLIT, HIPC_PREFILL_DIRECT, HIPC_PREFILL_GROUPS,
- * HIPC_DEC_FUSED_GLUE, HIPC_DEC_FUSED_ATTN, HIPC_GEMV_LEAN, HIPC_DEC_LEAN, HIPC_DEC_PREFETCH; a context starts from the environment
+ * HIPC_DEC_FUSED_GLUE, HIPC_DEC_FUSED_ATTN, HIPC_DEC_FUSED_ARGMAX, HIPC_GEMV_LEAN, HIPC_DEC_LEAN, HIPC_DEC_PREFETCH; a context starts from the environment
  * variables of the same names; value < 0 returns the choice to the library. */
 int hipc_set_option(hipc_ctx *ctx, const char *name, int value);
 

@@ -110,6 +110,7 @@ const OptionName kOptions[] = {
     {"HIPC_PREFILL_GROUPS", &Tuning::prefill_groups},
     {"HIPC_DEC_FUSED_GLUE", &Tuning::dec_fused_glue},
     {"HIPC_DEC_FUSED_ATTN", &Tuning::dec_fused_attn},
+    {"HIPC_DEC_FUSED_ARGMAX", &Tuning::dec_fused_argmax},
     {"HIPC_GEMV_LEAN", &Tuning::gemv_lean},
     {"HIPC_DEC_LEAN", &Tuning::dec_lean},
     {"HIPC_DEC_PREFETCH", &Tuning::dec_prefetch},

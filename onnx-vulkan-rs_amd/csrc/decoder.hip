@@ -699,6 +699,8 @@ __global__ void __launch_bounds__(256) dec_gelu_mul_kernel(const float *__restri
 }
 
 // argmax, smallest index on ties: per-workgroup candidates, then one workgroup picks and advances the state
+constexpr int kArgmaxParts = 256;   // workgroups of the separate scan over the logits
+constexpr int kArgmaxCap = 1024;    // candidates the token pick takes: the scan's, or one per workgroup of an lm_head launch that leaves them
 __global__ void __launch_bounds__(256)
 dec_argmax_partial_kernel(const float *__restrict__ logits, int n, float *__restrict__ pv, int *__restrict__ pi) {
     __shared__ float sv[4];
@@ -749,9 +751,17 @@ dec_pick_embed_kernel(const float *__restrict__ pv, const int *__restrict__ pi, 
     if (threadIdx.x < 64) {
         float best = -3.4e38f;
         int bi = 0x7fffffff;
-        for (int i = threadIdx.x; i < nparts; i += 64) {
-            if (pv[i] > best || (pv[i] == best && pi[i] < bi)) best = pv[i], bi = pi[i];
+        // up to kArgmaxCap candidates: a lane's sixteen are asked for together, then compared
+        float cv[kArgmaxCap / 64];
+        int ci[kArgmaxCap / 64];
+#pragma unroll
+        for (int u = 0; u < kArgmaxCap / 64; u++) {
+            const int i = min((int)threadIdx.x + 64 * u, nparts - 1);
+            cv[u] = pv[i], ci[u] = pi[i];
         }
+#pragma unroll
+        for (int u = 0; u < kArgmaxCap / 64; u++)
+            if ((int)threadIdx.x + 64 * u < nparts && (cv[u] > best || (cv[u] == best && ci[u] < bi))) best = cv[u], bi = ci[u];
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) {
             const float ov = __shfl_xor(best, off, 64);
@@ -832,7 +842,6 @@ struct hipc_decoder {
 
 namespace {
 
-constexpr int kArgmaxParts = 256;
 
 template <typename T>
 int dev_alloc(hipc_ctx *ctx, hipc_decoder *d, T **p, size_t count) {
@@ -922,7 +931,7 @@ int hipc_decoder_create(hipc_ctx *ctx, const hipc_decoder_config *cfg, hipc_deco
         A(&d->gu, (size_t)2 * c.ffn), A(&d->h, c.ffn), A(&d->logits, c.vocab);
         const size_t parts = (size_t)c.n_kv_heads * std::max(d->nsplit, kAttnSplits) * G;
         A(&d->part_ml, parts * 2), A(&d->part_o, parts * c.head_dim);
-        A(&d->am_v, kArgmaxParts), A(&d->am_i, kArgmaxParts);
+        A(&d->am_v, kArgmaxCap), A(&d->am_i, kArgmaxCap);
         A(&d->pf_sink, 4);
         A(&d->rope, (size_t)2 * c.head_dim), A(&d->x2, c.hidden);
         // options read when the decoder is created: dec_fused_glue = 0 keeps the separate norm / GELU
@@ -1285,19 +1294,27 @@ int hipc_decoder_step(hipc_ctx *ctx, hipc_decoder *d) {
                 HIPC_LAUNCHED(ctx);
             }
         }
+        GemvArgmax am;
+        am.v = d->am_v, am.i = d->am_i, am.capacity = ctx->tune.dec_fused_argmax == 0 ? 0 : kArgmaxCap;
         if (d->fused_glue) {
             // the unembedding's prologue adds the last branch to the stream and applies the final norm (every workgroup
             // for itself, while its first weight tiles are on their way)
             GemvPrologue pro;
             pro.mode = 2, pro.x = xc, pro.y = d->lean ? d->yd : d->y, pro.y_slices = d->lean ? d->down_slices : 1;
             pro.w_post = d->layers[c.n_layers - 1].norm[HIPC_DEC_NORM_POST_FFN], pro.w_in = d->final_norm, pro.eps = c.rms_eps;
-            if ((rc = nbits_gemv(ctx, xc, HIPC_F32, d->lm_head, d->logits, 1, terms, &pro)) != HIPC_OK) return rc;
+            if ((rc = nbits_gemv(ctx, xc, HIPC_F32, d->lm_head, d->logits, 1, terms, &pro, &am)) != HIPC_OK) return rc;
         } else {
-            if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms)) != HIPC_OK) return rc;
+            if ((rc = nbits_gemv(ctx, d->xn, HIPC_F32, d->lm_head, d->logits, 1, terms, nullptr, &am)) != HIPC_OK) return rc;
         }
-        hipLaunchKernelGGL((dec_argmax_partial_kernel), kArgmaxParts, 256, 0, s, d->logits, c.vocab, d->am_v, d->am_i);
-        HIPC_LAUNCHED(ctx);
-        hipLaunchKernelGGL((dec_pick_embed_kernel), 1, 256, 0, s, d->am_v, d->am_i, kArgmaxParts, d->state, d->history, c.max_seq, c.vocab, embed_args(d));
+        // the unembedding's workgroups leave their candidates themselves when its launch can carry that (the kernel
+        // for wide outputs); else a launch of its own scans the logits
+        int parts = am.parts;
+        if (parts == 0) {
+            parts = kArgmaxParts;
+            hipLaunchKernelGGL((dec_argmax_partial_kernel), kArgmaxParts, 256, 0, s, d->logits, c.vocab, d->am_v, d->am_i);
+            HIPC_LAUNCHED(ctx);
+        }
+        hipLaunchKernelGGL((dec_pick_embed_kernel), 1, 256, 0, s, d->am_v, d->am_i, parts, d->state, d->history, c.max_seq, c.vocab, embed_args(d));
         HIPC_LAUNCHED(ctx);
         if (!ctx->capturing) d->x_ready = true;
         return HIPC_OK;

@@ -63,6 +63,7 @@ struct Tuning {
     int prefill_groups = -1;  // HIPC_PREFILL_GROUPS 1 / 2: groups of four wavefronts per workgroup of the prefill tiles (2: each takes half of k)
     int prefill_direct = -1;  // HIPC_PREFILL_DIRECT 0: 128-row tiles keep the kernel that passes the weight through LDS (and are never 192 wide)
     int dec_fused_glue = -1;  // HIPC_DEC_FUSED_GLUE 0 keeps the separate norm / GELU kernels (read when a decoder is created)
+    int dec_fused_argmax = -1; // HIPC_DEC_FUSED_ARGMAX 0: a launch of its own scans the logits for the token pick
     int dec_fused_attn = -1;  // HIPC_DEC_FUSED_ATTN 0 keeps the three-kernel attention (read when a decoder is created)
     int gemv_lean = -1;       // HIPC_GEMV_LEAN      0: one-row products keep the streaming GEMV kernel
     int dec_lean = -1;        // HIPC_DEC_LEAN       0: the decoder keeps the streaming GEMV and its prologues (read when a decoder is created)
@@ -339,8 +340,19 @@ __host__ __device__ inline int attn_live_chunks(int span) {
 }
 // the transposed value cache's row length: max_seq rounded up to 64
 __host__ __device__ inline int attn_v_stride(int max_seq) { return (max_seq + 63) / 64 * 64; }
+// Optional epilogue of nbits_gemv for one f32 row: every workgroup of the wide kernel also leaves the largest of the
+// results it stored and its column (smallest column on ties; NaN never wins) in v[workgroup], i[workgroup]. `parts`
+// comes back as the number of workgroups that wrote a candidate, or 0 when the launch could not carry the epilogue
+// (another kernel took the product, k was split over workgroups, more workgroups than `capacity`): the caller then
+// scans Y itself.
+struct GemvArgmax {
+    float *v = nullptr;
+    int *i = nullptr;
+    int capacity = 0;
+    int parts = 0;
+};
 int nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
-               const GemvPrologue *pro = nullptr);
+               const GemvPrologue *pro = nullptr, GemvArgmax *am = nullptr);
 
 // ---- the latency-built kernel for one f32 row (gemv_lean.hip) -------------------------------------
 // A row "in operand order": per 32-k chunk c, NT terms x 4 k groups of 8 bf16 (16 bytes each), term

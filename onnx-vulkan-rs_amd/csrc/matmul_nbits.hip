@@ -182,6 +182,10 @@ struct GemvArgs {
     int nparts;   // ways the live chunks are divided among threads that share four channels
     int ny_slices; // norm prologue: ny is this many partial rows, K floats apart, that add up to y
     int pro_off;  // byte offset of the prologue's own LDS area
+    // argmax epilogue (one f32 row, k not split over workgroups): workgroup b leaves the largest result it stored and
+    // its column in am_v[b], am_i[b]; null: no epilogue
+    float *am_v;
+    int *am_i;
 };
 
 template <int SG>
@@ -266,6 +270,7 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
     HIPC_ARG_NOW(p.A); HIPC_ARG_NOW(p.Wq); HIPC_ARG_NOW(p.Sc); HIPC_ARG_NOW(p.Zb); HIPC_ARG_NOW(p.Y); HIPC_ARG_NOW(p.Ypart);
     HIPC_ARG_NOW(p.M); HIPC_ARG_NOW(p.K); HIPC_ARG_NOW(p.N); HIPC_ARG_NOW(p.n_tiles); HIPC_ARG_NOW(p.n_cg); HIPC_ARG_NOW(p.WK); HIPC_ARG_NOW(p.WN);
     HIPC_ARG_NOW(p.slice_tiles); HIPC_ARG_NOW(p.ksplit); HIPC_ARG_NOW(p.a_f16); HIPC_ARG_NOW(p.a_vec); HIPC_ARG_NOW(p.nib_mask); HIPC_ARG_NOW(p.magic);
+    HIPC_ARG_NOW(p.am_v); HIPC_ARG_NOW(p.am_i);
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int M = MC > 0 ? MC : p.M;
@@ -681,6 +686,28 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
             for (int r = 0; r < NR; r++) acc[t][r] = fmaf(s_q[t], fmaf(-zb_q[t], as_q[r], d_q[t][r]), acc[t][r]);
     };
 
+    // argmax epilogue: the largest result this lane has stored and its column (smallest column on ties; a NaN never wins)
+    float am_best = -3.4e38f;
+    int am_col = 0x7fffffff;
+    __shared__ float am_sv[16];
+    __shared__ int am_si[16];
+    auto argmax_out = [&]() {   // the workgroup's candidate: over the lanes, then over the wavefronts
+        if (!p.am_v) return;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(am_best, off, 64);
+            const int oc = __shfl_xor(am_col, off, 64);
+            if (ov > am_best || (ov == am_best && oc < am_col)) am_best = ov, am_col = oc;
+        }
+        if (lane == 0) am_sv[wave] = am_best, am_si[wave] = am_col;
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < nthreads / 64; w++)
+                if (am_sv[w] > am_best || (am_sv[w] == am_best && am_si[w] < am_col)) am_best = am_sv[w], am_col = am_si[w];
+            p.am_v[blockIdx.x] = am_best, p.am_i[blockIdx.x] = am_col;
+        }
+    };
+
     // one column group is done: reduce over the k wavefronts, store, clear
     auto group_end = [&](bool more_groups) {
         if (p.WK > 1) {
@@ -717,6 +744,7 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
                             static_cast<__half *>(p.Y)[(size_t)m * p.N + n] = __float2half(acc[t][r]);
                         } else {
                             static_cast<float *>(p.Y)[(size_t)m * p.N + n] = acc[t][r];
+                            if (p.am_v && (acc[t][r] > am_best || (acc[t][r] == am_best && n < am_col))) am_best = acc[t][r], am_col = n;   // (M is 1 there)
                         }
                     }
                 }
@@ -731,6 +759,7 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
             group_end(g + 1 < my_groups);
             ng += gstride;
         }
+        argmax_out();
         return;
     }
     int tile = tile0 + wk, ti = 0, gi = 0;
@@ -755,6 +784,7 @@ __global__ void __launch_bounds__(1024 / T / (NR == 4 ? 2 : 1)) mmnb_gemv_kernel
 #pragma unroll
         for (int d = 0; d < D; d++) step(st[d]);
     }
+    argmax_out();
 }
 
 __global__ void __launch_bounds__(256)
@@ -872,7 +902,8 @@ void launch_gemv_nt(const GemvArgs &a, int pro, int NT, int NR, int SG, dim3 gri
 
 // rows [0, M) with M <= 16 of one activation matrix against a prepacked weight
 int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int NT,
-                const GemvPrologue *pro = nullptr) {
+                const GemvPrologue *pro = nullptr, GemvArgmax *am = nullptr) {
+    if (am) am->parts = 0;
     HIPC_REQUIRE(ctx, w->interleave_half == 0, "MatMulNBits gemv: this weight was prepacked with interleaved halves for the decoder");
     // one plain f32 row on a narrow output: the kernel built for latency (gemv_lean.hip); the
     // gemv_lean option set to 0 keeps this kernel (tuning, tests)
@@ -960,6 +991,10 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
             HIPC_REQUIRE(ctx, lds <= 64 * 1024, "MatMulNBits gemv: LDS plan of %zu bytes does not fit", lds);
             a.a_vec = 1;
         }
+    }
+    if (am && am->v && am->i && M == 1 && !a.a_f16 && ksplit == 1 && (int)grid.x <= am->capacity) {
+        a.am_v = am->v, a.am_i = am->i;
+        am->parts = (int)grid.x;
     }
     if (T == 4)
         launch_gemv_nt<4>(a, mode, NT, NR, w->SG, grid, block, lds, ctx->stream);
@@ -1083,8 +1118,8 @@ void hipc::nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w) {
 }
 
 int hipc::nbits_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int M, int terms,
-                     const GemvPrologue *pro) {
-    return launch_gemv(ctx, A, a_dtype, w, Y, M, terms, pro);
+                     const GemvPrologue *pro, GemvArgmax *am) {
+    return launch_gemv(ctx, A, a_dtype, w, Y, M, terms, pro, am);
 }
 
 int64_t hipc::nbits_cols(const hipc_nbits_weight *w) { return w->N; }

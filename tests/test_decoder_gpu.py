@@ -40,6 +40,27 @@ def test_decode_steps_match_the_oracle(ctx, pkg, oracle):
     dec.destroy()
 
 
+@pytest.mark.parametrize("env", [{}, {"HIPC_DEC_FUSED_ARGMAX": 0}, {"HIPC_DEC_FUSED_GLUE": 0}], ids=["candidates-from-lm_head", "separate-scan", "separate-glue"])
+def test_the_token_is_the_argmax_of_the_logits_on_a_wide_vocabulary(ctx, pkg, route, env):
+    """A vocabulary wide enough for the unembedding to run on the kernel whose workgroups leave the argmax candidates
+    themselves (ragged: 32768 + 48 columns): the token the device picks is the first largest of the logits it stores,
+    step after step, and the same with a launch of its own scanning the logits."""
+    route(env)
+    cfg = dict(SMALL, vocab=32768 + 48)
+    w = pkg.decoder.build_weights(cfg, seed=21)
+    dec = pkg.decoder.Decoder(ctx, cfg, 24)
+    dec.load(w)
+    dec.reset(5, 0)
+    seen = set()
+    for pos in range(12):
+        dec.step()
+        tok, got_pos, logits, _ = dec.read(want_logits=True)
+        assert got_pos == pos + 1 and tok == int(np.argmax(logits)), (pos, tok, int(np.argmax(logits)))
+        seen.add(tok)
+    assert len(seen) > 1
+    dec.destroy()
+
+
 DEEP = [  # (head_dim, query heads, kv heads, first position): every head_dim / group size the chunk kernel is built for
     (256, 4, 1, 2046),   # crosses from 64 to 128 positions per workgroup at 2048
     (128, 8, 1, 4290),   # three passes per workgroup, the last one ragged
