@@ -746,7 +746,7 @@ dec_pick_embed_kernel(const float *__restrict__ pv, const int *__restrict__ pi, 
     __shared__ int next[2];
     // the upper two wavefronts work out the next position's rotary table (it follows from the position alone) while
     // the first picks the token
-    const int pos_now = st->pos;
+    const int pos_now = st->pos, token_now = st->token;   // (both read here, once: asked for again after the pick they would be a trip to memory on its critical path)
     dec_rope_table(e, pos_now >= max_hist ? pos_now : pos_now + 1);
     if (threadIdx.x < 64) {
         float best = -3.4e38f;
@@ -769,8 +769,8 @@ dec_pick_embed_kernel(const float *__restrict__ pv, const int *__restrict__ pi, 
             if (ov > best || (ov == best && oi < bi)) best = ov, bi = oi;
         }
         if (threadIdx.x == 0) {
-            const int pos = st->pos;
-            int token = st->token, new_pos = pos;
+            const int pos = pos_now;
+            int token = token_now, new_pos = pos;
             if (pos >= max_hist) {
                 st->overflow = 1;
             } else {
