@@ -2,7 +2,10 @@
 //
 // The reference has no tiled path for this shape: its kernels re-read the weight once per row
 // (crates/onnx-vulkan-core/src/shaders/matmul_nbits.rs:21-25). Here the weight is read once per
-// 64- or 128-row tile of A and the products run on the matrix cores:
+// 64- or 128-row tile of A and the products run on the matrix cores. Two kernels: the one further
+// down (mmnb_prefill_direct_kernel), which every shape takes by default, keeps the weight out of LDS;
+// the first one passes both operands through LDS and stays behind the prefill_direct option as the
+// control the other is tested against:
 //
 //   * a 256-thread workgroup owns a T x T tile of Y (T = 128, or 64 when that would leave CUs
 //     idle), four wavefronts as 2 x 2, each T/2 x T/2 as 32x32 accumulators of
