@@ -102,6 +102,22 @@ __device__ __forceinline__ void lean_ld8f(__amdgpu_buffer_rsrc_t r, uint32_t vof
 // remainder, of the second remainder (every remainder is exact in f32)
 typedef __attribute__((ext_vector_type(2))) __bf16 lbf16x2;
 typedef __attribute__((ext_vector_type(2))) float lf32x2;
+// The sum of the two bf16 halves of every word of NT operands (f32): what a product of the operands with ones
+// would give, on the vector unit (one v_dot2c_f32_bf16 per word).
+typedef __attribute__((ext_vector_type(2))) __bf16 lbf16pair;
+template <int NT>
+__device__ __forceinline__ float lean_term_sum(const uint4 (&op)[3]) {
+    const lbf16pair ones = __builtin_bit_cast(lbf16pair, 0x3f803f80u);
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        s0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(lbf16pair, op[t].x), ones, s0, false);
+        s1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(lbf16pair, op[t].y), ones, s1, false);
+        s0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(lbf16pair, op[t].z), ones, s0, false);
+        s1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(lbf16pair, op[t].w), ones, s1, false);
+    }
+    return s0 + s1;
+}
 template <int NT>
 __device__ __forceinline__ void lean_split8(const float (&av)[8], uint4 (&op)[3]) {
     uint32_t w[3][4];
@@ -156,10 +172,13 @@ constexpr int kLeanMaxSlices = 4;   // partial rows a norm prologue adds up at m
 //
 // The vector unit is what these kernels wait for (a wavefront alone on its SIMD issues one vector
 // instruction per four clocks, and every instruction of a prologue is on the critical path), so:
-// addresses are scalar (buffer loads), nothing is divided at run time, the sums over a quantisation
-// block's activations that take the weights' +128 bias out again are one more matrix-core product
-// against an all-ones operand instead of additions in every prologue, and values are split into
-// bf16 terms with the packed conversion.
+// addresses are scalar (buffer loads), nothing is divided at run time, and values are split into
+// bf16 terms with the packed conversion. The sums over a quantisation block's activations that take
+// the weights' +128 bias out again come from where they are cheapest: a prologue that holds eight
+// consecutive values per thread (PRO 0, 2) adds its terms up with eight dot instructions and two
+// steps inside a quad and leaves one sum per 32-k chunk in LDS (twelve matrix-core products per
+// wavefront less at three tiles: 0.1 us per launch); the others (PRO 3: one value per lane, PRO 4:
+// no prologue) multiply the operands with ones on the matrix cores.
 template <int SG, int NT, int PRO, int EPI, int KT>
 __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const LeanArgs p) {
     extern __shared__ uint4 lean_smem[];
@@ -256,6 +275,13 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
 
     uint4 *As = lean_smem;                                                     // [nch][NT][4] operands
     float *red = reinterpret_cast<float *>(As + (size_t)slice_tiles * 4 * NT * 4);   // [WN][16 columns][16 k wavefronts]; before that the norm's partial sums
+    // The sums of the split activations over every 32-k chunk, which take the weights' +128 bias and the zero
+    // points out again, are left here by the prologue that splits the row (four per tile, read back with one
+    // broadcast load). A row that arrives already split (PRO 4) has no prologue, and the attention join (PRO 3)
+    // holds one value per lane, whose sums over 32 lanes cost more than they save: those two take the sums from
+    // a second product against ones.
+    constexpr bool kSumsAhead = PRO == 0 || PRO == 2;
+    float *bsum = red + (size_t)p.WN * 256;   // [slice tiles][4 chunks]
     const int nthreads = blockDim.x;
     const int kbase = kt0 * 128;
     const int nitems = nch * 4;   // one item = 8 consecutive k of the row = one operand per term
@@ -267,6 +293,11 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
         uint4 *dst = As + (size_t)(item >> 2) * NT * 4 + (item & 3);
 #pragma unroll
         for (int t = 0; t < NT; t++) dst[4 * t] = op[t];
+        // the four items of a chunk sit in the four lanes of a quad (the number of items is a multiple of four)
+        float cs = lean_term_sum<NT>(op);
+        cs += lean_dpp<0xB1>(cs);
+        cs += lean_dpp<0x4E>(cs);
+        if ((item & 3) == 0) bsum[item >> 2] = cs;
     };
 
     if (PRO == 0) {
@@ -417,7 +448,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
     // matrix-core product (independent accumulators), then the per-block sums. The operand rows of a
     // lane: every group of four rows of the 16-row A operand holds the NT terms (row 4 q + t is term
     // t), so ONE product per chunk multiplies all terms and the result rows 0 .. NT-1 add up to the dot
-    // product; a second product against ones gives the chunk's sum of the split activations.
+    // product; where no prologue left the chunks' sums, a second product against ones gives them.
     const int term = min(i16 & 3, NT - 1);
     const uint32_t nib_mask = p.nib_mask;
     uint32_t magic;
@@ -426,6 +457,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
     // wavefront of a 1024-thread workgroup may hold: that instance reads a tile's operands when it multiplies it)
     constexpr bool kOperandsAhead = !(NT == 3 && KT == 4);
     uint4 aop[KT][4];
+    float4 bs[KT];
     const uint4 *a_lane = As + term * 4 + g4;
     if (PRO == 4) {
         const __amdgpu_buffer_rsrc_t r_a = lean_rsrc(p.a_split, (uint32_t)p.n_cg * 4u * NT * 64u);
@@ -439,6 +471,10 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
         for (int i = 0; i < KT; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) aop[i][j] = a_lane[(size_t)(tile_in_slice[i] * 4 + j) * NT * 4];
+        if (kSumsAhead) {
+#pragma unroll
+            for (int i = 0; i < KT; i++) bs[i] = reinterpret_cast<const float4 *>(bsum)[tile_in_slice[i]];
+        }
     }
     LEAN_STAMP_AFTER(aop[KT - 1][3].x, 4);
     const uint32_t one2 = 0x3f803f80u;   // bf16 1.0 twice
@@ -455,14 +491,18 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
             const bool first = (j % CPG) == 0;
             const lbf16x8 a = __builtin_bit_cast(lbf16x8, aop[i][j]);
             d[i][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(lbf16x8, bw), first ? lf32x4{0.f, 0.f, 0.f, 0.f} : d[i][g], 0, 0, 0);
-            e[i][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ones, first ? lf32x4{0.f, 0.f, 0.f, 0.f} : e[i][g], 0, 0, 0);
+            if (!kSumsAhead) e[i][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ones, first ? lf32x4{0.f, 0.f, 0.f, 0.f} : e[i][g], 0, 0, 0);
         }
     };
     auto fold_tile = [&](int i) {
 #pragma unroll
         for (int g = 0; g < SG; g++) {
             const float dsum = NT == 3 ? (d[i][g][0] + d[i][g][1]) + d[i][g][2] : d[i][g][0] + d[i][g][1];
-            const float asg = NT == 3 ? (e[i][g][0] + e[i][g][1]) + e[i][g][2] : e[i][g][0] + e[i][g][1];
+            float asg;
+            if (!kSumsAhead) asg = NT == 3 ? (e[i][g][0] + e[i][g][1]) + e[i][g][2] : e[i][g][0] + e[i][g][1];
+            else if (SG == 4) asg = g == 0 ? bs[i].x : g == 1 ? bs[i].y : g == 2 ? bs[i].z : bs[i].w;
+            else if (SG == 2) asg = g == 0 ? bs[i].x + bs[i].y : bs[i].z + bs[i].w;
+            else asg = (bs[i].x + bs[i].y) + (bs[i].z + bs[i].w);
             const float zb = (float)((sv[i].z >> (8 * g)) & 0xffu);
             acc = fmaf(sv[i].s[g] * tile_live[i], fmaf(-zb, asg, dsum), acc);
         }
@@ -480,6 +520,7 @@ __global__ void __launch_bounds__(PRO == 0 ? 1024 : 512) mmnb_lean_kernel(const 
             if (PRO != 4) {
 #pragma unroll
                 for (int j = 0; j < 4; j++) aop[i][j] = a_lane[(size_t)(tile_in_slice[i] * 4 + j) * NT * 4];
+                if (kSumsAhead) bs[i] = reinterpret_cast<const float4 *>(bsum)[tile_in_slice[i]];
             }
             multiply_tile(i);
             fold_tile(i);
@@ -616,6 +657,7 @@ int hipc::lean_gemv(hipc_ctx *ctx, const hipc_nbits_weight *w, const LeanPlan &p
     HIPC_REQUIRE(ctx, pro == 0 || threads <= 512, "MatMulNBits lean gemv: at most eight wavefronts with a prologue");
     size_t lds = (size_t)slice_tiles * 4 * NT * 4 * 16;
     lds += (size_t)pl.WN * 16 * 16 * 4;   // reduction area [WN][16][16]; the norm's partial sums [16][4][4] fit its first KiB
+    lds += (size_t)slice_tiles * 16;          // the chunks' activation sums
     HIPC_REQUIRE(ctx, lds <= 64 * 1024, "MatMulNBits lean gemv: LDS plan of %zu bytes does not fit", lds);
     if (a.pf.kind == 0) a.pf.rows = 0;
     const dim3 grid((unsigned)ceil_div(w->n_tiles, pl.WN), (unsigned)(pl.slices + a.pf.rows));

@@ -145,6 +145,9 @@ inline float gpu_model_rcp(float v) { return 1.f / v; }
 #define __builtin_amdgcn_rcpf gpu_model_rcp
 inline int gpu_model_sdot4(int, int, int c, bool) { return c; }
 #define __builtin_amdgcn_sdot4 gpu_model_sdot4
+template <typename P>
+inline float gpu_model_fdot2(P, P, float c, bool) { return c; }
+#define __builtin_amdgcn_fdot2_f32_bf16 gpu_model_fdot2
 inline uint32_t gpu_model_perm(uint32_t a, uint32_t, uint32_t) { return a; }
 #define __builtin_amdgcn_perm gpu_model_perm
 template <typename T>
