@@ -524,20 +524,22 @@ def bench_prefill(pkg, ctx, M=512, bs=128):
                                                     gbs=byts / ns, frac_hbm=byts / ns / HBM_PEAK_GBS,
                                                     frac_of_min_bound=min_bound_us(byts, flops, F16_PEAK_TFLOPS) / (ns / 1e3))
         if name == "qkv_2048x2560":
-            # the same product with f32 rows (two f16 rows each through the same kernel, plus a split and a join launch)
+            # the same product with f32 rows: two f16 rows each through the same kernel after a launch that splits them
+            # (accuracy_level unset), or one (a level that allows f16 activations)
             a32 = ctx.upload(pkg.synth.normal_f32(M * K, 41).reshape(M, K))
             y32 = ctx.alloc(4 * M * N)
-            run32 = lambda: pkg.ops.matmul_nbits_packed_device(ctx, a32, pkg.F32, w, y32, M)  # noqa: E731
-            run32()
-            ctx.flush()
-            ctx.capture_begin()
-            for _ in range(reps):
+            for level, label in ((0, "matmul_nbits_f32_M512_"), (2, "matmul_nbits_f32_level2_M512_")):
+                run32 = lambda: pkg.ops.matmul_nbits_packed_device(ctx, a32, pkg.F32, w, y32, M, level)  # noqa: E731,B023
                 run32()
-            g = ctx.capture_end()
-            warm_graph(ctx, g)
-            ns32, _ = median_ns(ctx, g, reps, samples=10, reps=4)
-            ctx.graph_destroy(g)
-            out["matmul_nbits_f32_M512_" + name] = dict(us=ns32 / 1e3, tflops=flops / ns32 / 1e3)
+                ctx.flush()
+                ctx.capture_begin()
+                for _ in range(reps):
+                    run32()
+                g = ctx.capture_end()
+                warm_graph(ctx, g)
+                ns32, _ = median_ns(ctx, g, reps, samples=10, reps=4)
+                ctx.graph_destroy(g)
+                out[label + name] = dict(us=ns32 / 1e3, tflops=flops / ns32 / 1e3)
             a32.free(), y32.free()
         w.destroy(), a.free(), y.free()
         ctx.flush()

@@ -162,8 +162,9 @@ int hipc_probe_int8_mfma(hipc_ctx *ctx, int random_operands, int waves_per_simd,
  *   Y      [M, N]  the dtype of A (crates/onnx-vulkan-frontend/src/shape.rs:497-512)
  * bits is fixed at 4; block_size is any positive multiple of 8, the reference's envelope (the
  * operator's own definition asks for a power of two >= 16); g_idx and bias are
- * refused as in the reference (interp.rs:447-464). `accuracy_level` must be 0
- * (unset) or 1..3: level 4 asks for int8 activations and is refused.
+ * refused as in the reference (interp.rs:447-464). `accuracy_level` is 0 (unset)
+ * or 1..4, a lower bound on the activations' precision that the reference never reads (it
+ * computes every level in f32): see hipc_matmul_nbits_packed for what each level gets here.
  * Buffer lengths are in elements and are checked against K, N and block_size
  * as the reference does (interp.rs:6455-6472); M*N == 0 is a no-op.
  */
@@ -182,13 +183,17 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
 void hipc_nbits_weight_destroy(hipc_ctx *ctx, hipc_nbits_weight *w);
 /* bytes of device memory the prepacked form occupies */
 size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w);
-/* MatMulNBits on a prepacked weight. `accuracy_level` as in the operator: 0 (unset), 2 or 3 let
- * f32 activations enter the matrix cores as two bf16 terms (16 significant bits, less error than
- * f32 accumulation over K adds); 1 pins f32 and uses three terms (all 24 bits); 4 is refused.
- * More than 16 rows of f16 (32 of f32) run a tiled matrix-core kernel whose accumulators are kept in
- * units of the open quantisation block's scale: there a scale of magnitude below 2^-64 counts as
- * 2^-64 (what such a block adds is below 2^-64 x 15 x sum |a|), and a column whose scales are all
- * below it is stored as 0. */
+/* MatMulNBits on a prepacked weight. `accuracy_level` as in the operator, a lower bound on what the
+ * activations may be reduced to (the reference never reads it and computes in f32). Up to 32 rows
+ * of f32: 0 (unset), 2, 3 and 4 enter the matrix cores as two bf16 terms (16 significant bits, less
+ * error than f32 accumulation over K adds), 1 pins f32 and uses three terms (all 24 bits).
+ * More than 16 rows of f16, or 32 of f32, run a tiled f16 matrix-core kernel; an f32 row travels
+ * as f16 terms of the row times the power of two that puts its largest value into [2^14, 2^15):
+ * two terms (22 bits) at level 0, one (11 bits of every value) at levels 2, 3 and 4, which allow
+ * f16, bf16 or int8 activations; level 1 keeps the three-term route, 16 rows at a time.
+ * The tiled kernel keeps its accumulators in units of the open quantisation block's scale: there a
+ * scale of magnitude below 2^-64 counts as 2^-64 (what such a block adds is below
+ * 2^-64 x 15 x sum |a|), and a column whose scales are all below it is stored as 0. */
 int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w,
                              void *Y, int64_t M, int accuracy_level);
 

@@ -1020,8 +1020,9 @@ int hipc_matmul_nbits(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, 
                       int64_t N, int64_t block_size, int accuracy_level) {
     return entry(ctx, [&]() -> int {
         HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
-        HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 3,
-                    "MatMulNBits: accuracy_level %d asks for quantised activations", accuracy_level);
+        // (the attribute is a lower bound on what the activations may be reduced to; the reference never reads it and
+        // computes every level in f32. Level 4 allows int8 activations: two bf16 terms are more than it asks for.)
+        HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 4, "MatMulNBits: accuracy_level %d is not one of 0..4", accuracy_level);
         int rc = check_nbits_shape(ctx, M, K, N, block_size, b_len, scales_len, zp, zp_len, scale_dtype);
         if (rc != HIPC_OK) return rc;
         if (M == 0 || N == 0) return HIPC_OK;
@@ -1141,20 +1142,22 @@ int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hi
     return entry(ctx, [&]() -> int {
         HIPC_REQUIRE(ctx, w, "MatMulNBits: null weight");
         HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
-        HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 3,
-                    "MatMulNBits: accuracy_level %d asks for quantised activations", accuracy_level);
+        // (the attribute is a lower bound on what the activations may be reduced to; the reference never reads it and
+        // computes every level in f32. Level 4 allows int8 activations: two bf16 terms are more than it asks for.)
+        HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 4, "MatMulNBits: accuracy_level %d is not one of 0..4", accuracy_level);
         HIPC_REQUIRE(ctx, M >= 0 && M < (int64_t(1) << 30), "MatMulNBits: bad M=%ld", (long)M);
         if (M == 0) return HIPC_OK;
         HIPC_REQUIRE(ctx, A && Y, "MatMulNBits: null operand");
         const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
         // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
-        // terms). Unset, or 2 / 3 (f16 / bf16 are enough): 2 terms. f16 activations are exact in 2.
+        // terms). Unset, or 2 / 3 / 4 (f16 / bf16 / int8 are enough): 2 terms. f16 activations are exact in 2.
         const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
         // many rows of f16: the tiled kernel reads the weight once per row tile instead of once per 16 rows
         if (a_dtype == HIPC_F16 && nbits_prefill_takes(A, w, M)) return nbits_prefill(ctx, A, w, Y, M);
-        // many rows of f32: two f16 rows each (22 bits) through the same kernel; accuracy_level 1 (f32 pinned: all 24
-        // bits) keeps the decode kernel's three-term route
-        if (a_dtype == HIPC_F32 && NT == 2 && nbits_prefill_f32_takes(A, w, M)) return nbits_prefill_f32(ctx, A, w, Y, M);
+        // many rows of f32: two f16 rows each (22 bits) through the same kernel, or one (11 bits beside the row's own
+        // power of two) where the operator's attribute allows f16, bf16 or int8 activations; accuracy_level 1 (f32
+        // pinned: all 24 bits) keeps the decode kernel's three-term route
+        if (a_dtype == HIPC_F32 && NT == 2 && nbits_prefill_f32_takes(A, w, M)) return nbits_prefill_f32(ctx, A, w, Y, M, accuracy_level >= 2 ? 1 : 2);
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int rows = (int)std::min<int64_t>(16, M - m0);
             int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,

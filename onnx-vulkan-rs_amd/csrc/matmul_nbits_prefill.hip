@@ -52,6 +52,14 @@ struct PrefillArgs {
     int ksplit, split_stages;
     float *Ypart;
     float *Yf32;   // when set, the result is written here as f32 and Y is not used (rows of f32 activations, see nbits_prefill_f32)
+    // Paired rows (set together; only the kernel that keeps the weight out of LDS, 128-row tiles): A holds the two
+    // f16 terms of `pair_rows` f32 rows, 32 rows of high terms followed by the 32 rows of their low terms, so that a
+    // wavefront's two row blocks are the two terms of the same 32 rows; it adds them and stores row r of the result
+    // times 2^exps[r] -- into Yf32, or unscaled into the k split's partials [split][pair_rows][N].
+    // exps without pair_rows: A holds one f16 term per f32 row and row r of the f32 result is stored times 2^exps[r]
+    // (any of the kernels; the k split's partials stay unscaled).
+    const int *exps;
+    int pair_rows;
 };
 
 // two f16 values as one word, the first in the low half
@@ -78,9 +86,15 @@ __device__ __forceinline__ uint4 dequant8(uint32_t w, uint32_t zb) {
 // the k split's partials. Which of the three, and whether the wavefront's square lies inside the matrix, is decided
 // once (asked per element, the same questions made 3000 instructions of this and 5 of the kernel's 45 us).
 template <int FM, int FN, bool CHECKED, typename OUT>
-__device__ __forceinline__ void prefill_store_as(OUT *__restrict__ dst, int M, int N, const f32x16 (&total)[FM][FN], int i0, int j0, int r32, int kg) {
+__device__ __forceinline__ void prefill_store_as(OUT *__restrict__ dst, int M, int N, const f32x16 (&total)[FM][FN], int i0, int j0, int r32, int kg,
+                                                 const int *__restrict__ exps = nullptr) {   // exps (f32 results only): row r times 2^exps[r]
 #pragma unroll
     for (int i = 0; i < FM; i++) {
+        int e[16];
+        if constexpr (sizeof(OUT) == 4) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) e[r] = exps ? exps[min(i0 + i * 32 + kg * 4 + (r >> 2) * 8 + (r & 3), M - 1)] : 0;
+        }
 #pragma unroll
         for (int j = 0; j < FN; j++) {
             const int gj = j0 + j * 32 + r32;
@@ -90,7 +104,7 @@ __device__ __forceinline__ void prefill_store_as(OUT *__restrict__ dst, int M, i
                 const int rf = (r >> 2) * 8 + (r & 3);   // (+ kg * 4, which is in `at`)
                 if (!CHECKED || (i0 + i * 32 + kg * 4 + rf < M && gj < N)) {
                     if constexpr (sizeof(OUT) == 2) at[(size_t)rf * N] = __float2half(total[i][j][r]);
-                    else at[(size_t)rf * N] = total[i][j][r];
+                    else at[(size_t)rf * N] = exps ? ldexpf(total[i][j][r], e[r]) : total[i][j][r];
                 }
             }
         }
@@ -101,12 +115,39 @@ __device__ __forceinline__ void prefill_store(const PrefillArgs &p, const f32x16
     const bool inside = i0 + FM * 32 <= p.M && j0 + FN * 32 <= p.N;
     float *f32_to = p.ksplit > 1 ? p.Ypart + (size_t)blockIdx.y * p.M * p.N : p.Yf32;
     if (f32_to) {
-        if (inside) prefill_store_as<FM, FN, false>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
-        else prefill_store_as<FM, FN, true>(f32_to, p.M, p.N, total, i0, j0, r32, kg);
+        const int *exps = p.ksplit > 1 ? nullptr : p.exps;
+        if (inside) prefill_store_as<FM, FN, false>(f32_to, p.M, p.N, total, i0, j0, r32, kg, exps);
+        else prefill_store_as<FM, FN, true>(f32_to, p.M, p.N, total, i0, j0, r32, kg, exps);
     } else {
         if (inside) prefill_store_as<FM, FN, false>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
         else prefill_store_as<FM, FN, true>(p.Y, p.M, p.N, total, i0, j0, r32, kg);
     }
+}
+
+// paired rows: one block of 32 result rows (first row i0 of the result) times 2^exps[row], or unscaled partials
+template <int FN, bool CHECKED>
+__device__ __forceinline__ void prefill_store_pairs_as(float *__restrict__ dst, const int *__restrict__ exps, int M, int N, const f32x16 (&total)[1][FN], int i0, int j0, int r32, int kg) {
+    int e[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) e[r] = exps ? exps[min(i0 + kg * 4 + (r >> 2) * 8 + (r & 3), M - 1)] : 0;
+#pragma unroll
+    for (int j = 0; j < FN; j++) {
+        const int gj = j0 + j * 32 + r32;
+        float *at = dst + (size_t)(i0 + kg * 4) * N + gj;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int rf = (r >> 2) * 8 + (r & 3);
+            if (!CHECKED || (i0 + kg * 4 + rf < M && gj < N)) at[(size_t)rf * N] = ldexpf(total[0][j][r], e[r]);
+        }
+    }
+}
+template <int FN>
+__device__ __forceinline__ void prefill_store_pairs(const PrefillArgs &p, const f32x16 (&total)[1][FN], int i0, int j0, int r32, int kg) {
+    const bool inside = i0 + 32 <= p.pair_rows && j0 + FN * 32 <= p.N;
+    float *to = p.ksplit > 1 ? p.Ypart + (size_t)blockIdx.y * p.pair_rows * p.N : p.Yf32;
+    const int *exps = p.ksplit > 1 ? nullptr : p.exps;
+    if (inside) prefill_store_pairs_as<FN, false>(to, exps, p.pair_rows, p.N, total, i0, j0, r32, kg);
+    else prefill_store_pairs_as<FN, true>(to, exps, p.pair_rows, p.N, total, i0, j0, r32, kg);
 }
 
 // FULL: K is a multiple of 128, so no stage is partial or missing and nothing needs masking.
@@ -571,6 +612,39 @@ __global__ void __launch_bounds__(256 * KG, KG > 1 ? 1 : MI * NJ == 1 ? 4 : MI *
         for (int i = 0; i < kF; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] *= scaled[j] ? unit[j] : 0.f;
+    if constexpr (MI == 2) {
+        if (p.pair_rows > 0) {
+            // paired rows: the wavefront's two row blocks are the two terms of the same 32 rows. Every group adds its
+            // own two, the second hands its sums to the first ([16-byte piece][thread] in LDS, as below), which adds
+            // them and stores.
+            f32x16 pair[1][NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) pair[0][j][r] = acc[0][j][r] + acc[1][j][r];
+            if constexpr (KG == 2) {
+                float4 *slot = reinterpret_cast<float4 *>(lds_raw);
+                if (grp > 0) {
+#pragma unroll
+                    for (int j = 0; j < NJ; j++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                            slot[(j * 4 + q) * 256 + tid] = make_float4(pair[0][j][4 * q], pair[0][j][4 * q + 1], pair[0][j][4 * q + 2], pair[0][j][4 * q + 3]);
+                }
+                __syncthreads();
+                if (grp > 0) return;
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const float4 o = slot[(j * 4 + q) * 256 + tid];
+                        pair[0][j][4 * q] += o.x, pair[0][j][4 * q + 1] += o.y, pair[0][j][4 * q + 2] += o.z, pair[0][j][4 * q + 3] += o.w;
+                    }
+            }
+            prefill_store_pairs<NJ>(p, pair, (i0 + wm * kWT) >> 1, j0 + wn * kWN, r32, kg);
+            return;
+        }
+    }
     if constexpr (KG > 1 && MI == 1) {
         // the later groups hand their accumulators to the first: [group - 1][16-byte piece][thread] in LDS (the A
         // buffers are done with: the last barrier of the loop is behind every read of them), added in group order
@@ -630,7 +704,8 @@ __global__ void __launch_bounds__(256 * KG, KG > 1 ? 1 : MI * NJ == 1 ? 4 : MI *
 // 16-byte store. (static: this file is compiled twice)
 template <bool VEC>
 static __global__ void __launch_bounds__(256)
-mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ Y, float *__restrict__ Yf32, long total, int ksplit) {
+mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ Y, float *__restrict__ Yf32, long total, int ksplit,
+                           const int *__restrict__ exps, int N) {   // exps: the f32 result's row r times 2^exps[r] (paired rows; VEC then has N a multiple of four)
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= total) return;
     if (VEC) {
@@ -638,6 +713,10 @@ mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ 
         for (int s = 1; s < ksplit; s++) {
             const float4 u = *reinterpret_cast<const float4 *>(part + (size_t)s * total + i);
             v.x += u.x, v.y += u.y, v.z += u.z, v.w += u.w;
+        }
+        if (exps) {
+            const int e = exps[i / N];
+            v = make_float4(ldexpf(v.x, e), ldexpf(v.y, e), ldexpf(v.z, e), ldexpf(v.w, e));
         }
         if (Yf32) {
             *reinterpret_cast<float4 *>(Yf32 + i) = v;
@@ -649,6 +728,7 @@ mmnb_prefill_reduce_kernel(const float *__restrict__ part, __half *__restrict__ 
     for (long j = i; j < min(i + 4, total); j++) {
         float v = part[j];
         for (int s = 1; s < ksplit; s++) v += part[(size_t)s * total + j];
+        if (exps) v = ldexpf(v, exps[j / N]);
         if (Yf32) Yf32[j] = v;
         else Y[j] = __float2half(v);
     }
@@ -693,12 +773,12 @@ int prefill_plan(hipc_ctx *ctx, PrefillArgs &a, int TM, int TN, bool may_split, 
 // the second launch of a k split
 int prefill_join_splits(hipc_ctx *ctx, const PrefillArgs &a) {
     if (a.ksplit > 1) {
-        const long total = (long)a.M * a.N;
-        const bool vec = total % 4 == 0 && (a.Yf32 ? aligned(a.Yf32, 16) : aligned(a.Y, 8));
+        const long total = (long)(a.pair_rows > 0 ? a.pair_rows : a.M) * a.N;
+        const bool vec = (a.exps ? a.N % 4 == 0 : total % 4 == 0) && (a.Yf32 ? aligned(a.Yf32, 16) : aligned(a.Y, 8));
         if (vec)
-            hipLaunchKernelGGL((mmnb_prefill_reduce_kernel<true>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit);
+            hipLaunchKernelGGL((mmnb_prefill_reduce_kernel<true>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit, a.exps, a.N);
         else
-            hipLaunchKernelGGL((mmnb_prefill_reduce_kernel<false>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit);
+            hipLaunchKernelGGL((mmnb_prefill_reduce_kernel<false>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, a.Ypart, a.Y, a.Yf32, total, a.ksplit, a.exps, a.N);
         HIPC_LAUNCHED(ctx);
     }
     return HIPC_OK;
@@ -824,6 +904,7 @@ int prefill_launch(hipc_ctx *ctx, const PrefillArgs &a) {
     const int64_t cus = std::max(1, ctx->cu_count);
     if (tile == 128 && tiles128 >= 256 && ctx->tune.prefill_direct != 0 && ceil_div(tiles192, cus) * 3 < ceil_div(tiles128, cus) * 2) tile = 192;
     if (forced == 64 || forced == 128 || (forced == 192 && ctx->tune.prefill_direct != 0)) tile = forced;
+    if (a.pair_rows > 0 && tile == 64) tile = 128;   // paired rows are the two row blocks of a wavefront: 128-row tiles
     return tile == 64 && ctx->tune.prefill_direct == 0 ? prefill_launch_tile<SG, 64>(ctx, a) : prefill_launch_wide(ctx, a, SG, tile);
 }
 
@@ -848,11 +929,20 @@ int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void
 // Rows of f32 activations for the f16 matrix cores: row m becomes two f16 rows, hi = f16(a 2^-e) and
 // lo = f16(a 2^-e - hi) (22 significant bits), with 2^e the row's own power of two that brings its
 // largest magnitude into [2^14, 2^15) -- exact, and no value of the row leaves the f16 range. The rows
-// are stored as A2[m] = hi, A2[M + m] = lo; one workgroup per row.
+// are stored as A2[m] = hi, A2[M + m] = lo; one workgroup per row. PAIRED: 32 rows of high terms are followed by the
+// 32 rows of their low terms (row m: hi at 64 (m / 32) + m % 32, lo 32 rows on), the grid covers a multiple of 32
+// rows and the rows past M are zeros.
+template <bool PAIRED, bool LOW = true>   // LOW false: the high terms alone, M rows
 static __global__ void __launch_bounds__(256)
 mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half *__restrict__ A2, int *__restrict__ exps) {
     __shared__ float red[4];
     const int m = blockIdx.x, tid = threadIdx.x;
+    const size_t hi_at = PAIRED ? (size_t)(64 * (m >> 5) + (m & 31)) : (size_t)m, lo_at = PAIRED ? hi_at + 32 : (size_t)M + m;
+    if (PAIRED && m >= M) {
+        uint4 *hi_row = reinterpret_cast<uint4 *>(A2 + hi_at * K), *lo_row = reinterpret_cast<uint4 *>(A2 + lo_at * K);
+        for (int c = tid; c < K / 8; c += 256) hi_row[c] = make_uint4(0u, 0u, 0u, 0u), lo_row[c] = make_uint4(0u, 0u, 0u, 0u);
+        return;
+    }
     const float4 *row = reinterpret_cast<const float4 *>(A + (size_t)m * K);   // (K is a multiple of 8 and A is aligned: see nbits_prefill_f32_takes)
     const int nv = K / 4;
     constexpr int kHeld = 4;   // 16-byte pieces a thread keeps between the two passes: rows up to 4096 values are read once
@@ -878,14 +968,14 @@ mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half
     const int e = (ef == 0 || ef == 255) ? 0 : ef - 127 - 14;
     if (tid == 0) exps[m] = e;
     const float down = __uint_as_float((uint32_t)(127 - e) << 23);   // 2^-e: e is in [-140, 113], 2^-e a normal number
-    uint2 *hi_row = reinterpret_cast<uint2 *>(A2 + (size_t)m * K), *lo_row = reinterpret_cast<uint2 *>(A2 + (size_t)(M + m) * K);
+    uint2 *hi_row = reinterpret_cast<uint2 *>(A2 + hi_at * K), *lo_row = reinterpret_cast<uint2 *>(A2 + lo_at * K);
     auto split4 = [&](const float4 &v, int c) {
         const float a[4] = {v.x * down, v.y * down, v.z * down, v.w * down};
         __half hi[4], lo[4];
 #pragma unroll
         for (int t = 0; t < 4; t++) hi[t] = __float2half(a[t]), lo[t] = __float2half(a[t] - __half2float(hi[t]));
         hi_row[c] = make_uint2(two_halves(hi[0], hi[1]), two_halves(hi[2], hi[3]));
-        lo_row[c] = make_uint2(two_halves(lo[0], lo[1]), two_halves(lo[2], lo[3]));
+        if (LOW) lo_row[c] = make_uint2(two_halves(lo[0], lo[1]), two_halves(lo[2], lo[3]));
     };
 #pragma unroll
     for (int u = 0; u < kHeld; u++)
@@ -907,33 +997,61 @@ mmnb_prefill_join_rows_kernel(const float *__restrict__ P, const int *__restrict
     }
 }
 
-// Many rows of f32 activations: each row as two f16 rows (22 bits) through the same tiled kernel, 2 M rows
-// of f32 results, and a last launch that adds the pairs and puts the rows' powers of two back. Twice the
-// products of the f16 case, against one pass over the whole weight per 16 rows on the decode kernel.
+// Many rows of f32 activations: each row as two f16 rows (22 bits) through the same tiled kernel. Twice the products
+// of the f16 case, against one pass over the whole weight per 16 rows on the decode kernel. With the kernel that
+// keeps the weight out of LDS the two terms of a row are the two row blocks of one wavefront, which adds them and
+// puts the rows' powers of two back itself; the kernel that stages both operands through LDS writes 2 M rows of f32
+// results and a last launch adds the pairs.
 bool nbits_prefill_f32_takes(const void *A, const hipc_nbits_weight *w, int64_t M) {
-    return M > 32 && w->K % 8 == 0 && aligned(A, 16) && 2 * M * w->K < (int64_t(1) << 31) && 2 * M * w->N < (int64_t(1) << 31);
+    return M > 32 && w->K % 8 == 0 && aligned(A, 16) && (2 * M + 64) * w->K < (int64_t(1) << 31) && 2 * M * w->N < (int64_t(1) << 31);
 }
 
-int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M) {
+int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M, int terms) {
     HIPC_REFUSE(ctx, !nbits_prefill_f32_takes(A, w, M), "MatMulNBits prefill: shape or alignment not taken by the tiled kernel");
-    const size_t a2_bytes = (size_t)2 * M * w->K * sizeof(__half), e_bytes = ((size_t)M * sizeof(int) + 255) & ~(size_t)255;
+    if (terms == 1) {
+        // one f16 term per row (11 bits beside the row's own power of two): M rows through the kernel, which scales
+        // the rows of its f32 result back itself (after a k split, the reduce launch does)
+        const size_t e_bytes = ((size_t)M * sizeof(int) + 255) & ~(size_t)255;
+        void *split = nullptr;
+        if (int rc = scratch_get(ctx, 2, (size_t)M * w->K * sizeof(__half) + e_bytes, &split)) return rc;
+        __half *A1 = reinterpret_cast<__half *>(static_cast<char *>(split) + e_bytes);
+        int *exps = static_cast<int *>(split);
+        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<false, false>), dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A1, exps);
+        HIPC_LAUNCHED(ctx);
+        PrefillArgs a{};
+        a.A = A1, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = nullptr, a.Yf32 = static_cast<float *>(Y), a.exps = exps;
+        a.M = (int)M, a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
+        switch (w->SG) {
+            case 4: return prefill_launch<4>(ctx, a);
+            case 2: return prefill_launch<2>(ctx, a);
+            default: return prefill_launch<1>(ctx, a);
+        }
+    }
+    const bool paired = ctx->tune.prefill_direct != 0;
+    const int64_t rows2 = paired ? 64 * ceil_div(M, 32) : 2 * M;
+    const size_t a2_bytes = (size_t)rows2 * w->K * sizeof(__half), e_bytes = ((size_t)M * sizeof(int) + 255) & ~(size_t)255;
     void *split = nullptr, *sums = nullptr;
     if (int rc = scratch_get(ctx, 2, a2_bytes + e_bytes, &split)) return rc;
-    if (int rc = scratch_get(ctx, 3, (size_t)2 * M * w->N * sizeof(float), &sums)) return rc;
+    if (!paired)
+        if (int rc = scratch_get(ctx, 3, (size_t)2 * M * w->N * sizeof(float), &sums)) return rc;
     __half *A2 = reinterpret_cast<__half *>(static_cast<char *>(split) + e_bytes);
     int *exps = static_cast<int *>(split);
-    hipLaunchKernelGGL(mmnb_prefill_split_rows_kernel, dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
+    if (paired)
+        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<true, true>), dim3((unsigned)(rows2 / 2)), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
+    else
+        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<false, true>), dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
     HIPC_LAUNCHED(ctx);
     PrefillArgs a{};
-    a.A = A2, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = nullptr, a.Yf32 = static_cast<float *>(sums);
-    a.M = (int)(2 * M), a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
+    a.A = A2, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = nullptr, a.Yf32 = static_cast<float *>(paired ? Y : sums);
+    a.M = (int)rows2, a.K = (int)w->K, a.N = (int)w->N, a.n_tiles = w->n_tiles, a.n_cg = w->n_cg;
+    if (paired) a.exps = exps, a.pair_rows = (int)M;
     int rc;
     switch (w->SG) {
         case 4: rc = prefill_launch<4>(ctx, a); break;
         case 2: rc = prefill_launch<2>(ctx, a); break;
         default: rc = prefill_launch<1>(ctx, a); break;
     }
-    if (rc != HIPC_OK) return rc;
+    if (rc != HIPC_OK || paired) return rc;
     const long total = (long)M * w->N;
     if (w->N % 4 == 0 && aligned(Y, 16))
         hipLaunchKernelGGL((mmnb_prefill_join_rows_kernel<true>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, static_cast<const float *>(sums), exps, (int)M, (int)w->N, static_cast<float *>(Y));

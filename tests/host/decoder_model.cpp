@@ -41,7 +41,7 @@ int scratch_get(hipc_ctx *ctx, int slot, size_t bytes, void **out) {
 bool nbits_prefill_takes(const void *, const hipc_nbits_weight *, int64_t) { return false; }
 int nbits_prefill(hipc_ctx *, const void *, const hipc_nbits_weight *, void *, int64_t) { return HIPC_ERR_UNSUPPORTED; }
 bool nbits_prefill_f32_takes(const void *, const hipc_nbits_weight *, int64_t) { return false; }
-int nbits_prefill_f32(hipc_ctx *, const void *, const hipc_nbits_weight *, void *, int64_t) { return HIPC_ERR_UNSUPPORTED; }
+int nbits_prefill_f32(hipc_ctx *, const void *, const hipc_nbits_weight *, void *, int64_t, int) { return HIPC_ERR_UNSUPPORTED; }
 }  // namespace hipc
 extern "C" {
 const char *hipGetErrorString(hipError_t) { return "model"; }

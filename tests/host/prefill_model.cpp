@@ -80,6 +80,8 @@ void product(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dt
                       a_dtype == HIPC_F16 ? "f16" : "f32", r.tile, r.direct, r.split, r.groups);
         gpu_model::reg().where = where;
         MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 0));
+        // (f32 rows at a level that allows f16 activations: one term per row, the kernel scales the result's rows)
+        if (a_dtype == HIPC_F32) MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 2));
     }
     ctx.tune.prefill_tile = ctx.tune.prefill_direct = ctx.tune.prefill_split = ctx.tune.prefill_groups = -1;
     gpu_model::release(A), gpu_model::release(Y);

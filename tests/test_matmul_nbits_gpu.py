@@ -204,8 +204,18 @@ F32_PREFILL = [  # (M, K, N, block_size, zero points)
 ]
 
 
+F32_ROUTES = [  # the default; the two terms of a row as the two row blocks of a wavefront (128 x 128 and 128 x 192 tiles, two k
+    # groups per workgroup, k split over workgroups, a forced 64-row tile that such rows cannot take); the kernel
+    # with both operands in LDS, whose 2 M result rows a last launch adds up
+    {}, {"HIPC_PREFILL_TILE": 128}, {"HIPC_PREFILL_TILE": 192}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 2},
+    {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2}, {"HIPC_PREFILL_TILE": 192, "HIPC_PREFILL_GROUPS": 2, "HIPC_PREFILL_SPLIT": 2},
+    {"HIPC_PREFILL_TILE": 64}, {"HIPC_PREFILL_DIRECT": 0}, {"HIPC_PREFILL_DIRECT": 0, "HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2},
+]
+
+
+@pytest.mark.parametrize("options", F32_ROUTES, ids=lambda v: str(v).replace(" ", ""))
 @pytest.mark.parametrize("shape", F32_PREFILL, ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
-def test_f32_rows_beyond_thirty_two_run_the_tiled_kernel(ctx, pkg, oracle, shape):
+def test_f32_rows_beyond_thirty_two_run_the_tiled_kernel(ctx, pkg, oracle, shape, options):
     """More than 32 rows of f32 activations (the reference's own element type, interp.rs:6455-6472) go through
     the tiled matrix-core kernel as two f16 rows each, scaled per row by a power of two: against the oracle at
     the operator's f32 tolerance, against the float64 product at 2e-5 of the row's largest output, and equal
@@ -218,7 +228,8 @@ def test_f32_rows_beyond_thirty_two_run_the_tiled_kernel(ctx, pkg, oracle, shape
     a[2] = 0
     want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
     w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
-    got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    with ctx.options(**options):
+        got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
     by_rows = np.concatenate([pkg.ops.matmul_nbits(ctx, a[i:i + 16], None, None, None, k, n, bs, weight=w) for i in range(0, m, 16)])
     w.destroy()
     assert got.dtype == np.float32 and got.shape == (m, n)
@@ -230,6 +241,37 @@ def test_f32_rows_beyond_thirty_two_run_the_tiled_kernel(ctx, pkg, oracle, shape
     big = np.abs(f64).max(axis=1, keepdims=True)
     assert np.all(np.abs(got - f64) <= 2e-5 * np.maximum(big, 1e-300)), float(np.max(np.abs(got - f64) / np.maximum(big, 1e-300)))
     assert np.all(np.abs(got - f64) <= np.abs(by_rows - f64).max(axis=1, keepdims=True) * 1.5 + 2e-6 * big)
+    assert np.all(got[2] == 0)
+
+
+@pytest.mark.parametrize("options", [{}, {"HIPC_PREFILL_TILE": 64}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_GROUPS": 2}, {"HIPC_PREFILL_TILE": 192},
+                                     {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2}, {"HIPC_PREFILL_DIRECT": 0}], ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("level", [2, 3, 4])
+@pytest.mark.parametrize("shape", F32_PREFILL, ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_f32_rows_at_a_level_that_allows_f16_activations(ctx, pkg, oracle, shape, level, options):
+    """accuracy_level 2, 3 and 4 allow the activations to be reduced to f16, bf16 or int8 (the reference never reads
+    the attribute and computes in f32). More than 32 rows of f32 then travel as ONE f16 row each: the row times the
+    power of two that puts its largest value into [2^14, 2^15), rounded to f16 (11 bits of every value, whatever the
+    row's size). The result is the operator on exactly those rounded rows, at the f32 tolerance -- and so within
+    what each of the three levels permits."""
+    m, k, n, bs, with_zp = shape
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=45, with_zp=with_zp)
+    a = pkg.synth.normal_f32(m * k, 46).reshape(m, k)
+    a[0] *= np.float32(3.0e7)
+    a[1] *= np.float32(1.0e-9)
+    a[2] = 0
+    mx = np.abs(a).max(axis=1, keepdims=True)
+    e = np.where(mx > 0, np.floor(np.log2(np.maximum(mx, np.float32(1e-30)))) - 14, 0).astype(np.int32)
+    rounded = np.ldexp(np.ldexp(a, -e).astype(np.float16).astype(np.float32), e).astype(np.float32)
+    assert np.all(np.abs(rounded - a) <= 2.0 ** -11 * mx)
+    want = oracle.matmul_nbits(rounded, B, scales, zp, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    with ctx.options(**options):
+        got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, accuracy_level=level, weight=w)
+    w.destroy()
+    assert got.dtype == np.float32 and got.shape == (m, n)
+    scale = np.maximum(np.abs(want).max(axis=1, keepdims=True), 1e-30)
+    assert np.all(np.abs(got - want) <= (1e-3 + 1e-4 * np.abs(want)) * np.maximum(scale / np.abs(want[3:]).max(), 1e-30) + 1e-4 * scale), worst(got, want)
     assert np.all(got[2] == 0)
 
 
@@ -272,8 +314,8 @@ def test_refusals_and_short_buffers(ctx, pkg):
     k, n, bs = 128, 16, 32
     B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=1)
     a = np.zeros((1, k), np.float32)
-    with pytest.raises(pkg.HipComputeError) as e:   # level 4 asks for int8 activations
-        pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs, accuracy_level=4)
+    with pytest.raises(pkg.HipComputeError) as e:   # the operator defines levels 0..4
+        pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs, accuracy_level=5)
     assert e.value.code == 2
     with pytest.raises(pkg.HipComputeError) as e:   # the weight is short for N (interp.rs:6465-6472)
         pkg.ops.matmul_nbits(ctx, a, B[: n - 1], scales, zp, k, n, bs)
@@ -297,8 +339,8 @@ def _unpack(B, zp, k, n, bs):
 
 @pytest.mark.parametrize("shape", [(1, 1152, 6912), (1, 6912, 1152), (8, 1152, 512), (1, 1152, 32768 + 48)], ids=lambda s: "M%d_K%d_N%d" % s)
 def test_accuracy_levels(ctx, pkg, oracle, shape):
-    """accuracy_level 0 (unset), 2 and 3 let an f32 activation enter the matrix cores as two bf16 terms;
-    1 pins f32 and sends all 24 bits (three terms). The last shape has more than 2048 column tiles, so
+    """accuracy_level 0 (unset), 2, 3 and 4 (a lower bound: the reference computes every level in f32) let
+    an f32 activation enter the matrix cores as two bf16 terms; 1 pins f32 and sends all 24 bits (three terms). The last shape has more than 2048 column tiles, so
     its one row takes the wide streaming kernel (the unembedding's route) and level 1 that kernel's
     three-term instance. Every level meets the operator's tolerance
     against the oracle; level 1 is held to a tighter bound against the float64 product -- 2e-5 of
@@ -313,14 +355,14 @@ def test_accuracy_levels(ctx, pkg, oracle, shape):
     f64 = rc.matmul_nbits_f64(a, nib, z, scales.reshape(n, -1), bs)
     w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
     err = {}
-    for level in (0, 1, 2, 3):
+    for level in (0, 1, 2, 3, 4):
         got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, accuracy_level=level, weight=w)
         assert close(got, want, RTOL32), (level, worst(got, want))
         err[level] = float(np.max(np.abs(got - f64)))
     w.destroy()
     assert err[1] <= 2e-5 * float(np.max(np.abs(f64))), err
     assert err[1] <= err[0] * 1.05 + 1e-7, err
-    assert err[2] == err[0] and err[3] == err[0], err     # the same kernel instance as the default
+    assert err[2] == err[0] and err[3] == err[0] and err[4] == err[0], err     # the same kernel instance as the default
 
 
 @pytest.mark.parametrize("shape", [(1, 1152, 6912, 32, True), (1, 6912, 1152, 32, True), (1, 2048, 2560, 128, False),
