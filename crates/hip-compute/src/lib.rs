@@ -409,7 +409,7 @@ impl HipContext {
 
     // -------------------------------------------------------------- MatMulNBits
 
-    /// `interp::matmul_nbits` (interp.rs:6429-6561) on the ONNX layout: `block_size == 16`, or a weight used once.
+    /// `interp::matmul_nbits` (interp.rs:6429-6561) on the ONNX layout: a weight used once (`prepack_matmul_nbits` takes every block size).
     pub fn matmul_nbits(&self, a: BufferSlice<'_>, a_dtype: DType, w: &NBitsOperands<'_>, y: BufferSlice<'_>, m: i64, accuracy_level: i32) -> Result<()> {
         let (zp, zp_len) = w.zero_points.map_or((ptr::null_mut(), 0), |(s, n)| (s.ptr(), n));
         self.check(unsafe {

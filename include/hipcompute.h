@@ -176,7 +176,9 @@ int hipc_matmul_nbits(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, 
 /* Repack a constant weight once (the role `packed_b` plays for MatMulInteger,
  * interp.rs:2712-2768; the reference feeds MatMulNBits the ONNX layout directly).
  * The operands are device pointers in the ONNX layout above and may be released
- * after the next flush. */
+ * after the next flush. A block_size below 32 or not a power of two has no tiled form:
+ * its handle holds copies of the tensors as they are and hipc_matmul_nbits_packed runs
+ * the kernel of hipc_matmul_nbits on them (the same results, bit for bit). */
 int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales,
                               int scale_dtype, size_t scales_len, const void *zp, size_t zp_len,
                               int64_t K, int64_t N, int64_t block_size, hipc_nbits_weight **out);

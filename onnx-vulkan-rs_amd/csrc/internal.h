@@ -150,6 +150,11 @@ struct hipc_nbits_weight {
     float *Sc = nullptr;
     uint8_t *Zb = nullptr;
     size_t bytes = 0;
+    // A block_size below 32 or not a power of two has no tiled form (a 32-k product step would straddle scale
+    // groups): the handle then keeps device copies of the operator's own tensors (Wq is null) and the product
+    // runs on the kernel that reads that layout. Only hipc_matmul_nbits_packed takes such a handle.
+    void *raw_B = nullptr, *raw_scales = nullptr, *raw_zp = nullptr;
+    int raw_scale_dtype = 0;
 };
 
 namespace hipc {
@@ -297,7 +302,7 @@ inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_
 // MatMulNBits pieces other operators of the library build on (the caller holds the lock)
 int nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype, size_t scales_len,
                   const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size, hipc_nbits_weight **out,
-                  int interleave_half = 0);
+                  int interleave_half = 0, bool any_block_size = false);   // any_block_size: may return a handle in the operator's layout
 void nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w);
 // rows [0, M), M <= 16, of A against a prepacked weight; `terms` = bf16 terms per activation (2 or 3)
 // What the single activation row of a decode GEMV is computed from (mode 0 / null: A as given):

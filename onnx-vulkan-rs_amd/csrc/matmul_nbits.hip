@@ -1041,7 +1041,7 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
                               hipc_nbits_weight **out) {
     if (!out) return HIPC_ERR_INVALID;
     return entry(ctx, [&]() -> int {
-        return hipc::nbits_prepack(ctx, B, b_len, scales, scale_dtype, scales_len, zp, zp_len, K, N, block_size, out);
+        return hipc::nbits_prepack(ctx, B, b_len, scales, scale_dtype, scales_len, zp, zp_len, K, N, block_size, out, 0, true);
     });
 }
 
@@ -1050,7 +1050,7 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
 // The same operations for callers inside the library that already hold the context's lock.
 int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype,
                         size_t scales_len, const void *zp, size_t zp_len, int64_t K, int64_t N, int64_t block_size,
-                        hipc_nbits_weight **out, int interleave_half) {
+                        hipc_nbits_weight **out, int interleave_half, bool any_block_size) {
     *out = nullptr;
     HIPC_REQUIRE(ctx, interleave_half == 0 || (interleave_half % 16 == 0 && 2 * (int64_t)interleave_half == N),
                  "MatMulNBits prepack: interleaved halves of %d columns do not make up N=%ld in whole tiles", interleave_half, (long)N);
@@ -1059,10 +1059,35 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
     if (rc != HIPC_OK) return rc;
     HIPC_REQUIRE(ctx, N > 0 && B && scales, "MatMulNBits prepack: empty weight");
     HIPC_REQUIRE(ctx, aligned(B, 4), "MatMulNBits: packed weight must be 4-byte aligned");
-    HIPC_REFUSE(ctx, block_size < 32 || !is_pow2(block_size),
-                "MatMulNBits prepack: block_size %ld (below 32, or not a power of two) only runs on the direct path", (long)block_size);
+    const bool tiled = block_size >= 32 && is_pow2(block_size);
+    HIPC_REFUSE(ctx, !tiled && (!any_block_size || interleave_half != 0),
+                "MatMulNBits prepack: block_size %ld (below 32, or not a power of two) has no tiled form", (long)block_size);
     hipc_nbits_weight *w = new hipc_nbits_weight();
     w->K = K, w->N = N, w->block_size = block_size;
+    if (!tiled) {
+        // the reference's envelope is every positive multiple of 8 (interp.rs:447-464): copies of the tensors as they are
+        const size_t esz = scale_dtype == HIPC_F16 ? 2 : 4;
+        const size_t sizes[3] = {b_len, scales_len * esz, zp ? zp_len : 0};
+        const void *from[3] = {B, scales, zp};
+        void **to[3] = {&w->raw_B, &w->raw_scales, &w->raw_zp};
+        hipError_t e = hipSuccess;
+        for (int i = 0; i < 3 && e == hipSuccess; i++) {
+            if (sizes[i] == 0) continue;
+            e = hipMalloc(to[i], (sizes[i] + 3) & ~(size_t)3);
+            if (e == hipSuccess) e = hipMemcpyAsync(*to[i], from[i], sizes[i], hipMemcpyDeviceToDevice, ctx->stream);
+        }
+        if (e != hipSuccess) {
+            for (int i = 0; i < 3; i++)
+                if (*to[i]) (void)hipFree(*to[i]);
+            delete w;
+            return fail(ctx, HIPC_ERR_BACKEND, "MatMulNBits prepack: %s", hipGetErrorString(e));
+        }
+        HIPC_LAUNCHED(ctx);
+        w->raw_scale_dtype = scale_dtype;
+        w->bytes = sizes[0] + sizes[1] + sizes[2];
+        *out = w;
+        return HIPC_OK;
+    }
     w->interleave_half = interleave_half;
     const int n_blocks = (int)ceil_div(K, block_size);
     const int n_chunks = (int)ceil_div(K, 32);
@@ -1115,6 +1140,8 @@ void hipc::nbits_release(hipc_ctx *ctx, hipc_nbits_weight *w) {
     if (w->Wq) ctx->deferred.push_back(w->Wq);
     if (w->Sc) ctx->deferred.push_back(w->Sc);
     if (w->Zb) ctx->deferred.push_back(w->Zb);
+    for (void *p : {w->raw_B, w->raw_scales, w->raw_zp})
+        if (p) ctx->deferred.push_back(p);
     delete w;
 }
 
@@ -1148,6 +1175,13 @@ int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hi
         HIPC_REQUIRE(ctx, M >= 0 && M < (int64_t(1) << 30), "MatMulNBits: bad M=%ld", (long)M);
         if (M == 0) return HIPC_OK;
         HIPC_REQUIRE(ctx, A && Y, "MatMulNBits: null operand");
+        if (!w->Wq) {   // a handle in the operator's own layout (block_size below 32 or not a power of two)
+            const bool af16 = a_dtype == HIPC_F16, sf16 = w->raw_scale_dtype == HIPC_F16;
+            if (af16 && sf16) return launch_direct<__half, __half>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+            if (af16) return launch_direct<__half, float>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+            if (sf16) return launch_direct<float, __half>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+            return launch_direct<float, float>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+        }
         const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
         // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
         // terms). Unset, or 2 / 3 / 4 (f16 / bf16 / int8 are enough): 2 terms. f16 activations are exact in 2.

@@ -106,7 +106,7 @@ void rows(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dtype
     gpu_model::reg().where = where;
     for (int level : {0, 1})
         MUST(hipc_matmul_nbits(&ctx, A, a_dtype, B, b_len, S, a_dtype, s_len, with_zp ? Z : nullptr, with_zp ? z_len : 0, Y, M, K, N, bs, level));
-    if (bs >= 32 && (bs & (bs - 1)) == 0) {
+    {   // (a block size without a tiled form: the handle's own copies of the tensors, exactly as long as they are)
         hipc_nbits_weight *w = nullptr;
         MUST(hipc_prepack_matmul_nbits(&ctx, B, b_len, S, a_dtype, s_len, with_zp ? Z : nullptr, with_zp ? z_len : 0, K, N, bs, &w));
         for (int level : {0, 1}) MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, level));

@@ -85,17 +85,27 @@ def test_seeded_shapes_both_paths(ctx, pkg, oracle, shape):
 
 @pytest.mark.parametrize("k,n,bs", [(208, 50, 16), (200, 33, 8), (240, 50, 24), (1000, 64, 40), (330, 17, 48)],
                          ids=lambda v: str(v))
-def test_small_and_odd_block_sizes_run_direct_and_refuse_prepack(ctx, pkg, oracle, k, n, bs):
+def test_small_and_odd_block_sizes(ctx, pkg, oracle, k, n, bs):
     """The reference accepts every block_size that is a positive multiple of 8 (interp.rs:447-464); those
     below 32 or not a power of two run on the kernel that reads the ONNX layout. 13 blocks of 16: odd,
-    zero-point rows off word boundaries; 8, 24, 40, 48: blocks that are no power of two, partial last block."""
+    zero-point rows off word boundaries; 8, 24, 40, 48: blocks that are no power of two, partial last block.
+    A handle for such a weight keeps the tensors as they are (the caller's copies may go) and gives the
+    same bits; one row, a few and more than 32 (no tiled kernel for them)."""
     B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=3)
-    a = pkg.synth.normal_f32(3 * k, 8).reshape(3, k)
-    got = pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs)
-    assert close(got, oracle.matmul_nbits(a, B, scales, zp, k, n, bs), RTOL32)
-    with pytest.raises(pkg.HipComputeError) as e:
-        pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
-    assert e.value.code == 2
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    for m in (1, 3, 40):
+        a = pkg.synth.normal_f32(m * k, 8 + m).reshape(m, k)
+        got = pkg.ops.matmul_nbits(ctx, a, B, scales, zp, k, n, bs)
+        assert close(got, oracle.matmul_nbits(a, B, scales, zp, k, n, bs), RTOL32)
+        by_handle = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+        assert np.array_equal(by_handle, got)
+    a16 = pkg.synth.normal_f32(5 * k, 9).reshape(5, k).astype(np.float16)
+    B16, s16, _ = pkg.synth.nbits_weight(n, k, bs, seed=4, with_zp=False, scale_dtype=np.float16)
+    w16 = pkg.ops.NBitsWeight(ctx, B16, s16, None, k, n, bs)
+    got = pkg.ops.matmul_nbits(ctx, a16, None, None, None, k, n, bs, weight=w16)
+    assert got.dtype == np.float16 and close(got, oracle.matmul_nbits(a16, B16, s16, None, k, n, bs), RTOL16)
+    assert w.nbytes == B.size + 4 * scales.size + zp.size
+    w.destroy(), w16.destroy()
 
 
 @pytest.mark.parametrize("shape", [(1, 2048, 2560, 128), (6, 1024, 300, 32), (40, 512, 128, 128)],
