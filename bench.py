@@ -207,7 +207,7 @@ def bench_lm_head(pkg, ctx, copies=3, accuracy_level=0):
     per = gemv_bytes(K, N)
     s.destroy()
     return dict(bound="hbm", achieved=per / med, peak=HBM_PEAK_GBS, unit="GB/s", frac=per / med / HBM_PEAK_GBS,
-                traffic=LM_HEAD_TRAFFIC_BYTES, kernel="mmnb_gemv_kernel (lm_head 1152->262144, M=1)", bytes_per_launch=per,
+                traffic=LM_HEAD_TRAFFIC_BYTES if accuracy_level == 0 else None, kernel="mmnb_gemv_kernel (lm_head 1152->262144, M=1)", bytes_per_launch=per,
                 avg_launch_us=med / 1e3, min_launch_us=mn / 1e3, accuracy_level=accuracy_level)
 
 
@@ -619,6 +619,9 @@ def main():
     if want("lm_head"):
         extras["lm_head_gemv"] = bench_lm_head(pkg, ctx)
         log(f"[bench] lm_head gemv: {extras['lm_head_gemv']['avg_launch_us']:.1f} us, {extras['lm_head_gemv']['achieved']:.0f} GB/s")
+        # the same launch with f32 pinned (accuracy_level = 1: three bf16 terms per activation, all 24 bits)
+        extras["lm_head_gemv_level1"] = bench_lm_head(pkg, ctx, accuracy_level=1)
+        log(f"[bench] lm_head gemv, level 1: {extras['lm_head_gemv_level1']['avg_launch_us']:.1f} us")
     if want("gemv"):
         extras["gemv_up_1152x6912"] = bench_single_gemv(pkg, ctx, 1152, 6912, cold_copies=104)
         extras["gemv_down_6912x1152"] = bench_single_gemv(pkg, ctx, 6912, 1152, cold_copies=104)
