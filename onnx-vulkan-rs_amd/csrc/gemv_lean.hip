@@ -613,15 +613,17 @@ int lean_launch_pro(hipc_ctx *ctx, const LeanArgs &a, int pro, int epi, dim3 gri
 
 }  // namespace
 
-bool hipc::lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int WN, LeanPlan *out, int max_waves) {
+bool hipc::lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int WN, LeanPlan *out, int max_waves, bool short_in_three) {
     if (w->K % 8 != 0 || slices < 1 || WN < 1 || WN > max_waves) return false;
     const int per_slice = (w->n_cg + slices - 1) / slices;   // k tiles a workgroup covers
-    // k tiles per wavefront: the fewest that fit the wavefronts a workgroup may have; three when the
-    // slice is short (a workgroup of three wavefronts then holds the row and all of them prepare it)
+    // k tiles per wavefront: the fewest that fit the wavefronts a workgroup may have. short_in_three: three when
+    // the slice is short (a workgroup of three wavefronts then holds the row and all of them take part in a norm or
+    // join prologue; the plain-row prologue is over sooner than two more tiles' products: 1152 -> 1536 as nine
+    // wavefronts of one tile each, 4.25 against 4.36 us over a token's stand-alone launches)
     const int max_wk = max_waves / WN;
     int KT = (per_slice + max_wk - 1) / max_wk;
     if (ctx->tune.gemv_t >= 1 && ctx->tune.gemv_t <= 4) KT = std::max(KT, ctx->tune.gemv_t);
-    else if (per_slice <= 12 && per_slice >= 3) KT = std::max(KT, 3);
+    else if (short_in_three && per_slice <= 12 && per_slice >= 3) KT = std::max(KT, 3);
     if (KT > 4) return false;
     LeanPlan pl{};
     pl.KT = KT, pl.WK = (per_slice + KT - 1) / KT, pl.WN = WN, pl.slices = slices;

@@ -441,7 +441,7 @@ struct LeanPlan {
     int WK, KT, WN, slices;
 };
 // false when the shape does not fit the kernel (k tiles per wavefront would exceed 4)
-bool lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int WN, LeanPlan *out, int max_waves = 16);
+bool lean_plan(hipc_ctx *ctx, const hipc_nbits_weight *w, int slices, int WN, LeanPlan *out, int max_waves = 16, bool short_in_three = true);
 // `a` carries the prologue / epilogue operands; weight and launch-shape fields are filled in here
 int lean_gemv(hipc_ctx *ctx, const hipc_nbits_weight *w, const LeanPlan &pl, LeanArgs a, int pro, int epi, int NT);
 // the prefetch description of a one-row product launched with plan `pl` (for the launch before it)

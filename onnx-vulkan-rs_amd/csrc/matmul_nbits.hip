@@ -913,7 +913,7 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
         // several column tiles per workgroup once that still leaves a workgroup for most CUs: the row is then prepared
         // (read, split into terms, written to LDS) by a half or a quarter as many workgroups (1152 -> 13824: 5.4 -> 5.0 us)
         const int WN = w->n_tiles >= 768 ? 4 : w->n_tiles >= 384 ? 2 : 1;
-        if (lean_plan(ctx, w, 1, WN, &pl)) {
+        if (lean_plan(ctx, w, 1, WN, &pl, 16, false)) {
             LeanArgs la{};
             la.A = static_cast<const float *>(A), la.Y = static_cast<float *>(Y);
             return lean_gemv(ctx, w, pl, la, 0, 0, NT);

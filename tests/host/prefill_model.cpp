@@ -142,7 +142,10 @@ int main() {
     // few rows: block sizes of the reference's envelope that only the ONNX-layout kernel takes (8, 24, 40), the
     // prepacked ones on the decode kernels; one row, a partial 16-row group, a full one; ragged K and N
     const int64_t few[][5] = {{1, 72, 16, 8, 1},   {3, 120, 50, 24, 1},  {16, 200, 33, 40, 0}, {1, 1000, 200, 32, 1}, {5, 384, 131, 64, 1},
-                              {16, 640, 96, 128, 0}, {1, 1152, 1536, 32, 1}, {2, 256, 1024, 256, 1}};
+                              {16, 640, 96, 128, 0}, {1, 1152, 1536, 32, 1}, {2, 256, 1024, 256, 1},
+                              // the stand-alone launches of a gemma3-1b token (one k tile per wavefront up to sixteen tiles,
+                              // four column tiles per workgroup on the widest, four k tiles per wavefront on the longest), a ragged k
+                              {1, 1024, 1152, 32, 1}, {1, 1152, 13824, 32, 1}, {1, 6912, 1152, 32, 1}, {1, 1480, 64, 32, 1}};
     for (const auto &s : few)
         for (int dt : {HIPC_F32, HIPC_F16}) rows(s[0], s[1], s[2], s[3], s[4] != 0, dt);
     gpu_model::Registry &g = gpu_model::reg();
