@@ -525,10 +525,10 @@ def bench_prefill(pkg, ctx, M=512, bs=128):
                                                     frac_of_min_bound=min_bound_us(byts, flops, F16_PEAK_TFLOPS) / (ns / 1e3))
         if name == "qkv_2048x2560":
             # the same product with f32 rows: two f16 rows each through the same kernel after a launch that splits them
-            # (accuracy_level unset), or one (a level that allows f16 activations)
+            # (accuracy_level unset), one (a level that allows f16 activations) or three (level 1: f32 pinned)
             a32 = ctx.upload(pkg.synth.normal_f32(M * K, 41).reshape(M, K))
             y32 = ctx.alloc(4 * M * N)
-            for level, label in ((0, "matmul_nbits_f32_M512_"), (2, "matmul_nbits_f32_level2_M512_")):
+            for level, label in ((0, "matmul_nbits_f32_M512_"), (2, "matmul_nbits_f32_level2_M512_"), (1, "matmul_nbits_f32_level1_M512_")):
                 run32 = lambda: pkg.ops.matmul_nbits_packed_device(ctx, a32, pkg.F32, w, y32, M, level)  # noqa: E731,B023
                 run32()
                 ctx.flush()

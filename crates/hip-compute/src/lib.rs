@@ -431,7 +431,7 @@ impl HipContext {
         Ok(NBitsWeight { raw })
     }
     /// MatMulNBits on a prepacked weight: decode rows on the GEMV kernels, more than 16 rows of f16 on the
-    /// tiled matrix-core kernel. `accuracy_level` as in the operator (0..4, a lower bound: 1 keeps all 24 bits; many f32 rows travel as two f16 terms, one from level 2 on).
+    /// tiled matrix-core kernel. `accuracy_level` as in the operator (0..4, a lower bound: 1 keeps all 24 bits; many f32 rows travel as two f16 terms, three at level 1, one from level 2 on).
     pub fn matmul_nbits_packed(&self, a: BufferSlice<'_>, a_dtype: DType, w: &NBitsWeight, y: BufferSlice<'_>, m: i64, accuracy_level: i32) -> Result<()> {
         self.check(unsafe { sys::hipc_matmul_nbits_packed(self.raw, a.ptr(), a_dtype.raw(), w.raw, y.ptr(), m, accuracy_level as c_int) })
     }

@@ -192,7 +192,7 @@ size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w);
  * More than 16 rows of f16, or 32 of f32, run a tiled f16 matrix-core kernel; an f32 row travels
  * as f16 terms of the row times the power of two that puts its largest value into [2^14, 2^15):
  * two terms (22 bits) at level 0, one (11 bits of every value) at levels 2, 3 and 4, which allow
- * f16, bf16 or int8 activations; level 1 keeps the three-term route, 16 rows at a time.
+ * f16, bf16 or int8 activations, three (every bit of the row's values) at level 1.
  * The tiled kernel keeps its accumulators in units of the open quantisation block's scale: there a
  * scale of magnitude below 2^-64 counts as 2^-64 (what such a block adds is below
  * 2^-64 x 15 x sum |a|), and a column whose scales are all below it is stored as 0. */

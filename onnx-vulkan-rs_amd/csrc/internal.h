@@ -455,7 +455,7 @@ bool nbits_prefill_takes(const void *A, const hipc_nbits_weight *w, int64_t M);
 int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M);
 // f32 activations, more than 32 rows: the same kernel on two f16 rows per row (see matmul_nbits_prefill.hip)
 bool nbits_prefill_f32_takes(const void *A, const hipc_nbits_weight *w, int64_t M);
-int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M, int terms);   // f16 terms per f32 row: 2 (22 bits) or 1 (11)
+int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M, int terms);   // f16 terms per f32 row: 2 (22 bits), 1 (11) or 3 (all 24)
 
 // offsets inside ctx->params
 constexpr size_t kParamRange = 0;   // 8 B  {bits(-min), bits(max)}

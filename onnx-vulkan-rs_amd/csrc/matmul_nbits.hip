@@ -1188,10 +1188,10 @@ int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hi
         const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
         // many rows of f16: the tiled kernel reads the weight once per row tile instead of once per 16 rows
         if (a_dtype == HIPC_F16 && nbits_prefill_takes(A, w, M)) return nbits_prefill(ctx, A, w, Y, M);
-        // many rows of f32: two f16 rows each (22 bits) through the same kernel, or one (11 bits beside the row's own
-        // power of two) where the operator's attribute allows f16, bf16 or int8 activations; accuracy_level 1 (f32
-        // pinned: all 24 bits) keeps the decode kernel's three-term route
-        if (a_dtype == HIPC_F32 && NT == 2 && nbits_prefill_f32_takes(A, w, M)) return nbits_prefill_f32(ctx, A, w, Y, M, accuracy_level >= 2 ? 1 : 2);
+        // many rows of f32: two f16 rows each (22 bits) through the same kernel; one (11 bits beside the row's own
+        // power of two) where the operator's attribute allows f16, bf16 or int8 activations; three (all 24 bits) at
+        // accuracy_level 1, which pins f32
+        if (a_dtype == HIPC_F32 && nbits_prefill_f32_takes(A, w, M)) return nbits_prefill_f32(ctx, A, w, Y, M, NT == 3 ? 3 : accuracy_level >= 2 ? 1 : 2);
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int rows = (int)std::min<int64_t>(16, M - m0);
             int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,

@@ -932,7 +932,7 @@ int nbits_prefill(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void
 // are stored as A2[m] = hi, A2[M + m] = lo; one workgroup per row. PAIRED: 32 rows of high terms are followed by the
 // 32 rows of their low terms (row m: hi at 64 (m / 32) + m % 32, lo 32 rows on), the grid covers a multiple of 32
 // rows and the rows past M are zeros.
-template <bool PAIRED, bool LOW = true>   // LOW false: the high terms alone, M rows
+template <bool PAIRED, int TERMS = 2>   // TERMS 1: the high terms alone, M rows; 3: a third term (all 24 bits of the row's values), rows 2 M + m
 static __global__ void __launch_bounds__(256)
 mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half *__restrict__ A2, int *__restrict__ exps) {
     __shared__ float red[4];
@@ -971,29 +971,41 @@ mmnb_prefill_split_rows_kernel(const float *__restrict__ A, int M, int K, __half
     uint2 *hi_row = reinterpret_cast<uint2 *>(A2 + hi_at * K), *lo_row = reinterpret_cast<uint2 *>(A2 + lo_at * K);
     auto split4 = [&](const float4 &v, int c) {
         const float a[4] = {v.x * down, v.y * down, v.z * down, v.w * down};
-        __half hi[4], lo[4];
+        __half hi[4], lo[4], lo2[4];
 #pragma unroll
-        for (int t = 0; t < 4; t++) hi[t] = __float2half(a[t]), lo[t] = __float2half(a[t] - __half2float(hi[t]));
+        for (int t = 0; t < 4; t++) {
+            hi[t] = __float2half(a[t]);
+            const float r = a[t] - __half2float(hi[t]);   // (exact, like the next one)
+            lo[t] = __float2half(r);
+            lo2[t] = __float2half(r - __half2float(lo[t]));
+        }
         hi_row[c] = make_uint2(two_halves(hi[0], hi[1]), two_halves(hi[2], hi[3]));
-        if (LOW) lo_row[c] = make_uint2(two_halves(lo[0], lo[1]), two_halves(lo[2], lo[3]));
+        if (TERMS >= 2) lo_row[c] = make_uint2(two_halves(lo[0], lo[1]), two_halves(lo[2], lo[3]));
+        if (TERMS == 3) lo_row[c + (size_t)M * (K / 4)] = make_uint2(two_halves(lo2[0], lo2[1]), two_halves(lo2[2], lo2[3]));
     };
 #pragma unroll
     for (int u = 0; u < kHeld; u++)
         if (tid + 256 * u < nv) split4(held[u], tid + 256 * u);
     for (int c = tid + 256 * kHeld; c < nv; c += 256) split4(row[c], c);
 }
-// Y[m] = (P[m] + P[M + m]) 2^e[m]
+// Y[m] = (P[m] + P[M + m]) 2^e[m], or with three terms (P[m] + (P[M + m] + P[2 M + m])) 2^e[m]: the small ones first
 template <bool VEC>   // VEC: N is a multiple of four and Y is aligned for 16-byte stores
 static __global__ void __launch_bounds__(256)
-mmnb_prefill_join_rows_kernel(const float *__restrict__ P, const int *__restrict__ exps, int M, int N, float *__restrict__ Y) {
-    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * (VEC ? 4 : 1);
-    if (i >= (long)M * N) return;
+mmnb_prefill_join_rows_kernel(const float *__restrict__ P, const int *__restrict__ exps, int M, int N, float *__restrict__ Y, int terms) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * (VEC ? 4 : 1), plane = (long)M * N;
+    if (i >= plane) return;
     const int e = exps[(int)(i / N)];
     if (VEC) {
-        const float4 a = *reinterpret_cast<const float4 *>(P + i), b = *reinterpret_cast<const float4 *>(P + i + (long)M * N);
+        const float4 a = *reinterpret_cast<const float4 *>(P + i);
+        float4 b = *reinterpret_cast<const float4 *>(P + i + plane);
+        if (terms == 3) {
+            const float4 c = *reinterpret_cast<const float4 *>(P + i + 2 * plane);
+            b = make_float4(b.x + c.x, b.y + c.y, b.z + c.z, b.w + c.w);
+        }
         *reinterpret_cast<float4 *>(Y + i) = make_float4(ldexpf(a.x + b.x, e), ldexpf(a.y + b.y, e), ldexpf(a.z + b.z, e), ldexpf(a.w + b.w, e));
     } else {
-        Y[i] = ldexpf(P[i] + P[i + (long)M * N], e);
+        const float b = terms == 3 ? P[i + plane] + P[i + 2 * plane] : P[i + plane];
+        Y[i] = ldexpf(P[i] + b, e);
     }
 }
 
@@ -1003,7 +1015,7 @@ mmnb_prefill_join_rows_kernel(const float *__restrict__ P, const int *__restrict
 // puts the rows' powers of two back itself; the kernel that stages both operands through LDS writes 2 M rows of f32
 // results and a last launch adds the pairs.
 bool nbits_prefill_f32_takes(const void *A, const hipc_nbits_weight *w, int64_t M) {
-    return M > 32 && w->K % 8 == 0 && aligned(A, 16) && (2 * M + 64) * w->K < (int64_t(1) << 31) && 2 * M * w->N < (int64_t(1) << 31);
+    return M > 32 && w->K % 8 == 0 && aligned(A, 16) && (3 * M + 64) * w->K < (int64_t(1) << 31) && 3 * M * w->N < (int64_t(1) << 31);
 }
 
 int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, void *Y, int64_t M, int terms) {
@@ -1016,7 +1028,7 @@ int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, 
         if (int rc = scratch_get(ctx, 2, (size_t)M * w->K * sizeof(__half) + e_bytes, &split)) return rc;
         __half *A1 = reinterpret_cast<__half *>(static_cast<char *>(split) + e_bytes);
         int *exps = static_cast<int *>(split);
-        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<false, false>), dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A1, exps);
+        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<false, 1>), dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A1, exps);
         HIPC_LAUNCHED(ctx);
         PrefillArgs a{};
         a.A = A1, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = nullptr, a.Yf32 = static_cast<float *>(Y), a.exps = exps;
@@ -1027,19 +1039,23 @@ int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, 
             default: return prefill_launch<1>(ctx, a);
         }
     }
-    const bool paired = ctx->tune.prefill_direct != 0;
-    const int64_t rows2 = paired ? 64 * ceil_div(M, 32) : 2 * M;
+    // two terms: the pairs of the kernel that keeps the weight out of LDS; three (f32 pinned: all 24 bits), or the
+    // kernel with both operands in LDS: `terms` M rows, and a launch that adds them
+    const bool paired = terms == 2 && ctx->tune.prefill_direct != 0;
+    const int64_t rows2 = paired ? 64 * ceil_div(M, 32) : terms * M;
     const size_t a2_bytes = (size_t)rows2 * w->K * sizeof(__half), e_bytes = ((size_t)M * sizeof(int) + 255) & ~(size_t)255;
     void *split = nullptr, *sums = nullptr;
     if (int rc = scratch_get(ctx, 2, a2_bytes + e_bytes, &split)) return rc;
     if (!paired)
-        if (int rc = scratch_get(ctx, 3, (size_t)2 * M * w->N * sizeof(float), &sums)) return rc;
+        if (int rc = scratch_get(ctx, 3, (size_t)terms * M * w->N * sizeof(float), &sums)) return rc;
     __half *A2 = reinterpret_cast<__half *>(static_cast<char *>(split) + e_bytes);
     int *exps = static_cast<int *>(split);
     if (paired)
-        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<true, true>), dim3((unsigned)(rows2 / 2)), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
+        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<true, 2>), dim3((unsigned)(rows2 / 2)), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
+    else if (terms == 3)
+        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<false, 3>), dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
     else
-        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<false, true>), dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
+        hipLaunchKernelGGL((mmnb_prefill_split_rows_kernel<false, 2>), dim3((unsigned)M), dim3(256), 0, ctx->stream, static_cast<const float *>(A), (int)M, (int)w->K, A2, exps);
     HIPC_LAUNCHED(ctx);
     PrefillArgs a{};
     a.A = A2, a.Wq = w->Wq, a.Sc = w->Sc, a.Zb = w->Zb, a.Y = nullptr, a.Yf32 = static_cast<float *>(paired ? Y : sums);
@@ -1054,9 +1070,9 @@ int nbits_prefill_f32(hipc_ctx *ctx, const void *A, const hipc_nbits_weight *w, 
     if (rc != HIPC_OK || paired) return rc;
     const long total = (long)M * w->N;
     if (w->N % 4 == 0 && aligned(Y, 16))
-        hipLaunchKernelGGL((mmnb_prefill_join_rows_kernel<true>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, static_cast<const float *>(sums), exps, (int)M, (int)w->N, static_cast<float *>(Y));
+        hipLaunchKernelGGL((mmnb_prefill_join_rows_kernel<true>), dim3((unsigned)ceil_div(total, 1024)), dim3(256), 0, ctx->stream, static_cast<const float *>(sums), exps, (int)M, (int)w->N, static_cast<float *>(Y), terms);
     else
-        hipLaunchKernelGGL((mmnb_prefill_join_rows_kernel<false>), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream, static_cast<const float *>(sums), exps, (int)M, (int)w->N, static_cast<float *>(Y));
+        hipLaunchKernelGGL((mmnb_prefill_join_rows_kernel<false>), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream, static_cast<const float *>(sums), exps, (int)M, (int)w->N, static_cast<float *>(Y), terms);
     HIPC_LAUNCHED(ctx);
     return HIPC_OK;
 }

@@ -82,6 +82,8 @@ void product(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dt
         MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 0));
         // (f32 rows at a level that allows f16 activations: one term per row, the kernel scales the result's rows)
         if (a_dtype == HIPC_F32) MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 2));
+        // (and with f32 pinned: three terms per row, 3 M rows and the launch that adds them)
+        if (a_dtype == HIPC_F32) MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 1));
     }
     ctx.tune.prefill_tile = ctx.tune.prefill_direct = ctx.tune.prefill_split = ctx.tune.prefill_groups = -1;
     gpu_model::release(A), gpu_model::release(Y);

@@ -285,6 +285,37 @@ def test_f32_rows_at_a_level_that_allows_f16_activations(ctx, pkg, oracle, shape
     assert np.all(got[2] == 0)
 
 
+@pytest.mark.parametrize("options", [{}, {"HIPC_PREFILL_TILE": 128, "HIPC_PREFILL_SPLIT": 2}, {"HIPC_PREFILL_TILE": 192}, {"HIPC_PREFILL_DIRECT": 0}],
+                         ids=lambda v: str(v).replace(" ", ""))
+@pytest.mark.parametrize("shape", F32_PREFILL, ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_f32_rows_with_f32_pinned(ctx, pkg, oracle, shape, options):
+    """accuracy_level 1 pins f32: more than 32 rows travel as THREE f16 rows each (every bit of the row's values
+    beside its power of two) through the tiled kernel, and a launch adds the three results. Against the oracle at
+    the operator's tolerance; against the float64 product no worse than the default's two terms, and within what f32
+    accumulation leaves."""
+    m, k, n, bs, with_zp = shape
+    B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=45, with_zp=with_zp)
+    a = pkg.synth.normal_f32(m * k, 46).reshape(m, k)
+    a[0] *= np.float32(3.0e7)
+    a[1] *= np.float32(1.0e-9)
+    a[2] = 0
+    want = oracle.matmul_nbits(a, B, scales, zp, k, n, bs)
+    w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+    with ctx.options(**options):
+        got = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, accuracy_level=1, weight=w)
+        two = pkg.ops.matmul_nbits(ctx, a, None, None, None, k, n, bs, weight=w)
+    w.destroy()
+    scale = np.maximum(np.abs(want).max(axis=1, keepdims=True), 1e-30)
+    assert np.all(np.abs(got - want) <= (1e-3 + 1e-4 * np.abs(want)) * np.maximum(scale / np.abs(want[3:]).max(), 1e-30) + 1e-4 * scale), worst(got, want)
+    nib, z = _unpack(B, zp if zp is not None else np.full((n, (-(-k // bs) + 1) // 2), 0x88, np.uint8), k, n, bs)
+    f64 = rc.matmul_nbits_f64(a, nib, z, scales.reshape(n, -1), bs)
+    big = np.maximum(np.abs(f64).max(axis=1, keepdims=True), 1e-300)
+    e3, e2 = np.abs(got - f64) / big, np.abs(two - f64) / big
+    assert e3.max() <= 2e-5, float(e3.max())
+    assert e3.max() <= e2.max() * 1.05 + 1e-7, (float(e3.max()), float(e2.max()))
+    assert np.all(got[2] == 0)
+
+
 @pytest.mark.parametrize("kn", [(2048, 11008), (11008, 2048), (2048, 2560)], ids=lambda s: "K%d_N%d" % s)
 def test_prefill_configuration_full_size(ctx, pkg, oracle, kn):
     """512 rows of f16 activations against block-128 symmetric weights with f16 scales (no zero
