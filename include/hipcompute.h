@@ -167,6 +167,10 @@ int hipc_probe_int8_mfma(hipc_ctx *ctx, int random_operands, int waves_per_simd,
  * computes every level in f32): see hipc_matmul_nbits_packed for what each level gets here.
  * Buffer lengths are in elements and are checked against K, N and block_size
  * as the reference does (interp.rs:6455-6472); M*N == 0 is a no-op.
+ * With more rows than the decode kernels take (16 of f16, 32 of f32) and a block_size that has a
+ * tiled form, the call first writes that form into the context's scratch memory and then runs the
+ * kernels of hipc_matmul_nbits_packed (the same results as a handle gives, bit for bit); a weight
+ * that is used again is better prepacked once.
  */
 int hipc_matmul_nbits(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, size_t b_len,
                       const void *scales, int scale_dtype, size_t scales_len, const void *zp,

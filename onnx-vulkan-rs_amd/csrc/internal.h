@@ -37,7 +37,7 @@
 
 namespace hipc {
 
-constexpr int kScratchSlots = 4;
+constexpr int kScratchSlots = 5;
 
 // grow-only device scratch reused by operators that need a temporary (packed
 // B of a raw call, the i32 accumulator of a QLinear op). One in-order stream

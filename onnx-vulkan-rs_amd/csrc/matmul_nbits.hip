@@ -1013,6 +1013,12 @@ int launch_gemv(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weig
 
 }  // namespace
 
+namespace {
+int packed_run(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int64_t M, int accuracy_level);
+int tiled_from_onnx_layout(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, const void *scales, int scale_dtype, const void *zp, void *Y,
+                           int64_t M, int64_t K, int64_t N, int64_t block_size, int accuracy_level, bool *taken);
+}  // namespace
+
 extern "C" {
 
 int hipc_matmul_nbits(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, size_t b_len, const void *scales,
@@ -1029,6 +1035,11 @@ int hipc_matmul_nbits(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, 
         HIPC_REQUIRE(ctx, A && B && scales && Y, "MatMulNBits: null operand");
         HIPC_REQUIRE(ctx, aligned(B, 4), "MatMulNBits: packed weight must be 4-byte aligned");
         const bool af16 = a_dtype == HIPC_F16, sf16 = scale_dtype == HIPC_F16;
+        // many rows: the tiled form of the weight written to scratch memory first, then the matrix-core kernels
+        // (this kernel reads the whole weight once per four rows)
+        bool taken = false;
+        rc = tiled_from_onnx_layout(ctx, A, a_dtype, B, scales, scale_dtype, zp, Y, M, K, N, block_size, accuracy_level, &taken);
+        if (taken) return rc;
         if (af16 && sf16) return launch_direct<__half, __half>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
         if (af16) return launch_direct<__half, float>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
         if (sf16) return launch_direct<float, __half>(ctx, A, B, scales, zp, Y, M, K, N, block_size);
@@ -1046,6 +1057,39 @@ int hipc_prepack_matmul_nbits(hipc_ctx *ctx, const void *B, size_t b_len, const 
 }
 
 }  // extern "C"
+
+namespace {
+
+// tile counts and scale grouping of the tiled form of a weight (K, N, block_size set; block_size a power of two >= 32), and
+// the bytes of its three arrays
+void tiled_geometry(hipc_nbits_weight *w, size_t *wq_bytes, size_t *sc_bytes, size_t *zb_bytes) {
+    const int n_chunks = (int)ceil_div(w->K, 32);
+    w->n_tiles = (int)ceil_div(w->N, 16);
+    w->n_cg = (int)ceil_div(n_chunks, 4);
+    const int cpb = (int)(w->block_size / 32);
+    w->SG = cpb >= 4 ? 1 : 4 / cpb;
+    const size_t tiles = (size_t)w->n_tiles * w->n_cg;
+    *wq_bytes = tiles * 1024, *sc_bytes = tiles * 16 * w->SG * 4, *zb_bytes = tiles * 16 * w->SG;
+}
+// the launch that writes the tiled form from the operator's tensors (device pointers)
+hipError_t tiled_fill(hipc_ctx *ctx, const hipc_nbits_weight *w, const void *B, const void *scales, int scale_dtype, const void *zp) {
+    const int n_blocks = (int)ceil_div(w->K, w->block_size);
+    const int cpb = (int)(w->block_size / 32);
+    const size_t tiles = (size_t)w->n_tiles * w->n_cg;
+    const int row_words = (int)(n_blocks * w->block_size / 8);
+    const int zp_row = (n_blocks + 1) / 2;
+    const long threads = (long)tiles * 64;
+    const dim3 grid((unsigned)ceil_div(threads, 256)), block(256);
+    if (scale_dtype == HIPC_F16)
+        hipLaunchKernelGGL((mmnb_prepack_kernel<__half>), grid, block, 0, ctx->stream, static_cast<const uint32_t *>(B), static_cast<const __half *>(scales), static_cast<const uint8_t *>(zp),
+            w->Wq, w->Sc, w->Zb, (int)w->N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, w->interleave_half);
+    else
+        hipLaunchKernelGGL((mmnb_prepack_kernel<float>), grid, block, 0, ctx->stream, static_cast<const uint32_t *>(B), static_cast<const float *>(scales), static_cast<const uint8_t *>(zp),
+            w->Wq, w->Sc, w->Zb, (int)w->N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, w->interleave_half);
+    return hipGetLastError();
+}
+
+}  // namespace
 
 // The same operations for callers inside the library that already hold the context's lock.
 int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *scales, int scale_dtype,
@@ -1089,14 +1133,8 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
         return HIPC_OK;
     }
     w->interleave_half = interleave_half;
-    const int n_blocks = (int)ceil_div(K, block_size);
-    const int n_chunks = (int)ceil_div(K, 32);
-    w->n_tiles = (int)ceil_div(N, 16);
-    w->n_cg = (int)ceil_div(n_chunks, 4);
-    const int cpb = (int)(block_size / 32);
-    w->SG = cpb >= 4 ? 1 : 4 / cpb;
-    const size_t tiles = (size_t)w->n_tiles * w->n_cg;
-    const size_t wq_bytes = tiles * 1024, sc_bytes = tiles * 16 * w->SG * 4, zb_bytes = tiles * 16 * w->SG;
+    size_t wq_bytes, sc_bytes, zb_bytes;
+    tiled_geometry(w, &wq_bytes, &sc_bytes, &zb_bytes);
     if (wq_bytes >= (size_t(1) << 32)) {
         delete w;
         return fail(ctx, HIPC_ERR_UNSUPPORTED, "MatMulNBits prepack: a %zu-byte weight exceeds the 4 GiB the kernel addresses", wq_bytes);
@@ -1115,17 +1153,7 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
         return fail(ctx, HIPC_ERR_BACKEND, "MatMulNBits prepack: %s", hipGetErrorString(e));
     }
     w->bytes = wq_bytes + sc_bytes + zb_bytes;
-    const int row_words = (int)(n_blocks * block_size / 8);
-    const int zp_row = (n_blocks + 1) / 2;
-    const long threads = (long)tiles * 64;
-    const dim3 grid((unsigned)ceil_div(threads, 256)), block(256);
-    if (scale_dtype == HIPC_F16)
-        hipLaunchKernelGGL((mmnb_prepack_kernel<__half>), grid, block, 0, ctx->stream, static_cast<const uint32_t *>(B), static_cast<const __half *>(scales), static_cast<const uint8_t *>(zp),
-            w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, interleave_half);
-    else
-        hipLaunchKernelGGL((mmnb_prepack_kernel<float>), grid, block, 0, ctx->stream, static_cast<const uint32_t *>(B), static_cast<const float *>(scales), static_cast<const uint8_t *>(zp),
-            w->Wq, w->Sc, w->Zb, (int)N, n_blocks, row_words, zp_row, (long)tiles, w->n_cg, log2i(cpb), w->SG, interleave_half);
-    e = hipGetLastError();
+    e = tiled_fill(ctx, w, B, scales, scale_dtype, zp);
     if (e != hipSuccess) {
         cleanup();
         return fail(ctx, HIPC_ERR_BACKEND, "MatMulNBits prepack launch: %s", hipGetErrorString(e));
@@ -1166,40 +1194,72 @@ size_t hipc_nbits_weight_bytes(const hipc_nbits_weight *w) { return w ? w->bytes
 
 int hipc_matmul_nbits_packed(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int64_t M,
                              int accuracy_level) {
-    return entry(ctx, [&]() -> int {
-        HIPC_REQUIRE(ctx, w, "MatMulNBits: null weight");
-        HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
-        // (the attribute is a lower bound on what the activations may be reduced to; the reference never reads it and
-        // computes every level in f32. Level 4 allows int8 activations: two bf16 terms are more than it asks for.)
-        HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 4, "MatMulNBits: accuracy_level %d is not one of 0..4", accuracy_level);
-        HIPC_REQUIRE(ctx, M >= 0 && M < (int64_t(1) << 30), "MatMulNBits: bad M=%ld", (long)M);
-        if (M == 0) return HIPC_OK;
-        HIPC_REQUIRE(ctx, A && Y, "MatMulNBits: null operand");
-        if (!w->Wq) {   // a handle in the operator's own layout (block_size below 32 or not a power of two)
-            const bool af16 = a_dtype == HIPC_F16, sf16 = w->raw_scale_dtype == HIPC_F16;
-            if (af16 && sf16) return launch_direct<__half, __half>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
-            if (af16) return launch_direct<__half, float>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
-            if (sf16) return launch_direct<float, __half>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
-            return launch_direct<float, float>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
-        }
-        const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
-        // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
-        // terms). Unset, or 2 / 3 / 4 (f16 / bf16 / int8 are enough): 2 terms. f16 activations are exact in 2.
-        const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
-        // many rows of f16: the tiled kernel reads the weight once per row tile instead of once per 16 rows
-        if (a_dtype == HIPC_F16 && nbits_prefill_takes(A, w, M)) return nbits_prefill(ctx, A, w, Y, M);
-        // many rows of f32: two f16 rows each (22 bits) through the same kernel; one (11 bits beside the row's own
-        // power of two) where the operator's attribute allows f16, bf16 or int8 activations; three (all 24 bits) at
-        // accuracy_level 1, which pins f32
-        if (a_dtype == HIPC_F32 && nbits_prefill_f32_takes(A, w, M)) return nbits_prefill_f32(ctx, A, w, Y, M, NT == 3 ? 3 : accuracy_level >= 2 ? 1 : 2);
-        for (int64_t m0 = 0; m0 < M; m0 += 16) {
-            const int rows = (int)std::min<int64_t>(16, M - m0);
-            int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,
-                                 static_cast<char *>(Y) + (size_t)m0 * w->N * esz, rows, NT);
-            if (rc != HIPC_OK) return rc;
-        }
-        return HIPC_OK;
-    });
+    return entry(ctx, [&]() -> int { return packed_run(ctx, A, a_dtype, w, Y, M, accuracy_level); });
 }
 
 }  // extern "C"
+
+namespace {
+
+int packed_run(hipc_ctx *ctx, const void *A, int a_dtype, const hipc_nbits_weight *w, void *Y, int64_t M, int accuracy_level) {
+    HIPC_REQUIRE(ctx, w, "MatMulNBits: null weight");
+    HIPC_REFUSE(ctx, a_dtype != HIPC_F32 && a_dtype != HIPC_F16, "MatMulNBits: A must be f32 or f16, got %d", a_dtype);
+    // (the attribute is a lower bound on what the activations may be reduced to; the reference never reads it and
+    // computes every level in f32. Level 4 allows int8 activations: two bf16 terms are more than it asks for.)
+    HIPC_REFUSE(ctx, accuracy_level < 0 || accuracy_level > 4, "MatMulNBits: accuracy_level %d is not one of 0..4", accuracy_level);
+    HIPC_REQUIRE(ctx, M >= 0 && M < (int64_t(1) << 30), "MatMulNBits: bad M=%ld", (long)M);
+    if (M == 0) return HIPC_OK;
+    HIPC_REQUIRE(ctx, A && Y, "MatMulNBits: null operand");
+    if (!w->Wq) {   // a handle in the operator's own layout (block_size below 32 or not a power of two)
+        const bool af16 = a_dtype == HIPC_F16, sf16 = w->raw_scale_dtype == HIPC_F16;
+        if (af16 && sf16) return launch_direct<__half, __half>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+        if (af16) return launch_direct<__half, float>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+        if (sf16) return launch_direct<float, __half>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+        return launch_direct<float, float>(ctx, A, w->raw_B, w->raw_scales, w->raw_zp, Y, M, w->K, w->N, w->block_size);
+    }
+    const size_t esz = a_dtype == HIPC_F16 ? 2 : 4;
+    // accuracy_level 1 pins f32 activations: all 24 bits go through the matrix cores (3 bf16
+    // terms). Unset, or 2 / 3 / 4 (f16 / bf16 / int8 are enough): 2 terms. f16 activations are exact in 2.
+    const int NT = (accuracy_level == 1 && a_dtype == HIPC_F32) ? 3 : 2;
+    // many rows of f16: the tiled kernel reads the weight once per row tile instead of once per 16 rows
+    if (a_dtype == HIPC_F16 && nbits_prefill_takes(A, w, M)) return nbits_prefill(ctx, A, w, Y, M);
+    // many rows of f32: two f16 rows each (22 bits) through the same kernel; one (11 bits beside the row's own
+    // power of two) where the operator's attribute allows f16, bf16 or int8 activations; three (all 24 bits) at
+    // accuracy_level 1, which pins f32
+    if (a_dtype == HIPC_F32 && nbits_prefill_f32_takes(A, w, M)) return nbits_prefill_f32(ctx, A, w, Y, M, NT == 3 ? 3 : accuracy_level >= 2 ? 1 : 2);
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+        const int rows = (int)std::min<int64_t>(16, M - m0);
+        int rc = launch_gemv(ctx, static_cast<const char *>(A) + (size_t)m0 * w->K * esz, a_dtype, w,
+                             static_cast<char *>(Y) + (size_t)m0 * w->N * esz, rows, NT);
+        if (rc != HIPC_OK) return rc;
+    }
+    return HIPC_OK;
+}
+
+// hipc_matmul_nbits with more rows than the decode kernels take, on a block size that has a tiled form: the tiled
+// arrays are written into scratch memory (they live until the next call of this kind on the stream) and the product
+// runs as on a prepacked handle. *taken is false where the shape stays on the kernel that reads the ONNX layout.
+int tiled_from_onnx_layout(hipc_ctx *ctx, const void *A, int a_dtype, const void *B, const void *scales, int scale_dtype, const void *zp, void *Y,
+                           int64_t M, int64_t K, int64_t N, int64_t block_size, int accuracy_level, bool *taken) {
+    *taken = false;
+    if (block_size < 32 || !is_pow2(block_size)) return HIPC_OK;
+    hipc_nbits_weight w;
+    w.K = K, w.N = N, w.block_size = block_size;
+    size_t wq_bytes, sc_bytes, zb_bytes;
+    tiled_geometry(&w, &wq_bytes, &sc_bytes, &zb_bytes);
+    if (wq_bytes >= (size_t(1) << 32)) return HIPC_OK;
+    // only where a tiled kernel will take the rows (otherwise sixteen rows at a time on the decode kernel: no gain)
+    const bool many = a_dtype == HIPC_F16 ? nbits_prefill_takes(A, &w, M) : nbits_prefill_f32_takes(A, &w, M);
+    if (!many) return HIPC_OK;
+    *taken = true;
+    const size_t wq_r = (wq_bytes + 255) & ~(size_t)255, sc_r = (sc_bytes + 255) & ~(size_t)255;
+    void *block = nullptr;
+    if (int rc = scratch_get(ctx, 4, wq_r + sc_r + zb_bytes, &block)) return rc;
+    w.Wq = static_cast<uint4 *>(block);
+    w.Sc = reinterpret_cast<float *>(static_cast<char *>(block) + wq_r);
+    w.Zb = reinterpret_cast<uint8_t *>(block) + wq_r + sc_r;
+    HIPC_TRY(ctx, tiled_fill(ctx, &w, B, scales, scale_dtype, zp));
+    return packed_run(ctx, A, a_dtype, &w, Y, M, accuracy_level);
+}
+
+}  // namespace

@@ -86,6 +86,9 @@ void product(int64_t M, int64_t K, int64_t N, int64_t bs, bool with_zp, int a_dt
         if (a_dtype == HIPC_F32) MUST(hipc_matmul_nbits_packed(&ctx, A, a_dtype, w, Y, M, 1));
     }
     ctx.tune.prefill_tile = ctx.tune.prefill_direct = ctx.tune.prefill_split = ctx.tune.prefill_groups = -1;
+    // the operator on the ONNX layout with this many rows: the tiled form goes to scratch memory first
+    gpu_model::reg().where = "many rows on the ONNX layout";
+    MUST(hipc_matmul_nbits(&ctx, A, a_dtype, B.data(), b_len, S.data(), a_dtype, s_len, with_zp ? Z.data() : nullptr, with_zp ? z_len : 0, Y, M, K, N, bs, 0));
     gpu_model::release(A), gpu_model::release(Y);
     hipc_nbits_weight_destroy(&ctx, w);
     for (void *p : ctx.deferred) gpu_model::release(p);

@@ -208,6 +208,25 @@ def test_block_scales_of_zero_and_of_very_different_size(ctx, pkg, oracle, bs, d
         assert np.all(err <= 2e-5 * big + 1e-3), float((err / big).max())
 
 
+@pytest.mark.parametrize("shape", [(100, 1000, 200, 32, True), (257, 640, 96, 128, False)], ids=lambda s: "M%d_K%d_N%d_bs%d_zp%d" % s)
+def test_many_rows_on_the_onnx_layout_take_the_tiled_kernels(ctx, pkg, oracle, shape):
+    """hipc_matmul_nbits (the reference's own calling convention: the ONNX tensors on every call) with more rows
+    than the decode kernels take writes the tiled form into scratch memory and runs the kernels of the prepacked
+    path: the same bits as a handle gives, f16 and f32 rows, twice in a row with different weights (the scratch
+    block is reused)."""
+    m, k, n, bs, with_zp = shape
+    for seed, dtype in ((61, np.float32), (62, np.float16), (63, np.float32)):   # (scales in the activations' type, as the operator has them)
+        B, scales, zp = pkg.synth.nbits_weight(n, k, bs, seed=seed, with_zp=with_zp, scale_dtype=dtype)
+        rows = pkg.synth.normal_f32(m * k, seed + 10).reshape(m, k).astype(dtype)
+        w = pkg.ops.NBitsWeight(ctx, B, scales, zp, k, n, bs)
+        got = pkg.ops.matmul_nbits(ctx, rows, B, scales, zp, k, n, bs)
+        by_handle = pkg.ops.matmul_nbits(ctx, rows, None, None, None, k, n, bs, weight=w)
+        w.destroy()
+        assert got.dtype == dtype and np.array_equal(got, by_handle)
+        want = oracle.matmul_nbits(rows, B, scales, zp, k, n, bs)
+        assert close(got, want, RTOL32 if dtype == np.float32 else RTOL16), worst(got, want)
+
+
 F32_PREFILL = [  # (M, K, N, block_size, zero points)
     (100, 1000, 200, 32, True), (130, 384, 131, 64, True), (257, 640, 96, 128, False), (33, 72, 16, 32, True),
     (512, 2048, 2560, 128, False),
