@@ -1120,13 +1120,13 @@ int hipc::nbits_prepack(hipc_ctx *ctx, const void *B, size_t b_len, const void *
             e = hipMalloc(to[i], (sizes[i] + 3) & ~(size_t)3);
             if (e == hipSuccess) e = hipMemcpyAsync(*to[i], from[i], sizes[i], hipMemcpyDeviceToDevice, ctx->stream);
         }
+        if (e == hipSuccess) e = hipGetLastError();
         if (e != hipSuccess) {
             for (int i = 0; i < 3; i++)
                 if (*to[i]) (void)hipFree(*to[i]);
             delete w;
             return fail(ctx, HIPC_ERR_BACKEND, "MatMulNBits prepack: %s", hipGetErrorString(e));
         }
-        HIPC_LAUNCHED(ctx);
         w->raw_scale_dtype = scale_dtype;
         w->bytes = sizes[0] + sizes[1] + sizes[2];
         *out = w;
